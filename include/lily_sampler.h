@@ -1,0 +1,234 @@
+/*
+ * lily_sampler.h - C ABI of the MI355X logits-to-token stage (liblily_sampler_hip.so).
+ *
+ * Every entry point states the reference interface it stands in for (paths relative
+ * to the reference checkout).  The reference encodes work into a Metal pass and runs
+ * it at commit; here every draw is ENQUEUED on the HIP stream the sampler was created
+ * on and returns at once.  Results appear in the device buffers in stream order; the
+ * caller synchronises the stream (or calls lily_sampler_synchronize) before reading.
+ * Nothing here allocates on the draw calls, reads device memory on the host, or
+ * synchronises, except where a function says so.
+ *
+ * Pointers named *_dev are device pointers borrowed for the duration of the enqueued
+ * work (the reference's "a pass holds buffers by address only").  A sampler and the
+ * objects made from it belong to one host thread at a time.
+ *
+ * Return value: 0 on success, a negative lily_status otherwise; lily_last_error()
+ * returns the message of the calling thread's last failure.
+ */
+#ifndef LILY_SAMPLER_H
+#define LILY_SAMPLER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LILY_SAMPLE_K_CAP 1024u          /* src/kernels/sample.rs:17 SAMPLE_K_CAP */
+#define LILY_CTRL_STRIDE 4u              /* src/kernels/spec.rs:15 CTRL_STRIDE */
+#define LILY_SLOT_ACCEPTED 0u            /* src/kernels/spec.rs:18 */
+#define LILY_SLOT_KEEP 1u                /* src/kernels/spec.rs:20 */
+#define LILY_NO_TOKEN 0xFFFFFFFFu        /* "no forced token" in lily_rows.forced */
+#define LILY_MAX_VERIFY_ROWS 8u
+
+typedef enum lily_status {
+    LILY_OK = 0,
+    LILY_ERR_INVALID_ARG = -1, /* null/misaligned pointer, zero size, bad enum */
+    LILY_ERR_PARAMS = -2,      /* SamplingParams::validate failed (sample.rs:57-79) */
+    LILY_ERR_VOCAB = -3,       /* scratch sized for a different vocabulary (sample.rs:264) */
+    LILY_ERR_HIP = -4,         /* a HIP runtime call failed; message holds hipGetErrorString */
+    LILY_ERR_NOMEM = -5,
+    LILY_ERR_RANGE = -6        /* index or size beyond a stated limit */
+} lily_status;
+
+typedef enum lily_dtype { LILY_F32 = 0, LILY_BF16 = 1 } lily_dtype;
+
+/* src/kernels/sample.rs:21-31 SamplingParams, field for field (top_k as u32). */
+typedef struct lily_sampling_params {
+    float temperature;        /* 0 = greedy */
+    uint32_t top_k;           /* 0 = off (capped at LILY_SAMPLE_K_CAP) */
+    float top_p;
+    float min_p;
+    float presence_penalty;
+    float frequency_penalty;
+    float repetition_penalty;
+    uint32_t reserved;        /* must be 0 */
+    uint64_t seed;
+} lily_sampling_params;
+
+typedef struct lily_bias {
+    uint32_t id;
+    float delta;
+} lily_bias;
+
+typedef struct lily_sampler lily_sampler_t;         /* MetalContext + ComputePass of the path */
+typedef struct lily_scratch lily_scratch_t;         /* src/kernels/sample.rs:116-128 SamplerScratch */
+typedef struct lily_draft_dists lily_draft_dists_t; /* src/kernels/sample.rs:186-190 DraftDists */
+
+/* src/kernels/sample.rs:193-197 DraftDist: one slot's device arrays. */
+typedef struct lily_draft_dist {
+    uint32_t* ids_dev;   /* [LILY_SAMPLE_K_CAP] kept ids, best first */
+    float* probs_dev;    /* [LILY_SAMPLE_K_CAP] probabilities over the kept mass */
+    uint32_t* count_dev; /* [1] kept count */
+} lily_draft_dist;
+
+const char* lily_last_error(void);
+
+/* ---- pure host helpers (no GPU) ---------------------------------------------------- */
+
+/* src/kernels/sample.rs:34-45 SamplingParams::greedy() */
+void lily_params_greedy(lily_sampling_params* out);
+/* src/kernels/sample.rs:47-49 is_greedy */
+int lily_params_is_greedy(const lily_sampling_params* p);
+/* src/kernels/sample.rs:51-55 uses_penalties */
+int lily_params_uses_penalties(const lily_sampling_params* p);
+/* src/kernels/sample.rs:57-79 validate: LILY_OK or LILY_ERR_PARAMS with the rule's message */
+int lily_params_validate(const lily_sampling_params* p);
+/* src/kernels/sample.rs:83-94 effective: the temperature and candidate count the kernel uses */
+void lily_params_effective(const lily_sampling_params* p, float* temperature, uint32_t* top_k);
+/* src/kernels/sample.rs:227-234 draft_params */
+void lily_draft_params(const lily_sampling_params* p, lily_sampling_params* out);
+/* src/kernels/sample.rs:220-222 draft_step */
+uint32_t lily_draft_step(uint32_t step);
+/* src/kernels/sample.rs:435-441 uniform_for */
+float lily_uniform_for(uint64_t seed, uint32_t step);
+/* src/kernels/spec.rs:23-40 slot_pos / slot_block / slot_count / ctrl_words */
+uint32_t lily_slot_pos(uint32_t i);
+uint32_t lily_slot_block(uint32_t i);
+uint32_t lily_slot_count(uint32_t i);
+uint32_t lily_ctrl_words(uint32_t chain);
+
+/* ---- sampler (context) --------------------------------------------------------------- */
+
+/* MetalContext::new + ctx.begin (src/metal.rs:400, :618): binds `device` and an existing
+ * hipStream_t (`hip_stream`; NULL = the device's default stream).  Allocates the
+ * workspace the multi-workgroup rows use.  Fails loudly if no HIP device is present. */
+int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out);
+void lily_sampler_destroy(lily_sampler_t* s);
+/* ComputePass::commit_wait (src/metal.rs:2290): blocks until the stream has drained. */
+int lily_sampler_synchronize(lily_sampler_t* s);
+
+/* ---- SamplerScratch ------------------------------------------------------------------- */
+
+/* SamplerScratch::new (sample.rs:131-143).  Device state: the emission histogram
+ * counts[vocab] and a vocab-bit map of the ids whose count is non-zero. */
+int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out);
+void lily_scratch_destroy(lily_scratch_t* sc);
+/* SamplerScratch::vocab (sample.rs:176-178) */
+uint32_t lily_scratch_vocab(const lily_scratch_t* sc);
+/* SamplerScratch::reset_counts (sample.rs:161-163); stream-ordered. */
+int lily_scratch_reset_counts(lily_scratch_t* sc);
+/* SamplerScratch::uncount (sample.rs:147-157): saturating, out-of-range ignored; stream-ordered. */
+int lily_scratch_uncount(lily_scratch_t* sc, uint32_t token);
+/* SamplerScratch::copy_counts_from (sample.rs:168-174): LILY_ERR_VOCAB on a size mismatch. */
+int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src);
+/* No counterpart in the reference (its histogram only ever grows by the kernel's own
+ * draws): counts[id] += multiplicity of id in ids_dev[0..n); ids >= vocab are ignored. */
+int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32_t n);
+/* scratch.counts.write_bytes / to_u32 as the reference's tests use them
+ * (tests/unit/kernels/sample.rs:66,166): host <-> device copies; both synchronise. */
+int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts);
+int lily_scratch_read_counts(lily_scratch_t* sc, uint32_t* host_counts);
+
+/* ---- DraftDists ----------------------------------------------------------------------- */
+
+/* DraftDists::new (sample.rs:200-206) / slot (sample.rs:208-214) */
+int lily_draft_dists_create(lily_sampler_t* s, uint32_t slots, lily_draft_dists_t** out);
+void lily_draft_dists_destroy(lily_draft_dists_t* d);
+int lily_draft_dists_slot(const lily_draft_dists_t* d, uint32_t i, lily_draft_dist* out);
+
+/* ---- single-row draws (the reference's call signature) --------------------------------- */
+
+/* sample_f32 (sample.rs:373-387): one draw from logits_dev[vocab] into out_dev[0].
+ * Greedy without penalties is the exact first-max argmax; otherwise penalties,
+ * temperature, top-k, top-p/min-p and the inverse-CDF draw on uniform_for(seed, step).
+ * Under penalties counts[out] += 1.  `scratch` may be NULL when params use no penalties. */
+int lily_sample_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                    lily_scratch_t* scratch, const lily_sampling_params* params, uint32_t step,
+                    uint32_t* out_dev);
+/* sample_draft_f32 (sample.rs:394-408): as lily_sample_f32, and the kept distribution
+ * goes to `dist`.  Greedy exports nothing. */
+int lily_sample_draft_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                          lily_scratch_t* scratch, const lily_sampling_params* params,
+                          uint32_t step, uint32_t* out_dev, const lily_draft_dist* dist);
+/* sample_spec_f32 (sample.rs:417-432): speculative draw against `dist` and the proposal
+ * draft_dev[0]; greedy is the plain argmax. */
+int lily_sample_spec_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                         lily_scratch_t* scratch, const lily_sampling_params* params,
+                         uint32_t step, const lily_draft_dist* dist, const uint32_t* draft_dev,
+                         uint32_t* out_dev);
+/* argmax_f32 (src/kernels/elementwise.rs:297-308): first max, lowest index on ties. */
+int lily_argmax_f32(lily_sampler_t* s, const float* x_dev, uint32_t n, uint32_t* out_dev);
+
+/* ---- speculative control --------------------------------------------------------------- */
+
+/* spec_accept (src/kernels/spec.rs:52-91): a = leading draws[a] == ids[a+1]; writes the
+ * control block (slots LILY_CTRL_STRIDE words apart). */
+int lily_spec_accept(lily_sampler_t* s, const uint32_t* draws_dev, const uint32_t* ids_dev,
+                     uint32_t m, uint32_t* ctrl_dev, uint32_t ctrl_words, uint32_t pos0,
+                     uint32_t ratio, uint32_t chain);
+/* copy_row (src/kernels/spec.rs:96-127) with a GPU-supplied row index: dst[0..words) =
+ * src[row_dev[0]][0..words); copies nothing when the index is >= rows. */
+int lily_copy_row_u32(lily_sampler_t* s, const uint32_t* src_dev, uint32_t rows, uint32_t words,
+                      const uint32_t* row_dev, uint32_t* dst_dev);
+/* The verify pass's draws (src/qwen4exp/model.rs:3008-3040) followed by spec_accept
+ * (src/qwen4exp/spec.rs:414-424): rows j < m-1 are speculative draws against dists slot j
+ * and proposal ids_dev[j+1] at step0+j, the last row a plain draw; row j sees the counts
+ * of rows before it.  verify_tokens_dev[m] receives the draws, ctrl_dev the control block. */
+int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype, uint32_t vocab,
+                     uint64_t row_stride, uint32_t m, lily_scratch_t* scratch,
+                     const lily_sampling_params* params, uint32_t step0,
+                     const lily_draft_dists_t* dists, const uint32_t* ids_dev,
+                     uint32_t* verify_tokens_dev, uint32_t* ctrl_dev, uint32_t ctrl_words,
+                     uint32_t pos0, uint32_t ratio, uint32_t chain);
+
+/* ---- batched rows ---------------------------------------------------------------------- */
+
+/* The per-row draw loop of a batched step (src/qwen4exp/batch.rs:583-593) as ONE launch:
+ * row r draws from logits + r*row_stride with params[r], steps[r] and scratch[r].
+ * Host arrays are read during the call; device arrays are borrowed until the work ran.
+ * Beyond the reference: bf16 logits, a per-row allow-bitmask, a per-row logit-bias list,
+ * a forced token, an explicit uniform and the chosen token's log-probability. */
+typedef struct lily_rows {
+    uint32_t rows;
+    uint32_t vocab;
+    uint32_t dtype;                      /* lily_dtype */
+    uint32_t reserved;                   /* must be 0 */
+    const void* logits_dev;              /* [rows][row_stride] */
+    uint64_t row_stride;                 /* elements between rows */
+    const lily_sampling_params* params;  /* host [rows] */
+    const uint32_t* steps;               /* host [rows] */
+    lily_scratch_t* const* scratch;      /* host [rows] or NULL; entries may be NULL; no
+                                            scratch may appear twice in one call */
+    const uint32_t* allow_dev;           /* packed bits, bit id&31 of word id>>5, or NULL */
+    uint64_t allow_stride;               /* words between rows; 0 = one mask for all rows */
+    const lily_bias* bias_dev;           /* concatenated per-row lists or NULL */
+    const uint32_t* bias_offsets;        /* host [rows+1] into bias_dev */
+    const uint32_t* forced;              /* host [rows] or NULL; LILY_NO_TOKEN = draw */
+    const float* uniforms;               /* host [rows] or NULL; NaN = uniform_for(seed, step) */
+    uint32_t* out_ids_dev;               /* [rows] */
+    float* out_logprobs_dev;             /* [rows] or NULL */
+    /* diagnostics, any may be NULL: the sorted top-k candidates before truncation */
+    uint32_t* dbg_ids_dev;               /* [rows][LILY_SAMPLE_K_CAP] */
+    float* dbg_probs_dev;                /* [rows][LILY_SAMPLE_K_CAP] exp(adjusted - top) */
+    uint32_t* dbg_counts_dev;            /* [rows][2] = candidates, kept */
+} lily_rows;
+
+int lily_sample_rows(lily_sampler_t* s, const lily_rows* batch);
+
+/* A resident batch: the row table is packed and uploaded once (lily_plan_set, which
+ * synchronises) and each lily_plan_run is a single launch with steps[r] + step_delta.
+ * No counterpart in the reference, whose encode call re-sends its constants per draw. */
+typedef struct lily_plan lily_plan_t;
+int lily_plan_create(lily_sampler_t* s, uint32_t max_rows, lily_plan_t** out);
+void lily_plan_destroy(lily_plan_t* p);
+int lily_plan_set(lily_plan_t* p, const lily_rows* batch);
+int lily_plan_run(lily_plan_t* p, uint32_t step_delta);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* LILY_SAMPLER_H */

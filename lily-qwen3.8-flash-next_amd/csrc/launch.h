@@ -1,0 +1,25 @@
+// launch.h - host-callable launchers defined in sampler_kernels.hip.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include "row_args.h"
+
+namespace lily {
+
+hipError_t launch_rows(hipStream_t stream, int dtype, uint32_t rows, const LaunchCfg& cfg,
+                       const InlineRows* inline_rows);
+hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t v);
+hipError_t launch_add_history(hipStream_t stream, uint32_t* counts, uint32_t* touched,
+                              uint32_t vocab, const uint32_t* ids, uint32_t n);
+hipError_t launch_uncount(hipStream_t stream, uint32_t* counts, uint32_t* touched, uint32_t vocab,
+                          uint32_t token);
+hipError_t launch_rebuild_touched(hipStream_t stream, const uint32_t* counts, uint32_t* touched,
+                                  uint32_t vocab);
+hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const uint32_t* ids,
+                              uint32_t* ctrl, uint32_t m, uint32_t pos0, uint32_t ratio,
+                              uint32_t chain);
+hipError_t launch_copy_row(hipStream_t stream, const uint32_t* src, uint32_t* dst, uint32_t words,
+                           uint32_t rows, const uint32_t* row_dev);
+
+}  // namespace lily

@@ -1,0 +1,911 @@
+// sampler_api.cpp - the C ABI of include/lily_sampler.h over the HIP kernels.
+//
+// Host-side work per draw is validation and packing one RowArgs per row; up to
+// INLINE_ROWS rows travel as kernel arguments, larger batches go through a pinned
+// staging ring and one asynchronous copy into the sampler's device row table.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/lily_sampler.h"
+#include "../../include/lily_sampler_math.h"
+#include "launch.h"
+
+using namespace lily;
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(LILY_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(call)                      \
+    do {                                   \
+        hipError_t e_ = (call);            \
+        if (e_ != hipSuccess) {            \
+            return hip_fail(e_, #call);    \
+        }                                  \
+    } while (0)
+
+constexpr uint32_t WS_ROWS = 256;       // rows that may span several workgroups
+constexpr uint32_t STAGE_SLOTS = 4;
+constexpr uint32_t TARGET_GROUPS = 512;  // workgroups a small batch is spread over
+
+}  // namespace
+
+struct lily_sampler {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    uint64_t* ws_cand = nullptr;
+    uint32_t* ws_n = nullptr;
+    float* ws_lse = nullptr;
+    uint32_t* ws_ticket = nullptr;
+    // Row table of lily_sample_rows batches above INLINE_ROWS.
+    RowArgs* table_dev = nullptr;
+    uint32_t table_cap = 0;
+    RowArgs* stage[STAGE_SLOTS] = {};
+    hipEvent_t stage_done[STAGE_SLOTS] = {};
+    bool stage_used[STAGE_SLOTS] = {};
+    uint32_t stage_cap = 0;
+    uint32_t stage_next = 0;
+    uint32_t force_path = 0;
+    uint32_t force_slices = 0;
+};
+
+struct lily_scratch {
+    lily_sampler* s = nullptr;
+    uint32_t vocab = 0;
+    uint32_t words = 0;
+    uint32_t* counts = nullptr;   // [vocab]
+    uint32_t* touched = nullptr;  // [words]
+};
+
+struct lily_draft_dists {
+    lily_sampler* s = nullptr;
+    uint32_t slots = 0;
+    uint32_t* ids = nullptr;
+    float* probs = nullptr;
+    uint32_t* counts = nullptr;
+};
+
+struct lily_plan {
+    lily_sampler* s = nullptr;
+    uint32_t max_rows = 0;
+    RowArgs* table_dev = nullptr;
+    uint32_t rows = 0;
+    uint32_t vocab = 0;
+    uint32_t dtype = 0;
+    uint32_t slices = 1;
+    uint32_t ws_k = 0;
+};
+
+namespace {
+
+bool samples(const lily_sampling_params* p) {
+    return !lily_params_is_greedy(p) || lily_params_uses_penalties(p);
+}
+
+struct RowExtras {
+    const uint32_t* allow = nullptr;
+    const lily_bias* bias = nullptr;
+    uint32_t n_bias = 0;
+    uint32_t forced = LILY_NO_TOKEN;
+    bool has_uniform = false;
+    float uniform = 0.0f, uniform2 = 0.0f;
+    float* out_logprob = nullptr;
+    uint32_t* dbg_ids = nullptr;
+    float* dbg_probs = nullptr;
+    uint32_t* dbg_counts = nullptr;
+};
+
+// Validates one row and packs it.  `mode` is the draw the caller asked for.
+int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scratch,
+             const lily_sampling_params* params, uint32_t step, uint32_t mode, uint32_t* out_id,
+             const lily_draft_dist* dist, const uint32_t* draft, const RowExtras& x) {
+    if (logits == nullptr || vocab == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "logits must be [V] with V > 0");
+    }
+    if (out_id == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "out must be U32 [1]");
+    }
+    if (params == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "params is null");
+    }
+    if (int rc = lily_params_validate(params)) {
+        return rc;
+    }
+    const bool pen = lily_params_uses_penalties(params) != 0;
+    if (scratch != nullptr && scratch->vocab != vocab) {
+        return fail(LILY_ERR_VOCAB, "sampler scratch sized for a different vocabulary");
+    }
+    if (pen && scratch == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "penalties need a sampler scratch");
+    }
+    if (x.forced != LILY_NO_TOKEN && x.forced >= vocab) {
+        return fail(LILY_ERR_RANGE, "forced token %u outside the vocabulary", x.forced);
+    }
+    std::memset(out, 0, sizeof *out);
+    float temperature;
+    uint32_t k;
+    lily_params_effective(params, &temperature, &k);
+    const bool extended = x.allow != nullptr || x.n_bias != 0 || x.out_logprob != nullptr ||
+                          x.forced != LILY_NO_TOKEN;
+    if (!samples(params) && !extended) {
+        mode = MODE_ARGMAX;  // sample.rs:382-385, :404-406, :428-430
+    } else if (!samples(params)) {
+        mode = MODE_PLAIN;   // greedy over the masked / biased row: a top-1 draw
+    }
+    if (mode == MODE_DRAFT || mode == MODE_SPEC) {
+        if (dist == nullptr || dist->ids_dev == nullptr || dist->probs_dev == nullptr ||
+            dist->count_dev == nullptr) {
+            return fail(LILY_ERR_INVALID_ARG, "draft distribution slot is null");
+        }
+        out->q_ids = dist->ids_dev;
+        out->q_probs = dist->probs_dev;
+        out->q_n = dist->count_dev;
+    }
+    if (mode == MODE_SPEC) {
+        if (draft == nullptr) {
+            return fail(LILY_ERR_INVALID_ARG, "draft must be U32 [1]");
+        }
+        out->draft = draft;
+    }
+    out->logits = logits;
+    out->allow = x.allow;
+    out->bias = x.n_bias ? x.bias : nullptr;
+    out->n_bias = x.bias ? x.n_bias : 0;
+    if (pen) {
+        out->counts = scratch->counts;
+        out->touched = scratch->touched;
+        out->flags |= F_PEN;
+    }
+    if (x.has_uniform) {
+        out->flags |= F_UNIFORM;
+        out->uniform = x.uniform;
+        out->uniform2 = x.uniform2;
+    }
+    if (x.forced != LILY_NO_TOKEN) {
+        out->flags |= F_FORCED;
+        out->forced = x.forced;
+    }
+    out->out_id = out_id;
+    out->out_logprob = x.out_logprob;
+    out->dbg_ids = x.dbg_ids;
+    out->dbg_probs = x.dbg_probs;
+    out->dbg_counts = x.dbg_counts;
+    out->seed = params->seed;
+    out->step = step;
+    out->k = k;
+    out->mode = mode;
+    out->temperature = temperature;
+    out->c2 = (float)(1.4426950408889634 / (double)temperature);
+    out->top_p = params->top_p;
+    out->min_p = params->min_p;
+    out->presence = params->presence_penalty;
+    out->frequency = params->frequency_penalty;
+    out->repetition = params->repetition_penalty;
+    return LILY_OK;
+}
+
+// Workgroups per row for a batch of `rows` whose largest candidate count is kmax.
+uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab) {
+    if (rows > WS_ROWS) {
+        return 1;
+    }
+    uint32_t sl = s->force_slices ? s->force_slices : TARGET_GROUPS / rows;
+    sl = sl < 1 ? 1 : sl;
+    sl = sl > MAX_SLICES ? MAX_SLICES : sl;
+    const uint32_t by_k = CAND_CAP / (kmax ? kmax : 1);
+    sl = sl > by_k ? by_k : sl;
+    const uint32_t by_len = (vocab + 2047u) / 2048u;
+    sl = sl > by_len ? by_len : sl;
+    return sl < 1 ? 1 : sl;
+}
+
+void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t slices,
+              uint32_t kmax, uint32_t step_delta, const RowArgs* table) {
+    std::memset(cfg, 0, sizeof *cfg);
+    cfg->table = table;
+    cfg->vocab = vocab;
+    cfg->slices = slices;
+    cfg->step_delta = step_delta;
+    cfg->ws_k = kmax ? kmax : 1;
+    cfg->ws_cand = s->ws_cand;
+    cfg->ws_n = s->ws_n;
+    cfg->ws_lse = s->ws_lse;
+    cfg->ws_ticket = s->ws_ticket;
+    cfg->path = s->force_path;
+}
+
+uint32_t max_k(const RowArgs* rows, uint32_t n) {
+    uint32_t k = 1;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (rows[i].mode != MODE_ARGMAX && rows[i].k > k) {
+            k = rows[i].k;
+        }
+    }
+    return k;
+}
+
+int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n) {
+    HIP_TRY(hipSetDevice(s->device));
+    const uint32_t kmax = max_k(rows.r, n);
+    LaunchCfg cfg;
+    fill_cfg(s, &cfg, vocab, choose_slices(s, n, kmax, vocab), kmax, 0, nullptr);
+    HIP_TRY(launch_rows(s->stream, dtype, n, cfg, &rows));
+    return LILY_OK;
+}
+
+int one_row(lily_sampler* s, const void* logits, int dtype, uint32_t vocab, lily_scratch* scratch,
+            const lily_sampling_params* params, uint32_t step, uint32_t mode, uint32_t* out,
+            const lily_draft_dist* dist, const uint32_t* draft) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    InlineRows rows;
+    RowExtras x;
+    if (int rc = pack_row(&rows.r[0], logits, vocab, scratch, params, step, mode, out, dist, draft, x)) {
+        return rc;
+    }
+    return launch_inline(s, dtype, vocab, rows, 1);
+}
+
+// Packs a lily_rows batch into `table[0..rows)`.
+int pack_batch(const lily_rows* b, RowArgs* table) {
+    if (b == nullptr || b->rows == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "empty batch");
+    }
+    if (b->dtype != LILY_F32 && b->dtype != LILY_BF16) {
+        return fail(LILY_ERR_INVALID_ARG, "dtype must be LILY_F32 or LILY_BF16");
+    }
+    if (b->logits_dev == nullptr || b->params == nullptr || b->out_ids_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "logits, params and out_ids are required");
+    }
+    if (b->row_stride < b->vocab) {
+        return fail(LILY_ERR_INVALID_ARG, "row_stride is shorter than the vocabulary");
+    }
+    if (b->bias_dev != nullptr && b->bias_offsets == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "bias needs bias_offsets");
+    }
+    const size_t es = b->dtype == LILY_BF16 ? 2 : 4;
+    const uint32_t words = (b->vocab + 31u) / 32u;
+    if (b->scratch != nullptr) {
+        for (uint32_t r = 0; r < b->rows; ++r) {
+            for (uint32_t q = 0; q < r && b->scratch[r] != nullptr; ++q) {
+                if (b->scratch[q] == b->scratch[r] &&
+                    lily_params_uses_penalties(&b->params[r])) {
+                    return fail(LILY_ERR_INVALID_ARG, "rows %u and %u share a scratch", q, r);
+                }
+            }
+        }
+    }
+    for (uint32_t r = 0; r < b->rows; ++r) {
+        RowExtras x;
+        if (b->allow_dev != nullptr) {
+            x.allow = b->allow_dev + (size_t)r * b->allow_stride;
+            if (b->allow_stride != 0 && b->allow_stride < words) {
+                return fail(LILY_ERR_INVALID_ARG, "allow_stride is shorter than the mask");
+            }
+        }
+        if (b->bias_dev != nullptr) {
+            const uint32_t lo = b->bias_offsets[r], hi = b->bias_offsets[r + 1];
+            if (hi < lo) {
+                return fail(LILY_ERR_INVALID_ARG, "bias_offsets must not decrease");
+            }
+            x.bias = b->bias_dev + lo;
+            x.n_bias = hi - lo;
+        }
+        if (b->forced != nullptr) {
+            x.forced = b->forced[r];
+        }
+        if (b->uniforms != nullptr && !std::isnan(b->uniforms[r])) {
+            x.has_uniform = true;
+            x.uniform = b->uniforms[r];
+            x.uniform2 = b->uniforms[r];
+        }
+        if (b->out_logprobs_dev != nullptr) {
+            x.out_logprob = b->out_logprobs_dev + r;
+        }
+        if (b->dbg_ids_dev != nullptr) {
+            x.dbg_ids = b->dbg_ids_dev + (size_t)r * LILY_SAMPLE_K_CAP;
+        }
+        if (b->dbg_probs_dev != nullptr) {
+            x.dbg_probs = b->dbg_probs_dev + (size_t)r * LILY_SAMPLE_K_CAP;
+        }
+        if (b->dbg_counts_dev != nullptr) {
+            x.dbg_counts = b->dbg_counts_dev + (size_t)r * 2;
+        }
+        const char* row = static_cast<const char*>(b->logits_dev) + (size_t)r * b->row_stride * es;
+        lily_scratch* sc = b->scratch ? b->scratch[r] : nullptr;
+        if (int rc = pack_row(&table[r], row, b->vocab, sc, &b->params[r],
+                              b->steps ? b->steps[r] : 0, MODE_PLAIN, b->out_ids_dev + r, nullptr,
+                              nullptr, x)) {
+            return rc;
+        }
+    }
+    return LILY_OK;
+}
+
+int ensure_table(lily_sampler* s, uint32_t rows) {
+    if (rows <= s->table_cap && rows <= s->stage_cap) {
+        return LILY_OK;
+    }
+    // Growing is rare (first large batch); drain the stream so nothing reads the old buffers.
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    uint32_t cap = 1024;
+    while (cap < rows) {
+        cap <<= 1;
+    }
+    if (s->table_dev) {
+        (void)hipFree(s->table_dev);
+        s->table_dev = nullptr;
+    }
+    for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {
+        if (s->stage[i]) {
+            (void)hipHostFree(s->stage[i]);
+            s->stage[i] = nullptr;
+        }
+        s->stage_used[i] = false;
+    }
+    s->table_cap = s->stage_cap = 0;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->table_dev), (size_t)cap * sizeof(RowArgs)));
+    for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&s->stage[i]), (size_t)cap * sizeof(RowArgs),
+                              hipHostMallocDefault));
+    }
+    s->table_cap = s->stage_cap = cap;
+    return LILY_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* lily_last_error(void) { return g_error; }
+
+// ---- pure host helpers
+
+void lily_params_greedy(lily_sampling_params* out) {
+    out->temperature = 0.0f;
+    out->top_k = 1;
+    out->top_p = 1.0f;
+    out->min_p = 0.0f;
+    out->presence_penalty = 0.0f;
+    out->frequency_penalty = 0.0f;
+    out->repetition_penalty = 1.0f;
+    out->reserved = 0;
+    out->seed = 0;
+}
+
+int lily_params_is_greedy(const lily_sampling_params* p) {
+    return p->temperature <= 0.0f || p->top_k == 1;
+}
+
+int lily_params_uses_penalties(const lily_sampling_params* p) {
+    return p->presence_penalty != 0.0f || p->frequency_penalty != 0.0f ||
+           p->repetition_penalty != 1.0f;
+}
+
+int lily_params_validate(const lily_sampling_params* p) {
+    if (!(std::isfinite(p->temperature) && p->temperature >= 0.0f)) {
+        return fail(LILY_ERR_PARAMS, "temperature must be a finite number >= 0");
+    }
+    if (!(std::isfinite(p->top_p) && p->top_p > 0.0f && p->top_p <= 1.0f)) {
+        return fail(LILY_ERR_PARAMS, "top_p must be in (0, 1]");
+    }
+    if (!(std::isfinite(p->min_p) && p->min_p >= 0.0f && p->min_p <= 1.0f)) {
+        return fail(LILY_ERR_PARAMS, "min_p must be in [0, 1]");
+    }
+    if (!(std::isfinite(p->repetition_penalty) && p->repetition_penalty > 0.0f)) {
+        return fail(LILY_ERR_PARAMS, "repetition_penalty must be > 0");
+    }
+    if (!(std::isfinite(p->presence_penalty) && std::isfinite(p->frequency_penalty))) {
+        return fail(LILY_ERR_PARAMS, "penalties must be finite");
+    }
+    return LILY_OK;
+}
+
+void lily_params_effective(const lily_sampling_params* p, float* temperature, uint32_t* top_k) {
+    if (lily_params_is_greedy(p)) {
+        *temperature = 1.0f;
+        *top_k = 1;
+    } else {
+        *temperature = p->temperature;
+        *top_k = p->top_k == 0 ? LILY_SAMPLE_K_CAP
+                               : (p->top_k < LILY_SAMPLE_K_CAP ? p->top_k : LILY_SAMPLE_K_CAP);
+    }
+}
+
+void lily_draft_params(const lily_sampling_params* p, lily_sampling_params* out) {
+    *out = *p;
+    out->presence_penalty = 0.0f;
+    out->frequency_penalty = 0.0f;
+    out->repetition_penalty = 1.0f;
+}
+
+uint32_t lily_draft_step(uint32_t step) { return lilym_draft_step(step); }
+float lily_uniform_for(uint64_t seed, uint32_t step) { return lilym_uniform_for(seed, step); }
+uint32_t lily_slot_pos(uint32_t i) { return 2 + 3 * i; }
+uint32_t lily_slot_block(uint32_t i) { return 3 + 3 * i; }
+uint32_t lily_slot_count(uint32_t i) { return 4 + 3 * i; }
+uint32_t lily_ctrl_words(uint32_t chain) { return (2 + 3 * chain) * LILY_CTRL_STRIDE; }
+
+// ---- sampler
+
+int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
+    if (out == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "out is null");
+    }
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) {
+        return fail(LILY_ERR_HIP, "no HIP device: %s", hipGetErrorString(e));
+    }
+    if (device < 0 || device >= n) {
+        return fail(LILY_ERR_RANGE, "device %d of %d", device, n);
+    }
+    HIP_TRY(hipSetDevice(device));
+    lily_sampler* s = new (std::nothrow) lily_sampler;
+    if (s == nullptr) {
+        return fail(LILY_ERR_NOMEM, "out of host memory");
+    }
+    s->device = device;
+    s->stream = static_cast<hipStream_t>(hip_stream);
+    if (const char* p = std::getenv("LILY_SAMPLER_PATH")) {
+        s->force_path = (uint32_t)std::atoi(p);
+    }
+    if (const char* p = std::getenv("LILY_SAMPLER_SLICES")) {
+        s->force_slices = (uint32_t)std::atoi(p);
+    }
+    const size_t slots = (size_t)WS_ROWS * MAX_SLICES;
+    hipError_t err = hipMalloc(reinterpret_cast<void**>(&s->ws_cand),
+                               (size_t)WS_ROWS * CAND_CAP * sizeof(uint64_t));
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_n), slots * 4);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 8);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
+    if (err == hipSuccess) err = hipMemset(s->ws_ticket, 0, WS_ROWS * 4);
+    for (uint32_t i = 0; i < STAGE_SLOTS && err == hipSuccess; ++i) {
+        err = hipEventCreateWithFlags(&s->stage_done[i], hipEventDisableTiming);
+    }
+    if (err != hipSuccess) {
+        lily_sampler_destroy(s);
+        return hip_fail(err, "sampler workspace");
+    }
+    *out = s;
+    return LILY_OK;
+}
+
+void lily_sampler_destroy(lily_sampler_t* s) {
+    if (s == nullptr) {
+        return;
+    }
+    (void)hipSetDevice(s->device);
+    (void)hipStreamSynchronize(s->stream);
+    (void)hipFree(s->ws_cand);
+    (void)hipFree(s->ws_n);
+    (void)hipFree(s->ws_lse);
+    (void)hipFree(s->ws_ticket);
+    (void)hipFree(s->table_dev);
+    for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {
+        if (s->stage[i]) (void)hipHostFree(s->stage[i]);
+        if (s->stage_done[i]) (void)hipEventDestroy(s->stage_done[i]);
+    }
+    delete s;
+}
+
+int lily_sampler_synchronize(lily_sampler_t* s) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    return LILY_OK;
+}
+
+// ---- scratch
+
+int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out) {
+    if (s == nullptr || out == nullptr || vocab == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch needs a sampler and a vocabulary > 0");
+    }
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(s->device));
+    lily_scratch* sc = new (std::nothrow) lily_scratch;
+    if (sc == nullptr) {
+        return fail(LILY_ERR_NOMEM, "out of host memory");
+    }
+    sc->s = s;
+    sc->vocab = vocab;
+    sc->words = (vocab + 31u) / 32u;
+    // One allocation: counts, then the bitmap (padded so the bitmap is 16-byte aligned).
+    const size_t count_bytes = (((size_t)vocab * 4) + 15) & ~(size_t)15;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts),
+                             count_bytes + (size_t)(sc->words + 4) * 4);
+    if (e != hipSuccess) {
+        delete sc;
+        return hip_fail(e, "scratch allocation");
+    }
+    sc->touched = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(sc->counts) + count_bytes);
+    *out = sc;
+    return lily_scratch_reset_counts(sc);
+}
+
+void lily_scratch_destroy(lily_scratch_t* sc) {
+    if (sc == nullptr) {
+        return;
+    }
+    (void)hipSetDevice(sc->s->device);
+    (void)hipStreamSynchronize(sc->s->stream);
+    (void)hipFree(sc->counts);
+    delete sc;
+}
+
+uint32_t lily_scratch_vocab(const lily_scratch_t* sc) { return sc ? sc->vocab : 0; }
+
+int lily_scratch_reset_counts(lily_scratch_t* sc) {
+    if (sc == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch is null");
+    }
+    HIP_TRY(hipSetDevice(sc->s->device));
+    HIP_TRY(launch_fill_u32(sc->s->stream, sc->counts, sc->vocab, 0));
+    HIP_TRY(launch_fill_u32(sc->s->stream, sc->touched, sc->words + 4, 0));
+    return LILY_OK;
+}
+
+int lily_scratch_uncount(lily_scratch_t* sc, uint32_t token) {
+    if (sc == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch is null");
+    }
+    if (token >= sc->vocab) {
+        return LILY_OK;  // sample.rs:149-151
+    }
+    HIP_TRY(hipSetDevice(sc->s->device));
+    HIP_TRY(launch_uncount(sc->s->stream, sc->counts, sc->touched, sc->vocab, token));
+    return LILY_OK;
+}
+
+int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src) {
+    if (dst == nullptr || src == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch is null");
+    }
+    if (dst->vocab != src->vocab) {
+        return fail(LILY_ERR_VOCAB, "sampler scratches for different vocabularies");
+    }
+    HIP_TRY(hipSetDevice(dst->s->device));
+    HIP_TRY(hipMemcpyAsync(dst->counts, src->counts, (size_t)src->vocab * 4, hipMemcpyDeviceToDevice,
+                           dst->s->stream));
+    HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)src->words * 4,
+                           hipMemcpyDeviceToDevice, dst->s->stream));
+    return LILY_OK;
+}
+
+int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32_t n) {
+    if (sc == nullptr || (ids_dev == nullptr && n != 0)) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch or ids is null");
+    }
+    HIP_TRY(hipSetDevice(sc->s->device));
+    HIP_TRY(launch_add_history(sc->s->stream, sc->counts, sc->touched, sc->vocab, ids_dev, n));
+    return LILY_OK;
+}
+
+int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts) {
+    if (sc == nullptr || host_counts == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch or counts is null");
+    }
+    HIP_TRY(hipSetDevice(sc->s->device));
+    HIP_TRY(hipStreamSynchronize(sc->s->stream));
+    HIP_TRY(hipMemcpy(sc->counts, host_counts, (size_t)sc->vocab * 4, hipMemcpyHostToDevice));
+    HIP_TRY(launch_rebuild_touched(sc->s->stream, sc->counts, sc->touched, sc->vocab));
+    HIP_TRY(hipStreamSynchronize(sc->s->stream));
+    return LILY_OK;
+}
+
+int lily_scratch_read_counts(lily_scratch_t* sc, uint32_t* host_counts) {
+    if (sc == nullptr || host_counts == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch or counts is null");
+    }
+    HIP_TRY(hipSetDevice(sc->s->device));
+    HIP_TRY(hipStreamSynchronize(sc->s->stream));
+    HIP_TRY(hipMemcpy(host_counts, sc->counts, (size_t)sc->vocab * 4, hipMemcpyDeviceToHost));
+    return LILY_OK;
+}
+
+// ---- draft distributions
+
+int lily_draft_dists_create(lily_sampler_t* s, uint32_t slots, lily_draft_dists_t** out) {
+    if (s == nullptr || out == nullptr || slots == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "draft dists need a sampler and slots > 0");
+    }
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(s->device));
+    lily_draft_dists* d = new (std::nothrow) lily_draft_dists;
+    if (d == nullptr) {
+        return fail(LILY_ERR_NOMEM, "out of host memory");
+    }
+    d->s = s;
+    d->slots = slots;
+    const size_t n = (size_t)slots * LILY_SAMPLE_K_CAP;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->ids), n * 8 + (size_t)slots * 4);
+    if (e != hipSuccess) {
+        delete d;
+        return hip_fail(e, "draft dists allocation");
+    }
+    d->probs = reinterpret_cast<float*>(d->ids + n);
+    d->counts = reinterpret_cast<uint32_t*>(d->probs + n);
+    e = hipMemsetAsync(d->ids, 0, n * 8 + (size_t)slots * 4, s->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(d->ids);
+        delete d;
+        return hip_fail(e, "draft dists clear");
+    }
+    *out = d;
+    return LILY_OK;
+}
+
+void lily_draft_dists_destroy(lily_draft_dists_t* d) {
+    if (d == nullptr) {
+        return;
+    }
+    (void)hipSetDevice(d->s->device);
+    (void)hipStreamSynchronize(d->s->stream);
+    (void)hipFree(d->ids);
+    delete d;
+}
+
+int lily_draft_dists_slot(const lily_draft_dists_t* d, uint32_t i, lily_draft_dist* out) {
+    if (d == nullptr || out == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "draft dists or out is null");
+    }
+    if (i >= d->slots) {
+        return fail(LILY_ERR_RANGE, "slot %u of %u", i, d->slots);
+    }
+    out->ids_dev = d->ids + (size_t)i * LILY_SAMPLE_K_CAP;
+    out->probs_dev = d->probs + (size_t)i * LILY_SAMPLE_K_CAP;
+    out->count_dev = d->counts + i;
+    return LILY_OK;
+}
+
+// ---- single-row draws
+
+int lily_sample_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                    lily_scratch_t* scratch, const lily_sampling_params* params, uint32_t step,
+                    uint32_t* out_dev) {
+    return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step, MODE_PLAIN, out_dev,
+                   nullptr, nullptr);
+}
+
+int lily_sample_draft_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                          lily_scratch_t* scratch, const lily_sampling_params* params,
+                          uint32_t step, uint32_t* out_dev, const lily_draft_dist* dist) {
+    return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step, MODE_DRAFT, out_dev, dist,
+                   nullptr);
+}
+
+int lily_sample_spec_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                         lily_scratch_t* scratch, const lily_sampling_params* params,
+                         uint32_t step, const lily_draft_dist* dist, const uint32_t* draft_dev,
+                         uint32_t* out_dev) {
+    return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step, MODE_SPEC, out_dev, dist,
+                   draft_dev);
+}
+
+int lily_argmax_f32(lily_sampler_t* s, const float* x_dev, uint32_t n, uint32_t* out_dev) {
+    lily_sampling_params g;
+    lily_params_greedy(&g);
+    if (n == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "empty argmax input");
+    }
+    return one_row(s, x_dev, LILY_F32, n, nullptr, &g, 0, MODE_PLAIN, out_dev, nullptr, nullptr);
+}
+
+// ---- speculative control
+
+int lily_spec_accept(lily_sampler_t* s, const uint32_t* draws_dev, const uint32_t* ids_dev,
+                     uint32_t m, uint32_t* ctrl_dev, uint32_t ctrl_words, uint32_t pos0,
+                     uint32_t ratio, uint32_t chain) {
+    if (s == nullptr || draws_dev == nullptr || ids_dev == nullptr || ctrl_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "spec_accept works on U32 tensors");
+    }
+    if (m == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "draws and ids must both hold the verified rows");
+    }
+    if (ctrl_words < lily_ctrl_words(chain)) {
+        return fail(LILY_ERR_RANGE, "control block too small for %u chain rows", chain);
+    }
+    if (ratio == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "indexer block ratio must be nonzero");
+    }
+    HIP_TRY(hipSetDevice(s->device));
+    HIP_TRY(launch_spec_accept(s->stream, draws_dev, ids_dev, ctrl_dev, m, pos0, ratio, chain));
+    return LILY_OK;
+}
+
+int lily_copy_row_u32(lily_sampler_t* s, const uint32_t* src_dev, uint32_t rows, uint32_t words,
+                      const uint32_t* row_dev, uint32_t* dst_dev) {
+    if (s == nullptr || src_dev == nullptr || row_dev == nullptr || dst_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "copy_row needs src, row and dst");
+    }
+    if (rows == 0 || words == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "src must be [rows, words] with both > 0");
+    }
+    HIP_TRY(hipSetDevice(s->device));
+    HIP_TRY(launch_copy_row(s->stream, src_dev, dst_dev, words, rows, row_dev));
+    return LILY_OK;
+}
+
+int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype, uint32_t vocab,
+                     uint64_t row_stride, uint32_t m, lily_scratch_t* scratch,
+                     const lily_sampling_params* params, uint32_t step0,
+                     const lily_draft_dists_t* dists, const uint32_t* ids_dev,
+                     uint32_t* verify_tokens_dev, uint32_t* ctrl_dev, uint32_t ctrl_words,
+                     uint32_t pos0, uint32_t ratio, uint32_t chain) {
+    if (s == nullptr || logits_dev == nullptr || ids_dev == nullptr || verify_tokens_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "verify needs logits, ids and verify_tokens");
+    }
+    if (m == 0 || m > LILY_MAX_VERIFY_ROWS) {
+        return fail(LILY_ERR_RANGE, "verify rows %u outside 1..%u", m, LILY_MAX_VERIFY_ROWS);
+    }
+    if (dtype != LILY_F32 && dtype != LILY_BF16) {
+        return fail(LILY_ERR_INVALID_ARG, "dtype must be LILY_F32 or LILY_BF16");
+    }
+    if (row_stride < vocab) {
+        return fail(LILY_ERR_INVALID_ARG, "row_stride is shorter than the vocabulary");
+    }
+    if (params == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "params is null");
+    }
+    const bool sampled = samples(params);
+    if (sampled && m > 1 && (dists == nullptr || dists->slots < m - 1)) {
+        return fail(LILY_ERR_RANGE, "verify needs %u draft distribution slots", m - 1);
+    }
+    const size_t es = dtype == LILY_BF16 ? 2 : 4;
+    // One launch per row: row j must see the counts of rows before it.
+    for (uint32_t j = 0; j < m; ++j) {
+        const char* row = static_cast<const char*>(logits_dev) + (size_t)j * row_stride * es;
+        InlineRows rows;
+        RowExtras x;
+        lily_draft_dist slot;
+        const bool spec = j + 1 < m && sampled;
+        if (spec) {
+            if (int rc = lily_draft_dists_slot(dists, j, &slot)) {
+                return rc;
+            }
+        }
+        if (int rc = pack_row(&rows.r[0], row, vocab, scratch, params, step0 + j,
+                              spec ? MODE_SPEC : MODE_PLAIN, verify_tokens_dev + j,
+                              spec ? &slot : nullptr, spec ? ids_dev + j + 1 : nullptr, x)) {
+            return rc;
+        }
+        if (int rc = launch_inline(s, dtype, vocab, rows, 1)) {
+            return rc;
+        }
+    }
+    if (ctrl_dev != nullptr) {
+        return lily_spec_accept(s, verify_tokens_dev, ids_dev, m, ctrl_dev, ctrl_words, pos0, ratio,
+                                chain);
+    }
+    return LILY_OK;
+}
+
+// ---- batched rows
+
+int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    if (b != nullptr && b->rows != 0 && b->rows <= (uint32_t)INLINE_ROWS) {
+        InlineRows rows;
+        if (int rc = pack_batch(b, rows.r)) {
+            return rc;
+        }
+        return launch_inline(s, (int)b->dtype, b->vocab, rows, b->rows);
+    }
+    if (b == nullptr || b->rows == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "empty batch");
+    }
+    HIP_TRY(hipSetDevice(s->device));
+    if (int rc = ensure_table(s, b->rows)) {
+        return rc;
+    }
+    const uint32_t slot = s->stage_next;
+    s->stage_next = (slot + 1) % STAGE_SLOTS;
+    if (s->stage_used[slot]) {
+        HIP_TRY(hipEventSynchronize(s->stage_done[slot]));
+    }
+    if (int rc = pack_batch(b, s->stage[slot])) {
+        return rc;
+    }
+    HIP_TRY(hipMemcpyAsync(s->table_dev, s->stage[slot], (size_t)b->rows * sizeof(RowArgs),
+                           hipMemcpyHostToDevice, s->stream));
+    HIP_TRY(hipEventRecord(s->stage_done[slot], s->stream));
+    s->stage_used[slot] = true;
+    const uint32_t kmax = max_k(s->stage[slot], b->rows);
+    LaunchCfg cfg;
+    fill_cfg(s, &cfg, b->vocab, choose_slices(s, b->rows, kmax, b->vocab), kmax, 0, s->table_dev);
+    HIP_TRY(launch_rows(s->stream, (int)b->dtype, b->rows, cfg, nullptr));
+    return LILY_OK;
+}
+
+int lily_plan_create(lily_sampler_t* s, uint32_t max_rows, lily_plan_t** out) {
+    if (s == nullptr || out == nullptr || max_rows == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "plan needs a sampler and max_rows > 0");
+    }
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(s->device));
+    lily_plan* p = new (std::nothrow) lily_plan;
+    if (p == nullptr) {
+        return fail(LILY_ERR_NOMEM, "out of host memory");
+    }
+    p->s = s;
+    p->max_rows = max_rows;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&p->table_dev),
+                             (size_t)max_rows * sizeof(RowArgs));
+    if (e != hipSuccess) {
+        delete p;
+        return hip_fail(e, "plan allocation");
+    }
+    *out = p;
+    return LILY_OK;
+}
+
+void lily_plan_destroy(lily_plan_t* p) {
+    if (p == nullptr) {
+        return;
+    }
+    (void)hipSetDevice(p->s->device);
+    (void)hipStreamSynchronize(p->s->stream);
+    (void)hipFree(p->table_dev);
+    delete p;
+}
+
+int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
+    if (p == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "plan is null");
+    }
+    if (b == nullptr || b->rows == 0 || b->rows > p->max_rows) {
+        return fail(LILY_ERR_RANGE, "batch rows outside 1..%u", p->max_rows);
+    }
+    std::vector<RowArgs> table(b->rows);
+    if (int rc = pack_batch(b, table.data())) {
+        return rc;
+    }
+    HIP_TRY(hipSetDevice(p->s->device));
+    HIP_TRY(hipStreamSynchronize(p->s->stream));
+    HIP_TRY(hipMemcpy(p->table_dev, table.data(), (size_t)b->rows * sizeof(RowArgs),
+                      hipMemcpyHostToDevice));
+    p->rows = b->rows;
+    p->vocab = b->vocab;
+    p->dtype = b->dtype;
+    p->ws_k = max_k(table.data(), b->rows);
+    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab);
+    return LILY_OK;
+}
+
+int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
+    if (p == nullptr || p->rows == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "plan is null or not set");
+    }
+    HIP_TRY(hipSetDevice(p->s->device));
+    LaunchCfg cfg;
+    fill_cfg(p->s, &cfg, p->vocab, p->slices, p->ws_k, step_delta, p->table_dev);
+    HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->rows, cfg, nullptr));
+    return LILY_OK;
+}
+
+}  // extern "C"

@@ -25,7 +25,7 @@
 // forced token, an explicit uniform, and the chosen token's log-probability
 // over the whole adjusted row in f64.
 //
-// Two exp() variants: EXP_LILY is lily_expf from include/lily_sampler_math.h
+// Two exp() variants: EXP_LILY is lilym_expf from include/lily_sampler_math.h
 // (bit-identical on the GPU), EXP_LIBM is the C library's expf, standing in
 // for the reference's platform libm (f32::exp).
 //
@@ -97,9 +97,9 @@ struct lo_result {
     double logprob;   // chosen token, over the full adjusted row
 };
 
-float lo_uniform_for(uint64_t seed, uint32_t step) { return lily_uniform_for(seed, step); }
-uint32_t lo_draft_step(uint32_t step) { return lily_draft_step(step); }
-float lo_expf(float x) { return lily_expf(x); }
+float lo_uniform_for(uint64_t seed, uint32_t step) { return lilym_uniform_for(seed, step); }
+uint32_t lo_draft_step(uint32_t step) { return lilym_draft_step(step); }
+float lo_expf(float x) { return lilym_expf(x); }
 
 int lo_is_greedy(const lo_params* p) { return p->temperature <= 0.0f || p->top_k == 1; }
 
@@ -139,7 +139,7 @@ void lo_draft_params(const lo_params* p, lo_params* out) {
 
 static inline float load_logit(const void* logits, int dtype, size_t i) {
     if (dtype == LO_BF16) {
-        return lily_bf16_to_f32(static_cast<const uint16_t*>(logits)[i]);
+        return lilym_bf16_to_f32(static_cast<const uint16_t*>(logits)[i]);
     }
     return static_cast<const float*>(logits)[i];
 }
@@ -217,8 +217,8 @@ int lo_sample(const void* logits, int dtype, size_t v, uint32_t* counts, const l
     std::vector<uint32_t> order(v);
     std::iota(order.begin(), order.end(), 0u);
     auto before = [&](uint32_t a, uint32_t b) {
-        const uint32_t ka = lily_order_key(adjusted[a]);
-        const uint32_t kb = lily_order_key(adjusted[b]);
+        const uint32_t ka = lilym_order_key(adjusted[a]);
+        const uint32_t kb = lilym_order_key(adjusted[b]);
         return ka != kb ? ka > kb : a < b;
     };
     if (ext && ext->sort_mode == LO_SORT_FULL) {
@@ -231,7 +231,7 @@ int lo_sample(const void* logits, int dtype, size_t v, uint32_t* counts, const l
     std::vector<float> probs(n);
     for (size_t i = 0; i < n; ++i) {
         const float d = adjusted[order[i]] - top;
-        probs[i] = libm ? std::exp(d) : lily_expf(d);
+        probs[i] = libm ? std::exp(d) : lilym_expf(d);
     }
     float total = 0.0f;
     for (size_t i = 0; i < n; ++i) total += probs[i];
@@ -243,7 +243,7 @@ int lo_sample(const void* logits, int dtype, size_t v, uint32_t* counts, const l
         cums.push_back(cum);
     }
     const float mass = cums.back();
-    const float u = (ext && ext->has_uniform) ? ext->uniform : lily_uniform_for(p->seed, step);
+    const float u = (ext && ext->has_uniform) ? ext->uniform : lilym_uniform_for(p->seed, step);
     const float target = u * mass;
     uint32_t chosen = order[cums.size() - 1];
     for (size_t i = 0; i < cums.size(); ++i) {
@@ -301,7 +301,7 @@ uint32_t lo_kept(const void* logits, int dtype, size_t v, const lo_params* p, ui
     std::vector<float> w(res.n_kept);
     for (uint32_t i = 0; i < res.n_kept; ++i) {
         const float d = load_logit(logits, dtype, cand[i]) / temperature - top;
-        w[i] = exp_mode == LO_EXP_LIBM ? std::exp(d) : lily_expf(d);
+        w[i] = exp_mode == LO_EXP_LIBM ? std::exp(d) : lilym_expf(d);
     }
     float mass = 0.0f;
     for (float x : w) mass += x;
@@ -329,7 +329,7 @@ uint32_t lo_spec(const uint32_t* p_ids, const float* p_probs, uint32_t pn, const
                  uint32_t* zero_residual, float* gap) {
     const float p_d = dist_at(p_ids, p_probs, pn, d);
     const float q_d = dist_at(q_ids, q_probs, qn, d);
-    const float u1 = has_u ? u1_in : lily_uniform_for(seed, step);
+    const float u1 = has_u ? u1_in : lilym_uniform_for(seed, step);
     if (accepted) *accepted = 0;
     if (zero_residual) *zero_residual = 0;
     if (gap) *gap = std::numeric_limits<float>::infinity();
@@ -343,7 +343,7 @@ uint32_t lo_spec(const uint32_t* p_ids, const float* p_probs, uint32_t pn, const
     }
     float total = 0.0f;
     for (float x : r) total += x;
-    const float u2 = has_u ? u2_in : lily_uniform_for(seed, lily_residual_step(step));
+    const float u2 = has_u ? u2_in : lilym_uniform_for(seed, lilym_residual_step(step));
     const float target = u2 * total;
     if (zero_residual && !(total > 0.0f)) *zero_residual = 1;
     float cum = 0.0f;
