@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the logits-to-token stage on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the sampler over one batch of synthetic logits already
+resident in HBM: the throughput configuration of BASELINE.json (1 024 rows x 151 936
+bf16 logits, top-k 64, top-p 0.9, T 0.8, penalties over a 2 048-id history per row,
+output = token ids + chosen-token log-probabilities).  The 4-row decode-step
+configuration (f32, 8 192-id history, k 20) is timed in the same run and reported in
+the same JSON line under "decode_b4".  The CPU oracle is timed on a bounded sample
+of the same rows on the host's cores as a reported baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "lily-qwen3.8-flash-next_amd", "python"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--rows", type=int, default=1024)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    return ap.parse_args()
+
+
+def time_steps(stream, fn, steps, warmup):
+    """Average milliseconds per call of fn, HIP events on the sampler's own stream."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for i in range(steps):
+        fn(warmup + i)
+    stop.record(stream)
+    stop.synchronize()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def make_scratches(LS, sampler, history, vocab, device):
+    import numpy as np
+    import torch
+    out = []
+    for h in history:
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(np.ascontiguousarray(h)).to(device))
+        out.append(sc)
+    return out
+
+
+def cpu_baseline(c, rows_total, seconds):
+    """The oracle (reference-faithful full-vocabulary sort) on this host's cores."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = max(1, min(cores, 16))
+    x, hist = c["logits"], c["history"]
+    vocab = x.shape[1]
+    ext, _ = O.make_ext(sort_mode=O.SORT_FULL, want_logprob=True)
+
+    def run(n):
+        n = min(n, rows_total)
+        counts = np.stack([np.bincount(hist[i], minlength=vocab).astype(np.uint32) for i in range(n)])
+        params = [O.params(**c["params"][i]) for i in range(n)]
+        t0 = time.perf_counter()
+        O.sample_rows(x[:n], counts, params, [3] * n, exts=[ext] * n, threads=cores)
+        return n, time.perf_counter() - t0
+
+    n, dt = run(cores)                       # probe: one row per core
+    per_round = max(dt, 1e-3)
+    want = int(max(cores, min(rows_total, cores * (seconds / per_round))))
+    n, dt = run(want)
+    return {"value": n / dt, "unit": "rows/s", "cores": cores, "kind": "port",
+            "sample": f"{n} of the {rows_total} rows, full-vocabulary index sort per row "
+                      f"(as tests/unit/kernels/sample.rs:31-34), id + f64 log-probability, "
+                      f"{dt:.1f} s wall"}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: rows are independent, so more GPUs only split the "
+              "batch; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    import lily_sampler as LS
+    import lily_workloads as W
+
+    if not torch.cuda.is_available():
+        print("no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda", 0)
+    stream = torch.cuda.Stream(device=device)
+    sampler = LS.Sampler(0, stream=stream)
+
+    # ---- throughput configuration: rows x 151 936 bf16
+    rows = a.rows
+    c5 = W.config5(rows=rows)
+    vocab = c5["logits"].shape[1]
+    history = c5["history"].shape[1]
+    logits = torch.from_numpy(c5["logits"].view(np.int16)).to(device).view(torch.bfloat16)
+    params = [LS.SamplingParams.greedy(**kw) for kw in c5["params"]]
+    scratches = make_scratches(LS, sampler, c5["history"], vocab, device)
+    out_ids = torch.zeros(rows, dtype=torch.int32, device=device)
+    out_lp = torch.zeros(rows, dtype=torch.float32, device=device)
+    torch.cuda.synchronize()
+    plan = sampler.plan(logits, params, [0] * rows, out_ids, scratch=scratches, out_logprobs=out_lp)
+    ms = time_steps(stream, lambda i: plan.run(i), a.steps, a.warmup)
+    bytes_row = W.algorithmic_bytes_per_row(vocab, 2, history=history, logprob=True)
+    achieved = rows * bytes_row / (ms * 1e-3) / 1e9
+    ids_host = out_ids.cpu().numpy()
+    assert ids_host.min() >= 0 and ids_host.max() < vocab
+    plan.close()
+
+    # ---- decode-step configuration: 4 x 151 936 f32, 8 192-id history
+    c2 = W.config2()
+    l2 = torch.from_numpy(c2["logits"]).to(device)
+    p2 = [LS.SamplingParams.greedy(**kw) for kw in c2["params"]]
+    s2 = make_scratches(LS, sampler, c2["history"], vocab, device)
+    o2 = torch.zeros(4, dtype=torch.int32, device=device)
+    torch.cuda.synchronize()
+    plan2 = sampler.plan(l2, p2, [0] * 4, o2, scratch=s2)
+    ms2 = time_steps(stream, lambda i: plan2.run(i), max(a.steps, 200), max(a.warmup, 20))
+    # the reference's call shape: host descriptors every step (lily_sample_rows)
+    ms2_call = time_steps(stream, lambda i: sampler.sample_rows(l2, p2, [i] * 4, o2, scratch=s2),
+                          max(a.steps, 200), max(a.warmup, 20))
+    bytes2 = 4 * W.algorithmic_bytes_per_row(vocab, 4, history=c2["history"].shape[1])
+    plan2.close()
+
+    line = {
+        "metric": "rows/s and us/step at B=4 and B=1024 x151,936 vocab; achieved HBM GB/s",
+        "value": rows / (ms * 1e-3),
+        "unit": "rows/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{rows} rows x {vocab} bf16 logits (90% N(0,2^2) + 10% Student-t(3)x4), "
+                        f"top-k 64, top-p 0.9, T 0.8, penalties over a {history}-id history per "
+                        "row, output ids + chosen-token logprobs (BASELINE config 5)",
+            "rows": rows, "vocab": vocab, "logits": "bf16",
+        },
+        "us_per_step": ms * 1e3,
+        "decode_b4": {
+            "workload": "4 rows x 151936 f32 logits, 8192-id Zipf history, rep 1.05 / pres 0.3 / "
+                        "freq 0.2, k 20, p 0.95, min_p 0.05, T 0.6 (BASELINE config 2)",
+            "us_per_step": ms2 * 1e3,
+            "us_per_step_host_descriptors": ms2_call * 1e3,
+            "rows_per_s": 4 / (ms2 * 1e-3),
+            "achieved_GBs": bytes2 / (ms2 * 1e-3) / 1e9,
+            "target_us": 20.0,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "kernel": "k_rows_table<bf16>",
+            "bytes_per_row": bytes_row,
+        },
+    }
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(c5, rows, a.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

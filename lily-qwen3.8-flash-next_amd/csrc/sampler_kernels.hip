@@ -401,8 +401,8 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
         if (tid == 0) {
             const uint32_t slot = pick_sequential(sh.cum, n_keep, u1 * mass);
             const uint32_t id = composite_id(sh.cand[slot]);
+            write_logprob<DT>(a, sh, id, vocab);  // before the id is counted
             emit(a, id);
-            write_logprob<DT>(a, sh, id, vocab);
         }
         return;
     }
@@ -423,8 +423,8 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
     __syncthreads();
     if (u1 * sh.q_d < sh.p_d) {
         if (tid == 0) {
-            emit(a, d);
             write_logprob<DT>(a, sh, d, vocab);
+            emit(a, d);
         }
         return;
     }
@@ -464,8 +464,8 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
             slot = pick_sequential(sh.cum, n_keep, u2 * mass);
         }
         const uint32_t id = composite_id(sh.cand[slot]);
-        emit(a, id);
         write_logprob<DT>(a, sh, id, vocab);
+        emit(a, id);
     }
 }
 
@@ -631,8 +631,8 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
     }
     if (a.flags & F_FORCED) {
         if (tid == 0) {
-            emit(a, a.forced);
             write_logprob<DT>(a, sh, a.forced, vocab);
+            emit(a, a.forced);
         }
         return;
     }

@@ -9,6 +9,7 @@ There is no fallback: if the library is missing, importing this module raises.
 """
 import ctypes as C
 import os
+import weakref
 
 import torch
 
@@ -211,9 +212,12 @@ class Sampler:
         h = C.c_void_p()
         _check(_lib.lily_sampler_create(device, C.c_void_p(self.stream.cuda_stream), C.byref(h)))
         self._h = h
+        self._children = weakref.WeakSet()  # scratches, dists, plans: closed before the sampler
 
     def close(self):
         if self._h:
+            for child in list(self._children):
+                child.close()
             _lib.lily_sampler_destroy(self._h)
             self._h = None
 
@@ -270,7 +274,7 @@ class Sampler:
         m, vocab = logits.shape
         dtype = BF16 if logits.dtype == torch.bfloat16 else F32
         _check(_lib.lily_spec_verify(
-            self._h, _ptr(logits), dtype, vocab, logits.stride(0), m,
+            self._h, _ptr(logits), dtype, vocab, logits.stride(0) if m > 1 else vocab, m,
             scratch._h if scratch else None, C.byref(params), step0,
             dists._h if dists else None, _ptr(ids, torch.int32), _ptr(verify_tokens, torch.int32),
             _ptr(ctrl, torch.int32) if ctrl is not None else None,
@@ -289,7 +293,7 @@ class Sampler:
         if logits.dtype not in (torch.float32, torch.bfloat16) or logits.stride(1) != 1:
             raise SamplerError(-1, "logits must be F32 or BF16 [rows, V], rows contiguous")
         r.logits_dev = logits.data_ptr()
-        r.row_stride = logits.stride(0)
+        r.row_stride = logits.stride(0) if rows > 1 else vocab  # a [1, V] view may carry any stride
         parr = (SamplingParams * rows)(*params)
         sarr = (C.c_uint32 * rows)(*[int(s) for s in steps])
         keep += [parr, sarr]
@@ -354,6 +358,7 @@ class Plan:
         h = C.c_void_p()
         _check(_lib.lily_plan_create(sampler._h, logits.shape[0], C.byref(h)))
         self._h = h
+        sampler._children.add(self)
         r, self._keep = sampler._rows(logits, params, steps, out_ids, **kw)
         _check(_lib.lily_plan_set(self._h, C.byref(r)))
 
@@ -380,6 +385,7 @@ class SamplerScratch:
         h = C.c_void_p()
         _check(_lib.lily_scratch_create(sampler._h, vocab, C.byref(h)))
         self._h = h
+        sampler._children.add(self)
 
     def close(self):
         if self._h:
@@ -428,6 +434,7 @@ class DraftDists:
         h = C.c_void_p()
         _check(_lib.lily_draft_dists_create(sampler._h, slots, C.byref(h)))
         self._h = h
+        sampler._children.add(self)
 
     def close(self):
         if self._h:
