@@ -7,8 +7,10 @@
 
 namespace lily {
 
-hipError_t launch_rows(hipStream_t stream, int dtype, uint32_t rows, const LaunchCfg& cfg,
-                       const InlineRows* inline_rows);
+// `excl`: some row has a mask, penalties or a bias list; `lse`: some row wants a log-probability.
+// `dyn_bytes`: dynamic LDS = candidate slots, then the slice's exclusion bitmap.
+hipError_t launch_rows(hipStream_t stream, int dtype, bool excl, bool lse, uint32_t rows,
+                       const LaunchCfg& cfg, const InlineRows* inline_rows, size_t dyn_bytes);
 hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t v);
 hipError_t launch_add_history(hipStream_t stream, uint32_t* counts, uint32_t* touched,
                               uint32_t vocab, const uint32_t* ids, uint32_t n);

@@ -70,13 +70,14 @@ struct LaunchCfg {
     uint32_t ws_k;          // candidate slots per (row, slice) in ws_cand
     uint64_t* ws_cand;      // [rows][slices][ws_k] (value key << 32 | ~id)
     uint32_t* ws_n;         // [rows][slices] candidates written
-    float* ws_lse;          // [rows][slices][2] running max, sum of exp2
+    double* ws_lse;         // [rows][slices][2] log2-domain reference, sum of 2^(x - reference)
     uint32_t* ws_ticket;    // [rows] arrival counter, left at 0
-    uint32_t path;          // 0 = automatic, 1 = force the exhaustive select
-    uint32_t pad;
+    uint32_t path;          // 0 = automatic, 1 = exhaustive select only, 2 = two-pass select only
+    uint32_t cand_cap;      // candidate slots at the start of dynamic LDS (the bitmap follows)
 };
 
-constexpr uint32_t CAND_CAP = 4096;   // candidates one workgroup holds in LDS
+constexpr uint32_t CAND_CAP = 2048;   // candidates a workgroup collects while scanning
+constexpr uint32_t MERGE_CAP = 4096;  // candidates the merging workgroup gathers (slices x k)
 constexpr uint32_t MAX_SLICES = 64;
 
 }  // namespace lily

@@ -54,7 +54,7 @@ struct lily_sampler {
     hipStream_t stream = nullptr;
     uint64_t* ws_cand = nullptr;
     uint32_t* ws_n = nullptr;
-    float* ws_lse = nullptr;
+    double* ws_lse = nullptr;
     uint32_t* ws_ticket = nullptr;
     // Row table of lily_sample_rows batches above INLINE_ROWS.
     RowArgs* table_dev = nullptr;
@@ -93,6 +93,9 @@ struct lily_plan {
     uint32_t dtype = 0;
     uint32_t slices = 1;
     uint32_t ws_k = 0;
+    bool excl = false;
+    bool lse = false;
+    size_t dyn_bytes = 0;
 };
 
 namespace {
@@ -211,7 +214,7 @@ uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint
     uint32_t sl = s->force_slices ? s->force_slices : TARGET_GROUPS / rows;
     sl = sl < 1 ? 1 : sl;
     sl = sl > MAX_SLICES ? MAX_SLICES : sl;
-    const uint32_t by_k = CAND_CAP / (kmax ? kmax : 1);
+    const uint32_t by_k = MERGE_CAP / (kmax ? kmax : 1);
     sl = sl > by_k ? by_k : sl;
     const uint32_t by_len = (vocab + 2047u) / 2048u;
     sl = sl > by_len ? by_len : sl;
@@ -231,6 +234,35 @@ void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t sl
     cfg->ws_lse = s->ws_lse;
     cfg->ws_ticket = s->ws_ticket;
     cfg->path = s->force_path;
+    cfg->cand_cap = CAND_CAP;
+}
+
+// What a launch over `rows` needs beyond the configuration: which kernel variant and
+// how much dynamic LDS (candidate slots, then the widest slice's exclusion bitmap; the
+// merging workgroup reuses both for up to slices x k gathered candidates).
+struct LaunchShape {
+    bool excl = false;
+    bool lse = false;
+    size_t dyn_bytes = 0;
+};
+
+LaunchShape shape_of(const RowArgs* rows, uint32_t n, int dtype, uint32_t vocab, uint32_t slices,
+                     uint32_t kmax) {
+    LaunchShape sh;
+    for (uint32_t i = 0; i < n; ++i) {
+        sh.excl = sh.excl || rows[i].allow != nullptr || (rows[i].flags & F_PEN) || rows[i].n_bias;
+        sh.lse = sh.lse || rows[i].out_logprob != nullptr;
+    }
+    const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
+    const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
+    const uint32_t per = (nch + slices - 1) / slices;
+    const size_t bitmap = sh.excl ? ((size_t)(per * e + 31) / 32 + 2) * 4 : 0;
+    sh.dyn_bytes = (size_t)CAND_CAP * 8 + bitmap;
+    const size_t merge = slices > 1 ? (size_t)slices * kmax * 8 : 0;
+    if (merge > sh.dyn_bytes) {
+        sh.dyn_bytes = merge;
+    }
+    return sh;
 }
 
 uint32_t max_k(const RowArgs* rows, uint32_t n) {
@@ -247,8 +279,10 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     HIP_TRY(hipSetDevice(s->device));
     const uint32_t kmax = max_k(rows.r, n);
     LaunchCfg cfg;
-    fill_cfg(s, &cfg, vocab, choose_slices(s, n, kmax, vocab), kmax, 0, nullptr);
-    HIP_TRY(launch_rows(s->stream, dtype, n, cfg, &rows));
+    const uint32_t slices = choose_slices(s, n, kmax, vocab);
+    fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
+    const LaunchShape shp = shape_of(rows.r, n, dtype, vocab, slices, kmax);
+    HIP_TRY(launch_rows(s->stream, dtype, shp.excl, shp.lse, n, cfg, &rows, shp.dyn_bytes));
     return LILY_OK;
 }
 
@@ -476,9 +510,9 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     }
     const size_t slots = (size_t)WS_ROWS * MAX_SLICES;
     hipError_t err = hipMalloc(reinterpret_cast<void**>(&s->ws_cand),
-                               (size_t)WS_ROWS * CAND_CAP * sizeof(uint64_t));
+                               (size_t)WS_ROWS * MERGE_CAP * sizeof(uint64_t));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_n), slots * 4);
-    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 8);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 16);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
     if (err == hipSuccess) err = hipMemset(s->ws_ticket, 0, WS_ROWS * 4);
     for (uint32_t i = 0; i < STAGE_SLOTS && err == hipSuccess; ++i) {
@@ -837,8 +871,11 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     s->stage_used[slot] = true;
     const uint32_t kmax = max_k(s->stage[slot], b->rows);
     LaunchCfg cfg;
-    fill_cfg(s, &cfg, b->vocab, choose_slices(s, b->rows, kmax, b->vocab), kmax, 0, s->table_dev);
-    HIP_TRY(launch_rows(s->stream, (int)b->dtype, b->rows, cfg, nullptr));
+    const uint32_t slices = choose_slices(s, b->rows, kmax, b->vocab);
+    fill_cfg(s, &cfg, b->vocab, slices, kmax, 0, s->table_dev);
+    const LaunchShape shp = shape_of(s->stage[slot], b->rows, (int)b->dtype, b->vocab, slices, kmax);
+    HIP_TRY(launch_rows(s->stream, (int)b->dtype, shp.excl, shp.lse, b->rows, cfg, nullptr,
+                        shp.dyn_bytes));
     return LILY_OK;
 }
 
@@ -894,6 +931,11 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->dtype = b->dtype;
     p->ws_k = max_k(table.data(), b->rows);
     p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab);
+    const LaunchShape shp = shape_of(table.data(), b->rows, (int)b->dtype, b->vocab, p->slices,
+                                     p->ws_k);
+    p->excl = shp.excl;
+    p->lse = shp.lse;
+    p->dyn_bytes = shp.dyn_bytes;
     return LILY_OK;
 }
 
@@ -904,7 +946,8 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     HIP_TRY(hipSetDevice(p->s->device));
     LaunchCfg cfg;
     fill_cfg(p->s, &cfg, p->vocab, p->slices, p->ws_k, step_delta, p->table_dev);
-    HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->rows, cfg, nullptr));
+    HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->excl, p->lse, p->rows, cfg, nullptr,
+                        p->dyn_bytes));
     return LILY_OK;
 }
 

@@ -1,16 +1,36 @@
 // sampler_kernels.hip - gfx950 kernels of the logits-to-token stage.
 //
 // One launch serves a batch of logits rows.  Row r is scanned by `slices`
-// workgroups (grid = slices x rows); each finds the exact top-k of its slice
-// as 64-bit composites (order key of the adjusted value << 32 | ~id, so a
-// greater composite is a better candidate and the lowest id wins a tie).  With
-// several slices the last workgroup to arrive (an atomic ticket, nobody waits)
-// merges them.  That workgroup then runs the tail: sort, softmax over the
-// candidates, the sequential top-p / min-p prefix, the draw, and for the
-// speculative modes the export or the accept / residual draw.
+// workgroups of 512 threads (grid = slices x rows).  Each workgroup finds the
+// exact top-k of its slice as 64-bit composites (order key of the adjusted value
+// << 32 | ~id: a greater composite is a better candidate, the lowest id wins a
+// tie).  With several slices the last workgroup to arrive (an atomic ticket,
+// nobody waits) merges them.  That workgroup then runs the tail: sort, softmax
+// over the candidates, the sequential top-p / min-p prefix, the draw, and for
+// the speculative modes the export or the accept / residual draw.
 //
-// Arithmetic that decides a token id follows tests/unit/kernels/sample.rs:8-54
-// of the reference operation for operation (IEEE division by the temperature,
+// How a slice is scanned (select_fast):
+//   * 16-byte loads, 8 bf16 or 4 f32 per lane, four loads in flight per lane.
+//   * Ids that need more than "widen and compare" - masked out, penalised
+//     (count > 0) or biased - are marked in an LDS bitmap built once per slice;
+//     the stream treats them as -inf and the few that are allowed are evaluated
+//     exactly afterwards ("specials").
+//   * The filter works on the value BEFORE the division by the temperature (the
+//     division is monotone), so the hot loop has no division.  Candidates that
+//     pass go to an LDS buffer; the exact arithmetic runs on those only.
+//   * k <= 64: single pass.  Every lane keeps its running maximum; the minimum
+//     over G >= k lane groups of the group maximum is a lower bound of the k-th
+//     largest value (G distinct elements reach it), refreshed every block of
+//     loads; elements at or above it (less a 4-ulp slack for values the division
+//     merges) are appended.
+//   * k > 64: two passes.  The k-th largest of the 4 096 per-lane-per-slot
+//     running maxima is the bound; the second pass (L2 / MALL hits) collects.
+//   * Too many candidates (huge tie classes, adversarial order) or a failed
+//     slack check: the slice is redone by select_exhaustive, a radix select over
+//     the composites that re-evaluates every element and is correct for any input.
+//
+// Arithmetic that decides a token id follows tests/unit/kernels/sample.rs:8-54 of
+// the reference operation for operation (IEEE division by the temperature,
 // left-to-right f32 sums, lilym_expf); see include/lily_sampler_math.h.
 #include <hip/hip_runtime.h>
 
@@ -21,10 +41,13 @@ namespace lily {
 
 constexpr int NT = 512;
 constexpr int NWAVE = NT / 64;
+constexpr int UNROLL = 4;
 constexpr uint32_t K_CAP = LILY_SAMPLE_K_CAP;
-constexpr float LOG2E = 1.4426950408889634f;
+constexpr float F32_LOWEST = -3.4028234663852886e38f;
 
 #define NEG_INF (-__builtin_huge_valf())
+
+extern __shared__ uint64_t dyn_lds[];  // candidates, then the exclusion bitmap
 
 // ------------------------------------------------------------------ small helpers
 
@@ -92,64 +115,93 @@ __device__ __forceinline__ double wave_sum_d(double v) {
     }
     return v;
 }
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int o) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, o);
+    const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), o);
+    return ((uint64_t)hi << 32) | lo;
+}
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
     for (int o = 32; o > 0; o >>= 1) {
-        const uint64_t w = __shfl_xor((unsigned long long)v, o);
+        const uint64_t w = shfl_xor_u64(v, o);
         v = w > v ? w : v;
     }
     return v;
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t w = __shfl_xor(v, o);
+        v = w < v ? w : v;
+    }
+    return v;
+}
+
+// The value 4 order-key steps below t, not below the lowest finite float.
+__device__ __forceinline__ float lower_by_slack(float t) {
+    if (!(t > F32_LOWEST)) {
+        return F32_LOWEST;
+    }
+    const uint32_t key = lilym_order_key(t) - 4u;
+    return fmaxf(lilym_key_value(key), F32_LOWEST);
 }
 
 // ------------------------------------------------------------------ shared memory
 
 struct Shared {
-    uint64_t cand[CAND_CAP];   // candidates / sort area
-    float prob[K_CAP];         // exp(adjusted - top) per sorted candidate
-    float cum[K_CAP];          // inclusive prefix of the kept ones
-    float res[K_CAP];          // residual of the speculative draw
+    float prob[K_CAP];   // exp(adjusted - top) per sorted candidate
+    float cum[K_CAP];    // inclusive prefix of the kept ones
+    float res[K_CAP];    // residual of the speculative draw
     uint32_t hist[256];
     double red_d[NWAVE];
     float red_f[NWAVE];
     uint64_t red_u[NWAVE];
-    uint64_t prefix;
+    uint32_t red_i[NWAVE];
+    float wthr[NWAVE];      // each wave's threshold statistic (single-pass select)
+    float wthr_f[NWAVE];    // each wave's last filter threshold
     uint32_t n_cand;
     uint32_t need;
     uint32_t sel_bin;
+    uint32_t bin_count;
     uint32_t all_taken;
     uint32_t n_keep;
-    uint32_t pick;
     uint32_t last;
     float mass;
     float p_d;
     float q_d;
-    float lse_m;               // row maximum of the adjusted values (log2 domain reference)
-    double lse_s;              // sum of exp2((adjusted - lse_m) * log2e)
+    double lse_mc;   // log2-domain reference of the row's sum of exponentials
+    double lse_s;    // sum of 2^(x * log2e / T - lse_mc) over the row
 };
 
-// Running (maximum, sum of 2^((x - maximum) * log2e)) of one thread.
-struct Lse {
-    float m;
+// Running sum of 2^(v*c - mc) of one thread with its own reference mc.
+struct LseAcc {
+    float mc;
     float s;
-    __device__ void init() {
-        m = NEG_INF;
+    __device__ __forceinline__ void init() {
+        mc = NEG_INF;
         s = 0.0f;
     }
-    __device__ void add(float adj) {
-        if (!(adj > NEG_INF)) {
-            return;
+    // Raises the reference to cover block maximum cm; returns the reference to subtract.
+    __device__ __forceinline__ float rebase(float cm, float c) {
+        const float mcn = fmaxf(mc, cm * c);
+        const float safe = fmaxf(mcn, F32_LOWEST);
+        s *= __builtin_amdgcn_exp2f(mc - safe);
+        mc = mcn;
+        return safe;
+    }
+    __device__ __forceinline__ void term(float v, float c, float safe) {
+        s += __builtin_amdgcn_exp2f(__builtin_fmaf(v, c, -safe));
+    }
+    __device__ __forceinline__ void add_one(float v, float c) {
+        if (v > NEG_INF) {
+            const float safe = rebase(v, c);
+            term(v, c, safe);
         }
-        if (adj > m) {
-            s = s * exp2f((m - adj) * LOG2E);
-            m = adj;
-        }
-        s += exp2f((adj - m) * LOG2E);
     }
 };
 
-// Workgroup-wide merge of the threads' Lse into sh.lse_m / sh.lse_s.
-__device__ void lse_reduce(Shared& sh, const Lse& l) {
+// Workgroup-wide merge of the threads' accumulators into sh.lse_mc / sh.lse_s.
+__device__ void lse_reduce(Shared& sh, const LseAcc& l) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    float m = wave_max_f(l.m);
+    float m = wave_max_f(l.mc);
     if (lane == 0) {
         sh.red_f[w] = m;
     }
@@ -159,8 +211,8 @@ __device__ void lse_reduce(Shared& sh, const Lse& l) {
         m = fmaxf(m, sh.red_f[i]);
     }
     double s = 0.0;
-    if (l.m > NEG_INF) {
-        s = (double)l.s * exp2((double)(l.m - m) * (double)LOG2E);
+    if (l.mc > NEG_INF) {
+        s = (double)l.s * exp2((double)l.mc - (double)m);
     }
     s = wave_sum_d(s);
     if (lane == 0) {
@@ -172,25 +224,494 @@ __device__ void lse_reduce(Shared& sh, const Lse& l) {
         for (int i = 0; i < NWAVE; ++i) {
             t += sh.red_d[i];
         }
-        sh.lse_m = m;
+        sh.lse_mc = (double)m;
         sh.lse_s = t;
     }
     __syncthreads();
 }
 
-// ------------------------------------------------------------------ exhaustive select
-//
-// The exact top-k of elements [e0, e1) by a radix select on the composite:
-// eight passes of 8 bits, each re-evaluating every element.  Slow and correct
-// for any input (ties, masks, few finite values); the other paths fall back to
-// it.  Leaves the winners (unsorted) in sh.cand[0 .. sh.n_cand).
-template <int DT>
-__device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, uint32_t k,
-                                  bool want_lse, Shared& sh) {
+// ------------------------------------------------------------------ radix-select plumbing
+
+// With sh.hist complete: finds the bin in which the count from bin 255 downwards
+// reaches `need`.  Leaves sh.sel_bin, sh.need (what is still needed inside that
+// bin), sh.bin_count, and sh.all_taken = 1 when fewer than `need` were counted.
+__device__ void find_bin(Shared& sh, uint32_t need) {
+    if (threadIdx.x < 64) {
+        const uint32_t lane = threadIdx.x;
+        uint32_t h[4], sum = 0;
+        for (int j = 0; j < 4; ++j) {
+            h[j] = sh.hist[255u - (4u * lane + j)];
+            sum += h[j];
+        }
+        uint32_t incl = sum;
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t t = __shfl_up(incl, o);
+            if ((int)lane >= o) {
+                incl += t;
+            }
+        }
+        const uint32_t excl = incl - sum;
+        const uint32_t total = __shfl(incl, 63);
+        if (excl < need && need <= incl) {
+            uint32_t seen = excl;
+            for (int j = 0; j < 4; ++j) {
+                if (seen + h[j] >= need) {
+                    sh.sel_bin = 255u - (4u * lane + j);
+                    sh.need = need - seen;
+                    sh.bin_count = h[j];
+                    break;
+                }
+                seen += h[j];
+            }
+        }
+        if (lane == 0) {
+            sh.all_taken = total < need ? 1u : 0u;
+        }
+    }
+    __syncthreads();
+}
+
+// The top-k of cand[0..n) (zeros are invalid) compacted, unsorted, to the front;
+// returns how many there are.
+__device__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     uint64_t prefix = 0, pmask = 0;
     uint32_t need = k;
-    Lse lse;
+    bool all = false;
+    for (int pass = 0; pass < 8; ++pass) {
+        const int shift = 56 - 8 * pass;
+        if (tid < 256) {
+            sh.hist[tid] = 0;
+        }
+        __syncthreads();
+        for (uint32_t i = tid; i < n; i += NT) {
+            const uint64_t c = cand[i];
+            if (c != 0 && (c & pmask) == prefix) {
+                atomicAdd(&sh.hist[(uint32_t)(c >> shift) & 255u], 1u);
+            }
+        }
+        __syncthreads();
+        find_bin(sh, need);
+        if (sh.all_taken != 0u) {
+            all = true;
+            break;
+        }
+        prefix |= (uint64_t)sh.sel_bin << shift;
+        pmask |= (uint64_t)255u << shift;
+        const bool whole_bin = sh.bin_count == sh.need;
+        need = sh.need;
+        if (whole_bin) {
+            break;
+        }
+    }
+    const uint64_t floor_c = all ? 1ull : prefix;
+    uint64_t mine[8];
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t i = tid + (uint32_t)j * NT;
+        mine[j] = i < n ? cand[i] : 0ull;
+    }
+    if (tid == 0) {
+        sh.n_cand = 0;
+    }
+    __syncthreads();
+    for (int j = 0; j < 8; ++j) {
+        if (mine[j] != 0 && mine[j] >= floor_c) {
+            cand[atomicAdd(&sh.n_cand, 1u)] = mine[j];
+        }
+    }
+    __syncthreads();
+    return sh.n_cand;
+}
+
+// The k-th largest of the workgroup's NT x 8 per-lane values (-inf = absent) by a
+// radix select on their order keys; F32_LOWEST when fewer than k are present.
+__device__ float wg_kth_largest(const float (&ms)[8], uint32_t k, Shared& sh) {
+    const uint32_t tid = threadIdx.x;
+    uint32_t keys[8];
+    for (int j = 0; j < 8; ++j) {
+        keys[j] = ms[j] > NEG_INF ? lilym_order_key(ms[j]) : 0u;
+    }
+    uint32_t prefix = 0, pmask = 0, need = k;
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        if (tid < 256) {
+            sh.hist[tid] = 0;
+        }
+        __syncthreads();
+        for (int j = 0; j < 8; ++j) {
+            if (keys[j] != 0u && (keys[j] & pmask) == prefix) {
+                atomicAdd(&sh.hist[(keys[j] >> shift) & 255u], 1u);
+            }
+        }
+        __syncthreads();
+        find_bin(sh, need);
+        if (sh.all_taken != 0u) {
+            return F32_LOWEST;
+        }
+        prefix |= sh.sel_bin << shift;
+        pmask |= 255u << shift;
+        need = sh.need;
+    }
+    return lilym_key_value(prefix);
+}
+
+// ------------------------------------------------------------------ slice geometry
+
+// A row is read in 16-byte chunks from the 16-byte boundary at or below its first
+// element; `pad` elements of chunk 0 lie before the row.  Chunk c holds ids
+// c*E - pad .. c*E - pad + E - 1.
+template <int DT>
+struct Geo {
+    static constexpr int E = DT == LILY_BF16 ? 8 : 4;
+    const char* base;   // 16-byte aligned
+    uint32_t pad;
+    uint32_t cb, ce;    // this slice's chunks
+    uint32_t full_lo, full_hi;  // chunks lying wholly inside the row
+    uint32_t vocab;
+    uint32_t id_lo, id_hi;      // this slice's ids
+
+    __device__ void init(const void* logits, uint32_t v, uint32_t s, uint32_t slices) {
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(logits);
+        pad = (uint32_t)(addr & 15u) / (16u / E);
+        base = reinterpret_cast<const char*>(addr & ~(uintptr_t)15u);
+        vocab = v;
+        const uint32_t nch = (pad + v + E - 1) / E;
+        const uint32_t per = (nch + slices - 1) / slices;
+        cb = min(s * per, nch);
+        ce = min(cb + per, nch);
+        full_lo = pad ? 1u : 0u;
+        full_hi = (pad + v) / E;
+        const int64_t lo = (int64_t)cb * E - pad, hi = (int64_t)ce * E - pad;
+        id_lo = (uint32_t)max(lo, (int64_t)0);
+        id_hi = (uint32_t)min(hi, (int64_t)v);
+        if (id_hi < id_lo) {
+            id_hi = id_lo;
+        }
+    }
+
+    // Chunk c as floats; positions outside the row or the slice read as -inf.
+    __device__ __forceinline__ void load(const void* logits, uint32_t c, float (&v)[E]) const {
+        if (c >= full_lo && c < full_hi && c < ce) {
+            const uint4 q = *reinterpret_cast<const uint4*>(base + (size_t)c * 16);
+            if (DT == LILY_BF16) {
+                v[0] = lilym_bits_f32(q.x << 16);
+                v[1] = lilym_bits_f32(q.x & 0xffff0000u);
+                v[2] = lilym_bits_f32(q.y << 16);
+                v[3] = lilym_bits_f32(q.y & 0xffff0000u);
+                v[4 % E] = lilym_bits_f32(q.z << 16);
+                v[5 % E] = lilym_bits_f32(q.z & 0xffff0000u);
+                v[6 % E] = lilym_bits_f32(q.w << 16);
+                v[7 % E] = lilym_bits_f32(q.w & 0xffff0000u);
+            } else {
+                v[0] = lilym_bits_f32(q.x);
+                v[1] = lilym_bits_f32(q.y);
+                v[2] = lilym_bits_f32(q.z);
+                v[3] = lilym_bits_f32(q.w);
+            }
+        } else {
+            for (int j = 0; j < E; ++j) {
+                const int64_t id = (int64_t)c * E - pad + j;
+                v[j] = (c < ce && id >= 0 && id < (int64_t)vocab)
+                           ? load_logit<DT>(logits, (uint32_t)id)
+                           : NEG_INF;
+            }
+        }
+    }
+
+    __device__ __forceinline__ uint32_t id_of(uint32_t c, int j) const {
+        return c * E - pad + (uint32_t)j;
+    }
+};
+
+// 32 bits of bitmap `words` (bit index = id) starting at id0 (may be negative or
+// run past the end: those bits read 0).
+__device__ __forceinline__ uint32_t bits32_at(const uint32_t* words, uint32_t nwords, int64_t id0) {
+    const int64_t wi = id0 >> 5;
+    const uint32_t sh = (uint32_t)(id0 & 31);
+    const uint32_t w0 = (wi >= 0 && wi < (int64_t)nwords) ? words[wi] : 0u;
+    if (sh == 0) {
+        return w0;
+    }
+    const uint32_t w1 = (wi + 1 >= 0 && wi + 1 < (int64_t)nwords) ? words[wi + 1] : 0u;
+    return (w0 >> sh) | (w1 << (32u - sh));
+}
+
+// Bits of [id0, id0 + 32) that are ids in [lo, hi).
+__device__ __forceinline__ uint32_t range32_at(uint32_t lo, uint32_t hi, int64_t id0) {
+    const int64_t a = (int64_t)lo - id0 > 0 ? (int64_t)lo - id0 : 0;
+    const int64_t b = (int64_t)hi - id0 < 32 ? (int64_t)hi - id0 : 32;
+    if (b <= a) {
+        return 0u;
+    }
+    const uint32_t upto_b = b >= 32 ? 0xffffffffu : ((1u << b) - 1u);
+    const uint32_t upto_a = a >= 32 ? 0xffffffffu : ((1u << a) - 1u);
+    return upto_b & ~upto_a;
+}
+
+// ------------------------------------------------------------------ fast select
+
+// Appends the lanes with `pass` set to the candidate buffer (wave-aggregated).
+__device__ __forceinline__ void append(bool pass, float v, uint32_t id, uint64_t* cand,
+                                       uint32_t cap, Shared& sh) {
+    const uint64_t mask = __ballot(pass);
+    if (mask == 0) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t rank =
+        __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+    const int leader = __builtin_ctzll(mask);
+    uint32_t base = 0;
+    if ((int)lane == leader) {
+        base = atomicAdd(&sh.n_cand, (uint32_t)__popcll(mask));
+    }
+    base = __shfl(base, leader);
+    if (pass) {
+        const uint32_t at = base + rank;
+        if (at < cap) {
+            cand[at] = ((uint64_t)lilym_order_key(v) << 32) | (uint32_t)(~id);
+        }
+    }
+}
+
+// The exact top-k of the slice in cand[0..n) as adjusted-value composites,
+// unsorted, n returned through sh.n_cand; false when the slice must be redone
+// exhaustively.  Also leaves the slice's log-sum-exp in sh when LSE.
+template <int DT, bool EXCL, bool LSE>
+__device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool two_pass,
+                            uint64_t* cand, uint32_t cap, uint32_t* excl, Shared& sh) {
+    constexpr int E = Geo<DT>::E;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const uint32_t nchunks = g.ce - g.cb;
+    const uint32_t nwords = (nchunks * E + 31u) / 32u;
+    const uint32_t row_words = (g.vocab + 31u) / 32u;
+    const float c2 = a.c2;
+
+    if (tid == 0) {
+        sh.n_cand = 0;
+    }
+    if (tid < NWAVE) {
+        sh.wthr[tid] = NEG_INF;
+        sh.wthr_f[tid] = F32_LOWEST;
+    }
+    if (EXCL) {
+        // Bit b of the slice bitmap <-> id cb*E - pad + b.  Set = not streamed.
+        for (uint32_t i = tid; i < nwords; i += NT) {
+            const int64_t id0 = (int64_t)g.cb * E - g.pad + (int64_t)i * 32;
+            uint32_t x = ~range32_at(g.id_lo, g.id_hi, id0);
+            if (a.allow != nullptr) {
+                x |= ~bits32_at(a.allow, row_words, id0);
+            }
+            if (a.flags & F_PEN) {
+                x |= bits32_at(a.touched, row_words, id0);
+            }
+            excl[i] = x;
+        }
+        __syncthreads();
+        for (uint32_t i = tid; i < a.n_bias; i += NT) {
+            const uint32_t id = a.bias[i].id;
+            if (id >= g.id_lo && id < g.id_hi) {
+                const uint32_t b = id + g.pad - g.cb * E;
+                atomicOr(&excl[b >> 5], 1u << (b & 31u));
+            }
+        }
+    }
+    __syncthreads();
+
+    // Lanes per group: the largest power of two with NT / L >= k groups (at most a wave).
+    uint32_t group = 64;
+    while (group > 1 && NT / group < k) {
+        group >>= 1;
+    }
+
+    float lane_max = NEG_INF;
+    float ms[8];
+    for (int j = 0; j < 8; ++j) {
+        ms[j] = NEG_INF;
+    }
+    LseAcc lse;
+    lse.init();
+    float thr_f = F32_LOWEST;
+    const uint8_t* excl_bytes = reinterpret_cast<const uint8_t*>(excl);
+
+    for (int pass = 0; pass < (two_pass ? 2 : 1); ++pass) {
+        const bool filter = !two_pass || pass == 1;
+        for (uint32_t c0 = g.cb; c0 < g.ce; c0 += NT * UNROLL) {
+            float v[UNROLL][E];
+            for (int u = 0; u < UNROLL; ++u) {
+                g.load(a.logits, c0 + u * NT + tid, v[u]);
+            }
+            if (EXCL) {
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t c = c0 + u * NT + tid;
+                    if (c < g.ce) {
+                        const uint32_t rel = c - g.cb;
+                        uint32_t m;
+                        if (E == 8) {
+                            m = excl_bytes[rel];
+                        } else {
+                            m = (excl_bytes[rel >> 1] >> ((rel & 1u) * 4u)) & 15u;
+                        }
+                        for (int j = 0; j < E; ++j) {
+                            v[u][j] = ((m >> j) & 1u) ? NEG_INF : v[u][j];
+                        }
+                    }
+                }
+            }
+            if (pass == 0) {
+                float cm = NEG_INF;
+                for (int u = 0; u < UNROLL; ++u) {
+                    for (int j = 0; j < E; ++j) {
+                        cm = fmaxf(cm, v[u][j]);
+                        if (two_pass) {
+                            const int slot = (E == 8) ? j : ((u & 1) * 4 + j);
+                            ms[slot] = fmaxf(ms[slot], v[u][j]);
+                        }
+                    }
+                }
+                lane_max = fmaxf(lane_max, cm);
+                if (LSE) {
+                    const float safe = lse.rebase(cm, c2);
+                    for (int u = 0; u < UNROLL; ++u) {
+                        for (int j = 0; j < E; ++j) {
+                            lse.term(v[u][j], c2, safe);
+                        }
+                    }
+                }
+                if (!two_pass) {
+                    // Lower bound of the k-th largest: min over groups of the group maximum.
+                    float t = lane_max;
+                    for (uint32_t o = 1; o < group; o <<= 1) {
+                        t = fmaxf(t, __shfl_xor(t, (int)o));
+                    }
+                    for (uint32_t o = group; o < 64; o <<= 1) {
+                        t = fminf(t, __shfl_xor(t, (int)o));
+                    }
+                    if (lane == 0) {
+                        __hip_atomic_store(&sh.wthr[w], t, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                    if (c0 == g.cb) {
+                        __syncthreads();  // every wave has published its first statistic
+                    }
+                    for (int i = 0; i < NWAVE; ++i) {
+                        // Other waves' values may be older: still lower bounds.
+                        t = fminf(t, __hip_atomic_load(&sh.wthr[i], __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_WORKGROUP));
+                    }
+                    thr_f = fmaxf(thr_f, lower_by_slack(t));
+                }
+            }
+            if (filter) {
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t c = c0 + u * NT + tid;
+                    for (int j = 0; j < E; ++j) {
+                        append(v[u][j] >= thr_f, v[u][j], g.id_of(c, j), cand, cap, sh);
+                    }
+                }
+            }
+        }
+        if (two_pass && pass == 0) {
+            thr_f = lower_by_slack(wg_kth_largest(ms, k, sh));
+        }
+    }
+    if (lane == 0) {
+        sh.wthr_f[w] = thr_f;
+    }
+    __syncthreads();
+    float filt = sh.wthr_f[0];
+    for (int i = 1; i < NWAVE; ++i) {
+        filt = fmaxf(filt, sh.wthr_f[i]);
+    }
+    uint32_t n = sh.n_cand;
+    if (n > cap) {
+        return false;
+    }
+    // Buffered composites hold the pre-temperature value: divide now, exactly.
+    for (uint32_t i = tid; i < n; i += NT) {
+        const uint64_t c = cand[i];
+        cand[i] = composite_of(composite_value(c) / a.temperature, composite_id(c));
+    }
+    if (EXCL) {
+        // Specials: excluded from the stream but allowed ids (penalised or biased).
+        for (uint32_t i = tid; i < nwords; i += NT) {
+            const int64_t id0 = (int64_t)g.cb * E - g.pad + (int64_t)i * 32;
+            uint32_t bits = excl[i] & range32_at(g.id_lo, g.id_hi, id0);
+            if (a.allow != nullptr) {
+                bits &= bits32_at(a.allow, row_words, id0);
+            }
+            while (bits != 0u) {
+                const int b = __builtin_ctz(bits);
+                bits &= bits - 1u;
+                const uint32_t id = (uint32_t)(id0 + b);
+                const float u = pre_temperature_of<DT>(a, id);
+                if (LSE) {
+                    lse.add_one(u, c2);
+                }
+                if (u >= filt) {
+                    const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                    if (at < cap) {
+                        cand[at] = composite_of(u / a.temperature, id);
+                    }
+                }
+            }
+        }
+    }
+    if (LSE) {
+        lse_reduce(sh, lse);
+    } else {
+        __syncthreads();
+    }
+    n = sh.n_cand;
+    if (n > cap) {
+        return false;
+    }
+    if (n > k) {
+        n = wg_select_topk(cand, n, k, sh);
+    }
+    // Every element that was not collected lies strictly below `filt`; it must also
+    // lie strictly below the k-th adjusted value, or the division has merged it
+    // into the boundary's tie class.
+    if (filt > F32_LOWEST && n > 0) {
+        uint32_t lowest = 0xffffffffu;
+        for (uint32_t i = tid; i < n; i += NT) {
+            lowest = min(lowest, (uint32_t)(cand[i] >> 32));
+        }
+        lowest = wave_min_u32(lowest);
+        if (lane == 0) {
+            sh.red_i[w] = lowest;
+        }
+        __syncthreads();
+        lowest = sh.red_i[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            lowest = min(lowest, sh.red_i[i]);
+        }
+        __syncthreads();
+        const float below = lilym_key_value(lilym_order_key(filt) - 1u) / a.temperature;
+        if (!(lilym_order_key(below) < lowest)) {
+            return false;
+        }
+    }
+    if (tid == 0) {
+        sh.n_cand = n;
+    }
+    __syncthreads();
+    return true;
+}
+
+// ------------------------------------------------------------------ exhaustive select
+//
+// The exact top-k of ids [id_lo, id_hi) by a radix select on the composite: up to
+// eight passes of 8 bits, each re-evaluating every element.  Slow and correct for
+// any input (ties, masks, few finite values).  Leaves the winners (unsorted) in
+// cand[0 .. sh.n_cand).
+template <int DT>
+__device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, uint32_t k,
+                                  bool want_lse, uint64_t* cand, uint32_t cap, Shared& sh) {
+    const uint32_t tid = threadIdx.x;
+    uint64_t prefix = 0, pmask = 0;
+    uint32_t need = k;
+    LseAcc lse;
     lse.init();
     bool take_all = false;
     for (int pass = 0; pass < 8 && !take_all; ++pass) {
@@ -200,35 +721,17 @@ __device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, ui
         }
         __syncthreads();
         for (uint32_t id = e0 + tid; id < e1; id += NT) {
-            const float adj = adjusted_of<DT>(a, id);
+            const float u = pre_temperature_of<DT>(a, id);
             if (pass == 0 && want_lse) {
-                lse.add(adj);
+                lse.add_one(u, a.c2);
             }
-            const uint64_t c = composite_of(adj, id);
+            const uint64_t c = composite_of(u / a.temperature, id);
             if (c != 0 && (c & pmask) == prefix) {
                 atomicAdd(&sh.hist[(uint32_t)(c >> shift) & 255u], 1u);
             }
         }
         __syncthreads();
-        if (tid == 0) {
-            uint32_t seen = 0, bin = 0;
-            bool found = false;
-            for (int b = 255; b >= 0; --b) {
-                const uint32_t h = sh.hist[b];
-                if (seen + h >= need) {
-                    bin = (uint32_t)b;
-                    found = true;
-                    break;
-                }
-                seen += h;
-            }
-            // Fewer valid elements than asked for (only possible on the first
-            // pass, where every valid element is counted): take them all.
-            sh.all_taken = found ? 0u : 1u;
-            sh.sel_bin = bin;
-            sh.need = found ? need - seen : 0u;
-        }
-        __syncthreads();
+        find_bin(sh, need);
         take_all = sh.all_taken != 0u;
         if (!take_all) {
             prefix |= (uint64_t)sh.sel_bin << shift;
@@ -248,8 +751,8 @@ __device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, ui
         const uint64_t c = composite_of(adjusted_of<DT>(a, id), id);
         if (c >= floor_c && c != 0) {
             const uint32_t at = atomicAdd(&sh.n_cand, 1u);
-            if (at < CAND_CAP) {
-                sh.cand[at] = c;
+            if (at < cap) {
+                cand[at] = c;
             }
         }
     }
@@ -258,14 +761,33 @@ __device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, ui
 
 // ------------------------------------------------------------------ sort
 
-// Bitonic sort, descending, of sh.cand[0..n) padded with zeros to a power of two.
-__device__ void sort_desc(Shared& sh, uint32_t n) {
-    uint32_t p = 2;
+// Descending sort of cand[0..n).  Up to 64 entries: one wave, in registers.
+// More: bitonic in LDS over the next power of two (the buffer holds it).
+__device__ void sort_desc(uint64_t* cand, uint32_t n) {
+    if (n <= 64) {
+        if (threadIdx.x < 64) {
+            const uint32_t lane = threadIdx.x;
+            uint64_t c = lane < n ? cand[lane] : 0ull;
+            for (uint32_t size = 2; size <= 64; size <<= 1) {
+                for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+                    const uint64_t o = shfl_xor_u64(c, (int)stride);
+                    const bool desc = (lane & size) == 0;
+                    const bool lower = (lane & stride) == 0;
+                    const bool take_max = lower == desc;
+                    c = take_max ? (o > c ? o : c) : (o < c ? o : c);
+                }
+            }
+            cand[lane] = c;
+        }
+        __syncthreads();
+        return;
+    }
+    uint32_t p = 128;
     while (p < n) {
         p <<= 1;
     }
     for (uint32_t i = n + threadIdx.x; i < p; i += NT) {
-        sh.cand[i] = 0;
+        cand[i] = 0;
     }
     __syncthreads();
     for (uint32_t size = 2; size <= p; size <<= 1) {
@@ -274,10 +796,10 @@ __device__ void sort_desc(Shared& sh, uint32_t n) {
                 const uint32_t pos = ((i / stride) * (stride << 1)) + (i % stride);
                 const uint32_t partner = pos + stride;
                 const bool desc = (pos & size) == 0;
-                const uint64_t x = sh.cand[pos], y = sh.cand[partner];
+                const uint64_t x = cand[pos], y = cand[partner];
                 if (desc ? x < y : x > y) {
-                    sh.cand[pos] = y;
-                    sh.cand[partner] = x;
+                    cand[pos] = y;
+                    cand[partner] = x;
                 }
             }
             __syncthreads();
@@ -305,6 +827,8 @@ __device__ uint32_t pick_sequential(const float* prefix, uint32_t n, float targe
     return n - 1;
 }
 
+// log p(id) = (u*c2 - mc - log2 s) * ln 2, with the id's exponent u*c2 formed exactly as
+// the row sum formed its terms, so the two cancel when the id carries all the mass.
 template <int DT>
 __device__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
     if (a.out_logprob == nullptr) {
@@ -312,26 +836,27 @@ __device__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, u
     }
     float lp = NEG_INF;
     if (id < vocab) {
-        const float adj = adjusted_of<DT>(a, id);
-        if (adj > NEG_INF) {
-            const double lse = (double)sh.lse_m + log(sh.lse_s);
-            lp = (float)((double)adj - lse);
+        const float u = pre_temperature_of<DT>(a, id);
+        if (u > NEG_INF) {
+            const double e = (double)u * (double)a.c2 - sh.lse_mc - log2(sh.lse_s);
+            lp = fminf((float)(e * 0.6931471805599453), 0.0f);  // the sum is approximate: clamp
         }
     }
     *a.out_logprob = lp;
 }
 
-// sh.cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
+// cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
 template <int DT>
-__device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, Shared& sh) {
+__device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, uint64_t* cand,
+                     Shared& sh) {
     const uint32_t tid = threadIdx.x;
     if (n == 0) {
         // No finite value anywhere: the oracle's order then starts at id 0.
         if (tid == 0) {
-            emit(a, 0);
             if (a.out_logprob) {
                 *a.out_logprob = NEG_INF;
             }
+            emit(a, 0);
             if (a.dbg_counts) {
                 a.dbg_counts[0] = 0;
                 a.dbg_counts[1] = 0;
@@ -342,14 +867,14 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
         }
         return;
     }
-    sort_desc(sh, n);
+    sort_desc(cand, n);
     const uint32_t k = min(a.k, n);
-    const float top = composite_value(sh.cand[0]);
+    const float top = composite_value(cand[0]);
     for (uint32_t i = tid; i < k; i += NT) {
-        const float p = lilym_expf(composite_value(sh.cand[i]) - top);
+        const float p = lilym_expf(composite_value(cand[i]) - top);
         sh.prob[i] = p;
         if (a.dbg_ids) {
-            a.dbg_ids[i] = composite_id(sh.cand[i]);
+            a.dbg_ids[i] = composite_id(cand[i]);
         }
         if (a.dbg_probs) {
             a.dbg_probs[i] = p;
@@ -389,7 +914,7 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
 
     if (a.mode == MODE_DRAFT) {
         for (uint32_t i = tid; i < n_keep; i += NT) {
-            a.q_ids[i] = composite_id(sh.cand[i]);
+            a.q_ids[i] = composite_id(cand[i]);
             a.q_probs[i] = sh.prob[i] / mass;
         }
         if (tid == 0) {
@@ -400,7 +925,7 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
     if (a.mode != MODE_SPEC) {
         if (tid == 0) {
             const uint32_t slot = pick_sequential(sh.cum, n_keep, u1 * mass);
-            const uint32_t id = composite_id(sh.cand[slot]);
+            const uint32_t id = composite_id(cand[slot]);
             write_logprob<DT>(a, sh, id, vocab);  // before the id is counted
             emit(a, id);
         }
@@ -411,7 +936,7 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
     const uint32_t d = *a.draft;
     const uint32_t qn = min(*a.q_n, K_CAP);
     for (uint32_t i = tid; i < n_keep; i += NT) {
-        if (composite_id(sh.cand[i]) == d) {
+        if (composite_id(cand[i]) == d) {
             sh.p_d = sh.prob[i] / mass;
         }
     }
@@ -429,7 +954,7 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
         return;
     }
     for (uint32_t i = tid; i < n_keep; i += NT) {
-        const uint32_t id = composite_id(sh.cand[i]);
+        const uint32_t id = composite_id(cand[i]);
         float q_i = 0.0f;
         for (uint32_t j = 0; j < qn; ++j) {
             if (a.q_ids[j] == id) {
@@ -463,7 +988,7 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
             // Only rounding gives a rejected proposal a massless residual: draw from p.
             slot = pick_sequential(sh.cum, n_keep, u2 * mass);
         }
-        const uint32_t id = composite_id(sh.cand[slot]);
+        const uint32_t id = composite_id(cand[slot]);
         write_logprob<DT>(a, sh, id, vocab);
         emit(a, id);
     }
@@ -472,24 +997,36 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
 // ------------------------------------------------------------------ argmax
 
 // First maximum under float comparison (NaN never wins, -0 == +0), lowest id on
-// ties: elementwise.metal:145-150.  Result: the best composite of [e0, e1).
+// ties: elementwise.metal:145-150.  Result: the best (value, id) of the slice as a
+// composite; id bits all zero when no element qualified.
 template <int DT>
-__device__ uint64_t slice_argmax(const RowArgs& a, uint32_t e0, uint32_t e1, Shared& sh) {
-    uint64_t best = 0;
-    for (uint32_t id = e0 + threadIdx.x; id < e1; id += NT) {
-        float v = load_logit<DT>(a.logits, id);
-        uint64_t c;
-        if (v != v) {
-            c = (uint64_t)(uint32_t)(~id);  // below every number, lowest id first
-        } else {
-            v = v + 0.0f;  // -0 -> +0
-            c = ((uint64_t)lilym_order_key(v) << 32) | (uint32_t)(~id);
+__device__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>& g, Shared& sh) {
+    constexpr int E = Geo<DT>::E;
+    const uint32_t tid = threadIdx.x;
+    float bv = NEG_INF;
+    uint32_t bi = 0xffffffffu;
+    for (uint32_t c0 = g.cb; c0 < g.ce; c0 += NT * UNROLL) {
+        float v[UNROLL][E];
+        for (int u = 0; u < UNROLL; ++u) {
+            g.load(a.logits, c0 + u * NT + tid, v[u]);
         }
-        best = c > best ? c : best;
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t c = c0 + u * NT + tid;
+            for (int j = 0; j < E; ++j) {
+                const uint32_t id = g.id_of(c, j);
+                const bool inside = c < g.ce && id < g.vocab;  // id wraps for the pad
+                const float x = v[u][j];
+                if (inside && (x > bv || (x == bv && id < bi))) {
+                    bv = x;
+                    bi = id;
+                }
+            }
+        }
     }
+    uint64_t best = ((uint64_t)lilym_order_key(bv + 0.0f) << 32) | (uint32_t)(~bi);
     best = wave_max_u64(best);
-    if ((threadIdx.x & 63) == 0) {
-        sh.red_u[threadIdx.x >> 6] = best;
+    if ((tid & 63u) == 0) {
+        sh.red_u[tid >> 6] = best;
     }
     __syncthreads();
     best = sh.red_u[0];
@@ -502,13 +1039,15 @@ __device__ uint64_t slice_argmax(const RowArgs& a, uint32_t e0, uint32_t e1, Sha
 
 // ------------------------------------------------------------------ the row kernel
 
-template <int DT>
+template <int DT, bool EXCL, bool LSE>
 __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     const uint32_t s = blockIdx.x, row = blockIdx.y, S = cfg.slices;
     const uint32_t vocab = cfg.vocab;
     const uint32_t step = a.step + cfg.step_delta;
-    const bool want_lse = a.out_logprob != nullptr;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    uint64_t* cand = dyn_lds;
+    uint32_t* excl = reinterpret_cast<uint32_t*>(dyn_lds + cfg.cand_cap);
 
     if ((a.flags & F_FORCED) && !want_lse) {
         if (s == 0 && tid == 0) {
@@ -517,22 +1056,19 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
         return;
     }
 
-    // Slice bounds in elements: equal slices, a multiple of 2048 long.
-    uint32_t len = (vocab + S - 1) / S;
-    len = (len + 2047u) & ~2047u;
-    const uint32_t e0 = min(s * len, vocab);
-    const uint32_t e1 = min(e0 + len, vocab);
+    Geo<DT> g;
+    g.init(a.logits, vocab, s, S);
 
     const bool argmax = a.mode == MODE_ARGMAX;
     uint64_t best = 0;
     if (argmax) {
-        best = slice_argmax<DT>(a, e0, e1, sh);
+        best = slice_argmax<DT>(a, g, sh);
     } else if (a.flags & F_FORCED) {
         // Only the row's log-sum-exp is needed.
-        Lse lse;
+        LseAcc lse;
         lse.init();
-        for (uint32_t id = e0 + tid; id < e1; id += NT) {
-            lse.add(adjusted_of<DT>(a, id));
+        for (uint32_t id = g.id_lo + tid; id < g.id_hi; id += NT) {
+            lse.add_one(pre_temperature_of<DT>(a, id), a.c2);
         }
         lse_reduce(sh, lse);
         if (tid == 0) {
@@ -540,10 +1076,21 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
         }
         __syncthreads();
     } else {
-        select_exhaustive<DT>(a, e0, e1, a.k, want_lse, sh);
+        bool done = false;
+        if (cfg.path != 1u) {
+            const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
+            if (EXCL || !special) {
+                const bool two_pass = a.k > 64u || cfg.path == 2u;
+                done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh);
+            }
+        }
+        if (!done) {
+            __syncthreads();
+            select_exhaustive<DT>(a, g.id_lo, g.id_hi, a.k, want_lse, cand, cfg.cand_cap, sh);
+        }
     }
 
-    uint32_t n = argmax ? 0u : min(sh.n_cand, CAND_CAP);
+    uint32_t n = argmax ? 0u : min(sh.n_cand, cfg.cand_cap);
     if (S > 1) {
         const size_t slot = (size_t)row * S + s;
         if (argmax) {
@@ -552,12 +1099,12 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
             }
         } else {
             for (uint32_t i = tid; i < n; i += NT) {
-                cfg.ws_cand[slot * cfg.ws_k + i] = sh.cand[i];
+                cfg.ws_cand[slot * cfg.ws_k + i] = cand[i];
             }
             if (tid == 0) {
                 cfg.ws_n[slot] = n;
-                cfg.ws_lse[2 * slot] = sh.lse_m;
-                cfg.ws_lse[2 * slot + 1] = (float)sh.lse_s;
+                cfg.ws_lse[2 * slot] = want_lse ? sh.lse_mc : 0.0;
+                cfg.ws_lse[2 * slot + 1] = want_lse ? sh.lse_s : 0.0;
             }
         }
         __threadfence();
@@ -583,7 +1130,7 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
                 best = c > best ? c : best;
             }
             best = wave_max_u64(best);
-            if ((tid & 63) == 0) {
+            if ((tid & 63u) == 0) {
                 sh.red_u[tid >> 6] = best;
             }
             __syncthreads();
@@ -597,35 +1144,42 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
             for (uint32_t t = 0; t < S; ++t) {
                 const uint32_t nt = __builtin_nontemporal_load(&cfg.ws_n[base + t]);
                 for (uint32_t i = tid; i < nt; i += NT) {
-                    sh.cand[total + i] =
+                    cand[total + i] =
                         __builtin_nontemporal_load(&cfg.ws_cand[(base + t) * cfg.ws_k + i]);
                 }
                 total += nt;
             }
-            n = total;
             if (want_lse && tid == 0) {
-                float m = NEG_INF;
+                double m = -__builtin_huge_val();
                 for (uint32_t t = 0; t < S; ++t) {
-                    m = fmaxf(m, __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t)]));
+                    const double st = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t) + 1]);
+                    if (st > 0.0) {
+                        m = fmax(m, __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t)]));
+                    }
                 }
                 double sum = 0.0;
                 for (uint32_t t = 0; t < S; ++t) {
-                    const float mt = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t)]);
-                    const float st = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t) + 1]);
-                    if (mt > NEG_INF) {
-                        sum += (double)st * exp2((double)(mt - m) * (double)LOG2E);
+                    const double mt = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t)]);
+                    const double st = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t) + 1]);
+                    if (st > 0.0) {
+                        sum += st * exp2(mt - m);
                     }
                 }
-                sh.lse_m = m;
+                sh.lse_mc = m;
                 sh.lse_s = sum;
             }
             __syncthreads();
+            n = total;
+            if (n > a.k) {
+                n = wg_select_topk(cand, n, a.k, sh);
+            }
         }
     }
 
     if (argmax) {
         if (tid == 0) {
-            *a.out_id = composite_id(best);
+            const uint32_t id = composite_id(best);
+            *a.out_id = id == 0xffffffffu ? 0u : id;
         }
         return;
     }
@@ -636,16 +1190,16 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
         }
         return;
     }
-    tail<DT>(a, vocab, step, n, sh);
+    tail<DT>(a, vocab, step, n, cand, sh);
 }
 
-template <int DT>
+template <int DT, bool EXCL, bool LSE>
 __global__ __launch_bounds__(NT) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
     __shared__ Shared sh;
-    row_body<DT>(rows.r[blockIdx.y], cfg, sh);
+    row_body<DT, EXCL, LSE>(rows.r[blockIdx.y], cfg, sh);
 }
 
-template <int DT>
+template <int DT, bool EXCL, bool LSE>
 __global__ __launch_bounds__(NT) void k_rows_table(LaunchCfg cfg) {
     __shared__ Shared sh;
     __shared__ RowArgs a;
@@ -655,7 +1209,7 @@ __global__ __launch_bounds__(NT) void k_rows_table(LaunchCfg cfg) {
             reinterpret_cast<const uint32_t*>(&cfg.table[blockIdx.y])[threadIdx.x];
     }
     __syncthreads();
-    row_body<DT>(a, cfg, sh);
+    row_body<DT, EXCL, LSE>(a, cfg, sh);
 }
 
 // ------------------------------------------------------------------ small kernels
@@ -741,23 +1295,33 @@ __global__ void k_copy_row_u32(const uint32_t* src, uint32_t* dst, uint32_t word
 
 // ------------------------------------------------------------------ launchers (host)
 
-hipError_t launch_rows(hipStream_t stream, int dtype, uint32_t rows, const LaunchCfg& cfg,
-                       const InlineRows* inline_rows) {
+template <int DT, bool EXCL, bool LSE>
+static hipError_t launch_variant(hipStream_t stream, uint32_t rows, const LaunchCfg& cfg,
+                                 const InlineRows* inline_rows, size_t dyn_bytes) {
     const dim3 grid(cfg.slices, rows), block(NT);
     if (inline_rows != nullptr) {
-        if (dtype == LILY_BF16) {
-            hipLaunchKernelGGL(k_rows_inline<LILY_BF16>, grid, block, 0, stream, *inline_rows, cfg);
-        } else {
-            hipLaunchKernelGGL(k_rows_inline<LILY_F32>, grid, block, 0, stream, *inline_rows, cfg);
-        }
+        hipLaunchKernelGGL((k_rows_inline<DT, EXCL, LSE>), grid, block, dyn_bytes, stream,
+                           *inline_rows, cfg);
     } else {
-        if (dtype == LILY_BF16) {
-            hipLaunchKernelGGL(k_rows_table<LILY_BF16>, grid, block, 0, stream, cfg);
-        } else {
-            hipLaunchKernelGGL(k_rows_table<LILY_F32>, grid, block, 0, stream, cfg);
-        }
+        hipLaunchKernelGGL((k_rows_table<DT, EXCL, LSE>), grid, block, dyn_bytes, stream, cfg);
     }
     return hipGetLastError();
+}
+
+hipError_t launch_rows(hipStream_t stream, int dtype, bool excl, bool lse, uint32_t rows,
+                       const LaunchCfg& cfg, const InlineRows* inline_rows, size_t dyn_bytes) {
+#define LILY_DISPATCH(DT)                                                                      \
+    if (excl) {                                                                                \
+        return lse ? launch_variant<DT, true, true>(stream, rows, cfg, inline_rows, dyn_bytes)  \
+                   : launch_variant<DT, true, false>(stream, rows, cfg, inline_rows, dyn_bytes); \
+    }                                                                                          \
+    return lse ? launch_variant<DT, false, true>(stream, rows, cfg, inline_rows, dyn_bytes)     \
+               : launch_variant<DT, false, false>(stream, rows, cfg, inline_rows, dyn_bytes);
+    if (dtype == LILY_BF16) {
+        LILY_DISPATCH(LILY_BF16)
+    }
+    LILY_DISPATCH(LILY_F32)
+#undef LILY_DISPATCH
 }
 
 hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t v) {
