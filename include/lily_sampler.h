@@ -110,6 +110,16 @@ void lily_sampler_destroy(lily_sampler_t* s);
 /* ComputePass::commit_wait (src/metal.rs:2290): blocks until the stream has drained. */
 int lily_sampler_synchronize(lily_sampler_t* s);
 
+/* Per-kernel profile transport of the reference (LILY_KERNEL_PROFILE, src/metal.rs:30-33,
+ * :140-198) at a finer grain: while trace_dev is set, thread 0 of every workgroup of the row
+ * kernels stores the 100 MHz device wall clock at 8 phase boundaries into
+ * trace_dev[(row * slices + slice) * 8 + phase] (u64; phases: 0 start, 1 bitmap built,
+ * 2 scan done, 3 specials done, 4 slice top-k done, 5 ticket taken, 6 merge done, 7 row
+ * done).  capacity_words bounds rows * slices * 8; larger launches run untraced.  NULL stops. */
+int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_t capacity_words);
+/* Workgroups per row the next launch of `rows` rows with candidate count k would use. */
+uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab);
+
 /* ---- SamplerScratch ------------------------------------------------------------------- */
 
 /* SamplerScratch::new (sample.rs:131-143).  Device state: the emission histogram

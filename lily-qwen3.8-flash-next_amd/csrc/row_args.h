@@ -74,10 +74,16 @@ struct LaunchCfg {
     uint32_t* ws_ticket;    // [rows] arrival counter, left at 0
     uint32_t path;          // 0 = automatic, 1 = exhaustive select only, 2 = two-pass select only
     uint32_t cand_cap;      // candidate slots at the start of dynamic LDS (the bitmap follows)
+    uint64_t* phase_trace;  // null, or [rows][slices][PHASE_SLOTS] 100 MHz timestamps
+    uint32_t excl_words;    // words reserved for the slice bitmap (the specials' id list follows)
+    uint32_t pad;
 };
+
+constexpr uint32_t PHASE_SLOTS = 8;
 
 constexpr uint32_t CAND_CAP = 2048;   // candidates a workgroup collects while scanning
 constexpr uint32_t MERGE_CAP = 4096;  // candidates the merging workgroup gathers (slices x k)
 constexpr uint32_t MAX_SLICES = 64;
+constexpr uint32_t SPECIAL_LIST_CAP = 2048;  // ids of penalised / biased tokens gathered per batch
 
 }  // namespace lily

@@ -66,6 +66,8 @@ struct lily_sampler {
     uint32_t stage_next = 0;
     uint32_t force_path = 0;
     uint32_t force_slices = 0;
+    uint64_t* phase_trace = nullptr;
+    uint64_t phase_words = 0;
 };
 
 struct lily_scratch {
@@ -96,6 +98,7 @@ struct lily_plan {
     bool excl = false;
     bool lse = false;
     size_t dyn_bytes = 0;
+    uint32_t excl_words = 0;
 };
 
 namespace {
@@ -237,6 +240,14 @@ void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t sl
     cfg->cand_cap = CAND_CAP;
 }
 
+// Attaches the phase trace when the launch fits the caller's buffer.
+void attach_trace(const lily_sampler* s, LaunchCfg* cfg, uint32_t rows) {
+    if (s->phase_trace != nullptr &&
+        (uint64_t)rows * cfg->slices * PHASE_SLOTS <= s->phase_words) {
+        cfg->phase_trace = s->phase_trace;
+    }
+}
+
 // What a launch over `rows` needs beyond the configuration: which kernel variant and
 // how much dynamic LDS (candidate slots, then the widest slice's exclusion bitmap; the
 // merging workgroup reuses both for up to slices x k gathered candidates).
@@ -244,6 +255,7 @@ struct LaunchShape {
     bool excl = false;
     bool lse = false;
     size_t dyn_bytes = 0;
+    uint32_t excl_words = 0;
 };
 
 LaunchShape shape_of(const RowArgs* rows, uint32_t n, int dtype, uint32_t vocab, uint32_t slices,
@@ -256,8 +268,13 @@ LaunchShape shape_of(const RowArgs* rows, uint32_t n, int dtype, uint32_t vocab,
     const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
     const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
     const uint32_t per = (nch + slices - 1) / slices;
-    const size_t bitmap = sh.excl ? ((size_t)(per * e + 31) / 32 + 2) * 4 : 0;
+    sh.excl_words = sh.excl ? (per * e + 31) / 32 + 2 : 0;
+    const size_t bitmap = sh.excl ? ((size_t)sh.excl_words + SPECIAL_LIST_CAP) * 4 : 0;
     sh.dyn_bytes = (size_t)CAND_CAP * 8 + bitmap;
+    const size_t tail = (size_t)LILY_SAMPLE_K_CAP * 8 + 3 * (size_t)LILY_SAMPLE_K_CAP * 4;
+    if (tail > sh.dyn_bytes) {
+        sh.dyn_bytes = tail;
+    }
     const size_t merge = slices > 1 ? (size_t)slices * kmax * 8 : 0;
     if (merge > sh.dyn_bytes) {
         sh.dyn_bytes = merge;
@@ -281,7 +298,9 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     LaunchCfg cfg;
     const uint32_t slices = choose_slices(s, n, kmax, vocab);
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
+    attach_trace(s, &cfg, n);
     const LaunchShape shp = shape_of(rows.r, n, dtype, vocab, slices, kmax);
+    cfg.excl_words = shp.excl_words;
     HIP_TRY(launch_rows(s->stream, dtype, shp.excl, shp.lse, n, cfg, &rows, shp.dyn_bytes));
     return LILY_OK;
 }
@@ -542,6 +561,22 @@ void lily_sampler_destroy(lily_sampler_t* s) {
         if (s->stage_done[i]) (void)hipEventDestroy(s->stage_done[i]);
     }
     delete s;
+}
+
+int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_t capacity_words) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    s->phase_trace = trace_dev;
+    s->phase_words = trace_dev ? capacity_words : 0;
+    return LILY_OK;
+}
+
+uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab) {
+    if (s == nullptr || rows == 0) {
+        return 0;
+    }
+    return choose_slices(s, rows, k ? k : 1, vocab);
 }
 
 int lily_sampler_synchronize(lily_sampler_t* s) {
@@ -873,7 +908,9 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     LaunchCfg cfg;
     const uint32_t slices = choose_slices(s, b->rows, kmax, b->vocab);
     fill_cfg(s, &cfg, b->vocab, slices, kmax, 0, s->table_dev);
+    attach_trace(s, &cfg, b->rows);
     const LaunchShape shp = shape_of(s->stage[slot], b->rows, (int)b->dtype, b->vocab, slices, kmax);
+    cfg.excl_words = shp.excl_words;
     HIP_TRY(launch_rows(s->stream, (int)b->dtype, shp.excl, shp.lse, b->rows, cfg, nullptr,
                         shp.dyn_bytes));
     return LILY_OK;
@@ -936,6 +973,7 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->excl = shp.excl;
     p->lse = shp.lse;
     p->dyn_bytes = shp.dyn_bytes;
+    p->excl_words = shp.excl_words;
     return LILY_OK;
 }
 
@@ -946,6 +984,8 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     HIP_TRY(hipSetDevice(p->s->device));
     LaunchCfg cfg;
     fill_cfg(p->s, &cfg, p->vocab, p->slices, p->ws_k, step_delta, p->table_dev);
+    attach_trace(p->s, &cfg, p->rows);
+    cfg.excl_words = p->excl_words;
     HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->excl, p->lse, p->rows, cfg, nullptr,
                         p->dyn_bytes));
     return LILY_OK;

@@ -51,16 +51,35 @@ extern __shared__ uint64_t dyn_lds[];  // candidates, then the exclusion bitmap
 
 // ------------------------------------------------------------------ small helpers
 
+// Loads through a pointer known to be device memory: global_load instead of flat_load
+// (the row's pointers arrive through LDS, so the compiler cannot tell by itself).
+#define LILY_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <class T>
+__device__ __forceinline__ T gload(const T* p) {
+    return *(const LILY_GLOBAL T*)p;
+}
+// Device-scope accesses that go through to memory, for data another workgroup (on any
+// XCD, behind another L2) will read after taking the row's ticket.
+template <class T>
+__device__ __forceinline__ void store_through(T* p, T v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class T>
+__device__ __forceinline__ T load_through(const T* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int DT>
 __device__ __forceinline__ float load_logit(const void* p, uint32_t i) {
     if (DT == LILY_BF16) {
-        return lilym_bits_f32((uint32_t) static_cast<const uint16_t*>(p)[i] << 16);
+        return lilym_bits_f32((uint32_t)gload(static_cast<const uint16_t*>(p) + i) << 16);
     }
-    return static_cast<const float*>(p)[i];
+    return gload(static_cast<const float*>(p) + i);
 }
 
 __device__ __forceinline__ bool bit_of(const uint32_t* words, uint32_t id) {
-    return (words[id >> 5] >> (id & 31u)) & 1u;
+    return (gload(words + (id >> 5)) >> (id & 31u)) & 1u;
 }
 
 __device__ __forceinline__ uint64_t composite_of(float adj, uint32_t id) {
@@ -74,28 +93,33 @@ __device__ __forceinline__ float composite_value(uint64_t c) {
     return lilym_key_value((uint32_t)(c >> 32));
 }
 
-// The value before the temperature, exactly as the oracle's map: bias (list
-// order), mask, penalties.
+// The oracle's map on a loaded logit l with emission count c: bias (list order), mask,
+// penalties; the division by the temperature is the caller's.
+__device__ __forceinline__ float finish_pre_temperature(const RowArgs& a, uint32_t id, float l,
+                                                        uint32_t c, bool allowed) {
+    for (uint32_t j = 0; j < a.n_bias; ++j) {
+        const uint32_t bid = gload(&a.bias[j].id);
+        if (bid == id) {
+            l += gload(&a.bias[j].delta);
+        }
+    }
+    if (!allowed) {
+        return NEG_INF;
+    }
+    if (c > 0u) {
+        l = l > 0.0f ? l / a.repetition : l * a.repetition;
+        l -= a.presence + a.frequency * (float)c;
+    }
+    return l;
+}
+
+// The value before the temperature of one id, loads included.
 template <int DT>
 __device__ float pre_temperature_of(const RowArgs& a, uint32_t id) {
     float l = load_logit<DT>(a.logits, id);
-    for (uint32_t j = 0; j < a.n_bias; ++j) {
-        const lily_bias b = a.bias[j];
-        if (b.id == id) {
-            l += b.delta;
-        }
-    }
-    if (a.allow != nullptr && !bit_of(a.allow, id)) {
-        return NEG_INF;
-    }
-    if ((a.flags & F_PEN) && bit_of(a.touched, id)) {
-        const uint32_t c = a.counts[id];
-        if (c > 0u) {
-            l = l > 0.0f ? l / a.repetition : l * a.repetition;
-            l -= a.presence + a.frequency * (float)c;
-        }
-    }
-    return l;
+    const uint32_t c = (a.flags & F_PEN) ? gload(a.counts + id) : 0u;
+    const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
+    return finish_pre_temperature(a, id, l, c, allowed);
 }
 
 template <int DT>
@@ -147,9 +171,11 @@ __device__ __forceinline__ float lower_by_slack(float t) {
 // ------------------------------------------------------------------ shared memory
 
 struct Shared {
-    float prob[K_CAP];   // exp(adjusted - top) per sorted candidate
-    float cum[K_CAP];    // inclusive prefix of the kept ones
-    float res[K_CAP];    // residual of the speculative draw
+    // The tail's arrays live in dynamic LDS behind the (by then at most K_CAP) sorted
+    // candidates; see tail_arrays().
+    float* prob;         // [K_CAP] exp(adjusted - top) per sorted candidate
+    float* cum;          // [K_CAP] inclusive prefix of the kept ones
+    float* res;          // [K_CAP] residual of the speculative draw
     uint32_t hist[256];
     double red_d[NWAVE];
     float red_f[NWAVE];
@@ -323,6 +349,38 @@ __device__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Share
     return sh.n_cand;
 }
 
+// Small sets (n <= NT): every thread ranks one candidate against all the others (each a
+// broadcast LDS read); the rank is the candidate's place in descending order, so the
+// top-k come out sorted.  Returns how many there are (zeros are dropped).
+__device__ uint32_t wg_rank_select(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
+    const uint32_t tid = threadIdx.x;
+    const uint64_t mine = tid < n ? cand[tid] : 0ull;
+    uint32_t rank = 0;
+    for (uint32_t j = 0; j < n; ++j) {
+        rank += cand[j] > mine ? 1u : 0u;
+    }
+    if (tid == 0) {
+        sh.n_cand = 0;
+    }
+    __syncthreads();
+    if (mine != 0ull && rank < k) {
+        cand[rank] = mine;  // composites are distinct: ranks are too
+        atomicAdd(&sh.n_cand, 1u);
+    }
+    __syncthreads();
+    return sh.n_cand;
+}
+
+// Top-k of cand[0..n) to the front; `sorted` tells whether they are in descending order.
+__device__ uint32_t select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh, bool& sorted) {
+    if (n <= 256u) {
+        sorted = true;
+        return wg_rank_select(cand, n, k, sh);
+    }
+    sorted = false;
+    return wg_select_topk(cand, n, k, sh);
+}
+
 // The k-th largest of the workgroup's NT x 8 per-lane values (-inf = absent) by a
 // radix select on their order keys; F32_LOWEST when fewer than k are present.
 __device__ float wg_kth_largest(const float (&ms)[8], uint32_t k, Shared& sh) {
@@ -392,7 +450,7 @@ struct Geo {
     // Chunk c as floats; positions outside the row or the slice read as -inf.
     __device__ __forceinline__ void load(const void* logits, uint32_t c, float (&v)[E]) const {
         if (c >= full_lo && c < full_hi && c < ce) {
-            const uint4 q = *reinterpret_cast<const uint4*>(base + (size_t)c * 16);
+            const u32x4 q = gload(reinterpret_cast<const u32x4*>(base + (size_t)c * 16));
             if (DT == LILY_BF16) {
                 v[0] = lilym_bits_f32(q.x << 16);
                 v[1] = lilym_bits_f32(q.x & 0xffff0000u);
@@ -428,11 +486,11 @@ struct Geo {
 __device__ __forceinline__ uint32_t bits32_at(const uint32_t* words, uint32_t nwords, int64_t id0) {
     const int64_t wi = id0 >> 5;
     const uint32_t sh = (uint32_t)(id0 & 31);
-    const uint32_t w0 = (wi >= 0 && wi < (int64_t)nwords) ? words[wi] : 0u;
+    const uint32_t w0 = (wi >= 0 && wi < (int64_t)nwords) ? gload(words + wi) : 0u;
     if (sh == 0) {
         return w0;
     }
-    const uint32_t w1 = (wi + 1 >= 0 && wi + 1 < (int64_t)nwords) ? words[wi + 1] : 0u;
+    const uint32_t w1 = (wi + 1 >= 0 && wi + 1 < (int64_t)nwords) ? gload(words + wi + 1) : 0u;
     return (w0 >> sh) | (w1 << (32u - sh));
 }
 
@@ -449,6 +507,15 @@ __device__ __forceinline__ uint32_t range32_at(uint32_t lo, uint32_t hi, int64_t
 }
 
 // ------------------------------------------------------------------ fast select
+
+// Diagnostic: thread 0 stamps the 100 MHz wall clock at phase i (see LaunchCfg::phase_trace).
+__device__ __forceinline__ void phase(const LaunchCfg& cfg, uint32_t i) {
+    if (cfg.phase_trace != nullptr && threadIdx.x == 0) {
+        cfg.phase_trace[((size_t)blockIdx.y * cfg.slices + blockIdx.x) * PHASE_SLOTS + i] =
+            wall_clock64();
+    }
+}
+
 
 // Appends the lanes with `pass` set to the candidate buffer (wave-aggregated).
 __device__ __forceinline__ void append(bool pass, float v, uint32_t id, uint64_t* cand,
@@ -479,7 +546,8 @@ __device__ __forceinline__ void append(bool pass, float v, uint32_t id, uint64_t
 // exhaustively.  Also leaves the slice's log-sum-exp in sh when LSE.
 template <int DT, bool EXCL, bool LSE>
 __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool two_pass,
-                            uint64_t* cand, uint32_t cap, uint32_t* excl, Shared& sh) {
+                            uint64_t* cand, uint32_t cap, uint32_t* excl, Shared& sh,
+                            const LaunchCfg& cfg, bool& sorted) {
     constexpr int E = Geo<DT>::E;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const uint32_t nchunks = g.ce - g.cb;
@@ -496,20 +564,31 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
     }
     if (EXCL) {
         // Bit b of the slice bitmap <-> id cb*E - pad + b.  Set = not streamed.
-        for (uint32_t i = tid; i < nwords; i += NT) {
-            const int64_t id0 = (int64_t)g.cb * E - g.pad + (int64_t)i * 32;
-            uint32_t x = ~range32_at(g.id_lo, g.id_hi, id0);
-            if (a.allow != nullptr) {
-                x |= ~bits32_at(a.allow, row_words, id0);
+        for (uint32_t i0 = tid; i0 < nwords; i0 += 4 * NT) {
+            uint32_t x[4];
+            for (int q = 0; q < 4; ++q) {  // four words' loads in flight before any store
+                const uint32_t i = i0 + (uint32_t)q * NT;
+                const int64_t id0 = (int64_t)g.cb * E - g.pad + (int64_t)i * 32;
+                x[q] = ~range32_at(g.id_lo, g.id_hi, id0);
+                if (i < nwords) {
+                    if (a.allow != nullptr) {
+                        x[q] |= ~bits32_at(a.allow, row_words, id0);
+                    }
+                    if (a.flags & F_PEN) {
+                        x[q] |= bits32_at(a.touched, row_words, id0);
+                    }
+                }
             }
-            if (a.flags & F_PEN) {
-                x |= bits32_at(a.touched, row_words, id0);
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t i = i0 + (uint32_t)q * NT;
+                if (i < nwords) {
+                    excl[i] = x[q];
+                }
             }
-            excl[i] = x;
         }
         __syncthreads();
         for (uint32_t i = tid; i < a.n_bias; i += NT) {
-            const uint32_t id = a.bias[i].id;
+            const uint32_t id = gload(&a.bias[i].id);
             if (id >= g.id_lo && id < g.id_hi) {
                 const uint32_t b = id + g.pad - g.cb * E;
                 atomicOr(&excl[b >> 5], 1u << (b & 31u));
@@ -517,6 +596,8 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
         }
     }
     __syncthreads();
+
+    phase(cfg, 1);
 
     // Lanes per group: the largest power of two with NT / L >= k groups (at most a wave).
     uint32_t group = 64;
@@ -553,7 +634,9 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
                             m = (excl_bytes[rel >> 1] >> ((rel & 1u) * 4u)) & 15u;
                         }
                         for (int j = 0; j < E; ++j) {
-                            v[u][j] = ((m >> j) & 1u) ? NEG_INF : v[u][j];
+                            // all-ones when bit j is set: the element reads as -inf
+                            const uint32_t on = (uint32_t)((int32_t)(m << (31 - j)) >> 31);
+                            v[u][j] = lilym_bits_f32((lilym_f32_bits(v[u][j]) & ~on) | (0xff800000u & on));
                         }
                     }
                 }
@@ -619,6 +702,7 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
         sh.wthr_f[w] = thr_f;
     }
     __syncthreads();
+    phase(cfg, 2);
     float filt = sh.wthr_f[0];
     for (int i = 1; i < NWAVE; ++i) {
         filt = fmaxf(filt, sh.wthr_f[i]);
@@ -633,26 +717,81 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
         cand[i] = composite_of(composite_value(c) / a.temperature, composite_id(c));
     }
     if (EXCL) {
-        // Specials: excluded from the stream but allowed ids (penalised or biased).
-        for (uint32_t i = tid; i < nwords; i += NT) {
-            const int64_t id0 = (int64_t)g.cb * E - g.pad + (int64_t)i * 32;
-            uint32_t bits = excl[i] & range32_at(g.id_lo, g.id_hi, id0);
+        // Specials: ids kept out of the stream that are allowed (penalised or biased).
+        // Their ids are compacted into an LDS list, then the workgroup walks the list four
+        // ids per thread at a time, so the gathers of a batch (logit, count) are
+        // independent loads and the work is balanced.
+        const bool pen = (a.flags & F_PEN) != 0;
+        const int64_t slice_id0 = (int64_t)g.cb * E - g.pad;
+        auto special_bits = [&](uint32_t i) -> uint32_t {
+            const int64_t id0 = slice_id0 + (int64_t)i * 32;
+            uint32_t b = excl[i] & range32_at(g.id_lo, g.id_hi, id0);
             if (a.allow != nullptr) {
-                bits &= bits32_at(a.allow, row_words, id0);
+                b &= bits32_at(a.allow, row_words, id0);
             }
-            while (bits != 0u) {
-                const int b = __builtin_ctz(bits);
-                bits &= bits - 1u;
-                const uint32_t id = (uint32_t)(id0 + b);
-                const float u = pre_temperature_of<DT>(a, id);
-                if (LSE) {
-                    lse.add_one(u, c2);
+            return b;
+        };
+        auto process = [&](uint32_t id, float l, uint32_t cnt) {
+            const float u = finish_pre_temperature(a, id, l, cnt, true);
+            if (LSE) {
+                lse.add_one(u, c2);
+            }
+            if (u >= filt) {
+                const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                if (at < cap) {
+                    cand[at] = composite_of(u / a.temperature, id);
                 }
-                if (u >= filt) {
-                    const uint32_t at = atomicAdd(&sh.n_cand, 1u);
-                    if (at < cap) {
-                        cand[at] = composite_of(u / a.temperature, id);
+            }
+        };
+        if (tid == 0) {
+            sh.need = 0;
+        }
+        __syncthreads();
+        uint32_t* list = excl + cfg.excl_words;  // SPECIAL_LIST_CAP ids behind the bitmap
+        const uint32_t list_cap = SPECIAL_LIST_CAP;
+        for (uint32_t i0 = 0; i0 < nwords; i0 += NT) {
+            const uint32_t i = i0 + tid;
+            uint32_t bits = i < nwords ? special_bits(i) : 0u;
+            while (__ballot(bits != 0u) != 0ull) {
+                const bool has = bits != 0u;
+                const uint32_t id = has ? (uint32_t)(slice_id0 + (int64_t)i * 32 + __builtin_ctz(bits)) : 0u;
+                bits &= bits - 1u;
+                const uint64_t mask = __ballot(has);
+                const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+                    (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                const int leader = __builtin_ctzll(mask);
+                uint32_t base = 0;
+                if ((int)lane == leader) {
+                    base = atomicAdd(&sh.need, (uint32_t)__popcll(mask));
+                }
+                base = __shfl(base, leader);
+                if (has) {
+                    if (base + rank < list_cap) {
+                        list[base + rank] = id;
+                    } else {  // more specials than the list holds: one at a time
+                        process(id, load_logit<DT>(a.logits, id), pen ? gload(a.counts + id) : 0u);
                     }
+                }
+            }
+        }
+        __syncthreads();
+        const uint32_t m = min(sh.need, list_cap);
+        for (uint32_t i0 = tid; i0 < m; i0 += 4 * NT) {
+            uint32_t ids[4];
+            float l[4];
+            uint32_t cnt[4];
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t i = i0 + (uint32_t)q * NT;
+                ids[q] = i < m ? list[i] : 0xffffffffu;
+            }
+            for (int q = 0; q < 4; ++q) {
+                const bool ok = ids[q] != 0xffffffffu;
+                l[q] = ok ? load_logit<DT>(a.logits, ids[q]) : 0.0f;
+                cnt[q] = (ok && pen) ? gload(a.counts + ids[q]) : 0u;
+            }
+            for (int q = 0; q < 4; ++q) {
+                if (ids[q] != 0xffffffffu) {
+                    process(ids[q], l[q], cnt[q]);
                 }
             }
         }
@@ -663,11 +802,13 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
         __syncthreads();
     }
     n = sh.n_cand;
+    phase(cfg, 3);
     if (n > cap) {
         return false;
     }
+    sorted = false;
     if (n > k) {
-        n = wg_select_topk(cand, n, k, sh);
+        n = select_topk(cand, n, k, sh, sorted);
     }
     // Every element that was not collected lies strictly below `filt`; it must also
     // lie strictly below the k-th adjusted value, or the division has merged it
@@ -847,8 +988,8 @@ __device__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, u
 
 // cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
 template <int DT>
-__device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, uint64_t* cand,
-                     Shared& sh) {
+__device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
+                     uint64_t* cand, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     if (n == 0) {
         // No finite value anywhere: the oracle's order then starts at id 0.
@@ -867,7 +1008,9 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
         }
         return;
     }
-    sort_desc(cand, n);
+    if (!sorted) {
+        sort_desc(cand, n);
+    }
     const uint32_t k = min(a.k, n);
     const float top = composite_value(cand[0]);
     for (uint32_t i = tid; i < k; i += NT) {
@@ -1058,9 +1201,11 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
 
     Geo<DT> g;
     g.init(a.logits, vocab, s, S);
+    phase(cfg, 0);
 
     const bool argmax = a.mode == MODE_ARGMAX;
     uint64_t best = 0;
+    bool sorted = false;
     if (argmax) {
         best = slice_argmax<DT>(a, g, sh);
     } else if (a.flags & F_FORCED) {
@@ -1081,52 +1226,57 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
             const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
             if (EXCL || !special) {
                 const bool two_pass = a.k > 64u || cfg.path == 2u;
-                done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh);
+                done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh, cfg,
+                                                  sorted);
             }
         }
         if (!done) {
             __syncthreads();
+            sorted = false;
             select_exhaustive<DT>(a, g.id_lo, g.id_hi, a.k, want_lse, cand, cfg.cand_cap, sh);
         }
     }
 
     uint32_t n = argmax ? 0u : min(sh.n_cand, cfg.cand_cap);
+    phase(cfg, 4);
     if (S > 1) {
         const size_t slot = (size_t)row * S + s;
+        // Partials go through to memory (no dirty L2 lines to write back), the wave waits
+        // for its stores, the workgroup meets, and one thread takes the row's ticket.
         if (argmax) {
             if (tid == 0) {
-                cfg.ws_cand[slot * cfg.ws_k] = best;
+                store_through(&cfg.ws_cand[slot * cfg.ws_k], best);
             }
         } else {
             for (uint32_t i = tid; i < n; i += NT) {
-                cfg.ws_cand[slot * cfg.ws_k + i] = cand[i];
+                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], cand[i]);
             }
             if (tid == 0) {
-                cfg.ws_n[slot] = n;
-                cfg.ws_lse[2 * slot] = want_lse ? sh.lse_mc : 0.0;
-                cfg.ws_lse[2 * slot + 1] = want_lse ? sh.lse_s : 0.0;
+                store_through(&cfg.ws_n[slot], n);
+                store_through(&cfg.ws_lse[2 * slot], want_lse ? sh.lse_mc : 0.0);
+                store_through(&cfg.ws_lse[2 * slot + 1], want_lse ? sh.lse_s : 0.0);
             }
         }
-        __threadfence();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) {
-            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_ACQ_REL,
+            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
                                                       __HIP_MEMORY_SCOPE_AGENT);
             sh.last = (t == S - 1) ? 1u : 0u;
         }
         __syncthreads();
+        phase(cfg, 5);
         if (sh.last == 0u) {
             return;
         }
-        __threadfence();
         if (tid == 0) {
-            cfg.ws_ticket[row] = 0;
+            store_through(&cfg.ws_ticket[row], 0u);
         }
         const size_t base = (size_t)row * S;
         if (argmax) {
             best = 0;
             for (uint32_t t = tid; t < S; t += NT) {
-                const uint64_t c = __builtin_nontemporal_load(&cfg.ws_cand[(base + t) * cfg.ws_k]);
+                const uint64_t c = load_through(&cfg.ws_cand[(base + t) * cfg.ws_k]);
                 best = c > best ? c : best;
             }
             best = wave_max_u64(best);
@@ -1139,43 +1289,44 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
                 best = sh.red_u[i] > best ? sh.red_u[i] : best;
             }
         } else {
-            // Gather every slice's candidates; merge the log-sum-exp partials.
-            uint32_t total = 0;
-            for (uint32_t t = 0; t < S; ++t) {
-                const uint32_t nt = __builtin_nontemporal_load(&cfg.ws_n[base + t]);
-                for (uint32_t i = tid; i < nt; i += NT) {
-                    cand[total + i] =
-                        __builtin_nontemporal_load(&cfg.ws_cand[(base + t) * cfg.ws_k + i]);
-                }
-                total += nt;
+            // Gather every slice's candidates (absent slots read as 0 = invalid) and merge
+            // the log-sum-exp partials, all slices at once.
+            if (tid < S) {
+                sh.hist[tid] = load_through(&cfg.ws_n[base + tid]);
             }
-            if (want_lse && tid == 0) {
-                double m = -__builtin_huge_val();
-                for (uint32_t t = 0; t < S; ++t) {
-                    const double st = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t) + 1]);
-                    if (st > 0.0) {
-                        m = fmax(m, __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t)]));
+            if (want_lse && tid < 64) {
+                double mt = -__builtin_huge_val(), st = 0.0;
+                if (tid < S) {
+                    mt = load_through(&cfg.ws_lse[2 * (base + tid)]);
+                    st = load_through(&cfg.ws_lse[2 * (base + tid) + 1]);
+                    if (!(st > 0.0)) {
+                        mt = -__builtin_huge_val();
                     }
                 }
-                double sum = 0.0;
-                for (uint32_t t = 0; t < S; ++t) {
-                    const double mt = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t)]);
-                    const double st = __builtin_nontemporal_load(&cfg.ws_lse[2 * (base + t) + 1]);
-                    if (st > 0.0) {
-                        sum += st * exp2(mt - m);
-                    }
+                double m = mt;
+                for (int o = 32; o > 0; o >>= 1) {
+                    m = fmax(m, __shfl_xor(m, o));
                 }
-                sh.lse_mc = m;
-                sh.lse_s = sum;
+                const double sum = wave_sum_d(st > 0.0 ? st * exp2(mt - m) : 0.0);
+                if (tid == 0) {
+                    sh.lse_mc = m;
+                    sh.lse_s = sum;
+                }
             }
             __syncthreads();
-            n = total;
-            if (n > a.k) {
-                n = wg_select_topk(cand, n, a.k, sh);
+            const uint32_t slots = S * cfg.ws_k;
+            for (uint32_t j = tid; j < slots; j += NT) {
+                const uint32_t t = j / cfg.ws_k, i = j - t * cfg.ws_k;
+                cand[j] = i < sh.hist[t] ? load_through(&cfg.ws_cand[(base + t) * cfg.ws_k + i]) : 0ull;
             }
+            __syncthreads();
+            n = slots;
+            sorted = false;
+            n = select_topk(cand, n, a.k, sh, sorted);
         }
     }
 
+    phase(cfg, 6);
     if (argmax) {
         if (tid == 0) {
             const uint32_t id = composite_id(best);
@@ -1190,13 +1341,37 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
         }
         return;
     }
-    tail<DT>(a, vocab, step, n, cand, sh);
+    tail<DT>(a, vocab, step, n, sorted, cand, sh);
+    phase(cfg, 7);
+}
+
+// Dynamic LDS: [0, cand_cap) candidates while scanning, then the bitmap.  In the tail the
+// first K_CAP slots hold the sorted candidates and the three float arrays follow them
+// (the launcher sizes the region for at least K_CAP * 8 + 3 * K_CAP * 4 bytes).
+__device__ __forceinline__ void tail_arrays(Shared& sh) {
+    float* f = reinterpret_cast<float*>(dyn_lds + K_CAP);
+    sh.prob = f;
+    sh.cum = f + K_CAP;
+    sh.res = f + 2 * K_CAP;
 }
 
 template <int DT, bool EXCL, bool LSE>
 __global__ __launch_bounds__(NT) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
     __shared__ Shared sh;
-    row_body<DT, EXCL, LSE>(rows.r[blockIdx.y], cfg, sh);
+    __shared__ RowArgs a;
+    // The row's arguments from the kernel-argument segment into LDS (a dynamic index into
+    // the by-value array would copy all of it to scratch memory).
+    for (int r = 0; r < INLINE_ROWS; ++r) {
+        if (r == (int)blockIdx.y && threadIdx.x < sizeof(RowArgs) / 4) {
+            reinterpret_cast<uint32_t*>(&a)[threadIdx.x] =
+                reinterpret_cast<const uint32_t*>(&rows.r[r])[threadIdx.x];
+        }
+    }
+    if (threadIdx.x == 0) {
+        tail_arrays(sh);
+    }
+    __syncthreads();
+    row_body<DT, EXCL, LSE>(a, cfg, sh);
 }
 
 template <int DT, bool EXCL, bool LSE>
@@ -1206,7 +1381,10 @@ __global__ __launch_bounds__(NT) void k_rows_table(LaunchCfg cfg) {
     // One coalesced copy of the row's arguments into LDS.
     if (threadIdx.x < sizeof(RowArgs) / 4) {
         reinterpret_cast<uint32_t*>(&a)[threadIdx.x] =
-            reinterpret_cast<const uint32_t*>(&cfg.table[blockIdx.y])[threadIdx.x];
+            gload(reinterpret_cast<const uint32_t*>(&cfg.table[blockIdx.y]) + threadIdx.x);
+    }
+    if (threadIdx.x == 0) {
+        tail_arrays(sh);
     }
     __syncthreads();
     row_body<DT, EXCL, LSE>(a, cfg, sh);

@@ -108,6 +108,8 @@ def _load():
     for n in ("lily_slot_pos", "lily_slot_block", "lily_slot_count", "lily_ctrl_words"):
         getattr(L, n).restype = C.c_uint32
         getattr(L, n).argtypes = [C.c_uint32]
+    L.lily_sampler_slices_for.restype = C.c_uint32
+    L.lily_sampler_slices_for.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32]
     L.lily_scratch_vocab.restype = C.c_uint32
     L.lily_scratch_vocab.argtypes = [C.c_void_p]
     vp, u32, u64 = C.c_void_p, C.c_uint32, C.c_uint64
@@ -115,6 +117,7 @@ def _load():
     sigs = {
         "lily_sampler_create": [C.c_int, vp, C.POINTER(vp)],
         "lily_sampler_synchronize": [vp],
+        "lily_sampler_set_phase_trace": [vp, vp, u64],
         "lily_scratch_create": [vp, u32, C.POINTER(vp)],
         "lily_scratch_reset_counts": [vp],
         "lily_scratch_uncount": [vp, u32],
@@ -226,6 +229,16 @@ class Sampler:
             self.close()
         except Exception:
             pass
+
+    def set_phase_trace(self, trace):
+        """trace: device int64 tensor (or None); see lily_sampler_set_phase_trace."""
+        self._trace = trace
+        _check(_lib.lily_sampler_set_phase_trace(
+            self._h, _ptr(trace, torch.int64) if trace is not None else None,
+            trace.numel() if trace is not None else 0))
+
+    def slices_for(self, rows, k, vocab):
+        return int(_lib.lily_sampler_slices_for(self._h, rows, k, vocab))
 
     def synchronize(self):
         """ComputePass::commit_wait."""
