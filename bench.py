@@ -21,6 +21,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "lily-qwen3.8-flash-next_amd", "python"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per 1024-row launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised
+# in profiles/k_rows_table_bf16_config5_b1024.md (valid for --rows 1024 only).
+MEASURED_TRAFFIC_BYTES = 738.1e6
 
 
 def parse():
@@ -31,6 +34,9 @@ def parse():
     ap.add_argument("--rows", type=int, default=1024)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 256 MiB device copy (a known-size kernel that counter runs "
+                         "under rocprofv3 --pmc are scaled by)")
     return ap.parse_args()
 
 
@@ -83,11 +89,15 @@ def cpu_baseline(c, rows_total, seconds):
         return n, time.perf_counter() - t0
 
     n, dt = run(cores)                       # probe: one row per core
-    per_round = max(dt, 1e-3)
-    want = int(max(cores, min(rows_total, cores * (seconds / per_round))))
-    n, dt = run(want)
+    total_rows, total_dt = 0, 0.0
+    chunk = int(max(cores, min(rows_total, cores * max(1.0, 2.0 / max(dt, 1e-3)))))
+    while total_dt < seconds:                # bounded sample: about `seconds` of wall time
+        n, dt = run(chunk)
+        total_rows += n
+        total_dt += dt
+    n, dt = total_rows, total_dt
     return {"value": n / dt, "unit": "rows/s", "cores": cores, "kind": "port",
-            "sample": f"{n} of the {rows_total} rows, full-vocabulary index sort per row "
+            "sample": f"{n} row draws (rows 0..{min(chunk, rows_total) - 1} of the {rows_total}, repeated), full-vocabulary index sort per row "
                       f"(as tests/unit/kernels/sample.rs:31-34), id + f64 log-probability, "
                       f"{dt:.1f} s wall"}
 
@@ -128,6 +138,14 @@ def main():
     ids_host = out_ids.cpu().numpy()
     assert ids_host.min() >= 0 and ids_host.max() < vocab
     plan.close()
+
+    if a.copy_probe:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)                      # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- decode-step configuration: 4 x 151 936 f32, 8 192-id history
     c2 = W.config2()
@@ -179,7 +197,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES if rows == 1024 else None,
             "kernel": "k_rows_table<bf16>",
             "bytes_per_row": bytes_row,
         },
