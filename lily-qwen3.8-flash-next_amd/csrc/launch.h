@@ -12,12 +12,10 @@ namespace lily {
 hipError_t launch_rows(hipStream_t stream, int dtype, bool excl, bool lse, uint32_t rows,
                        const LaunchCfg& cfg, const InlineRows* inline_rows, size_t dyn_bytes);
 hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t v);
-hipError_t launch_add_history(hipStream_t stream, uint32_t* counts, uint32_t* touched,
-                              uint32_t vocab, const uint32_t* ids, uint32_t n);
-hipError_t launch_uncount(hipStream_t stream, uint32_t* counts, uint32_t* touched, uint32_t vocab,
-                          uint32_t token);
-hipError_t launch_rebuild_touched(hipStream_t stream, const uint32_t* counts, uint32_t* touched,
-                                  uint32_t vocab);
+hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const uint32_t* ids,
+                              uint32_t n);
+hipError_t launch_uncount(hipStream_t stream, const ScratchView& sc, uint32_t token);
+hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc);
 hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const uint32_t* ids,
                               uint32_t* ctrl, uint32_t m, uint32_t pos0, uint32_t ratio,
                               uint32_t chain);

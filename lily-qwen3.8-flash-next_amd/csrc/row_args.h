@@ -19,13 +19,23 @@ enum : uint32_t {
     F_PEN = 1u,      // penalties on: read counts, count the emitted id
     F_UNIFORM = 2u,  // use `uniform` (and `uniform2`) instead of the seeded draws
     F_FORCED = 4u,   // emit `forced`
+    F_STREAM = 8u,   // eligible for the streaming select (k <= 64, no allow-mask, short bias list)
+};
+
+// One entry of a scratch's list of the ids that were ever counted.
+struct alignas(8) CountPair {
+    uint32_t id;
+    uint32_t count;
 };
 
 struct alignas(16) RowArgs {
     const void* logits;        // this row's first element
     const uint32_t* allow;     // packed allow bits or null
     uint32_t* counts;          // dense emission histogram or null
-    uint32_t* touched;         // bit per id with counts[id] != 0, or null
+    uint32_t* touched;         // bit per id that is in `pairs` (set with the first count), or null
+    CountPair* pairs;          // the listed ids with their counts (a count may have gone back to 0)
+    uint32_t* n_pairs;         // [1] entries appended so far (above pairs_cap: the list is unusable)
+    uint32_t* pos;             // [vocab] pairs index of a listed id
     const lily_bias* bias;     // n_bias pairs or null
     uint32_t* out_id;
     float* out_logprob;        // or null
@@ -52,9 +62,21 @@ struct alignas(16) RowArgs {
     float repetition;
     float uniform;
     float uniform2;
-    float pad;
+    uint32_t pairs_cap;
+    uint32_t pad[2];
 };
-static_assert(sizeof(RowArgs) == 192, "RowArgs layout");
+static_assert(sizeof(RowArgs) == 224, "RowArgs layout");
+
+// A scratch's device state as the small maintenance kernels take it.
+struct ScratchView {
+    uint32_t* counts;    // [vocab]
+    uint32_t* touched;   // [ceil(vocab / 32) + 4]
+    CountPair* pairs;    // [pairs_cap]
+    uint32_t* n_pairs;   // [1]
+    uint32_t* pos;       // [vocab]
+    uint32_t vocab;
+    uint32_t pairs_cap;
+};
 
 constexpr int INLINE_ROWS = 8;
 struct InlineRows {
@@ -72,18 +94,45 @@ struct LaunchCfg {
     uint32_t* ws_n;         // [rows][slices] candidates written
     double* ws_lse;         // [rows][slices][2] log2-domain reference, sum of 2^(x - reference)
     uint32_t* ws_ticket;    // [rows] arrival counter, left at 0
-    uint32_t path;          // 0 = automatic, 1 = exhaustive select only, 2 = two-pass select only
+    uint32_t path;          // 0 = automatic, 1 = exhaustive select only, 2 = two-pass select only,
+                            // 3 = no streaming select
     uint32_t cand_cap;      // candidate slots at the start of dynamic LDS (the bitmap follows)
     uint64_t* phase_trace;  // null, or [rows][slices][PHASE_SLOTS] 100 MHz timestamps
     uint32_t excl_words;    // words reserved for the slice bitmap (the specials' id list follows)
+    uint32_t list_cap;      // ids the specials' list holds
+    uint32_t old_layout;    // dynamic LDS holds cand_cap candidates + the bitmap + the id list
     uint32_t pad;
+    uint32_t* path_stats;   // null, or [4] counters: slices finished by the streaming select, the
+                            // bitmap select, the exhaustive select; [3] unused
 };
 
-constexpr uint32_t PHASE_SLOTS = 8;
+constexpr uint32_t PHASE_SLOTS = 16;
 
 constexpr uint32_t CAND_CAP = 2048;   // candidates a workgroup collects while scanning
 constexpr uint32_t MERGE_CAP = 4096;  // candidates the merging workgroup gathers (slices x k)
 constexpr uint32_t MAX_SLICES = 64;
 constexpr uint32_t SPECIAL_LIST_CAP = 2048;  // ids of penalised / biased tokens gathered per batch
+
+// Streaming select (k <= STREAM_K_MAX, no allow-mask): dynamic LDS layout in bytes.
+constexpr uint32_t STREAM_K_MAX = 64;
+constexpr uint32_t STREAM_UNROLL = 4;      // 16-byte chunks per thread per block
+constexpr uint32_t Q_CAP = 768;            // queued chunks (those holding a value at or above the bound)
+constexpr uint32_t SPEC_CAP = 3072;        // penalised / biased ids of one slice
+constexpr uint32_t FC_CAP = 1024;          // final candidates
+constexpr uint32_t DROP_CAP = 128;         // penalised / biased ids found inside queued chunks
+constexpr uint32_t MAX_BUCKETS = 64;       // blocks of one slice
+constexpr uint32_t STREAM_BIAS_CAP = 64;   // bias pairs kept in LDS
+constexpr uint32_t SPEC_ID_BITS = 20;      // packed entry: id | min(count, 4095) << 20
+constexpr uint32_t OFF_QRAW = 0;
+constexpr uint32_t OFF_QIDX = OFF_QRAW + Q_CAP * 16;
+constexpr uint32_t OFF_SPEC = OFF_QIDX + Q_CAP * 4;
+constexpr uint32_t OFF_FC = OFF_SPEC + SPEC_CAP * 4;
+constexpr uint32_t OFF_DROP = OFF_FC + FC_CAP * 8;
+constexpr uint32_t OFF_DMASK = OFF_DROP + DROP_CAP * 4;       // a byte per queue slot
+constexpr uint32_t OFF_BKT = OFF_DMASK + Q_CAP;               // [MAX_BUCKETS + 1] offsets
+constexpr uint32_t OFF_BFILL = OFF_BKT + (MAX_BUCKETS + 4) * 4;   // [MAX_BUCKETS] fill counters
+constexpr uint32_t OFF_BIAS = OFF_BFILL + MAX_BUCKETS * 4;    // ids then deltas
+constexpr uint32_t STREAM_LDS_BYTES = OFF_BIAS + STREAM_BIAS_CAP * 8;
+static_assert(OFF_FC % 8 == 0 && STREAM_LDS_BYTES % 16 == 0, "stream LDS layout");
 
 }  // namespace lily

@@ -43,7 +43,8 @@ int hip_fail(hipError_t e, const char* what) {
         }                                  \
     } while (0)
 
-constexpr uint32_t WS_ROWS = 256;       // rows that may span several workgroups
+constexpr uint32_t WS_ROWS = 4096;      // rows that may span several workgroups
+constexpr uint32_t WS_SLOTS = 1u << 20; // candidate slots of the workspace (rows x slices x k)
 constexpr uint32_t STAGE_SLOTS = 4;
 constexpr uint32_t TARGET_GROUPS = 512;  // workgroups a small batch is spread over
 
@@ -68,14 +69,19 @@ struct lily_sampler {
     uint32_t force_slices = 0;
     uint64_t* phase_trace = nullptr;
     uint64_t phase_words = 0;
+    uint32_t* path_stats = nullptr;
 };
 
 struct lily_scratch {
     lily_sampler* s = nullptr;
     uint32_t vocab = 0;
     uint32_t words = 0;
-    uint32_t* counts = nullptr;   // [vocab]
-    uint32_t* touched = nullptr;  // [words]
+    uint32_t pairs_cap = 0;
+    uint32_t* counts = nullptr;   // [vocab]; the one allocation, the rest follows it
+    uint32_t* pos = nullptr;      // [vocab] pairs index of a listed id
+    uint32_t* touched = nullptr;  // [words + 4] bit per listed id
+    CountPair* pairs = nullptr;   // [pairs_cap] listed ids with their counts
+    uint32_t* n_pairs = nullptr;  // [1]
 };
 
 struct lily_draft_dists {
@@ -99,9 +105,25 @@ struct lily_plan {
     bool lse = false;
     size_t dyn_bytes = 0;
     uint32_t excl_words = 0;
+    bool old_layout = false;
+    uint32_t cand_cap = 0;
 };
 
 namespace {
+
+constexpr uint32_t PAIRS_CAP = 16384;  // listed ids a scratch keeps (more: the list is not used)
+
+ScratchView view_of(const lily_scratch* sc) {
+    ScratchView v;
+    v.counts = sc->counts;
+    v.touched = sc->touched;
+    v.pairs = sc->pairs;
+    v.n_pairs = sc->n_pairs;
+    v.pos = sc->pos;
+    v.vocab = sc->vocab;
+    v.pairs_cap = sc->pairs_cap;
+    return v;
+}
 
 bool samples(const lily_sampling_params* p) {
     return !lily_params_is_greedy(p) || lily_params_uses_penalties(p);
@@ -179,6 +201,10 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
     if (pen) {
         out->counts = scratch->counts;
         out->touched = scratch->touched;
+        out->pairs = scratch->pairs;
+        out->n_pairs = scratch->n_pairs;
+        out->pos = scratch->pos;
+        out->pairs_cap = scratch->pairs_cap;
         out->flags |= F_PEN;
     }
     if (x.has_uniform) {
@@ -206,6 +232,10 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
     out->presence = params->presence_penalty;
     out->frequency = params->frequency_penalty;
     out->repetition = params->repetition_penalty;
+    if (mode != MODE_ARGMAX && k <= STREAM_K_MAX && x.allow == nullptr &&
+        out->n_bias <= STREAM_BIAS_CAP && vocab <= (1u << SPEC_ID_BITS)) {
+        out->flags |= F_STREAM;
+    }
     return LILY_OK;
 }
 
@@ -214,13 +244,15 @@ uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint
     if (rows > WS_ROWS) {
         return 1;
     }
-    uint32_t sl = s->force_slices ? s->force_slices : TARGET_GROUPS / rows;
+    uint32_t sl = s->force_slices ? s->force_slices : (TARGET_GROUPS + rows - 1) / rows;
     sl = sl < 1 ? 1 : sl;
     sl = sl > MAX_SLICES ? MAX_SLICES : sl;
     const uint32_t by_k = MERGE_CAP / (kmax ? kmax : 1);
     sl = sl > by_k ? by_k : sl;
     const uint32_t by_len = (vocab + 2047u) / 2048u;
     sl = sl > by_len ? by_len : sl;
+    const uint64_t by_ws = (uint64_t)WS_SLOTS / ((uint64_t)rows * (kmax ? kmax : 1));
+    sl = sl > by_ws ? (uint32_t)by_ws : sl;
     return sl < 1 ? 1 : sl;
 }
 
@@ -238,6 +270,9 @@ void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t sl
     cfg->ws_ticket = s->ws_ticket;
     cfg->path = s->force_path;
     cfg->cand_cap = CAND_CAP;
+    cfg->path_stats = s->path_stats;
+    if (const char* d = std::getenv("LILY_DBG")) cfg->pad = (uint32_t)std::atoi(d);  // DBG
+    cfg->list_cap = SPECIAL_LIST_CAP;
 }
 
 // Attaches the phase trace when the launch fits the caller's buffer.
@@ -254,23 +289,42 @@ void attach_trace(const lily_sampler* s, LaunchCfg* cfg, uint32_t rows) {
 struct LaunchShape {
     bool excl = false;
     bool lse = false;
+    bool old_layout = false;
     size_t dyn_bytes = 0;
     uint32_t excl_words = 0;
+    uint32_t cand_cap = 0;
 };
 
-LaunchShape shape_of(const RowArgs* rows, uint32_t n, int dtype, uint32_t vocab, uint32_t slices,
-                     uint32_t kmax) {
+LaunchShape shape_of(const lily_sampler* s, const RowArgs* rows, uint32_t n, int dtype,
+                     uint32_t vocab, uint32_t slices, uint32_t kmax) {
     LaunchShape sh;
+    bool any_stream = false, any_old = false, masked = false;
     for (uint32_t i = 0; i < n; ++i) {
         sh.excl = sh.excl || rows[i].allow != nullptr || (rows[i].flags & F_PEN) || rows[i].n_bias;
         sh.lse = sh.lse || rows[i].out_logprob != nullptr;
+        if (rows[i].mode == MODE_ARGMAX) {
+            continue;
+        }
+        const bool stream = (rows[i].flags & F_STREAM) && s->force_path == 0;
+        any_stream = any_stream || stream;
+        any_old = any_old || !stream;
+        masked = masked || rows[i].allow != nullptr;
     }
-    const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
-    const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
-    const uint32_t per = (nch + slices - 1) / slices;
-    sh.excl_words = sh.excl ? (per * e + 31) / 32 + 2 : 0;
-    const size_t bitmap = sh.excl ? ((size_t)sh.excl_words + SPECIAL_LIST_CAP) * 4 : 0;
-    sh.dyn_bytes = (size_t)CAND_CAP * 8 + bitmap;
+    // Rows outside the streaming select need the candidate buffer, the id list and (rows with
+    // an allow-mask) the slice bitmap; a launch of streaming rows only falls back to the
+    // exhaustive select.
+    sh.old_layout = any_old;
+    if (any_old) {
+        const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
+        const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
+        const uint32_t per = (nch + slices - 1) / slices;
+        sh.excl_words = masked ? (per * e + 31) / 32 + 2 : 0;
+        const size_t extra = sh.excl ? ((size_t)sh.excl_words + SPECIAL_LIST_CAP) * 4 : 0;
+        sh.dyn_bytes = (size_t)CAND_CAP * 8 + extra;
+    }
+    if (any_stream && STREAM_LDS_BYTES > sh.dyn_bytes) {
+        sh.dyn_bytes = STREAM_LDS_BYTES;
+    }
     const size_t tail = (size_t)LILY_SAMPLE_K_CAP * 8 + 3 * (size_t)LILY_SAMPLE_K_CAP * 4;
     if (tail > sh.dyn_bytes) {
         sh.dyn_bytes = tail;
@@ -279,6 +333,8 @@ LaunchShape shape_of(const RowArgs* rows, uint32_t n, int dtype, uint32_t vocab,
     if (merge > sh.dyn_bytes) {
         sh.dyn_bytes = merge;
     }
+    const size_t cap = sh.dyn_bytes / 8;
+    sh.cand_cap = any_old ? CAND_CAP : (uint32_t)(cap < CAND_CAP ? cap : CAND_CAP);
     return sh;
 }
 
@@ -299,8 +355,10 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     const uint32_t slices = choose_slices(s, n, kmax, vocab);
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
     attach_trace(s, &cfg, n);
-    const LaunchShape shp = shape_of(rows.r, n, dtype, vocab, slices, kmax);
+    const LaunchShape shp = shape_of(s, rows.r, n, dtype, vocab, slices, kmax);
     cfg.excl_words = shp.excl_words;
+    cfg.old_layout = shp.old_layout ? 1u : 0u;
+    cfg.cand_cap = shp.cand_cap;
     HIP_TRY(launch_rows(s->stream, dtype, shp.excl, shp.lse, n, cfg, &rows, shp.dyn_bytes));
     return LILY_OK;
 }
@@ -529,7 +587,7 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     }
     const size_t slots = (size_t)WS_ROWS * MAX_SLICES;
     hipError_t err = hipMalloc(reinterpret_cast<void**>(&s->ws_cand),
-                               (size_t)WS_ROWS * MERGE_CAP * sizeof(uint64_t));
+                               (size_t)WS_SLOTS * sizeof(uint64_t));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_n), slots * 4);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 16);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
@@ -572,6 +630,14 @@ int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_
     return LILY_OK;
 }
 
+int lily_sampler_set_path_stats(lily_sampler_t* s, uint32_t* stats_dev) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    s->path_stats = stats_dev;
+    return LILY_OK;
+}
+
 uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab) {
     if (s == nullptr || rows == 0) {
         return 0;
@@ -602,15 +668,27 @@ int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out)
     sc->s = s;
     sc->vocab = vocab;
     sc->words = (vocab + 31u) / 32u;
-    // One allocation: counts, then the bitmap (padded so the bitmap is 16-byte aligned).
-    const size_t count_bytes = (((size_t)vocab * 4) + 15) & ~(size_t)15;
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts),
-                             count_bytes + (size_t)(sc->words + 4) * 4);
+    sc->pairs_cap = vocab < PAIRS_CAP ? vocab : PAIRS_CAP;
+    // One allocation: counts, pos, the bitmap, the list, its length (each 16-byte aligned).
+    const size_t dense = (((size_t)vocab * 4) + 15) & ~(size_t)15;
+    const size_t bitmap = (((size_t)(sc->words + 4) * 4) + 15) & ~(size_t)15;
+    const size_t list = (size_t)sc->pairs_cap * sizeof(CountPair);
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts), 2 * dense + bitmap + list + 16);
     if (e != hipSuccess) {
         delete sc;
         return hip_fail(e, "scratch allocation");
     }
-    sc->touched = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(sc->counts) + count_bytes);
+    char* base = reinterpret_cast<char*>(sc->counts);
+    sc->pos = reinterpret_cast<uint32_t*>(base + dense);
+    sc->touched = reinterpret_cast<uint32_t*>(base + 2 * dense);
+    sc->pairs = reinterpret_cast<CountPair*>(base + 2 * dense + bitmap);
+    sc->n_pairs = reinterpret_cast<uint32_t*>(base + 2 * dense + bitmap + list);
+    e = hipMemsetAsync(sc->pos, 0, dense, s->stream);  // never read before written; defined anyway
+    if (e != hipSuccess) {
+        (void)hipFree(sc->counts);
+        delete sc;
+        return hip_fail(e, "scratch clear");
+    }
     *out = sc;
     return lily_scratch_reset_counts(sc);
 }
@@ -634,6 +712,7 @@ int lily_scratch_reset_counts(lily_scratch_t* sc) {
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->counts, sc->vocab, 0));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->touched, sc->words + 4, 0));
+    HIP_TRY(launch_fill_u32(sc->s->stream, sc->n_pairs, 1, 0));
     return LILY_OK;
 }
 
@@ -645,7 +724,7 @@ int lily_scratch_uncount(lily_scratch_t* sc, uint32_t token) {
         return LILY_OK;  // sample.rs:149-151
     }
     HIP_TRY(hipSetDevice(sc->s->device));
-    HIP_TRY(launch_uncount(sc->s->stream, sc->counts, sc->touched, sc->vocab, token));
+    HIP_TRY(launch_uncount(sc->s->stream, view_of(sc), token));
     return LILY_OK;
 }
 
@@ -661,6 +740,11 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
                            dst->s->stream));
     HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)src->words * 4,
                            hipMemcpyDeviceToDevice, dst->s->stream));
+    HIP_TRY(hipMemcpyAsync(dst->pos, src->pos, (size_t)src->vocab * 4, hipMemcpyDeviceToDevice,
+                           dst->s->stream));
+    HIP_TRY(hipMemcpyAsync(dst->pairs, src->pairs, (size_t)src->pairs_cap * sizeof(CountPair),
+                           hipMemcpyDeviceToDevice, dst->s->stream));
+    HIP_TRY(hipMemcpyAsync(dst->n_pairs, src->n_pairs, 4, hipMemcpyDeviceToDevice, dst->s->stream));
     return LILY_OK;
 }
 
@@ -669,7 +753,7 @@ int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32
         return fail(LILY_ERR_INVALID_ARG, "scratch or ids is null");
     }
     HIP_TRY(hipSetDevice(sc->s->device));
-    HIP_TRY(launch_add_history(sc->s->stream, sc->counts, sc->touched, sc->vocab, ids_dev, n));
+    HIP_TRY(launch_add_history(sc->s->stream, view_of(sc), ids_dev, n));
     return LILY_OK;
 }
 
@@ -680,7 +764,7 @@ int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts) {
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     HIP_TRY(hipMemcpy(sc->counts, host_counts, (size_t)sc->vocab * 4, hipMemcpyHostToDevice));
-    HIP_TRY(launch_rebuild_touched(sc->s->stream, sc->counts, sc->touched, sc->vocab));
+    HIP_TRY(launch_rebuild_listed(sc->s->stream, view_of(sc)));
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     return LILY_OK;
 }
@@ -909,8 +993,11 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     const uint32_t slices = choose_slices(s, b->rows, kmax, b->vocab);
     fill_cfg(s, &cfg, b->vocab, slices, kmax, 0, s->table_dev);
     attach_trace(s, &cfg, b->rows);
-    const LaunchShape shp = shape_of(s->stage[slot], b->rows, (int)b->dtype, b->vocab, slices, kmax);
+    const LaunchShape shp =
+        shape_of(s, s->stage[slot], b->rows, (int)b->dtype, b->vocab, slices, kmax);
     cfg.excl_words = shp.excl_words;
+    cfg.old_layout = shp.old_layout ? 1u : 0u;
+    cfg.cand_cap = shp.cand_cap;
     HIP_TRY(launch_rows(s->stream, (int)b->dtype, shp.excl, shp.lse, b->rows, cfg, nullptr,
                         shp.dyn_bytes));
     return LILY_OK;
@@ -968,12 +1055,14 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->dtype = b->dtype;
     p->ws_k = max_k(table.data(), b->rows);
     p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab);
-    const LaunchShape shp = shape_of(table.data(), b->rows, (int)b->dtype, b->vocab, p->slices,
-                                     p->ws_k);
+    const LaunchShape shp = shape_of(p->s, table.data(), b->rows, (int)b->dtype, b->vocab,
+                                     p->slices, p->ws_k);
     p->excl = shp.excl;
     p->lse = shp.lse;
     p->dyn_bytes = shp.dyn_bytes;
     p->excl_words = shp.excl_words;
+    p->old_layout = shp.old_layout;
+    p->cand_cap = shp.cand_cap;
     return LILY_OK;
 }
 
@@ -986,6 +1075,8 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     fill_cfg(p->s, &cfg, p->vocab, p->slices, p->ws_k, step_delta, p->table_dev);
     attach_trace(p->s, &cfg, p->rows);
     cfg.excl_words = p->excl_words;
+    cfg.old_layout = p->old_layout ? 1u : 0u;
+    cfg.cand_cap = p->cand_cap;
     HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->excl, p->lse, p->rows, cfg, nullptr,
                         p->dyn_bytes));
     return LILY_OK;

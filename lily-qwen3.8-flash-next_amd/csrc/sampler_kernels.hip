@@ -39,9 +39,10 @@
 
 namespace lily {
 
-constexpr int NT = 512;
+constexpr int NT = 256;
 constexpr int NWAVE = NT / 64;
 constexpr int UNROLL = 4;
+constexpr bool PREFETCH = false;  // keep block b+1 in flight while block b is processed
 constexpr uint32_t K_CAP = LILY_SAMPLE_K_CAP;
 constexpr float F32_LOWEST = -3.4028234663852886e38f;
 
@@ -54,6 +55,7 @@ extern __shared__ uint64_t dyn_lds[];  // candidates, then the exclusion bitmap
 // Loads through a pointer known to be device memory: global_load instead of flat_load
 // (the row's pointers arrive through LDS, so the compiler cannot tell by itself).
 #define LILY_GLOBAL __attribute__((address_space(1)))
+#define LILY_CONST __attribute__((address_space(4)))
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <class T>
 __device__ __forceinline__ T gload(const T* p) {
@@ -115,7 +117,7 @@ __device__ __forceinline__ float finish_pre_temperature(const RowArgs& a, uint32
 
 // The value before the temperature of one id, loads included.
 template <int DT>
-__device__ float pre_temperature_of(const RowArgs& a, uint32_t id) {
+__device__ __forceinline__ float pre_temperature_of(const RowArgs& a, uint32_t id) {
     float l = load_logit<DT>(a.logits, id);
     const uint32_t c = (a.flags & F_PEN) ? gload(a.counts + id) : 0u;
     const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
@@ -195,6 +197,12 @@ struct Shared {
     float q_d;
     double lse_mc;   // log2-domain reference of the row's sum of exponentials
     double lse_s;    // sum of 2^(x * log2e / T - lse_mc) over the row
+    // streaming select
+    float bound[2][NWAVE];   // each wave's lower bound of its share of the k-th largest (two parities)
+    uint32_t qfill[NWAVE];   // chunks each wave queued
+    uint32_t n_fc;           // final candidates
+    uint32_t n_drop;         // listed ids found inside queued chunks
+    uint32_t fail;
 };
 
 // Running sum of 2^(v*c - mc) of one thread with its own reference mc.
@@ -225,7 +233,7 @@ struct LseAcc {
 };
 
 // Workgroup-wide merge of the threads' accumulators into sh.lse_mc / sh.lse_s.
-__device__ void lse_reduce(Shared& sh, const LseAcc& l) {
+__device__ __forceinline__ void lse_reduce(Shared& sh, const LseAcc& l) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     float m = wave_max_f(l.mc);
     if (lane == 0) {
@@ -261,7 +269,7 @@ __device__ void lse_reduce(Shared& sh, const LseAcc& l) {
 // With sh.hist complete: finds the bin in which the count from bin 255 downwards
 // reaches `need`.  Leaves sh.sel_bin, sh.need (what is still needed inside that
 // bin), sh.bin_count, and sh.all_taken = 1 when fewer than `need` were counted.
-__device__ void find_bin(Shared& sh, uint32_t need) {
+__device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
     if (threadIdx.x < 64) {
         const uint32_t lane = threadIdx.x;
         uint32_t h[4], sum = 0;
@@ -299,7 +307,7 @@ __device__ void find_bin(Shared& sh, uint32_t need) {
 
 // The top-k of cand[0..n) (zeros are invalid) compacted, unsorted, to the front;
 // returns how many there are.
-__device__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
+__device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     uint64_t prefix = 0, pmask = 0;
     uint32_t need = k;
@@ -331,8 +339,9 @@ __device__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Share
         }
     }
     const uint64_t floor_c = all ? 1ull : prefix;
-    uint64_t mine[8];
-    for (int j = 0; j < 8; ++j) {
+    constexpr int PER = MERGE_CAP / NT;  // n <= MERGE_CAP
+    uint64_t mine[PER];
+    for (int j = 0; j < PER; ++j) {
         const uint32_t i = tid + (uint32_t)j * NT;
         mine[j] = i < n ? cand[i] : 0ull;
     }
@@ -340,7 +349,7 @@ __device__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Share
         sh.n_cand = 0;
     }
     __syncthreads();
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < PER; ++j) {
         if (mine[j] != 0 && mine[j] >= floor_c) {
             cand[atomicAdd(&sh.n_cand, 1u)] = mine[j];
         }
@@ -352,7 +361,7 @@ __device__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Share
 // Small sets (n <= NT): every thread ranks one candidate against all the others (each a
 // broadcast LDS read); the rank is the candidate's place in descending order, so the
 // top-k come out sorted.  Returns how many there are (zeros are dropped).
-__device__ uint32_t wg_rank_select(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
+__device__ __forceinline__ uint32_t wg_rank_select(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     const uint64_t mine = tid < n ? cand[tid] : 0ull;
     uint32_t rank = 0;
@@ -372,7 +381,7 @@ __device__ uint32_t wg_rank_select(uint64_t* cand, uint32_t n, uint32_t k, Share
 }
 
 // Top-k of cand[0..n) to the front; `sorted` tells whether they are in descending order.
-__device__ uint32_t select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh, bool& sorted) {
+__device__ __forceinline__ uint32_t select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh, bool& sorted) {
     if (n <= 256u) {
         sorted = true;
         return wg_rank_select(cand, n, k, sh);
@@ -383,7 +392,7 @@ __device__ uint32_t select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& 
 
 // The k-th largest of the workgroup's NT x 8 per-lane values (-inf = absent) by a
 // radix select on their order keys; F32_LOWEST when fewer than k are present.
-__device__ float wg_kth_largest(const float (&ms)[8], uint32_t k, Shared& sh) {
+__device__ __forceinline__ float wg_kth_largest(const float (&ms)[8], uint32_t k, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     uint32_t keys[8];
     for (int j = 0; j < 8; ++j) {
@@ -427,6 +436,9 @@ struct Geo {
     uint32_t full_lo, full_hi;  // chunks lying wholly inside the row
     uint32_t vocab;
     uint32_t id_lo, id_hi;      // this slice's ids
+    uint32_t main_lo, main_hi;  // this slice's chunks that are streamed
+    uint32_t edge_lo_end;       // ids [id_lo, edge_lo_end) and [edge_hi_begin, id_hi) are edges
+    uint32_t edge_hi_begin;
 
     __device__ void init(const void* logits, uint32_t v, uint32_t s, uint32_t slices) {
         const uintptr_t addr = reinterpret_cast<uintptr_t>(logits);
@@ -445,35 +457,28 @@ struct Geo {
         if (id_hi < id_lo) {
             id_hi = id_lo;
         }
+        main_lo = max(cb, full_lo);
+        main_hi = max(min(ce, full_hi), main_lo);
+        if (main_hi > main_lo) {
+            edge_lo_end = main_lo * E - pad;
+            edge_hi_begin = main_hi * E - pad;
+        } else {
+            edge_lo_end = id_hi;  // nothing is streamed: every id is an edge
+            edge_hi_begin = id_hi;
+        }
     }
 
-    // Chunk c as floats; positions outside the row or the slice read as -inf.
-    __device__ __forceinline__ void load(const void* logits, uint32_t c, float (&v)[E]) const {
-        if (c >= full_lo && c < full_hi && c < ce) {
-            const u32x4 q = gload(reinterpret_cast<const u32x4*>(base + (size_t)c * 16));
-            if (DT == LILY_BF16) {
-                v[0] = lilym_bits_f32(q.x << 16);
-                v[1] = lilym_bits_f32(q.x & 0xffff0000u);
-                v[2] = lilym_bits_f32(q.y << 16);
-                v[3] = lilym_bits_f32(q.y & 0xffff0000u);
-                v[4 % E] = lilym_bits_f32(q.z << 16);
-                v[5 % E] = lilym_bits_f32(q.z & 0xffff0000u);
-                v[6 % E] = lilym_bits_f32(q.w << 16);
-                v[7 % E] = lilym_bits_f32(q.w & 0xffff0000u);
-            } else {
-                v[0] = lilym_bits_f32(q.x);
-                v[1] = lilym_bits_f32(q.y);
-                v[2] = lilym_bits_f32(q.z);
-                v[3] = lilym_bits_f32(q.w);
-            }
-        } else {
-            for (int j = 0; j < E; ++j) {
-                const int64_t id = (int64_t)c * E - pad + j;
-                v[j] = (c < ce && id >= 0 && id < (int64_t)vocab)
-                           ? load_logit<DT>(logits, (uint32_t)id)
-                           : NEG_INF;
-            }
+    // Chunk c as its 16 raw bytes when it lies wholly inside the row and the slice
+    // (main_lo <= c < main_hi), else sixteen bytes of -inf.  The few ids of partial chunks
+    // at the ends of a row (edge_*) are not streamed; callers evaluate them one by one.
+    __device__ __forceinline__ u32x4 load_raw(uint32_t c) const {
+        u32x4 q;
+        const uint32_t ninf = DT == LILY_BF16 ? 0xff80ff80u : 0xff800000u;
+        q.x = q.y = q.z = q.w = ninf;
+        if (c >= main_lo && c < main_hi) {
+            q = gload(reinterpret_cast<const u32x4*>(base + (size_t)c * 16));
         }
+        return q;
     }
 
     __device__ __forceinline__ uint32_t id_of(uint32_t c, int j) const {
@@ -516,13 +521,31 @@ __device__ __forceinline__ void phase(const LaunchCfg& cfg, uint32_t i) {
     }
 }
 
-
-// Appends the lanes with `pass` set to the candidate buffer (wave-aggregated).
-__device__ __forceinline__ void append(bool pass, float v, uint32_t id, uint64_t* cand,
-                                       uint32_t cap, Shared& sh) {
+// Appends the lanes with `pass` set to this wave's own region of the candidate buffer
+// (`region`, `seg` slots); `count` is the wave's fill, the same in every lane.  No atomics:
+// the slot is the fill plus the lane's rank among the passing lanes.
+__device__ __forceinline__ void append(bool pass, float v, uint32_t id, uint64_t* region,
+                                       uint32_t seg, uint32_t& count) {
     const uint64_t mask = __ballot(pass);
     if (mask == 0) {
         return;
+    }
+    const uint32_t rank =
+        __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+    const uint32_t at = count + rank;
+    if (pass && at < seg) {
+        region[at] = ((uint64_t)lilym_order_key(v) << 32) | (uint32_t)(~id);
+    }
+    count += (uint32_t)__popcll(mask);
+}
+
+// Appends ids to the specials list (wave-aggregated); returns false for a lane whose id
+// did not fit.
+__device__ __forceinline__ bool list_push(bool has, uint32_t id, uint32_t* list, uint32_t list_cap,
+                                          Shared& sh) {
+    const uint64_t mask = __ballot(has);
+    if (mask == 0) {
+        return true;
     }
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t rank =
@@ -530,51 +553,191 @@ __device__ __forceinline__ void append(bool pass, float v, uint32_t id, uint64_t
     const int leader = __builtin_ctzll(mask);
     uint32_t base = 0;
     if ((int)lane == leader) {
-        base = atomicAdd(&sh.n_cand, (uint32_t)__popcll(mask));
+        base = atomicAdd(&sh.need, (uint32_t)__popcll(mask));
     }
     base = __shfl(base, leader);
-    if (pass) {
-        const uint32_t at = base + rank;
-        if (at < cap) {
-            cand[at] = ((uint64_t)lilym_order_key(v) << 32) | (uint32_t)(~id);
+    if (has) {
+        if (base + rank < list_cap) {
+            list[base + rank] = id;
+            return true;
+        }
+        return false;
+    }
+    return true;
+}
+
+// One wave's sum of 2^(v*c - ref) with a reference that is the same in every lane.
+struct WaveLse {
+    float ref;
+    float s;
+    __device__ __forceinline__ void init() {
+        ref = F32_LOWEST;
+        s = 0.0f;
+    }
+    // Adds the E terms of one load whose lane maximum is m; skipped by the whole wave when
+    // every term is below 2^-40 of the reference.
+    template <int E>
+    __device__ __forceinline__ void add(const float (&v)[E], float m, float c) {
+        if (__ballot(__builtin_fmaf(m, c, -ref) > 60.0f) != 0ull) {
+            // A term would dwarf the reference: raise it to the wave's maximum (rare).
+            const float nref = fmaxf(ref, wave_max_f(m * c));
+            s *= __builtin_amdgcn_exp2f(ref - nref);
+            ref = nref;
+        }
+        if (__ballot(__builtin_fmaf(m, c, -ref) > -40.0f) == 0ull) {
+            return;
+        }
+        for (int j = 0; j < E; ++j) {
+            s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
+        }
+    }
+    // As add() on the raw 16 bytes of one load (unpacked only when the wave does not skip
+    // it); an inactive lane contributes nothing.
+    template <int DT>
+    __device__ __forceinline__ void add_chunk(const u32x4& q, float m, float c, bool active);
+};
+
+// Workgroup-wide merge of per-thread (reference, sum) pairs: returns through `m`, `sum`
+// (double, valid in every thread).
+__device__ __forceinline__ void wg_merge_lse(Shared& sh, float mc, float s_in, double& m_out, double& sum_out) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    float m = wave_max_f(s_in > 0.0f ? mc : NEG_INF);
+    if (lane == 0) {
+        sh.red_f[w] = m;
+    }
+    __syncthreads();
+    m = sh.red_f[0];
+    for (int i = 1; i < NWAVE; ++i) {
+        m = fmaxf(m, sh.red_f[i]);
+    }
+    double s = 0.0;
+    if (s_in > 0.0f) {
+        s = (double)s_in * exp2((double)mc - (double)m);
+    }
+    s = wave_sum_d(s);
+    if (lane == 0) {
+        sh.red_d[w] = s;
+    }
+    __syncthreads();
+    double t = 0.0;
+    for (int i = 0; i < NWAVE; ++i) {
+        t += sh.red_d[i];
+    }
+    __syncthreads();
+    m_out = (double)m;
+    sum_out = t;
+}
+
+template <int DT>
+__device__ __forceinline__ void unpack(const u32x4 q, float (&v)[Geo<DT>::E]) {
+    if (DT == LILY_BF16) {
+        v[0] = lilym_bits_f32(q.x << 16);
+        v[1] = lilym_bits_f32(q.x & 0xffff0000u);
+        v[2] = lilym_bits_f32(q.y << 16);
+        v[3] = lilym_bits_f32(q.y & 0xffff0000u);
+        v[4 % Geo<DT>::E] = lilym_bits_f32(q.z << 16);
+        v[5 % Geo<DT>::E] = lilym_bits_f32(q.z & 0xffff0000u);
+        v[6 % Geo<DT>::E] = lilym_bits_f32(q.w << 16);
+        v[7 % Geo<DT>::E] = lilym_bits_f32(q.w & 0xffff0000u);
+    } else {
+        v[0] = lilym_bits_f32(q.x);
+        v[1] = lilym_bits_f32(q.y);
+        v[2] = lilym_bits_f32(q.z);
+        v[3] = lilym_bits_f32(q.w);
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void WaveLse::add_chunk(const u32x4& q, float m, float c, bool active) {
+    constexpr int E = DT == LILY_BF16 ? 8 : 4;
+    m = active ? m : NEG_INF;
+    if (__ballot(__builtin_fmaf(m, c, -ref) > 60.0f) != 0ull) {
+        const float nref = fmaxf(ref, wave_max_f(m * c));
+        s *= __builtin_amdgcn_exp2f(ref - nref);
+        ref = nref;
+    }
+    if (__ballot(__builtin_fmaf(m, c, -ref) > -40.0f) == 0ull) {
+        return;
+    }
+    if (active) {
+        float v[E];
+        unpack<DT>(q, v);
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
         }
     }
 }
 
-// The exact top-k of the slice in cand[0..n) as adjusted-value composites,
-// unsorted, n returned through sh.n_cand; false when the slice must be redone
-// exhaustively.  Also leaves the slice's log-sum-exp in sh when LSE.
+__device__ __forceinline__ bool in_bias_list(const RowArgs& a, uint32_t id) {
+    for (uint32_t j = 0; j < a.n_bias; ++j) {
+        if (gload(&a.bias[j].id) == id) {
+            return true;
+        }
+    }
+    return false;
+}
+
+// The exact top-k of the slice in cand[0..n) as adjusted-value composites (n through
+// sh.n_cand, `sorted` tells whether they are in order); false when the slice must be
+// redone exhaustively.  Also leaves the slice's log-sum-exp in sh when LSE.
+//
+// Rows with an allow-mask keep every masked, penalised or biased id out of the stream
+// through the LDS bitmap (`mask_stream`).  Rows with penalties or a bias list only are
+// streamed raw ("patch"): candidates that turn out to be penalised or biased are
+// dropped, all such ids are evaluated exactly afterwards and re-enter with their true
+// value, the row sum is corrected by their raw and true terms, and the a-posteriori
+// check below covers the case where a raw value had lifted the threshold too far.
 template <int DT, bool EXCL, bool LSE>
-__device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool two_pass,
+__device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool two_pass,
                             uint64_t* cand, uint32_t cap, uint32_t* excl, Shared& sh,
                             const LaunchCfg& cfg, bool& sorted) {
     constexpr int E = Geo<DT>::E;
+    constexpr int U = UNROLL;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const uint32_t nchunks = g.ce - g.cb;
     const uint32_t nwords = (nchunks * E + 31u) / 32u;
     const uint32_t row_words = (g.vocab + 31u) / 32u;
+    const uint32_t nblocks = (nchunks + NT * U - 1) / (NT * U);
+    const int64_t slice_id0 = (int64_t)g.cb * E - g.pad;
     const float c2 = a.c2;
+    const bool pen = (a.flags & F_PEN) != 0;
+    const bool special_row = EXCL && (a.allow != nullptr || pen || a.n_bias != 0);
+    const bool mask_stream = EXCL && a.allow != nullptr;
+    const bool patch = special_row && !mask_stream;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    uint32_t* list = excl + cfg.excl_words;
+    const uint32_t list_cap = cfg.list_cap;
+
+    auto fetch = [&](u32x4 (&dst)[U], uint32_t b) {
+        for (int u = 0; u < U; ++u) {
+            dst[u] = g.load_raw(g.cb + (b * U + u) * NT + tid);
+        }
+    };
+    u32x4 cur[U], nxt[U];
+    if (nblocks > 0) {
+        fetch(cur, 0);  // in flight while the bitmap is built
+    }
 
     if (tid == 0) {
         sh.n_cand = 0;
+        sh.need = 0;
     }
     if (tid < NWAVE) {
         sh.wthr[tid] = NEG_INF;
         sh.wthr_f[tid] = F32_LOWEST;
     }
-    if (EXCL) {
+    if (mask_stream) {
         // Bit b of the slice bitmap <-> id cb*E - pad + b.  Set = not streamed.
         for (uint32_t i0 = tid; i0 < nwords; i0 += 4 * NT) {
             uint32_t x[4];
             for (int q = 0; q < 4; ++q) {  // four words' loads in flight before any store
                 const uint32_t i = i0 + (uint32_t)q * NT;
-                const int64_t id0 = (int64_t)g.cb * E - g.pad + (int64_t)i * 32;
+                const int64_t id0 = slice_id0 + (int64_t)i * 32;
                 x[q] = ~range32_at(g.id_lo, g.id_hi, id0);
                 if (i < nwords) {
-                    if (a.allow != nullptr) {
-                        x[q] |= ~bits32_at(a.allow, row_words, id0);
-                    }
-                    if (a.flags & F_PEN) {
+                    x[q] |= ~bits32_at(a.allow, row_words, id0);
+                    if (pen) {
                         x[q] |= bits32_at(a.touched, row_words, id0);
                     }
                 }
@@ -596,7 +759,6 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
         }
     }
     __syncthreads();
-
     phase(cfg, 1);
 
     // Lanes per group: the largest power of two with NT / L >= k groups (at most a wave).
@@ -610,22 +772,99 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
     for (int j = 0; j < 8; ++j) {
         ms[j] = NEG_INF;
     }
-    LseAcc lse;
-    lse.init();
+    WaveLse wl;
+    wl.init();
     float thr_f = F32_LOWEST;
     const uint8_t* excl_bytes = reinterpret_cast<const uint8_t*>(excl);
+    // While scanning, wave w appends to cand[w * seg, (w + 1) * seg); wcount is its fill.
+    const uint32_t seg = cap / NWAVE;
+    uint64_t* region = cand + w * seg;
+    uint32_t wcount = 0;
 
-    for (int pass = 0; pass < (two_pass ? 2 : 1); ++pass) {
-        const bool filter = !two_pass || pass == 1;
-        for (uint32_t c0 = g.cb; c0 < g.ce; c0 += NT * UNROLL) {
-            float v[UNROLL][E];
-            for (int u = 0; u < UNROLL; ++u) {
-                g.load(a.logits, c0 + u * NT + tid, v[u]);
+    // Lower bound of the k-th largest value from the lanes' running maxima: the minimum
+    // over groups of the group maximum (other waves' entries may be older: still bounds).
+    auto update_threshold = [&](bool first) {
+        float t = lane_max;
+        for (uint32_t o = 1; o < group; o <<= 1) {
+            t = fmaxf(t, __shfl_xor(t, (int)o));
+        }
+        for (uint32_t o = group; o < 64; o <<= 1) {
+            t = fminf(t, __shfl_xor(t, (int)o));
+        }
+        if (lane == 0) {
+            __hip_atomic_store(&sh.wthr[w], t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        if (first) {
+            __syncthreads();  // every wave has published its first statistic
+        }
+        for (int i = 0; i < NWAVE; ++i) {
+            t = fminf(t, __hip_atomic_load(&sh.wthr[i], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP));
+        }
+        thr_f = fmaxf(thr_f, lower_by_slack(t));
+    };
+
+    // Stages of the scan.  Single pass (k <= 64): MAIN.  Two passes: BOUND then COLLECT.
+    // A failed a-posteriori check re-enters at COLLECT with a fixed threshold.
+    enum { MAIN = 0, BOUND = 1, COLLECT = 2 };
+    int stage = two_pass ? BOUND : MAIN;
+    bool have_first = nblocks > 0;
+
+    LseAcc lse_true, lse_raw;  // specials: true terms, and (patch) the raw terms streamed
+    lse_true.init();
+    lse_raw.init();
+    bool lse_done = !want_lse;
+    bool rescued = false;
+
+    for (int round = 0; round < 4; ++round) {
+        const bool stats = stage == MAIN;
+        const bool submax = stage == BOUND;
+        const bool lse_on = want_lse && stage != COLLECT;
+        const bool filter = stage != BOUND;
+        // One pass over the slice, double-buffered: block b+1 is in flight while b is
+        // processed.
+        if (nblocks > 0 && !have_first) {
+            fetch(cur, 0);
+        }
+        have_first = false;
+        if (stats && nblocks > 0) {
+            // Block 0's own maxima first, so that its elements already meet a real threshold.
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t c = g.cb + (uint32_t)u * NT + tid;
+                float v[E];
+                unpack<DT>(cur[u], v);
+                if (mask_stream && c >= g.main_lo && c < g.main_hi) {
+                    const uint32_t rel = c - g.cb;
+                    const uint32_t m = E == 8 ? excl_bytes[rel]
+                                              : ((excl_bytes[rel >> 1] >> ((rel & 1u) * 4u)) & 15u);
+#pragma unroll
+                    for (int j = 0; j < E; ++j) {
+                        v[j] = ((m >> j) & 1u) ? NEG_INF : v[j];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    lane_max = fmaxf(lane_max, v[j]);
+                }
             }
-            if (EXCL) {
-                for (int u = 0; u < UNROLL; ++u) {
-                    const uint32_t c = c0 + u * NT + tid;
-                    if (c < g.ce) {
+            update_threshold(true);
+        }
+        for (uint32_t b = 0; b < nblocks; ++b) {
+            if (PREFETCH) {
+                if (b + 1 < nblocks) {
+                    fetch(nxt, b + 1);
+                }
+            } else if (b > 0) {
+                fetch(cur, b);
+            }
+            {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t c = g.cb + (b * U + u) * NT + tid;
+                    float v[E];
+                    unpack<DT>(cur[u], v);
+                    if (mask_stream && c >= g.main_lo && c < g.main_hi) {
                         const uint32_t rel = c - g.cb;
                         uint32_t m;
                         if (E == 8) {
@@ -633,190 +872,910 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
                         } else {
                             m = (excl_bytes[rel >> 1] >> ((rel & 1u) * 4u)) & 15u;
                         }
+#pragma unroll
                         for (int j = 0; j < E; ++j) {
                             // all-ones when bit j is set: the element reads as -inf
                             const uint32_t on = (uint32_t)((int32_t)(m << (31 - j)) >> 31);
-                            v[u][j] = lilym_bits_f32((lilym_f32_bits(v[u][j]) & ~on) | (0xff800000u & on));
+                            v[j] = lilym_bits_f32((lilym_f32_bits(v[j]) & ~on) | (0xff800000u & on));
                         }
                     }
-                }
-            }
-            if (pass == 0) {
-                float cm = NEG_INF;
-                for (int u = 0; u < UNROLL; ++u) {
-                    for (int j = 0; j < E; ++j) {
-                        cm = fmaxf(cm, v[u][j]);
-                        if (two_pass) {
-                            const int slot = (E == 8) ? j : ((u & 1) * 4 + j);
-                            ms[slot] = fmaxf(ms[slot], v[u][j]);
-                        }
+                    float m8 = v[0];
+#pragma unroll
+                    for (int j = 1; j < E; ++j) {
+                        m8 = fmaxf(m8, v[j]);
                     }
-                }
-                lane_max = fmaxf(lane_max, cm);
-                if (LSE) {
-                    const float safe = lse.rebase(cm, c2);
-                    for (int u = 0; u < UNROLL; ++u) {
+                    if (stats) {
+                        lane_max = fmaxf(lane_max, m8);
+                    }
+                    if (submax) {
+#pragma unroll
                         for (int j = 0; j < E; ++j) {
-                            lse.term(v[u][j], c2, safe);
+                            const int slot = (E == 8) ? j : ((u & 1) * 4 + j);
+                            ms[slot] = fmaxf(ms[slot], v[j]);
+                        }
+                    }
+                    if (LSE && lse_on) {
+                        wl.template add<E>(v, m8, c2);
+                    }
+                    if (filter && __ballot(m8 >= thr_f) != 0ull) {
+#pragma unroll
+                        for (int j = 0; j < E; ++j) {
+                            append(v[j] >= thr_f, v[j], g.id_of(c, j), region, seg, wcount);
                         }
                     }
                 }
-                if (!two_pass) {
-                    // Lower bound of the k-th largest: min over groups of the group maximum.
-                    float t = lane_max;
-                    for (uint32_t o = 1; o < group; o <<= 1) {
-                        t = fmaxf(t, __shfl_xor(t, (int)o));
-                    }
-                    for (uint32_t o = group; o < 64; o <<= 1) {
-                        t = fminf(t, __shfl_xor(t, (int)o));
-                    }
-                    if (lane == 0) {
-                        __hip_atomic_store(&sh.wthr[w], t, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_WORKGROUP);
-                    }
-                    if (c0 == g.cb) {
-                        __syncthreads();  // every wave has published its first statistic
-                    }
-                    for (int i = 0; i < NWAVE; ++i) {
-                        // Other waves' values may be older: still lower bounds.
-                        t = fminf(t, __hip_atomic_load(&sh.wthr[i], __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_WORKGROUP));
-                    }
-                    thr_f = fmaxf(thr_f, lower_by_slack(t));
+            }
+            if (stats) {
+                update_threshold(false);
+            }
+            if (PREFETCH) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    cur[u] = nxt[u];
                 }
             }
-            if (filter) {
-                for (int u = 0; u < UNROLL; ++u) {
-                    const uint32_t c = c0 + u * NT + tid;
-                    for (int j = 0; j < E; ++j) {
-                        append(v[u][j] >= thr_f, v[u][j], g.id_of(c, j), cand, cap, sh);
+        }
+        if (stage == MAIN && nblocks == 0) {
+            update_threshold(true);  // keeps the barrier count the same in every workgroup
+        }
+        if (stage == BOUND) {
+            // The k-th largest of the NT x 8 sub-stream maxima bounds the k-th largest
+            // element; a margin covers maxima that belong to ids evaluated separately.
+            const uint32_t kb = patch ? min(k + k / 8u + 16u, (uint32_t)(NT * 8)) : k;
+            thr_f = lower_by_slack(wg_kth_largest(ms, kb, sh));
+            stage = COLLECT;
+            continue;
+        }
+        if (round == 0 || (two_pass && round == 1)) {
+            phase(cfg, 2);
+        }
+
+        if (lane == 0) {
+            sh.wthr_f[w] = thr_f;
+        }
+        __syncthreads();
+        float filt = sh.wthr_f[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            filt = fmaxf(filt, sh.wthr_f[i]);
+        }
+        // Close the gaps between the waves' regions (entries travel through registers).
+        if (lane == 0) {
+            sh.red_i[w] = wcount;
+        }
+        __syncthreads();
+        uint32_t n = 0, my_base = 0;
+        bool overflow = false;
+        for (int i = 0; i < NWAVE; ++i) {
+            const uint32_t ci = sh.red_i[i];
+            overflow = overflow || ci > seg;
+            if ((uint32_t)i == w) {
+                my_base = n;
+            }
+            n += min(ci, seg);
+        }
+        if (overflow) {
+            return false;
+        }
+        {
+            constexpr int PERW = CAND_CAP / NT;  // a wave moves its own region, PERW per lane
+            uint64_t keep[PERW];
+            const uint32_t mine = min(wcount, seg);
+#pragma unroll
+            for (int q = 0; q < PERW; ++q) {
+                const uint32_t i = lane + (uint32_t)q * 64u;
+                keep[q] = i < mine ? region[i] : 0ull;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < PERW; ++q) {
+                const uint32_t i = lane + (uint32_t)q * 64u;
+                if (i < mine) {
+                    cand[my_base + i] = keep[q];
+                }
+            }
+        }
+        if (tid == 0) {
+            sh.n_cand = n;
+        }
+        wcount = 0;
+        __syncthreads();
+        // Buffered composites hold the pre-temperature value: divide now, exactly.  In
+        // patch mode a candidate that is penalised or biased carried its raw value: drop
+        // it, the specials below bring it back with the true one.
+        for (uint32_t i = tid; i < n; i += NT) {
+            const uint64_t c = cand[i];
+            const uint32_t id = composite_id(c);
+            const bool drop = patch && ((pen && bit_of(a.touched, id)) || in_bias_list(a, id));
+            cand[i] = drop ? 0ull : composite_of(composite_value(c) / a.temperature, id);
+        }
+        phase(cfg, 8);
+        if (special_row) {
+            // Specials: the ids that need exact evaluation, compacted into an LDS list and
+            // walked four per thread at a time so a batch's gathers are independent loads.
+            if (tid == 0) {
+                sh.need = 0;
+            }
+            __syncthreads();
+            auto one = [&](uint32_t id, float l, uint32_t cnt) {
+                const float u = finish_pre_temperature(a, id, l, cnt, true);
+                if (!lse_done) {
+                    lse_true.add_one(u, c2);
+                    if (patch) {
+                        lse_raw.add_one(l, c2);
+                    }
+                }
+                if (u >= filt) {
+                    const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                    if (at < cap) {
+                        cand[at] = composite_of(u / a.temperature, id);
+                    }
+                }
+            };
+            auto slow_one = [&](uint32_t id) {
+                one(id, load_logit<DT>(a.logits, id), pen ? gload(a.counts + id) : 0u);
+            };
+            for (uint32_t i0 = 0; i0 < nwords; i0 += NT) {
+                const uint32_t i = i0 + tid;
+                const int64_t id0 = slice_id0 + (int64_t)i * 32;
+                uint32_t bits = 0;
+                if (i < nwords) {
+                    if (mask_stream) {
+                        bits = excl[i] & range32_at(g.id_lo, g.id_hi, id0) &
+                               bits32_at(a.allow, row_words, id0);
+                    } else if (pen) {
+                        bits = bits32_at(a.touched, row_words, id0) &
+                               range32_at(g.id_lo, g.id_hi, id0);
+                    }
+                }
+                while (__ballot(bits != 0u) != 0ull) {
+                    const bool has = bits != 0u;
+                    const uint32_t id = has ? (uint32_t)(id0 + __builtin_ctz(bits)) : 0u;
+                    bits &= bits - 1u;
+                    if (!list_push(has, id, list, list_cap, sh)) {
+                        slow_one(id);  // more specials than the list holds
+                    }
+                }
+            }
+            if (patch) {
+                // Biased ids that are not penalised (those are listed already), once each.
+                for (uint32_t i0 = 0; i0 < a.n_bias; i0 += NT) {
+                    const uint32_t i = i0 + tid;
+                    bool has = false;
+                    uint32_t id = 0;
+                    if (i < a.n_bias) {
+                        id = gload(&a.bias[i].id);
+                        has = id >= g.id_lo && id < g.id_hi && !(pen && bit_of(a.touched, id));
+                        for (uint32_t j = 0; has && j < i; ++j) {
+                            has = gload(&a.bias[j].id) != id;
+                        }
+                    }
+                    if (!list_push(has, id, list, list_cap, sh)) {
+                        slow_one(id);
+                    }
+                }
+            }
+            __syncthreads();
+            phase(cfg, 9);
+            const uint32_t m = min(sh.need, list_cap);
+            for (uint32_t i0 = tid; i0 < m; i0 += 4 * NT) {
+                uint32_t ids[4];
+                float l[4];
+                uint32_t cnt[4];
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t i = i0 + (uint32_t)q * NT;
+                    ids[q] = i < m ? list[i] : 0xffffffffu;
+                }
+                for (int q = 0; q < 4; ++q) {
+                    const bool ok = ids[q] != 0xffffffffu;
+                    l[q] = ok ? load_logit<DT>(a.logits, ids[q]) : 0.0f;
+                    cnt[q] = (ok && pen) ? gload(a.counts + ids[q]) : 0u;
+                }
+                for (int q = 0; q < 4; ++q) {
+                    if (ids[q] != 0xffffffffu) {
+                        one(ids[q], l[q], cnt[q]);
                     }
                 }
             }
         }
-        if (two_pass && pass == 0) {
-            thr_f = lower_by_slack(wg_kth_largest(ms, k, sh));
+        phase(cfg, 10);
+        // Edge ids (partial 16-byte chunks at the row's ends) were not streamed: the ones
+        // that are not specials (those were just handled) enter here with their raw value.
+        for (int side = 0; side < 2; ++side) {
+            const uint32_t lo = side == 0 ? g.id_lo : g.edge_hi_begin;
+            const uint32_t hi = side == 0 ? g.edge_lo_end : g.id_hi;
+            for (uint32_t id = lo + tid; id < hi; id += NT) {
+                const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
+                const bool is_special =
+                    special_row && ((pen && bit_of(a.touched, id)) || in_bias_list(a, id));
+                if (allowed && !is_special) {
+                    const float u = load_logit<DT>(a.logits, id);
+                    if (!lse_done) {
+                        lse_true.add_one(u, c2);
+                    }
+                    if (u >= filt && u > NEG_INF) {
+                        const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                        if (at < cap) {
+                            cand[at] = composite_of(u / a.temperature, id);
+                        }
+                    }
+                }
+            }
         }
+        phase(cfg, 11);
+        if (!lse_done) {
+            // Row sum = streamed sum - raw terms of the specials (patch) + their true terms.
+            double m_s, s_s, m_t, s_t, m_r = 0.0, s_r = 0.0;
+            wg_merge_lse(sh, wl.ref, wl.s, m_s, s_s);
+            wg_merge_lse(sh, lse_true.mc, lse_true.s, m_t, s_t);
+            if (patch) {
+                wg_merge_lse(sh, lse_raw.mc, lse_raw.s, m_r, s_r);
+            }
+            double rest = s_s;
+            bool bad = false;
+            if (patch && s_r > 0.0) {
+                rest = s_s - s_r * exp2(m_r - m_s);
+                bad = !(rest > 0.05 * s_s);  // cancellation: the streamed sum is too coarse
+            }
+            if (cfg.phase_trace != nullptr && tid == 0) {  // DEBUG
+                uint64_t* t = cfg.phase_trace + ((size_t)blockIdx.y * cfg.slices + blockIdx.x) * PHASE_SLOTS;
+                __builtin_memcpy(&t[13], &s_s, 8); __builtin_memcpy(&t[14], &s_r, 8); double dd = m_r - m_s; __builtin_memcpy(&t[15], &dd, 8);
+            }
+            if (bad) {
+                phase(cfg, 12);
+                // Rare: penalised ids held nearly all the raw mass.  Redo the sum exactly.
+                LseAcc exact;
+                exact.init();
+                for (uint32_t id = g.id_lo + tid; id < g.id_hi; id += NT) {
+                    exact.add_one(pre_temperature_of<DT>(a, id), c2);
+                }
+                double m_e, s_e;
+                wg_merge_lse(sh, exact.mc, exact.s, m_e, s_e);
+                if (tid == 0) {
+                    sh.lse_mc = m_e;
+                    sh.lse_s = s_e;
+                }
+            } else if (tid == 0) {
+                const bool has_s = rest > 0.0, has_t = s_t > 0.0;
+                const double m = has_s && has_t ? fmax(m_s, m_t) : (has_s ? m_s : m_t);
+                double total = 0.0;
+                if (has_s) {
+                    total += rest * exp2(m_s - m);
+                }
+                if (has_t) {
+                    total += s_t * exp2(m_t - m);
+                }
+                sh.lse_mc = m;
+                sh.lse_s = total;
+            }
+            lse_done = true;
+        }
+        __syncthreads();
+        n = sh.n_cand;
+        phase(cfg, 3);
+        if (n > cap) {
+            return false;
+        }
+        sorted = false;
+        n = select_topk(cand, n, k, sh, sorted);  // also drops the zeros
+        // Every element that was not collected lies strictly below `filt`.  The result is
+        // exact if k candidates were found and the k-th lies strictly above anything the
+        // division could map an uncollected value to.
+        bool good = true;
+        float lowest_value = 0.0f;
+        if (filt > F32_LOWEST) {
+            uint32_t lowest = 0xffffffffu;
+            for (uint32_t i = tid; i < n; i += NT) {
+                lowest = min(lowest, (uint32_t)(cand[i] >> 32));
+            }
+            lowest = wave_min_u32(lowest);
+            if (lane == 0) {
+                sh.red_i[w] = lowest;
+            }
+            __syncthreads();
+            lowest = sh.red_i[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                lowest = min(lowest, sh.red_i[i]);
+            }
+            __syncthreads();
+            const float below = lilym_key_value(lilym_order_key(filt) - 1u) / a.temperature;
+            good = n >= k && lilym_order_key(below) < lowest;
+            lowest_value = n > 0 ? lilym_key_value(lowest) : 0.0f;
+        }
+        if (good) {
+            if (tid == 0) {
+                sh.n_cand = n;
+            }
+            __syncthreads();
+            return true;
+        }
+        if (rescued || n < k) {
+            return false;
+        }
+        // k true candidates exist, so everything at or above the k-th of them (taken back
+        // before the division, with slack) is enough: collect exactly that.
+        rescued = true;
+        stage = COLLECT;
+        thr_f = lower_by_slack(lower_by_slack(lowest_value * a.temperature));
+        if (tid == 0) {
+            sh.n_cand = 0;
+        }
+        __syncthreads();
     }
-    if (lane == 0) {
-        sh.wthr_f[w] = thr_f;
+    return false;
+}
+
+
+// ------------------------------------------------------------------ streaming select
+//
+// The select of rows with k <= STREAM_K_MAX and no allow-mask.  One pass, one barrier per
+// block of NT x STREAM_UNROLL chunks, every 16-byte chunk read from memory once:
+//
+//   * Bound.  Each lane keeps the maximum of what it has seen; each wave takes the kw-th
+//     largest of its 64 lane maxima (kw = ceil(k' / NWAVE), a 16-step ballot search on the
+//     top half of the order key).  At least k' distinct elements are at or above the
+//     minimum of the waves' values, so that minimum is a lower bound of the k'-th largest
+//     value; it is refreshed after every block and is the same in every wave while a
+//     block is processed, which makes the run reproducible.
+//   * Owner side.  A lane whose chunk holds a value at or above the bound appends the whole
+//     chunk (16 raw bytes + its index) to its wave's queue and leaves it out of the running
+//     sum of exponentials; all other chunks only feed the lane maximum and the sum.
+//   * Listed ids (penalised: the scratch's (id, count) list; biased: the row's bias list)
+//     are sorted into per-block buckets in LDS before the scan.  While block b streams,
+//     thread t also loads the chunk of "its" listed id of block b (the same cache lines
+//     the owners are loading), evaluates the id exactly, offers it as a candidate, adds its
+//     true term to the sum and - when the chunk was not queued, which it can tell from the
+//     chunk's maximum and the block's bound - books the raw term the owner added, to be
+//     taken off at the end.  Listed ids inside queued chunks go to a short drop list.
+//   * After the scan the queued chunks are expanded: elements that are not on the drop list
+//     add their term and, at or above the final bound, become candidates.
+//
+// Values are compared before the division by the temperature; candidates are divided
+// exactly and the caller's check (k-th candidate strictly above anything a value below
+// the bound can map to) decides whether the result stands.  Any overflow returns false.
+
+struct StreamLds {
+    u32x4* qraw;
+    uint32_t* qidx;
+    uint32_t* spec;
+    uint64_t* fc;
+    uint32_t* drop;
+    uint32_t* dmask;   // per queue slot, a byte: bit j set = element j is a listed id
+    uint32_t* bkt;
+    uint32_t* bfill;
+    uint32_t* bias_id;
+    float* bias_delta;
+    __device__ __forceinline__ void init() {
+        char* b = reinterpret_cast<char*>(dyn_lds);
+        qraw = reinterpret_cast<u32x4*>(b + OFF_QRAW);
+        qidx = reinterpret_cast<uint32_t*>(b + OFF_QIDX);
+        spec = reinterpret_cast<uint32_t*>(b + OFF_SPEC);
+        fc = reinterpret_cast<uint64_t*>(b + OFF_FC);
+        drop = reinterpret_cast<uint32_t*>(b + OFF_DROP);
+        dmask = reinterpret_cast<uint32_t*>(b + OFF_DMASK);
+        bkt = reinterpret_cast<uint32_t*>(b + OFF_BKT);
+        bfill = reinterpret_cast<uint32_t*>(b + OFF_BFILL);
+        bias_id = reinterpret_cast<uint32_t*>(b + OFF_BIAS);
+        bias_delta = reinterpret_cast<float*>(b + OFF_BIAS + STREAM_BIAS_CAP * 4);
+    }
+};
+
+// 2^(v*c - ref) as a double for any argument (0 below 2^-1000).
+__device__ __forceinline__ double term_d(float v, float c, float ref) {
+    float d = __builtin_fmaf(v, c, -ref);
+    if (!(d > -1000.0f)) {
+        return 0.0;  // far below the reference, -inf, NaN
+    }
+    d = fminf(d, 1000.0f);
+    const float di = __builtin_floorf(d);
+    const float fr = d - di;
+    return __builtin_ldexp((double)__builtin_amdgcn_exp2f(fr), (int)di);
+}
+
+// The largest 16-bit prefix P with at least `need` lanes holding key16 >= P; 0 when fewer
+// than `need` lanes hold a non-zero key.
+__device__ __forceinline__ uint32_t wave_kth_key16(uint32_t key16, uint32_t need) {
+    uint32_t P = 0;
+#pragma unroll
+    for (int bit = 15; bit >= 0; --bit) {
+        const uint32_t c = P | (1u << bit);
+        const uint32_t cnt = (uint32_t)__popcll(__ballot(key16 >= c));
+        P = cnt >= need ? c : P;
+    }
+    return P;
+}
+
+__device__ __forceinline__ double wg_sum_d(Shared& sh, double v) {
+    v = wave_sum_d(v);
+    if ((threadIdx.x & 63u) == 0) {
+        sh.red_d[threadIdx.x >> 6] = v;
     }
     __syncthreads();
-    phase(cfg, 2);
-    float filt = sh.wthr_f[0];
-    for (int i = 1; i < NWAVE; ++i) {
-        filt = fmaxf(filt, sh.wthr_f[i]);
+    double t = 0.0;
+    for (int i = 0; i < NWAVE; ++i) {
+        t += sh.red_d[i];
     }
-    uint32_t n = sh.n_cand;
-    if (n > cap) {
-        return false;
+    __syncthreads();
+    return t;
+}
+
+// Records why the streaming select gave up (bit `why` of path_stats[3]) and returns false.
+__device__ __forceinline__ bool stream_fail(const LaunchCfg& cfg, uint32_t why) {
+    if (cfg.path_stats != nullptr && threadIdx.x == 0) {
+        atomicOr(&cfg.path_stats[3], 1u << why);
     }
-    // Buffered composites hold the pre-temperature value: divide now, exactly.
-    for (uint32_t i = tid; i < n; i += NT) {
-        const uint64_t c = cand[i];
-        cand[i] = composite_of(composite_value(c) / a.temperature, composite_id(c));
+    return false;
+}
+
+template <int DT, bool LSE>
+__device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g, uint32_t k, Shared& sh,
+                                              const LaunchCfg& cfg, bool& sorted) {
+    constexpr int E = Geo<DT>::E;
+    constexpr int U = STREAM_UNROLL;
+    constexpr uint32_t BLOCK = NT * U;
+    constexpr uint32_t QSEG = Q_CAP / NWAVE;
+    constexpr uint32_t NONE = 0xffffffffu;
+    constexpr uint32_t ID_MASK = (1u << SPEC_ID_BITS) - 1u;
+    constexpr int PREG = 12;  // listed ids a thread keeps in registers between the two bucket passes
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const uint32_t nchunks = g.ce - g.cb;
+    const uint32_t nblocks = (nchunks + BLOCK - 1) / BLOCK;
+    const bool pen = (a.flags & F_PEN) != 0;
+    const uint32_t n_bias = a.n_bias;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    const float c2 = a.c2;
+    if (nblocks > MAX_BUCKETS || n_bias > STREAM_BIAS_CAP || g.vocab > (1u << SPEC_ID_BITS)) {
+        return stream_fail(cfg, 1u);
     }
-    if (EXCL) {
-        // Specials: ids kept out of the stream that are allowed (penalised or biased).
-        // Their ids are compacted into an LDS list, then the workgroup walks the list four
-        // ids per thread at a time, so the gathers of a batch (logit, count) are
-        // independent loads and the work is balanced.
-        const bool pen = (a.flags & F_PEN) != 0;
-        const int64_t slice_id0 = (int64_t)g.cb * E - g.pad;
-        auto special_bits = [&](uint32_t i) -> uint32_t {
-            const int64_t id0 = slice_id0 + (int64_t)i * 32;
-            uint32_t b = excl[i] & range32_at(g.id_lo, g.id_hi, id0);
-            if (a.allow != nullptr) {
-                b &= bits32_at(a.allow, row_words, id0);
-            }
-            return b;
-        };
-        auto process = [&](uint32_t id, float l, uint32_t cnt) {
-            const float u = finish_pre_temperature(a, id, l, cnt, true);
-            if (LSE) {
-                lse.add_one(u, c2);
-            }
-            if (u >= filt) {
-                const uint32_t at = atomicAdd(&sh.n_cand, 1u);
-                if (at < cap) {
-                    cand[at] = composite_of(u / a.temperature, id);
-                }
-            }
-        };
-        if (tid == 0) {
-            sh.need = 0;
+    StreamLds L;
+    L.init();
+
+    auto fetch = [&](u32x4 (&dst)[U], uint32_t b) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            dst[u] = g.load_raw(g.cb + (b * U + u) * NT + tid);
         }
-        __syncthreads();
-        uint32_t* list = excl + cfg.excl_words;  // SPECIAL_LIST_CAP ids behind the bitmap
-        const uint32_t list_cap = SPECIAL_LIST_CAP;
-        for (uint32_t i0 = 0; i0 < nwords; i0 += NT) {
-            const uint32_t i = i0 + tid;
-            uint32_t bits = i < nwords ? special_bits(i) : 0u;
-            while (__ballot(bits != 0u) != 0ull) {
-                const bool has = bits != 0u;
-                const uint32_t id = has ? (uint32_t)(slice_id0 + (int64_t)i * 32 + __builtin_ctz(bits)) : 0u;
-                bits &= bits - 1u;
-                const uint64_t mask = __ballot(has);
-                const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
-                    (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
-                const int leader = __builtin_ctzll(mask);
-                uint32_t base = 0;
-                if ((int)lane == leader) {
-                    base = atomicAdd(&sh.need, (uint32_t)__popcll(mask));
-                }
-                base = __shfl(base, leader);
-                if (has) {
-                    if (base + rank < list_cap) {
-                        list[base + rank] = id;
-                    } else {  // more specials than the list holds: one at a time
-                        process(id, load_logit<DT>(a.logits, id), pen ? gload(a.counts + id) : 0u);
+    };
+    u32x4 cur[U], nxt[U];
+    if (nblocks > 0) {
+        fetch(cur, 0);  // in flight while the listed ids are bucketed
+    }
+
+    // ---- the slice's listed ids, bucketed by block
+    // The first PREG x NT list entries are requested together with the list's length (the
+    // list's memory is valid up to pairs_cap whatever the length turns out to be).
+    uint32_t n_pairs = 0;
+    uint64_t early[PREG];
+    if (pen) {
+        n_pairs = gload(a.n_pairs);
+#pragma unroll
+        for (int q = 0; q < PREG; ++q) {
+            const uint32_t p = (uint32_t)q * NT + tid;
+            early[q] = p < a.pairs_cap ? gload(reinterpret_cast<const uint64_t*>(a.pairs) + p)
+                                       : ~0ull;
+        }
+    }
+    if (tid <= MAX_BUCKETS) {
+        L.bkt[tid] = 0;
+    }
+    if (tid < MAX_BUCKETS) {
+        L.bfill[tid] = 0;
+    }
+    if (tid < Q_CAP / 4) {
+        L.dmask[tid] = 0;
+    }
+    if (tid == 0) {
+        sh.n_fc = 0;
+        sh.n_drop = 0;
+        sh.fail = 0;
+    }
+    for (uint32_t i = tid; i < n_bias; i += NT) {
+        L.bias_id[i] = gload(&a.bias[i].id);
+        L.bias_delta[i] = gload(&a.bias[i].delta);
+    }
+    __syncthreads();
+    if (n_pairs > a.pairs_cap) {
+        return stream_fail(cfg, 2u);  // the list overflowed: the bitmap and the counts hold the truth
+    }
+    const bool listed_row = n_pairs != 0 || n_bias != 0;
+    // Block of a streamed id of this slice, NONE for ids outside it or in a partial chunk.
+    auto block_of = [&](uint32_t id) -> uint32_t {
+        if (id >= g.vocab) {
+            return NONE;
+        }
+        const uint32_t c = (id + g.pad) / E;
+        if (c < g.main_lo || c >= g.main_hi) {
+            return NONE;
+        }
+        return (c - g.cb) / BLOCK;
+    };
+    // The bias entry i opens a bucket slot when it is the first of its id and the id is
+    // not on the scratch's list (that entry covers it).
+    auto bias_block = [&](uint32_t i) -> uint32_t {
+        const uint32_t id = L.bias_id[i];
+        for (uint32_t j = 0; j < i; ++j) {
+            if (L.bias_id[j] == id) {
+                return NONE;
+            }
+        }
+        const uint32_t b = block_of(id);
+        if (b != NONE && pen && bit_of(a.touched, id)) {
+            return NONE;
+        }
+        return b;
+    };
+    if (listed_row) {
+        uint32_t packed[PREG];  // id | min(count, 4095) << 20, NONE when not of this slice
+        uint32_t blk[PREG];
+#pragma unroll
+        for (int q = 0; q < PREG; ++q) {
+            const uint32_t p = (uint32_t)q * NT + tid;
+            packed[q] = NONE;
+            blk[q] = NONE;
+            if (p < n_pairs) {
+                const uint32_t id = (uint32_t)early[q];
+                blk[q] = block_of(id);
+                packed[q] = id | (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS);
+            }
+        }
+        for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+            for (int q = 0; q < PREG; ++q) {
+                if (blk[q] != NONE) {
+                    if (pass == 0) {
+                        atomicAdd(&L.bkt[blk[q]], 1u);
+                    } else {
+                        L.spec[L.bkt[blk[q]] + atomicAdd(&L.bfill[blk[q]], 1u)] = packed[q];
                     }
                 }
             }
-        }
-        __syncthreads();
-        const uint32_t m = min(sh.need, list_cap);
-        for (uint32_t i0 = tid; i0 < m; i0 += 4 * NT) {
-            uint32_t ids[4];
-            float l[4];
-            uint32_t cnt[4];
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t i = i0 + (uint32_t)q * NT;
-                ids[q] = i < m ? list[i] : 0xffffffffu;
+            for (uint32_t p = PREG * NT + tid; p < n_pairs; p += NT) {  // lists beyond the registers
+                const uint64_t e = gload(reinterpret_cast<const uint64_t*>(a.pairs) + p);
+                const uint32_t id = (uint32_t)e;
+                const uint32_t b = block_of(id);
+                if (b != NONE) {
+                    if (pass == 0) {
+                        atomicAdd(&L.bkt[b], 1u);
+                    } else {
+                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] =
+                            id | (min((uint32_t)(e >> 32), 4095u) << SPEC_ID_BITS);
+                    }
+                }
             }
-            for (int q = 0; q < 4; ++q) {
-                const bool ok = ids[q] != 0xffffffffu;
-                l[q] = ok ? load_logit<DT>(a.logits, ids[q]) : 0.0f;
-                cnt[q] = (ok && pen) ? gload(a.counts + ids[q]) : 0u;
+            for (uint32_t i = tid; i < n_bias; i += NT) {
+                const uint32_t b = bias_block(i);
+                if (b != NONE) {
+                    if (pass == 0) {
+                        atomicAdd(&L.bkt[b], 1u);
+                    } else {
+                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = L.bias_id[i];
+                    }
+                }
             }
-            for (int q = 0; q < 4; ++q) {
-                if (ids[q] != 0xffffffffu) {
-                    process(ids[q], l[q], cnt[q]);
+            __syncthreads();
+            if (pass == 0) {
+                if (tid < 64) {  // counts -> exclusive offsets, total in bkt[MAX_BUCKETS]
+                    const uint32_t cnt = L.bkt[tid];
+                    uint32_t incl = cnt;
+                    for (int o = 1; o < 64; o <<= 1) {
+                        const uint32_t t = __shfl_up(incl, o);
+                        if ((int)tid >= o) {
+                            incl += t;
+                        }
+                    }
+                    L.bkt[tid] = incl - cnt;
+                    if (tid == 63) {
+                        L.bkt[MAX_BUCKETS] = incl;
+                    }
+                }
+                __syncthreads();
+                if (L.bkt[MAX_BUCKETS] > SPEC_CAP) {
+                    return stream_fail(cfg, 3u);
                 }
             }
         }
     }
-    if (LSE) {
-        lse_reduce(sh, lse);
-    } else {
+    phase(cfg, 1);
+
+    // ---- scan
+    const uint32_t keff = min(k + k / 8u + 2u, 64u * NWAVE);
+    const uint32_t kw = (keff + NWAVE - 1) / NWAVE;
+    float lane_max = NEG_INF;
+    float T = F32_LOWEST;       // the block's bound, the same in every thread
+    float ref_s = 0.0f;         // reference of the double sums
+    uint32_t wq = 0;            // this wave's queue fill
+    WaveLse wl;
+    wl.init();
+    double acc_t = 0.0, acc_r = 0.0, acc_q = 0.0;
+    uint32_t parity = 0;
+
+    // Brings T up to date with everything the lanes have seen, the current block included.
+    auto refresh_bound = [&](bool first) {
+        const uint32_t key16 = lane_max > NEG_INF ? (lilym_order_key(lane_max) >> 16) : 0u;
+        const uint32_t P = wave_kth_key16(key16, kw);
+        const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
+        float wm = 0.0f;
+        if (first) {
+            wm = wave_max_f(lane_max);
+        }
+        if (lane == 0) {
+            sh.bound[parity][w] = mine;
+            if (first) {
+                sh.red_f[w] = wm;
+            }
+        }
         __syncthreads();
+        float t = sh.bound[parity][0];
+        for (int i = 1; i < NWAVE; ++i) {
+            t = fminf(t, sh.bound[parity][i]);
+        }
+        parity ^= 1u;
+        T = fmaxf(T, lower_by_slack(t));
+        if (first) {
+            float m = sh.red_f[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                m = fmaxf(m, sh.red_f[i]);
+            }
+            // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
+            ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
+        }
+    };
+
+    struct Listed {
+        uint32_t ent;
+        float raw;
+        u32x4 chunk;
+    };
+    auto listed_fetch = [&](Listed& r, uint32_t b, uint32_t round) {
+        r.ent = NONE;
+        r.raw = 0.0f;
+        r.chunk = u32x4{0u, 0u, 0u, 0u};
+        const uint32_t lo = L.bkt[b], hi = L.bkt[b + 1];
+        const uint32_t e = lo + round * NT + ((tid + NT - ((b * 64u) % NT)) % NT);
+        if (e < hi) {
+            r.ent = L.spec[e];
+            const uint32_t id = r.ent & ID_MASK;
+            const uint32_t c = (id + g.pad) / E;
+            r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (size_t)c * 16));
+            r.raw = load_logit<DT>(a.logits, id);
+        }
+    };
+    auto listed_process = [&](const Listed& r) {
+        if (r.ent == NONE) {
+            return;
+        }
+        const uint32_t id = r.ent & ID_MASK;
+        uint32_t cnt = r.ent >> SPEC_ID_BITS;
+        if (cnt == 4095u) {
+            cnt = gload(a.counts + id);
+        }
+        float v[E];
+        unpack<DT>(r.chunk, v);
+        float m8 = v[0];
+#pragma unroll
+        for (int j = 1; j < E; ++j) {
+            m8 = fmaxf(m8, v[j]);
+        }
+        const bool queued = m8 >= T;  // the owner's test, on the same bits
+        float t = r.raw;
+        for (uint32_t j = 0; j < n_bias; ++j) {
+            if (L.bias_id[j] == id) {
+                t += L.bias_delta[j];
+            }
+        }
+        if (cnt > 0u) {
+            t = t > 0.0f ? t / a.repetition : t * a.repetition;
+            t -= a.presence + a.frequency * (float)cnt;
+        }
+        if (want_lse) {
+            acc_t += term_d(t, c2, ref_s);
+            if (!queued) {
+                acc_r += term_d(r.raw, c2, ref_s);
+            }
+        }
+        if (queued) {
+            const uint32_t at = atomicAdd(&sh.n_drop, 1u);
+            if (at < DROP_CAP) {
+                L.drop[at] = id;
+            }
+        }
+        if (t >= T && t > NEG_INF) {
+            const uint32_t at = atomicAdd(&sh.n_fc, 1u);
+            if (at < FC_CAP) {
+                L.fc[at] = composite_of(t / a.temperature, id);
+            }
+        }
+    };
+
+    Listed lcur, lnxt;
+    lcur.ent = NONE;
+    if (nblocks > 0 && listed_row) {
+        listed_fetch(lcur, 0, 0);
     }
-    n = sh.n_cand;
+    if (nblocks == 0) {
+        refresh_bound(true);  // the same barriers in every workgroup
+    }
+    for (uint32_t b = 0; b < nblocks; ++b) {
+        const bool more = b + 1 < nblocks;
+        if (more) {
+            fetch(nxt, b + 1);
+            if (listed_row) {
+                listed_fetch(lnxt, b + 1, 0);
+            }
+        }
+        // The block's own maxima enter the bound before the block is filtered.
+        float m8[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float v[E];
+            unpack<DT>(cur[u], v);
+            m8[u] = v[0];
+#pragma unroll
+            for (int j = 1; j < E; ++j) {
+                m8[u] = fmaxf(m8[u], v[j]);
+            }
+            lane_max = fmaxf(lane_max, m8[u]);
+        }
+        refresh_bound(b == 0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t c = g.cb + (b * U + u) * NT + tid;
+            const bool pass = m8[u] >= T;
+            const uint64_t mask = __ballot(pass);
+            if (mask != 0ull) {
+                const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+                    (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                const uint32_t at = wq + rank;
+                if (pass && at < QSEG) {
+                    L.qraw[w * QSEG + at] = cur[u];
+                    L.qidx[w * QSEG + at] = c;
+                }
+                wq += (uint32_t)__popcll(mask);
+            }
+            if (LSE && want_lse) {
+                wl.template add_chunk<DT>(cur[u], m8[u], c2, !pass);
+            }
+        }
+        if (listed_row) {
+            listed_process(lcur);
+            const uint32_t n_b = L.bkt[b + 1] - L.bkt[b];
+            for (uint32_t round = 1; round * NT < n_b; ++round) {
+                Listed extra;
+                listed_fetch(extra, b, round);
+                listed_process(extra);
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                cur[u] = nxt[u];
+            }
+            lcur = lnxt;
+        }
+    }
+    phase(cfg, 2);
+
+    // ---- after the scan
+    if (lane == 0) {
+        sh.qfill[w] = wq;
+    }
+    __syncthreads();
+    const float filt = T;
+    {
+        bool overflow = sh.n_drop > DROP_CAP;
+        for (int i = 0; i < NWAVE; ++i) {
+            overflow = overflow || sh.qfill[i] > QSEG;
+        }
+        if (overflow) {
+            return stream_fail(cfg, 4u);
+        }
+    }
+    // Listed ids inside queued chunks: mark their element in the chunk's queue slot.  A
+    // wave's segment is in ascending chunk order, so the slot is found by bisection.
+    for (uint32_t d = tid; d < sh.n_drop; d += NT) {
+        const uint32_t id = L.drop[d];
+        const uint32_t c = (id + g.pad) / E, j = (id + g.pad) % E;
+        const uint32_t ow = ((c - g.cb) % NT) / 64u;
+        uint32_t lo = ow * QSEG, hi = lo + sh.qfill[ow];
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (L.qidx[mid] < c) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        atomicOr(&L.dmask[lo >> 2], (1u << j) << ((lo & 3u) * 8u));
+    }
+    __syncthreads();
+    auto offer = [&](float u, uint32_t id) {
+        if (u >= filt && u > NEG_INF) {
+            const uint32_t at = atomicAdd(&sh.n_fc, 1u);
+            if (at < FC_CAP) {
+                L.fc[at] = composite_of(u / a.temperature, id);
+            }
+        }
+    };
+    for (int ww = 0; ww < NWAVE; ++ww) {
+        const uint32_t n_e = sh.qfill[ww] * E;
+        for (uint32_t e = tid; e < n_e; e += NT) {
+            const uint32_t slot = (uint32_t)ww * QSEG + e / E, j = e % E;
+            const uint32_t id = g.id_of(L.qidx[slot], (int)j);
+            float v;
+            if (DT == LILY_BF16) {
+                v = lilym_bits_f32((uint32_t)reinterpret_cast<const uint16_t*>(L.qraw + slot)[j] << 16);
+            } else {
+                v = reinterpret_cast<const float*>(L.qraw + slot)[j];
+            }
+            const bool dropped = (L.dmask[slot >> 2] >> ((slot & 3u) * 8u + j)) & 1u;
+            if (!dropped) {
+                if (want_lse) {
+                    acc_q += term_d(v, c2, ref_s);
+                }
+                offer(v, id);
+            }
+        }
+    }
+    phase(cfg, 8);
+    // Ids of partial 16-byte chunks at the row's ends were not streamed: exact, one by one.
+    for (int side = 0; side < 2; ++side) {
+        const uint32_t lo = side == 0 ? g.id_lo : g.edge_hi_begin;
+        const uint32_t hi = side == 0 ? g.edge_lo_end : g.id_hi;
+        for (uint32_t id = lo + tid; id < hi; id += NT) {
+            const float u = pre_temperature_of<DT>(a, id);
+            if (want_lse) {
+                acc_q += term_d(u, c2, ref_s);
+            }
+            offer(u, id);
+        }
+    }
+    phase(cfg, 9);
+    if (cfg.phase_trace != nullptr && tid == 0) {  // DBG
+        uint64_t* t = cfg.phase_trace + ((size_t)blockIdx.y * cfg.slices + blockIdx.x) * PHASE_SLOTS;
+        t[13] = sh.n_drop; t[14] = sh.qfill[0] + sh.qfill[1] + sh.qfill[2] + sh.qfill[3]; t[15] = sh.n_fc;
+    }
+    if (want_lse) {
+        double m_s, s_s;
+        wg_merge_lse(sh, wl.ref, wl.s, m_s, s_s);
+        const double streamed = s_s > 0.0 ? s_s * exp2(m_s - (double)ref_s) : 0.0;
+        const double booked = wg_sum_d(sh, acc_r);
+        const double exact = wg_sum_d(sh, acc_t + acc_q);
+        const double rest = streamed - booked;
+        // Listed ids held nearly all of what was streamed: the difference is too coarse.
+        const bool coarse = booked > 0.0 && !(rest > 0.05 * streamed);
+        phase(cfg, 10);
+        if (coarse) {
+            phase(cfg, 11);
+            LseAcc all;
+            all.init();
+            for (uint32_t id = g.id_lo + tid; id < g.id_hi; id += NT) {
+                all.add_one(pre_temperature_of<DT>(a, id), c2);
+            }
+            double m_e, s_e;
+            wg_merge_lse(sh, all.mc, all.s, m_e, s_e);
+            if (tid == 0) {
+                sh.lse_mc = m_e;
+                sh.lse_s = s_e;
+            }
+        } else if (tid == 0) {
+            sh.lse_mc = (double)ref_s;
+            sh.lse_s = (rest > 0.0 ? rest : 0.0) + exact;
+        }
+    }
+    __syncthreads();
+    uint32_t n = sh.n_fc;
     phase(cfg, 3);
-    if (n > cap) {
-        return false;
+    if (n > FC_CAP) {
+        return stream_fail(cfg, 5u);
     }
     sorted = false;
-    if (n > k) {
-        n = select_topk(cand, n, k, sh, sorted);
-    }
-    // Every element that was not collected lies strictly below `filt`; it must also
-    // lie strictly below the k-th adjusted value, or the division has merged it
-    // into the boundary's tie class.
-    if (filt > F32_LOWEST && n > 0) {
+    n = select_topk(L.fc, n, k, sh, sorted);
+    // Everything that is not a candidate lies strictly below `filt`: the result is exact if
+    // k candidates were found and the k-th lies strictly above anything the division can
+    // map such a value to.
+    if (filt > F32_LOWEST) {
         uint32_t lowest = 0xffffffffu;
         for (uint32_t i = tid; i < n; i += NT) {
-            lowest = min(lowest, (uint32_t)(cand[i] >> 32));
+            lowest = min(lowest, (uint32_t)(L.fc[i] >> 32));
         }
         lowest = wave_min_u32(lowest);
         if (lane == 0) {
@@ -829,8 +1788,22 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
         }
         __syncthreads();
         const float below = lilym_key_value(lilym_order_key(filt) - 1u) / a.temperature;
-        if (!(lilym_order_key(below) < lowest)) {
-            return false;
+        if (!(n >= k && lilym_order_key(below) < lowest)) {
+            return stream_fail(cfg, 6u);
+        }
+    }
+    // The caller and the tail expect the candidates at the start of dynamic LDS.
+    uint64_t* cand = dyn_lds;
+    uint64_t keep[(STREAM_K_MAX + NT - 1) / NT];
+    for (uint32_t q = 0; q * NT < STREAM_K_MAX; ++q) {
+        const uint32_t i = q * NT + tid;
+        keep[q] = i < n ? L.fc[i] : 0ull;
+    }
+    __syncthreads();
+    for (uint32_t q = 0; q * NT < STREAM_K_MAX; ++q) {
+        const uint32_t i = q * NT + tid;
+        if (i < n) {
+            cand[i] = keep[q];
         }
     }
     if (tid == 0) {
@@ -847,7 +1820,7 @@ __device__ bool select_fast(const RowArgs& a, const Geo<DT>& g, uint32_t k, bool
 // any input (ties, masks, few finite values).  Leaves the winners (unsorted) in
 // cand[0 .. sh.n_cand).
 template <int DT>
-__device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, uint32_t k,
+__device__ __forceinline__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, uint32_t k,
                                   bool want_lse, uint64_t* cand, uint32_t cap, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     uint64_t prefix = 0, pmask = 0;
@@ -904,7 +1877,7 @@ __device__ void select_exhaustive(const RowArgs& a, uint32_t e0, uint32_t e1, ui
 
 // Descending sort of cand[0..n).  Up to 64 entries: one wave, in registers.
 // More: bitonic in LDS over the next power of two (the buffer holds it).
-__device__ void sort_desc(uint64_t* cand, uint32_t n) {
+__device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
     if (n <= 64) {
         if (threadIdx.x < 64) {
             const uint32_t lane = threadIdx.x;
@@ -950,16 +1923,38 @@ __device__ void sort_desc(uint64_t* cand, uint32_t n) {
 
 // ------------------------------------------------------------------ tail
 
+// Counts one emission of `id` in a scratch: the dense count, and the id's entry in the list
+// (appended with the first count; `touched` marks the listed ids).
+__device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched, CountPair* pairs,
+                                            uint32_t* n_pairs, uint32_t* pos, uint32_t pairs_cap,
+                                            uint32_t id) {
+    const uint32_t before = atomicAdd(&counts[id], 1u);
+    const uint32_t bit = 1u << (id & 31u);
+    const uint32_t bits = atomicOr(&touched[id >> 5], bit);
+    if ((bits & bit) == 0u) {
+        const uint32_t p = atomicAdd(n_pairs, 1u);
+        if (p < pairs_cap) {
+            pairs[p].id = id;
+            pairs[p].count = before + 1u;
+            pos[id] = p;
+        }
+    } else {
+        const uint32_t p = pos[id];
+        if (p < pairs_cap && pairs[p].id == id) {
+            pairs[p].count = before + 1u;
+        }
+    }
+}
+
 __device__ __forceinline__ void emit(const RowArgs& a, uint32_t id) {
     *a.out_id = id;
     if (a.flags & F_PEN) {
-        atomicAdd(&a.counts[id], 1u);
-        atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
+        count_token(a.counts, a.touched, a.pairs, a.n_pairs, a.pos, a.pairs_cap, id);
     }
 }
 
 // First slot of prefix[0..n) whose value exceeds target, else the last slot.
-__device__ uint32_t pick_sequential(const float* prefix, uint32_t n, float target) {
+__device__ __forceinline__ uint32_t pick_sequential(const float* prefix, uint32_t n, float target) {
     for (uint32_t i = 0; i < n; ++i) {
         if (target < prefix[i]) {
             return i;
@@ -971,7 +1966,7 @@ __device__ uint32_t pick_sequential(const float* prefix, uint32_t n, float targe
 // log p(id) = (u*c2 - mc - log2 s) * ln 2, with the id's exponent u*c2 formed exactly as
 // the row sum formed its terms, so the two cancel when the id carries all the mass.
 template <int DT>
-__device__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
+__device__ __forceinline__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
     if (a.out_logprob == nullptr) {
         return;
     }
@@ -988,7 +1983,7 @@ __device__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, u
 
 // cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
 template <int DT>
-__device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
+__device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
                      uint64_t* cand, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     if (n == 0) {
@@ -1143,26 +2138,39 @@ __device__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n
 // ties: elementwise.metal:145-150.  Result: the best (value, id) of the slice as a
 // composite; id bits all zero when no element qualified.
 template <int DT>
-__device__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>& g, Shared& sh) {
+__device__ __forceinline__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>& g, Shared& sh) {
     constexpr int E = Geo<DT>::E;
     const uint32_t tid = threadIdx.x;
     float bv = NEG_INF;
     uint32_t bi = 0xffffffffu;
     for (uint32_t c0 = g.cb; c0 < g.ce; c0 += NT * UNROLL) {
-        float v[UNROLL][E];
+        u32x4 raw[UNROLL];
         for (int u = 0; u < UNROLL; ++u) {
-            g.load(a.logits, c0 + u * NT + tid, v[u]);
+            raw[u] = g.load_raw(c0 + u * NT + tid);
         }
         for (int u = 0; u < UNROLL; ++u) {
             const uint32_t c = c0 + u * NT + tid;
+            float v[E];
+            unpack<DT>(raw[u], v);
             for (int j = 0; j < E; ++j) {
                 const uint32_t id = g.id_of(c, j);
-                const bool inside = c < g.ce && id < g.vocab;  // id wraps for the pad
-                const float x = v[u][j];
+                const bool inside = c >= g.main_lo && c < g.main_hi;
+                const float x = v[j];
                 if (inside && (x > bv || (x == bv && id < bi))) {
                     bv = x;
                     bi = id;
                 }
+            }
+        }
+    }
+    for (int side = 0; side < 2; ++side) {
+        const uint32_t lo = side == 0 ? g.id_lo : g.edge_hi_begin;
+        const uint32_t hi = side == 0 ? g.edge_lo_end : g.id_hi;
+        for (uint32_t id = lo + tid; id < hi; id += NT) {
+            const float x = load_logit<DT>(a.logits, id);
+            if (x > bv || (x == bv && id < bi)) {
+                bv = x;
+                bi = id;
             }
         }
     }
@@ -1183,7 +2191,7 @@ __device__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>& g, Shared& sh)
 // ------------------------------------------------------------------ the row kernel
 
 template <int DT, bool EXCL, bool LSE>
-__device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
+__device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
     const uint32_t tid = threadIdx.x;
     const uint32_t s = blockIdx.x, row = blockIdx.y, S = cfg.slices;
     const uint32_t vocab = cfg.vocab;
@@ -1222,13 +2230,25 @@ __device__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
         __syncthreads();
     } else {
         bool done = false;
-        if (cfg.path != 1u) {
+        uint32_t took = 2;
+        if (cfg.path == 0u && (a.flags & F_STREAM)) {
+            done = select_stream<DT, LSE>(a, g, a.k, sh, cfg, sorted);
+            took = done ? 0u : took;
+            if (!done) {
+                __syncthreads();
+            }
+        }
+        if (!done && cfg.path != 1u && cfg.old_layout != 0u) {
             const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
             if (EXCL || !special) {
                 const bool two_pass = a.k > 64u || cfg.path == 2u;
                 done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh, cfg,
                                                   sorted);
+                took = done ? 1u : took;
             }
+        }
+        if (cfg.path_stats != nullptr && tid == 0) {
+            atomicAdd(&cfg.path_stats[took], 1u);
         }
         if (!done) {
             __syncthreads();
@@ -1355,18 +2375,26 @@ __device__ __forceinline__ void tail_arrays(Shared& sh) {
     sh.res = f + 2 * K_CAP;
 }
 
-template <int DT, bool EXCL, bool LSE>
-__global__ __launch_bounds__(NT) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
-    __shared__ Shared sh;
-    __shared__ RowArgs a;
-    // The row's arguments from the kernel-argument segment into LDS (a dynamic index into
-    // the by-value array would copy all of it to scratch memory).
-    for (int r = 0; r < INLINE_ROWS; ++r) {
-        if (r == (int)blockIdx.y && threadIdx.x < sizeof(RowArgs) / 4) {
-            reinterpret_cast<uint32_t*>(&a)[threadIdx.x] =
-                reinterpret_cast<const uint32_t*>(&rows.r[r])[threadIdx.x];
-        }
+// The row's arguments are the same for every thread: read through the constant address
+// space they arrive by scalar loads and stay in scalar registers.
+__device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowArgs* src) {
+    static_assert(sizeof(RowArgs) % 16 == 0, "RowArgs is copied in 16-byte pieces");
+    const LILY_CONST u32x4* from = (const LILY_CONST u32x4*)src;
+    u32x4* to = reinterpret_cast<u32x4*>(&a);
+    for (unsigned i = 0; i < sizeof(RowArgs) / 16; ++i) {
+        to[i] = from[i];
     }
+}
+
+template <int DT, bool EXCL, bool LSE>
+__global__ __launch_bounds__(NT, 4) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
+    __shared__ Shared sh;
+    // `rows` is the first kernel argument: index it in the kernel-argument segment itself
+    // (indexing the by-value copy would move all of it to scratch memory).
+    const LILY_CONST RowArgs* table =
+        (const LILY_CONST RowArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+    RowArgs a;
+    load_row_args(a, table + blockIdx.y);
     if (threadIdx.x == 0) {
         tail_arrays(sh);
     }
@@ -1375,14 +2403,11 @@ __global__ __launch_bounds__(NT) void k_rows_inline(InlineRows rows, LaunchCfg c
 }
 
 template <int DT, bool EXCL, bool LSE>
-__global__ __launch_bounds__(NT) void k_rows_table(LaunchCfg cfg) {
+__global__ __launch_bounds__(NT, 4) void k_rows_table(LaunchCfg cfg) {
     __shared__ Shared sh;
-    __shared__ RowArgs a;
-    // One coalesced copy of the row's arguments into LDS.
-    if (threadIdx.x < sizeof(RowArgs) / 4) {
-        reinterpret_cast<uint32_t*>(&a)[threadIdx.x] =
-            gload(reinterpret_cast<const uint32_t*>(&cfg.table[blockIdx.y]) + threadIdx.x);
-    }
+    const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
+    RowArgs a;
+    load_row_args(a, table + blockIdx.y);
     if (threadIdx.x == 0) {
         tail_arrays(sh);
     }
@@ -1399,43 +2424,71 @@ __global__ void k_fill_u32(uint32_t* p, uint32_t n, uint32_t v) {
     }
 }
 
-__global__ void k_add_history(uint32_t* counts, uint32_t* touched, uint32_t vocab,
-                              const uint32_t* ids, uint32_t n) {
+// counts[id] += 1 per occurrence; ids counted for the first time join the list (their
+// count is filled in by k_refresh_pairs once every occurrence has been added).
+__global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         const uint32_t id = ids[i];
-        if (id < vocab) {
-            atomicAdd(&counts[id], 1u);
-            atomicOr(&touched[id >> 5], 1u << (id & 31u));
-        }
-    }
-}
-
-__global__ void k_uncount(uint32_t* counts, uint32_t* touched, uint32_t vocab, uint32_t token) {
-    if (blockIdx.x == 0 && threadIdx.x == 0 && token < vocab) {
-        const uint32_t c = counts[token];
-        if (c > 0u) {
-            counts[token] = c - 1u;
-            if (c == 1u) {
-                touched[token >> 5] &= ~(1u << (token & 31u));
+        if (id < sc.vocab) {
+            atomicAdd(&sc.counts[id], 1u);
+            const uint32_t bit = 1u << (id & 31u);
+            const uint32_t bits = atomicOr(&sc.touched[id >> 5], bit);
+            if ((bits & bit) == 0u) {
+                const uint32_t p = atomicAdd(sc.n_pairs, 1u);
+                if (p < sc.pairs_cap) {
+                    sc.pairs[p].id = id;
+                    sc.pos[id] = p;
+                }
             }
         }
     }
 }
 
-// touched[w] = bits of the non-zero counts in word w (after counts were written whole).
-__global__ void k_rebuild_touched(const uint32_t* counts, uint32_t* touched, uint32_t vocab) {
+// pairs[p].count = counts[pairs[p].id] for every listed id.
+__global__ void k_refresh_pairs(ScratchView sc) {
+    const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t n = min(*sc.n_pairs, sc.pairs_cap);
+    if (p < n) {
+        sc.pairs[p].count = sc.counts[sc.pairs[p].id];
+    }
+}
+
+// Saturating decrement; the id stays listed (with a count that may now be 0).
+__global__ void k_uncount(ScratchView sc, uint32_t token) {
+    if (blockIdx.x == 0 && threadIdx.x == 0 && token < sc.vocab) {
+        const uint32_t c = sc.counts[token];
+        if (c > 0u) {
+            sc.counts[token] = c - 1u;
+            const uint32_t p = sc.pos[token];
+            if (((sc.touched[token >> 5] >> (token & 31u)) & 1u) && p < sc.pairs_cap &&
+                sc.pairs[p].id == token) {
+                sc.pairs[p].count = c - 1u;
+            }
+        }
+    }
+}
+
+// After counts were written whole: touched[w] = bits of the non-zero counts in word w, and
+// the list is rebuilt from them (n_pairs was cleared before the launch).
+__global__ void k_rebuild_listed(ScratchView sc) {
     const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
-    const uint32_t words = (vocab + 31u) / 32u;
+    const uint32_t words = (sc.vocab + 31u) / 32u;
     if (w < words) {
         uint32_t bits = 0;
         for (uint32_t b = 0; b < 32u; ++b) {
             const uint32_t id = w * 32u + b;
-            if (id < vocab && counts[id] != 0u) {
+            if (id < sc.vocab && sc.counts[id] != 0u) {
                 bits |= 1u << b;
+                const uint32_t p = atomicAdd(sc.n_pairs, 1u);
+                if (p < sc.pairs_cap) {
+                    sc.pairs[p].id = id;
+                    sc.pairs[p].count = sc.counts[id];
+                    sc.pos[id] = p;
+                }
             }
         }
-        touched[w] = bits;
+        sc.touched[w] = bits;
     }
 }
 
@@ -1510,27 +2563,25 @@ hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t
     return hipGetLastError();
 }
 
-hipError_t launch_add_history(hipStream_t stream, uint32_t* counts, uint32_t* touched,
-                              uint32_t vocab, const uint32_t* ids, uint32_t n) {
+hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const uint32_t* ids,
+                              uint32_t n) {
     if (n == 0) {
         return hipSuccess;
     }
-    hipLaunchKernelGGL(k_add_history, dim3((n + 255) / 256), dim3(256), 0, stream, counts, touched,
-                       vocab, ids, n);
+    hipLaunchKernelGGL(k_add_history, dim3((n + 255) / 256), dim3(256), 0, stream, sc, ids, n);
+    hipLaunchKernelGGL(k_refresh_pairs, dim3((sc.pairs_cap + 255) / 256), dim3(256), 0, stream, sc);
     return hipGetLastError();
 }
 
-hipError_t launch_uncount(hipStream_t stream, uint32_t* counts, uint32_t* touched, uint32_t vocab,
-                          uint32_t token) {
-    hipLaunchKernelGGL(k_uncount, dim3(1), dim3(64), 0, stream, counts, touched, vocab, token);
+hipError_t launch_uncount(hipStream_t stream, const ScratchView& sc, uint32_t token) {
+    hipLaunchKernelGGL(k_uncount, dim3(1), dim3(64), 0, stream, sc, token);
     return hipGetLastError();
 }
 
-hipError_t launch_rebuild_touched(hipStream_t stream, const uint32_t* counts, uint32_t* touched,
-                                  uint32_t vocab) {
-    const uint32_t words = (vocab + 31u) / 32u;
-    hipLaunchKernelGGL(k_rebuild_touched, dim3((words + 255) / 256), dim3(256), 0, stream, counts,
-                       touched, vocab);
+hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc) {
+    const uint32_t words = (sc.vocab + 31u) / 32u;
+    hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(256), 0, stream, sc.n_pairs, 1u, 0u);
+    hipLaunchKernelGGL(k_rebuild_listed, dim3((words + 255) / 256), dim3(256), 0, stream, sc);
     return hipGetLastError();
 }
 

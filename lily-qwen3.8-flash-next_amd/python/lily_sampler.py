@@ -118,6 +118,7 @@ def _load():
         "lily_sampler_create": [C.c_int, vp, C.POINTER(vp)],
         "lily_sampler_synchronize": [vp],
         "lily_sampler_set_phase_trace": [vp, vp, u64],
+        "lily_sampler_set_path_stats": [vp, vp],
         "lily_scratch_create": [vp, u32, C.POINTER(vp)],
         "lily_scratch_reset_counts": [vp],
         "lily_scratch_uncount": [vp, u32],
@@ -236,6 +237,12 @@ class Sampler:
         _check(_lib.lily_sampler_set_phase_trace(
             self._h, _ptr(trace, torch.int64) if trace is not None else None,
             trace.numel() if trace is not None else 0))
+
+    def set_path_stats(self, stats):
+        """stats: device int32 tensor of 4 counters (or None); see lily_sampler_set_path_stats."""
+        self._stats = stats
+        _check(_lib.lily_sampler_set_path_stats(
+            self._h, _ptr(stats, torch.int32) if stats is not None else None))
 
     def slices_for(self, rows, k, vocab):
         return int(_lib.lily_sampler_slices_for(self._h, rows, k, vocab))

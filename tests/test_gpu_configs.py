@@ -243,7 +243,9 @@ def test_config5_full_size_properties(sampler):
         for s in sc:
             s.close()
     a, b = outs
-    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    assert np.array_equal(a[0], b[0])           # token ids replay exactly
+    # log-probabilities are sums whose order depends on wave arrival: equal to tolerance
+    assert np.allclose(a[1], b[1], rtol=0, atol=2e-6)
     ids, lps, cand, cnt, probs = a
     assert np.all(cnt[:, 0] == 64) and np.all(cnt[:, 1] >= 1) and np.all(cnt[:, 1] <= 64)
     for i in range(rows):
