@@ -7,9 +7,10 @@
 
 namespace lily {
 
-// `excl`: some row has a mask, penalties or a bias list; `lse`: some row wants a log-probability.
-// `dyn_bytes`: dynamic LDS = candidate slots, then the slice's exclusion bitmap.
-hipError_t launch_rows(hipStream_t stream, int dtype, bool excl, bool lse, uint32_t rows,
+// `kind`: 0 = no row has a mask, penalties or a bias list, 1 = some row has, 2 = every sampled
+// row takes the streaming select; `lse`: some row wants a log-probability.
+// `dyn_bytes`: dynamic LDS (see shape_of in sampler_api.cpp).
+hipError_t launch_rows(hipStream_t stream, int dtype, int kind, bool lse, uint32_t rows,
                        const LaunchCfg& cfg, const InlineRows* inline_rows, size_t dyn_bytes);
 hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t v);
 hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const uint32_t* ids,

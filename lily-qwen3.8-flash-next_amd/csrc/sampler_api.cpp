@@ -101,7 +101,7 @@ struct lily_plan {
     uint32_t dtype = 0;
     uint32_t slices = 1;
     uint32_t ws_k = 0;
-    bool excl = false;
+    int kind = 0;
     bool lse = false;
     size_t dyn_bytes = 0;
     uint32_t excl_words = 0;
@@ -271,7 +271,6 @@ void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t sl
     cfg->path = s->force_path;
     cfg->cand_cap = CAND_CAP;
     cfg->path_stats = s->path_stats;
-    if (const char* d = std::getenv("LILY_DBG")) cfg->pad = (uint32_t)std::atoi(d);  // DBG
     cfg->list_cap = SPECIAL_LIST_CAP;
 }
 
@@ -293,6 +292,7 @@ struct LaunchShape {
     size_t dyn_bytes = 0;
     uint32_t excl_words = 0;
     uint32_t cand_cap = 0;
+    int kind() const { return old_layout ? (excl ? 1 : 0) : 2; }
 };
 
 LaunchShape shape_of(const lily_sampler* s, const RowArgs* rows, uint32_t n, int dtype,
@@ -359,7 +359,7 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     cfg.excl_words = shp.excl_words;
     cfg.old_layout = shp.old_layout ? 1u : 0u;
     cfg.cand_cap = shp.cand_cap;
-    HIP_TRY(launch_rows(s->stream, dtype, shp.excl, shp.lse, n, cfg, &rows, shp.dyn_bytes));
+    HIP_TRY(launch_rows(s->stream, dtype, shp.kind(), shp.lse, n, cfg, &rows, shp.dyn_bytes));
     return LILY_OK;
 }
 
@@ -998,7 +998,7 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     cfg.excl_words = shp.excl_words;
     cfg.old_layout = shp.old_layout ? 1u : 0u;
     cfg.cand_cap = shp.cand_cap;
-    HIP_TRY(launch_rows(s->stream, (int)b->dtype, shp.excl, shp.lse, b->rows, cfg, nullptr,
+    HIP_TRY(launch_rows(s->stream, (int)b->dtype, shp.kind(), shp.lse, b->rows, cfg, nullptr,
                         shp.dyn_bytes));
     return LILY_OK;
 }
@@ -1057,7 +1057,7 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab);
     const LaunchShape shp = shape_of(p->s, table.data(), b->rows, (int)b->dtype, b->vocab,
                                      p->slices, p->ws_k);
-    p->excl = shp.excl;
+    p->kind = shp.kind();
     p->lse = shp.lse;
     p->dyn_bytes = shp.dyn_bytes;
     p->excl_words = shp.excl_words;
@@ -1077,7 +1077,7 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     cfg.excl_words = p->excl_words;
     cfg.old_layout = p->old_layout ? 1u : 0u;
     cfg.cand_cap = p->cand_cap;
-    HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->excl, p->lse, p->rows, cfg, nullptr,
+    HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->kind, p->lse, p->rows, cfg, nullptr,
                         p->dyn_bytes));
     return LILY_OK;
 }

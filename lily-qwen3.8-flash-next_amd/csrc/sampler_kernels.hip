@@ -365,7 +365,19 @@ __device__ __forceinline__ uint32_t wg_rank_select(uint64_t* cand, uint32_t n, u
     const uint32_t tid = threadIdx.x;
     const uint64_t mine = tid < n ? cand[tid] : 0ull;
     uint32_t rank = 0;
-    for (uint32_t j = 0; j < n; ++j) {
+    uint32_t j = 0;
+    for (; j + 8 <= n; j += 8) {  // eight independent broadcast reads at a time
+        uint64_t c[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            c[q] = cand[j + q];
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            rank += c[q] > mine ? 1u : 0u;
+        }
+    }
+    for (; j < n; ++j) {
         rank += cand[j] > mine ? 1u : 0u;
     }
     if (tid == 0) {
@@ -591,8 +603,26 @@ struct WaveLse {
             s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
         }
     }
-    // As add() on the raw 16 bytes of one load (unpacked only when the wave does not skip
-    // it); an inactive lane contributes nothing.
+    // As add(); an inactive lane contributes nothing.
+    template <int E>
+    __device__ __forceinline__ void add_if(const float (&v)[E], float m, float c, bool active) {
+        const float d = __builtin_fmaf(active ? m : NEG_INF, c, -ref);
+        if (__ballot(d > 60.0f) != 0ull) {
+            const float nref = fmaxf(ref, wave_max_f(active ? m * c : NEG_INF));
+            s *= __builtin_amdgcn_exp2f(ref - nref);
+            ref = nref;
+        } else if (__ballot(d > -40.0f) == 0ull) {
+            return;
+        }
+        if (active) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
+            }
+        }
+    }
+    // As add_if() on the raw 16 bytes of one load (unpacked only when the wave does not skip
+    // it).
     template <int DT>
     __device__ __forceinline__ void add_chunk(const u32x4& q, float m, float c, bool active);
 };
@@ -647,26 +677,37 @@ __device__ __forceinline__ void unpack(const u32x4 q, float (&v)[Geo<DT>::E]) {
     }
 }
 
+// max(a, b, c) / max(a, b) as single instructions (NaN operands lose, as with fmaxf); the
+// compiler's fmaxf adds a canonicalising instruction per operand in front of each.
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float max2_raw(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
+// The largest element of one 16-byte chunk.
+template <int DT>
+__device__ __forceinline__ float chunk_max(const u32x4& q) {
+    float v[Geo<DT>::E];
+    unpack<DT>(q, v);
+    if (DT == LILY_BF16) {
+        return max2_raw(max3_raw(v[0], v[1], v[2]),
+                        max3_raw(v[3], v[4 % Geo<DT>::E], max3_raw(v[5 % Geo<DT>::E], v[6 % Geo<DT>::E], v[7 % Geo<DT>::E])));
+    }
+    return max2_raw(max3_raw(v[0], v[1], v[2]), v[3]);
+}
+
 template <int DT>
 __device__ __forceinline__ void WaveLse::add_chunk(const u32x4& q, float m, float c, bool active) {
     constexpr int E = DT == LILY_BF16 ? 8 : 4;
-    m = active ? m : NEG_INF;
-    if (__ballot(__builtin_fmaf(m, c, -ref) > 60.0f) != 0ull) {
-        const float nref = fmaxf(ref, wave_max_f(m * c));
-        s *= __builtin_amdgcn_exp2f(ref - nref);
-        ref = nref;
-    }
-    if (__ballot(__builtin_fmaf(m, c, -ref) > -40.0f) == 0ull) {
-        return;
-    }
-    if (active) {
-        float v[E];
-        unpack<DT>(q, v);
-#pragma unroll
-        for (int j = 0; j < E; ++j) {
-            s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
-        }
-    }
+    float v[E];
+    unpack<DT>(q, v);
+    add_if<E>(v, m, c, active);
 }
 
 __device__ __forceinline__ bool in_bias_list(const RowArgs& a, uint32_t id) {
@@ -1335,14 +1376,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             dst[u] = g.load_raw(g.cb + (b * U + u) * NT + tid);
         }
     };
-    u32x4 cur[U], nxt[U];
-    if (nblocks > 0) {
-        fetch(cur, 0);  // in flight while the listed ids are bucketed
-    }
-
     // ---- the slice's listed ids, bucketed by block
     // The first PREG x NT list entries are requested together with the list's length (the
-    // list's memory is valid up to pairs_cap whatever the length turns out to be).
+    // list's memory is valid up to pairs_cap whatever the length turns out to be), ahead of
+    // the first block of the row, which is then in flight while the ids are bucketed.
     uint32_t n_pairs = 0;
     uint64_t early[PREG];
     if (pen) {
@@ -1353,6 +1390,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             early[q] = p < a.pairs_cap ? gload(reinterpret_cast<const uint64_t*>(a.pairs) + p)
                                        : ~0ull;
         }
+    }
+    u32x4 cur[U], nxt[U];
+    if (nblocks > 0) {
+        fetch(cur, 0);
     }
     if (tid <= MAX_BUCKETS) {
         L.bkt[tid] = 0;
@@ -1373,6 +1414,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         L.bias_delta[i] = gload(&a.bias[i].delta);
     }
     __syncthreads();
+    phase(cfg, 13);
     if (n_pairs > a.pairs_cap) {
         return stream_fail(cfg, 2u);  // the list overflowed: the bitmap and the counts hold the truth
     }
@@ -1405,26 +1447,24 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     };
     if (listed_row) {
         uint32_t packed[PREG];  // id | min(count, 4095) << 20, NONE when not of this slice
-        uint32_t blk[PREG];
 #pragma unroll
         for (int q = 0; q < PREG; ++q) {
             const uint32_t p = (uint32_t)q * NT + tid;
             packed[q] = NONE;
-            blk[q] = NONE;
-            if (p < n_pairs) {
-                const uint32_t id = (uint32_t)early[q];
-                blk[q] = block_of(id);
-                packed[q] = id | (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS);
+            if (p < n_pairs && block_of((uint32_t)early[q]) != NONE) {
+                packed[q] = (uint32_t)early[q] |
+                            (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS);
             }
         }
         for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
             for (int q = 0; q < PREG; ++q) {
-                if (blk[q] != NONE) {
+                if (packed[q] != NONE) {
+                    const uint32_t b = block_of(packed[q] & ID_MASK);
                     if (pass == 0) {
-                        atomicAdd(&L.bkt[blk[q]], 1u);
+                        atomicAdd(&L.bkt[b], 1u);
                     } else {
-                        L.spec[L.bkt[blk[q]] + atomicAdd(&L.bfill[blk[q]], 1u)] = packed[q];
+                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = packed[q];
                     }
                 }
             }
@@ -1453,6 +1493,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
             __syncthreads();
             if (pass == 0) {
+                phase(cfg, 14);
                 if (tid < 64) {  // counts -> exclusive offsets, total in bkt[MAX_BUCKETS]
                     const uint32_t cnt = L.bkt[tid];
                     uint32_t incl = cnt;
@@ -1468,6 +1509,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     }
                 }
                 __syncthreads();
+                phase(cfg, 15);
                 if (L.bkt[MAX_BUCKETS] > SPEC_CAP) {
                     return stream_fail(cfg, 3u);
                 }
@@ -1548,14 +1590,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (cnt == 4095u) {
             cnt = gload(a.counts + id);
         }
-        float v[E];
-        unpack<DT>(r.chunk, v);
-        float m8 = v[0];
-#pragma unroll
-        for (int j = 1; j < E; ++j) {
-            m8 = fmaxf(m8, v[j]);
-        }
-        const bool queued = m8 >= T;  // the owner's test, on the same bits
+        const bool queued = chunk_max<DT>(r.chunk) >= T;  // the owner's test, on the same bits
         float t = r.raw;
         for (uint32_t j = 0; j < n_bias; ++j) {
             if (L.bias_id[j] == id) {
@@ -1586,11 +1621,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
     };
 
-    Listed lcur, lnxt;
+    // Block b + 1 is requested before block b is worked on, so the arithmetic (eight
+    // exponentials per chunk when a log-probability is wanted) runs under the loads.
+    Listed lcur;
     lcur.ent = NONE;
-    if (nblocks > 0 && listed_row) {
-        listed_fetch(lcur, 0, 0);
-    }
     if (nblocks == 0) {
         refresh_bound(true);  // the same barriers in every workgroup
     }
@@ -1598,24 +1632,27 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const bool more = b + 1 < nblocks;
         if (more) {
             fetch(nxt, b + 1);
-            if (listed_row) {
-                listed_fetch(lnxt, b + 1, 0);
-            }
         }
-        // The block's own maxima enter the bound before the block is filtered.
+        if (listed_row) {
+            listed_fetch(lcur, b, 0);
+        }
+        // The block's own maxima enter the bound before the block is filtered.  Chunks below
+        // the previous bound cannot be queued: their terms are summed here, while unpacked.
+        const float T_prev = T;
         float m8[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            float v[E];
-            unpack<DT>(cur[u], v);
-            m8[u] = v[0];
-#pragma unroll
-            for (int j = 1; j < E; ++j) {
-                m8[u] = fmaxf(m8[u], v[j]);
+            m8[u] = chunk_max<DT>(cur[u]);
+            lane_max = max2_raw(lane_max, m8[u]);
+            if (LSE && want_lse) {
+                wl.template add_chunk<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
             }
-            lane_max = fmaxf(lane_max, m8[u]);
         }
-        refresh_bound(b == 0);
+        // The bound moves most in the first blocks: refresh it for each of them, then for
+        // every fourth block (each refresh is a ballot search and a barrier).
+        if (b < 4u || (b & 3u) == 0u) {
+            refresh_bound(b == 0);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t c = g.cb + (b * U + u) * NT + tid;
@@ -1632,7 +1669,11 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 wq += (uint32_t)__popcll(mask);
             }
             if (LSE && want_lse) {
-                wl.template add_chunk<DT>(cur[u], m8[u], c2, !pass);
+                // At or above the previous bound but below the new one: not queued after all.
+                const bool late = m8[u] >= T_prev && !pass;
+                if (__ballot(late) != 0ull) {
+                    wl.template add_chunk<DT>(cur[u], m8[u], c2, late);
+                }
             }
         }
         if (listed_row) {
@@ -1649,7 +1690,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             for (int u = 0; u < U; ++u) {
                 cur[u] = nxt[u];
             }
-            lcur = lnxt;
         }
     }
     phase(cfg, 2);
@@ -1695,23 +1735,51 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
     };
-    for (int ww = 0; ww < NWAVE; ++ww) {
-        const uint32_t n_e = sh.qfill[ww] * E;
-        for (uint32_t e = tid; e < n_e; e += NT) {
-            const uint32_t slot = (uint32_t)ww * QSEG + e / E, j = e % E;
-            const uint32_t id = g.id_of(L.qidx[slot], (int)j);
-            float v;
-            if (DT == LILY_BF16) {
-                v = lilym_bits_f32((uint32_t)reinterpret_cast<const uint16_t*>(L.qraw + slot)[j] << 16);
-            } else {
-                v = reinterpret_cast<const float*>(L.qraw + slot)[j];
-            }
-            const bool dropped = (L.dmask[slot >> 2] >> ((slot & 3u) * 8u + j)) & 1u;
-            if (!dropped) {
-                if (want_lse) {
-                    acc_q += term_d(v, c2, ref_s);
+    {
+        // Element e of the queue: slot = the e / E-th queued chunk, counting through the
+        // waves' segments in order.  Four independent elements per thread per step.
+        uint32_t seg_end[NWAVE], total = 0;
+#pragma unroll
+        for (int i = 0; i < NWAVE; ++i) {
+            total += sh.qfill[i];
+            seg_end[i] = total;
+        }
+        const uint32_t n_e = total * E;
+        for (uint32_t e0 = tid; e0 < n_e; e0 += 4 * NT) {
+            uint32_t ids[4];
+            float vs[4];
+            bool ok[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t e = e0 + (uint32_t)q * NT;
+                ok[q] = e < n_e;
+                const uint32_t ch = ok[q] ? e / E : 0u, j = e % E;
+                uint32_t ww = 0, before = 0;
+#pragma unroll
+                for (int i = 0; i + 1 < NWAVE; ++i) {
+                    if (ch >= seg_end[i]) {
+                        ww = (uint32_t)i + 1u;
+                        before = seg_end[i];
+                    }
                 }
-                offer(v, id);
+                const uint32_t slot = ww * QSEG + (ch - before);
+                ids[q] = g.id_of(L.qidx[slot], (int)j);
+                if (DT == LILY_BF16) {
+                    vs[q] = lilym_bits_f32(
+                        (uint32_t)reinterpret_cast<const uint16_t*>(L.qraw + slot)[j] << 16);
+                } else {
+                    vs[q] = reinterpret_cast<const float*>(L.qraw + slot)[j];
+                }
+                ok[q] = ok[q] && !((L.dmask[slot >> 2] >> ((slot & 3u) * 8u + j)) & 1u);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (ok[q]) {
+                    if (want_lse) {
+                        acc_q += term_d(vs[q], c2, ref_s);
+                    }
+                    offer(vs[q], ids[q]);
+                }
             }
         }
     }
@@ -1729,10 +1797,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
     }
     phase(cfg, 9);
-    if (cfg.phase_trace != nullptr && tid == 0) {  // DBG
-        uint64_t* t = cfg.phase_trace + ((size_t)blockIdx.y * cfg.slices + blockIdx.x) * PHASE_SLOTS;
-        t[13] = sh.n_drop; t[14] = sh.qfill[0] + sh.qfill[1] + sh.qfill[2] + sh.qfill[3]; t[15] = sh.n_fc;
-    }
     if (want_lse) {
         double m_s, s_s;
         wg_merge_lse(sh, wl.ref, wl.s, m_s, s_s);
@@ -1769,6 +1833,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     }
     sorted = false;
     n = select_topk(L.fc, n, k, sh, sorted);
+    phase(cfg, 12);
     // Everything that is not a candidate lies strictly below `filt`: the result is exact if
     // k candidates were found and the k-th lies strictly above anything the division can
     // map such a value to.
@@ -2008,6 +2073,65 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     }
     const uint32_t k = min(a.k, n);
     const float top = composite_value(cand[0]);
+    if (k <= 64u && a.mode != MODE_SPEC) {
+        // One wave, a candidate per lane.  The sums keep the reference's left-to-right f32
+        // order: every lane runs the same chain of 64 additions on values read lane by lane
+        // (lanes past k hold 0, which changes nothing), so nothing waits on LDS.
+        if (tid >= 64u) {
+            return;
+        }
+        const uint32_t lane = tid;
+        const uint64_t c = lane < k ? cand[lane] : 0ull;
+        const float p = lane < k ? lilym_expf(composite_value(c) - top) : 0.0f;
+        if (lane < k) {
+            if (a.dbg_ids) {
+                a.dbg_ids[lane] = composite_id(c);
+            }
+            if (a.dbg_probs) {
+                a.dbg_probs[lane] = p;
+            }
+        }
+        const int pbits = (int)lilym_f32_bits(p);
+        float total = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 64; ++i) {
+            total += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, i));
+        }
+        const float limit = a.top_p * total;
+        float cum = 0.0f, before = 0.0f, mine = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 64; ++i) {
+            before = lane == (uint32_t)i ? cum : before;
+            cum += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, i));
+            mine = lane == (uint32_t)i ? cum : mine;
+        }
+        const bool stop = lane >= 1u && lane < k && !(before < limit && p >= a.min_p);
+        const uint64_t stops = __ballot(stop);
+        const uint32_t kept = stops != 0ull ? (uint32_t)__builtin_ctzll(stops) : k;
+        const float mass = __shfl(mine, (int)kept - 1);
+        if (lane == 0 && a.dbg_counts) {
+            a.dbg_counts[0] = k;
+            a.dbg_counts[1] = kept;
+        }
+        if (a.mode == MODE_DRAFT) {
+            if (lane < kept) {
+                a.q_ids[lane] = composite_id(c);
+                a.q_probs[lane] = p / mass;
+            }
+            if (lane == 0) {
+                *a.q_n = kept;
+            }
+        }
+        const float u1 = (a.flags & F_UNIFORM) ? a.uniform : lilym_uniform_for(a.seed, step);
+        const uint64_t hits = __ballot(lane < kept && u1 * mass < mine);
+        const uint32_t slot = hits != 0ull ? (uint32_t)__builtin_ctzll(hits) : kept - 1u;
+        const uint32_t id = ~(uint32_t)__shfl((int)(uint32_t)c, (int)slot);
+        if (lane == 0) {
+            write_logprob<DT>(a, sh, id, vocab);  // before the id is counted
+            emit(a, id);
+        }
+        return;
+    }
     for (uint32_t i = tid; i < k; i += NT) {
         const float p = lilym_expf(composite_value(cand[i]) - top);
         sh.prob[i] = p;
@@ -2190,8 +2314,11 @@ __device__ __forceinline__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>
 
 // ------------------------------------------------------------------ the row kernel
 
-template <int DT, bool EXCL, bool LSE>
+template <int DT, int KIND, bool LSE>
 __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
+    // KIND: 0 = rows without masks, penalties or bias lists, 1 = rows with any of them (the
+    // bitmap select is compiled for them), 2 = streaming rows only (no bitmap select at all).
+    constexpr bool EXCL = KIND == 1;
     const uint32_t tid = threadIdx.x;
     const uint32_t s = blockIdx.x, row = blockIdx.y, S = cfg.slices;
     const uint32_t vocab = cfg.vocab;
@@ -2238,7 +2365,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
                 __syncthreads();
             }
         }
-        if (!done && cfg.path != 1u && cfg.old_layout != 0u) {
+        if (KIND != 2 && !done && cfg.path != 1u && cfg.old_layout != 0u) {
             const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
             if (EXCL || !special) {
                 const bool two_pass = a.k > 64u || cfg.path == 2u;
@@ -2386,7 +2513,7 @@ __device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowAr
     }
 }
 
-template <int DT, bool EXCL, bool LSE>
+template <int DT, int KIND, bool LSE>
 __global__ __launch_bounds__(NT, 4) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
     __shared__ Shared sh;
     // `rows` is the first kernel argument: index it in the kernel-argument segment itself
@@ -2399,10 +2526,10 @@ __global__ __launch_bounds__(NT, 4) void k_rows_inline(InlineRows rows, LaunchCf
         tail_arrays(sh);
     }
     __syncthreads();
-    row_body<DT, EXCL, LSE>(a, cfg, sh);
+    row_body<DT, KIND, LSE>(a, cfg, sh);
 }
 
-template <int DT, bool EXCL, bool LSE>
+template <int DT, int KIND, bool LSE>
 __global__ __launch_bounds__(NT, 4) void k_rows_table(LaunchCfg cfg) {
     __shared__ Shared sh;
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
@@ -2412,7 +2539,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_table(LaunchCfg cfg) {
         tail_arrays(sh);
     }
     __syncthreads();
-    row_body<DT, EXCL, LSE>(a, cfg, sh);
+    row_body<DT, KIND, LSE>(a, cfg, sh);
 }
 
 // ------------------------------------------------------------------ small kernels
@@ -2526,28 +2653,33 @@ __global__ void k_copy_row_u32(const uint32_t* src, uint32_t* dst, uint32_t word
 
 // ------------------------------------------------------------------ launchers (host)
 
-template <int DT, bool EXCL, bool LSE>
+template <int DT, int KIND, bool LSE>
 static hipError_t launch_variant(hipStream_t stream, uint32_t rows, const LaunchCfg& cfg,
                                  const InlineRows* inline_rows, size_t dyn_bytes) {
     const dim3 grid(cfg.slices, rows), block(NT);
     if (inline_rows != nullptr) {
-        hipLaunchKernelGGL((k_rows_inline<DT, EXCL, LSE>), grid, block, dyn_bytes, stream,
+        hipLaunchKernelGGL((k_rows_inline<DT, KIND, LSE>), grid, block, dyn_bytes, stream,
                            *inline_rows, cfg);
     } else {
-        hipLaunchKernelGGL((k_rows_table<DT, EXCL, LSE>), grid, block, dyn_bytes, stream, cfg);
+        hipLaunchKernelGGL((k_rows_table<DT, KIND, LSE>), grid, block, dyn_bytes, stream, cfg);
     }
     return hipGetLastError();
 }
 
-hipError_t launch_rows(hipStream_t stream, int dtype, bool excl, bool lse, uint32_t rows,
+hipError_t launch_rows(hipStream_t stream, int dtype, int kind, bool lse, uint32_t rows,
                        const LaunchCfg& cfg, const InlineRows* inline_rows, size_t dyn_bytes) {
-#define LILY_DISPATCH(DT)                                                                      \
-    if (excl) {                                                                                \
-        return lse ? launch_variant<DT, true, true>(stream, rows, cfg, inline_rows, dyn_bytes)  \
-                   : launch_variant<DT, true, false>(stream, rows, cfg, inline_rows, dyn_bytes); \
-    }                                                                                          \
-    return lse ? launch_variant<DT, false, true>(stream, rows, cfg, inline_rows, dyn_bytes)     \
-               : launch_variant<DT, false, false>(stream, rows, cfg, inline_rows, dyn_bytes);
+#define LILY_DISPATCH(DT)                                                                     \
+    switch (kind) {                                                                           \
+        case 0:                                                                               \
+            return lse ? launch_variant<DT, 0, true>(stream, rows, cfg, inline_rows, dyn_bytes)  \
+                       : launch_variant<DT, 0, false>(stream, rows, cfg, inline_rows, dyn_bytes); \
+        case 1:                                                                               \
+            return lse ? launch_variant<DT, 1, true>(stream, rows, cfg, inline_rows, dyn_bytes)  \
+                       : launch_variant<DT, 1, false>(stream, rows, cfg, inline_rows, dyn_bytes); \
+        default:                                                                              \
+            return lse ? launch_variant<DT, 2, true>(stream, rows, cfg, inline_rows, dyn_bytes)  \
+                       : launch_variant<DT, 2, false>(stream, rows, cfg, inline_rows, dyn_bytes); \
+    }
     if (dtype == LILY_BF16) {
         LILY_DISPATCH(LILY_BF16)
     }
