@@ -63,7 +63,8 @@ struct alignas(16) RowArgs {
     float uniform;
     float uniform2;
     uint32_t pairs_cap;
-    uint32_t pad[2];
+    uint32_t pairs_hint;       // host's upper bound of n_pairs when the row was packed (saves loads only)
+    uint32_t pad;
 };
 static_assert(sizeof(RowArgs) == 224, "RowArgs layout");
 
@@ -101,7 +102,7 @@ struct LaunchCfg {
     uint32_t excl_words;    // words reserved for the slice bitmap (the specials' id list follows)
     uint32_t list_cap;      // ids the specials' list holds
     uint32_t old_layout;    // dynamic LDS holds cand_cap candidates + the bitmap + the id list
-    uint32_t pad;
+    uint32_t hint_growth;   // added to every row's pairs_hint (draws since the table was packed)
     uint32_t* path_stats;   // null, or [4] counters: slices finished by the streaming select, the
                             // bitmap select, the exhaustive select; [3] unused
 };

@@ -82,6 +82,7 @@ struct lily_scratch {
     uint32_t* touched = nullptr;  // [words + 4] bit per listed id
     CountPair* pairs = nullptr;   // [pairs_cap] listed ids with their counts
     uint32_t* n_pairs = nullptr;  // [1]
+    uint64_t listed_bound = 0;    // host's upper bound of *n_pairs (ids added + draws enqueued)
 };
 
 struct lily_draft_dists {
@@ -107,6 +108,8 @@ struct lily_plan {
     uint32_t excl_words = 0;
     bool old_layout = false;
     uint32_t cand_cap = 0;
+    uint32_t runs = 0;                       // launches since the table was packed
+    std::vector<lily_scratch*> penalised;    // scratches whose rows count their draws
 };
 
 namespace {
@@ -205,6 +208,9 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
         out->n_pairs = scratch->n_pairs;
         out->pos = scratch->pos;
         out->pairs_cap = scratch->pairs_cap;
+        out->pairs_hint = (uint32_t)(scratch->listed_bound < scratch->pairs_cap
+                                         ? scratch->listed_bound : scratch->pairs_cap);
+        scratch->listed_bound += 1;  // this draw may list one more id
         out->flags |= F_PEN;
     }
     if (x.has_uniform) {
@@ -713,6 +719,7 @@ int lily_scratch_reset_counts(lily_scratch_t* sc) {
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->counts, sc->vocab, 0));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->touched, sc->words + 4, 0));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->n_pairs, 1, 0));
+    sc->listed_bound = 0;
     return LILY_OK;
 }
 
@@ -745,6 +752,7 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
     HIP_TRY(hipMemcpyAsync(dst->pairs, src->pairs, (size_t)src->pairs_cap * sizeof(CountPair),
                            hipMemcpyDeviceToDevice, dst->s->stream));
     HIP_TRY(hipMemcpyAsync(dst->n_pairs, src->n_pairs, 4, hipMemcpyDeviceToDevice, dst->s->stream));
+    dst->listed_bound = src->listed_bound;
     return LILY_OK;
 }
 
@@ -754,6 +762,7 @@ int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32
     }
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(launch_add_history(sc->s->stream, view_of(sc), ids_dev, n));
+    sc->listed_bound += n;
     return LILY_OK;
 }
 
@@ -765,6 +774,7 @@ int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts) {
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     HIP_TRY(hipMemcpy(sc->counts, host_counts, (size_t)sc->vocab * 4, hipMemcpyHostToDevice));
     HIP_TRY(launch_rebuild_listed(sc->s->stream, view_of(sc)));
+    sc->listed_bound = sc->vocab;
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     return LILY_OK;
 }
@@ -1063,6 +1073,13 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->excl_words = shp.excl_words;
     p->old_layout = shp.old_layout;
     p->cand_cap = shp.cand_cap;
+    p->runs = 0;
+    p->penalised.clear();
+    for (uint32_t r = 0; r < b->rows; ++r) {
+        if (b->scratch != nullptr && b->scratch[r] != nullptr && (table[r].flags & F_PEN)) {
+            p->penalised.push_back(b->scratch[r]);
+        }
+    }
     return LILY_OK;
 }
 
@@ -1077,6 +1094,11 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     cfg.excl_words = p->excl_words;
     cfg.old_layout = p->old_layout ? 1u : 0u;
     cfg.cand_cap = p->cand_cap;
+    cfg.hint_growth = p->runs;
+    p->runs += 1;
+    for (lily_scratch* sc : p->penalised) {
+        sc->listed_bound += 1;
+    }
     HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->kind, p->lse, p->rows, cfg, nullptr,
                         p->dyn_bytes));
     return LILY_OK;

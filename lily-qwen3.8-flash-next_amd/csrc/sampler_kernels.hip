@@ -203,6 +203,7 @@ struct Shared {
     uint32_t n_fc;           // final candidates
     uint32_t n_drop;         // listed ids found inside queued chunks
     uint32_t fail;
+    double red3[3][NWAVE];
 };
 
 // Running sum of 2^(v*c - mc) of one thread with its own reference mc.
@@ -625,6 +626,19 @@ struct WaveLse {
     // it).
     template <int DT>
     __device__ __forceinline__ void add_chunk(const u32x4& q, float m, float c, bool active);
+    // Block-wise use: prepare() once with the largest value the lane will add in the block
+    // (raises the reference when some lane's would dwarf it), then add_prepared() per load.
+    float skip_below;  // a load whose maximum is below this adds nothing that matters
+    __device__ __forceinline__ void prepare(float block_max, float c, float inv_c) {
+        if (__ballot(__builtin_fmaf(block_max, c, -ref) > 60.0f) != 0ull) {
+            const float nref = fmaxf(ref, wave_max_f(block_max * c));
+            s *= __builtin_amdgcn_exp2f(ref - nref);
+            ref = nref;
+        }
+        skip_below = (ref - 41.0f) * inv_c;
+    }
+    template <int DT>
+    __device__ __forceinline__ void add_prepared(const u32x4& q, float m, float c, bool active);
 };
 
 // Workgroup-wide merge of per-thread (reference, sum) pairs: returns through `m`, `sum`
@@ -700,6 +714,23 @@ __device__ __forceinline__ float chunk_max(const u32x4& q) {
                         max3_raw(v[3], v[4 % Geo<DT>::E], max3_raw(v[5 % Geo<DT>::E], v[6 % Geo<DT>::E], v[7 % Geo<DT>::E])));
     }
     return max2_raw(max3_raw(v[0], v[1], v[2]), v[3]);
+}
+
+template <int DT>
+__device__ __forceinline__ void WaveLse::add_prepared(const u32x4& q, float m, float c, bool active) {
+    constexpr int E = DT == LILY_BF16 ? 8 : 4;
+    active = active && m > skip_below;
+    if (__ballot(active) == 0ull) {
+        return;
+    }
+    if (active) {
+        float v[E];
+        unpack<DT>(q, v);
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
+        }
+    }
 }
 
 template <int DT>
@@ -1370,30 +1401,43 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     StreamLds L;
     L.init();
 
+    // Blocks lying wholly inside the streamed chunks are loaded without per-load checks.
     auto fetch = [&](u32x4 (&dst)[U], uint32_t b) {
+        const uint32_t c0 = g.cb + b * BLOCK;
+        if (c0 >= g.main_lo && c0 + BLOCK <= g.main_hi) {
+            const uint32_t off = (c0 + tid) << 4;  // the stream path's rows are below 4 GiB
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            dst[u] = g.load_raw(g.cb + (b * U + u) * NT + tid);
+            for (int u = 0; u < U; ++u) {
+                dst[u] = gload(reinterpret_cast<const u32x4*>(g.base + (off + (uint32_t)u * NT * 16u)));
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                dst[u] = g.load_raw(c0 + (uint32_t)u * NT + tid);
+            }
         }
     };
     // ---- the slice's listed ids, bucketed by block
     // The first PREG x NT list entries are requested together with the list's length (the
     // list's memory is valid up to pairs_cap whatever the length turns out to be), ahead of
     // the first block of the row, which is then in flight while the ids are bucketed.
-    uint32_t n_pairs = 0;
+    uint32_t n_pairs = 0, loaded = 0;
     uint64_t early[PREG];
     if (pen) {
         n_pairs = gload(a.n_pairs);
+        // The host's bound of the length says how much to request; a longer list is still
+        // read completely (by the loop further down), a shorter one costs idle loads.
+        const uint64_t want = ((uint64_t)a.pairs_hint + cfg.hint_growth + NT - 1) / NT * NT;
+        loaded = (uint32_t)min(want, (uint64_t)min(a.pairs_cap, (uint32_t)(PREG * NT)));
 #pragma unroll
         for (int q = 0; q < PREG; ++q) {
             const uint32_t p = (uint32_t)q * NT + tid;
-            early[q] = p < a.pairs_cap ? gload(reinterpret_cast<const uint64_t*>(a.pairs) + p)
-                                       : ~0ull;
+            early[q] = p < loaded ? gload(reinterpret_cast<const uint64_t*>(a.pairs) + p) : ~0ull;
         }
     }
-    u32x4 cur[U], nxt[U];
+    u32x4 buf_a[U], buf_b[U];
     if (nblocks > 0) {
-        fetch(cur, 0);
+        fetch(buf_a, 0);
     }
     if (tid <= MAX_BUCKETS) {
         L.bkt[tid] = 0;
@@ -1451,7 +1495,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         for (int q = 0; q < PREG; ++q) {
             const uint32_t p = (uint32_t)q * NT + tid;
             packed[q] = NONE;
-            if (p < n_pairs && block_of((uint32_t)early[q]) != NONE) {
+            if (p < n_pairs && p < loaded && block_of((uint32_t)early[q]) != NONE) {
                 packed[q] = (uint32_t)early[q] |
                             (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS);
             }
@@ -1468,7 +1512,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     }
                 }
             }
-            for (uint32_t p = PREG * NT + tid; p < n_pairs; p += NT) {  // lists beyond the registers
+            for (uint32_t p = loaded + tid; p < n_pairs; p += NT) {  // what the registers do not hold
                 const uint64_t e = gload(reinterpret_cast<const uint64_t*>(a.pairs) + p);
                 const uint32_t id = (uint32_t)e;
                 const uint32_t b = block_of(id);
@@ -1621,31 +1665,32 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
     };
 
-    // Block b + 1 is requested before block b is worked on, so the arithmetic (eight
-    // exponentials per chunk when a log-probability is wanted) runs under the loads.
-    Listed lcur;
-    lcur.ent = NONE;
-    if (nblocks == 0) {
-        refresh_bound(true);  // the same barriers in every workgroup
-    }
-    for (uint32_t b = 0; b < nblocks; ++b) {
-        const bool more = b + 1 < nblocks;
-        if (more) {
-            fetch(nxt, b + 1);
-        }
+    // Block b + 1 is requested before block b is worked on (two register buffers that swap
+    // roles), so the arithmetic - eight exponentials per chunk when a log-probability is
+    // wanted - runs under the loads.
+    const float inv_c2 = a.temperature * 0.6931471805599453f;
+    auto work = [&](const u32x4 (&cur)[U], uint32_t b) {
+        Listed lcur;
+        lcur.ent = NONE;
         if (listed_row) {
             listed_fetch(lcur, b, 0);
         }
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
-        // the previous bound cannot be queued: their terms are summed here, while unpacked.
+        // the previous bound cannot be queued: their terms are summed right away.
         const float T_prev = T;
         float m8[U];
+        float sum_max = NEG_INF;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             m8[u] = chunk_max<DT>(cur[u]);
             lane_max = max2_raw(lane_max, m8[u]);
-            if (LSE && want_lse) {
-                wl.template add_chunk<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
+            sum_max = max2_raw(sum_max, m8[u] >= T_prev ? NEG_INF : m8[u]);
+        }
+        if (LSE && want_lse) {
+            wl.prepare(sum_max, c2, inv_c2);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                wl.template add_prepared<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
             }
         }
         // The bound moves most in the first blocks: refresh it for each of them, then for
@@ -1685,11 +1730,20 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 listed_process(extra);
             }
         }
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                cur[u] = nxt[u];
+    };
+    if (nblocks == 0) {
+        refresh_bound(true);  // the same barriers in every workgroup
+    }
+    for (uint32_t b = 0; b < nblocks; b += 2) {
+        if (b + 1 < nblocks) {
+            fetch(buf_b, b + 1);
+        }
+        work(buf_a, b);
+        if (b + 1 < nblocks) {
+            if (b + 2 < nblocks) {
+                fetch(buf_a, b + 2);
             }
+            work(buf_b, b + 1);
         }
     }
     phase(cfg, 2);
@@ -1736,49 +1790,36 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
     };
     {
-        // Element e of the queue: slot = the e / E-th queued chunk, counting through the
-        // waves' segments in order.  Four independent elements per thread per step.
+        // One thread per queued chunk (the waves' segments counted through in order): its
+        // elements that are not listed ids add their term and are offered.
         uint32_t seg_end[NWAVE], total = 0;
 #pragma unroll
         for (int i = 0; i < NWAVE; ++i) {
             total += sh.qfill[i];
             seg_end[i] = total;
         }
-        const uint32_t n_e = total * E;
-        for (uint32_t e0 = tid; e0 < n_e; e0 += 4 * NT) {
-            uint32_t ids[4];
-            float vs[4];
-            bool ok[4];
+        for (uint32_t ch = tid; ch < total; ch += NT) {
+            uint32_t ww = 0, before = 0;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t e = e0 + (uint32_t)q * NT;
-                ok[q] = e < n_e;
-                const uint32_t ch = ok[q] ? e / E : 0u, j = e % E;
-                uint32_t ww = 0, before = 0;
-#pragma unroll
-                for (int i = 0; i + 1 < NWAVE; ++i) {
-                    if (ch >= seg_end[i]) {
-                        ww = (uint32_t)i + 1u;
-                        before = seg_end[i];
-                    }
+            for (int i = 0; i + 1 < NWAVE; ++i) {
+                if (ch >= seg_end[i]) {
+                    ww = (uint32_t)i + 1u;
+                    before = seg_end[i];
                 }
-                const uint32_t slot = ww * QSEG + (ch - before);
-                ids[q] = g.id_of(L.qidx[slot], (int)j);
-                if (DT == LILY_BF16) {
-                    vs[q] = lilym_bits_f32(
-                        (uint32_t)reinterpret_cast<const uint16_t*>(L.qraw + slot)[j] << 16);
-                } else {
-                    vs[q] = reinterpret_cast<const float*>(L.qraw + slot)[j];
-                }
-                ok[q] = ok[q] && !((L.dmask[slot >> 2] >> ((slot & 3u) * 8u + j)) & 1u);
             }
+            const uint32_t slot = ww * QSEG + (ch - before);
+            const u32x4 q = L.qraw[slot];
+            const uint32_t c = L.qidx[slot];
+            const uint32_t dm = (L.dmask[slot >> 2] >> ((slot & 3u) * 8u)) & 0xffu;
+            float v[E];
+            unpack<DT>(q, v);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                if (ok[q]) {
+            for (int j = 0; j < E; ++j) {
+                if (!((dm >> j) & 1u)) {
                     if (want_lse) {
-                        acc_q += term_d(vs[q], c2, ref_s);
+                        acc_q += term_d(v[j], c2, ref_s);
                     }
-                    offer(vs[q], ids[q]);
+                    offer(v[j], g.id_of(c, j));
                 }
             }
         }
@@ -1798,11 +1839,35 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     }
     phase(cfg, 9);
     if (want_lse) {
-        double m_s, s_s;
-        wg_merge_lse(sh, wl.ref, wl.s, m_s, s_s);
-        const double streamed = s_s > 0.0 ? s_s * exp2(m_s - (double)ref_s) : 0.0;
-        const double booked = wg_sum_d(sh, acc_r);
-        const double exact = wg_sum_d(sh, acc_t + acc_q);
+        // Everything relative to ref_s: this lane's streamed sum is rescaled from its wave's
+        // reference, then the three sums are reduced together.
+        double part[3];
+        {
+            float d = wl.ref - ref_s;
+            d = fminf(fmaxf(d, -1000.0f), 1000.0f);
+            const float di = __builtin_floorf(d);
+            part[0] = wl.s > 0.0f ? (double)wl.s * __builtin_ldexp(
+                                        (double)__builtin_amdgcn_exp2f(d - di), (int)di)
+                                  : 0.0;
+        }
+        part[1] = acc_r;
+        part[2] = acc_t + acc_q;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            part[i] = wave_sum_d(part[i]);
+            if (lane == 0) {
+                sh.red3[i][w] = part[i];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            part[i] = 0.0;
+            for (int ww = 0; ww < NWAVE; ++ww) {
+                part[i] += sh.red3[i][ww];
+            }
+        }
+        const double streamed = part[0], booked = part[1], exact = part[2];
         const double rest = streamed - booked;
         // Listed ids held nearly all of what was streamed: the difference is too coarse.
         const bool coarse = booked > 0.0 && !(rest > 0.05 * streamed);
@@ -2001,11 +2066,11 @@ __device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched,
         if (p < pairs_cap) {
             pairs[p].id = id;
             pairs[p].count = before + 1u;
-            pos[id] = p;
         }
+        pos[id] = p < pairs_cap ? p : 0xffffffffu;  // listed ids always have a meaningful pos
     } else {
         const uint32_t p = pos[id];
-        if (p < pairs_cap && pairs[p].id == id) {
+        if (p < pairs_cap) {
             pairs[p].count = before + 1u;
         }
     }
@@ -2044,6 +2109,53 @@ __device__ __forceinline__ void write_logprob(const RowArgs& a, const Shared& sh
         }
     }
     *a.out_logprob = lp;
+}
+
+// Emits `id` and, when asked, its log-probability, with the memory operations of both in one
+// round trip: the count's atomic increment returns the count the penalties used, the bitmap's
+// atomic OR tells whether the id is listed already, and the logit and the list position load
+// beside them.
+template <int DT>
+__device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
+    *a.out_id = id;
+    const bool pen = (a.flags & F_PEN) != 0;
+    const bool want = a.out_logprob != nullptr;
+    if (id >= vocab) {
+        if (want) {
+            *a.out_logprob = NEG_INF;
+        }
+        return;
+    }
+    uint32_t before = 0, bits = 0, p = 0xffffffffu;
+    const uint32_t bit = 1u << (id & 31u);
+    if (pen) {
+        before = atomicAdd(&a.counts[id], 1u);
+        bits = atomicOr(&a.touched[id >> 5], bit);
+        p = gload(a.pos + id);
+    }
+    if (want) {
+        const float l = load_logit<DT>(a.logits, id);
+        const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
+        const float u = finish_pre_temperature(a, id, l, before, allowed);
+        float lp = NEG_INF;
+        if (u > NEG_INF) {
+            const double e = (double)u * (double)a.c2 - sh.lse_mc - log2(sh.lse_s);
+            lp = fminf((float)(e * 0.6931471805599453), 0.0f);  // the sum is approximate: clamp
+        }
+        *a.out_logprob = lp;
+    }
+    if (pen) {
+        if ((bits & bit) == 0u) {
+            const uint32_t at = atomicAdd(a.n_pairs, 1u);
+            if (at < a.pairs_cap) {
+                a.pairs[at].id = id;
+                a.pairs[at].count = before + 1u;
+            }
+            a.pos[id] = at < a.pairs_cap ? at : 0xffffffffu;
+        } else if (p < a.pairs_cap) {
+            a.pairs[p].count = before + 1u;
+        }
+    }
 }
 
 // cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
@@ -2127,8 +2239,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         const uint32_t slot = hits != 0ull ? (uint32_t)__builtin_ctzll(hits) : kept - 1u;
         const uint32_t id = ~(uint32_t)__shfl((int)(uint32_t)c, (int)slot);
         if (lane == 0) {
-            write_logprob<DT>(a, sh, id, vocab);  // before the id is counted
-            emit(a, id);
+            finish_token<DT>(a, sh, id, vocab);
         }
         return;
     }
@@ -2188,8 +2299,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         if (tid == 0) {
             const uint32_t slot = pick_sequential(sh.cum, n_keep, u1 * mass);
             const uint32_t id = composite_id(cand[slot]);
-            write_logprob<DT>(a, sh, id, vocab);  // before the id is counted
-            emit(a, id);
+            finish_token<DT>(a, sh, id, vocab);
         }
         return;
     }
@@ -2210,8 +2320,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     __syncthreads();
     if (u1 * sh.q_d < sh.p_d) {
         if (tid == 0) {
-            write_logprob<DT>(a, sh, d, vocab);
-            emit(a, d);
+            finish_token<DT>(a, sh, d, vocab);
         }
         return;
     }
@@ -2251,8 +2360,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             slot = pick_sequential(sh.cum, n_keep, u2 * mass);
         }
         const uint32_t id = composite_id(cand[slot]);
-        write_logprob<DT>(a, sh, id, vocab);
-        emit(a, id);
+        finish_token<DT>(a, sh, id, vocab);
     }
 }
 
@@ -2483,8 +2591,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
     }
     if (a.flags & F_FORCED) {
         if (tid == 0) {
-            write_logprob<DT>(a, sh, a.forced, vocab);
-            emit(a, a.forced);
+            finish_token<DT>(a, sh, a.forced, vocab);
         }
         return;
     }
@@ -2565,8 +2672,8 @@ __global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
                 const uint32_t p = atomicAdd(sc.n_pairs, 1u);
                 if (p < sc.pairs_cap) {
                     sc.pairs[p].id = id;
-                    sc.pos[id] = p;
                 }
+                sc.pos[id] = p < sc.pairs_cap ? p : 0xffffffffu;
             }
         }
     }
@@ -2588,8 +2695,7 @@ __global__ void k_uncount(ScratchView sc, uint32_t token) {
         if (c > 0u) {
             sc.counts[token] = c - 1u;
             const uint32_t p = sc.pos[token];
-            if (((sc.touched[token >> 5] >> (token & 31u)) & 1u) && p < sc.pairs_cap &&
-                sc.pairs[p].id == token) {
+            if (((sc.touched[token >> 5] >> (token & 31u)) & 1u) && p < sc.pairs_cap) {
                 sc.pairs[p].count = c - 1u;
             }
         }
@@ -2611,8 +2717,8 @@ __global__ void k_rebuild_listed(ScratchView sc) {
                 if (p < sc.pairs_cap) {
                     sc.pairs[p].id = id;
                     sc.pairs[p].count = sc.counts[id];
-                    sc.pos[id] = p;
                 }
+                sc.pos[id] = p < sc.pairs_cap ? p : 0xffffffffu;
             }
         }
         sc.touched[w] = bits;
