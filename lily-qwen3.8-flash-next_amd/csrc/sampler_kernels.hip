@@ -2503,11 +2503,11 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
                 store_through(&cfg.ws_cand[slot * cfg.ws_k], best);
             }
         } else {
-            for (uint32_t i = tid; i < n; i += NT) {
-                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], cand[i]);
+            // Every slot is written (0 = no candidate), so the merge needs no counts.
+            for (uint32_t i = tid; i < cfg.ws_k; i += NT) {
+                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], i < n ? cand[i] : (uint64_t)0);
             }
             if (tid == 0) {
-                store_through(&cfg.ws_n[slot], n);
                 store_through(&cfg.ws_lse[2 * slot], want_lse ? sh.lse_mc : 0.0);
                 store_through(&cfg.ws_lse[2 * slot + 1], want_lse ? sh.lse_s : 0.0);
             }
@@ -2544,10 +2544,15 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
                 best = sh.red_u[i] > best ? sh.red_u[i] : best;
             }
         } else {
-            // Gather every slice's candidates (absent slots read as 0 = invalid) and merge
-            // the log-sum-exp partials, all slices at once.
-            if (tid < S) {
-                sh.hist[tid] = load_through(&cfg.ws_n[base + tid]);
+            // Gather every slice's candidates (0 = no candidate) and the log-sum-exp partials
+            // in one round trip.
+            constexpr int PER = MERGE_CAP / NT;
+            const uint32_t slots = S * cfg.ws_k;
+            uint64_t mine[PER];
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const uint32_t j = tid + (uint32_t)q * NT;
+                mine[q] = j < slots ? load_through(&cfg.ws_cand[base * cfg.ws_k + j]) : 0ull;
             }
             if (want_lse && tid < 64) {
                 double mt = -__builtin_huge_val(), st = 0.0;
@@ -2568,14 +2573,35 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
                     sh.lse_s = sum;
                 }
             }
-            __syncthreads();
-            const uint32_t slots = S * cfg.ws_k;
-            for (uint32_t j = tid; j < slots; j += NT) {
-                const uint32_t t = j / cfg.ws_k, i = j - t * cfg.ws_k;
-                cand[j] = i < sh.hist[t] ? load_through(&cfg.ws_cand[(base + t) * cfg.ws_k + i]) : 0ull;
+            // A bound of the k-th largest from the lanes' best entries (as in the streaming
+            // select: each wave's ceil(k / NWAVE)-th largest lane maximum, the minimum over the
+            // waves), then only entries at or above it are ranked.
+            uint64_t best_mine = 0;
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                best_mine = mine[q] > best_mine ? mine[q] : best_mine;
+            }
+            const uint32_t kw = (a.k + NWAVE - 1) / NWAVE;
+            const uint32_t P = kw <= 64u ? wave_kth_key16((uint32_t)(best_mine >> 48), kw) : 0u;
+            if ((tid & 63u) == 0) {
+                sh.red_i[tid >> 6] = P;
+            }
+            if (tid == 0) {
+                sh.n_cand = 0;
             }
             __syncthreads();
-            n = slots;
+            uint32_t bound = sh.red_i[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                bound = min(bound, sh.red_i[i]);
+            }
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                if (mine[q] != 0ull && (uint32_t)(mine[q] >> 48) >= bound) {
+                    cand[atomicAdd(&sh.n_cand, 1u)] = mine[q];
+                }
+            }
+            __syncthreads();
+            n = sh.n_cand;
             sorted = false;
             n = select_topk(cand, n, a.k, sh, sorted);
         }
