@@ -199,6 +199,7 @@ struct Shared {
     double lse_s;    // sum of 2^(x * log2e / T - lse_mc) over the row
     // streaming select
     float bound[2][NWAVE];   // each wave's lower bound of its share of the k-th largest (two parities)
+    float wmax[2][NWAVE];    // each wave's largest value so far
     uint32_t qfill[NWAVE];   // chunks each wave queued
     uint32_t n_fc;           // final candidates
     uint32_t n_drop;         // listed ids found inside queued chunks
@@ -628,14 +629,13 @@ struct WaveLse {
     __device__ __forceinline__ void add_chunk(const u32x4& q, float m, float c, bool active);
     // Block-wise use: prepare() once with the largest value the lane will add in the block
     // (raises the reference when some lane's would dwarf it), then add_prepared() per load.
-    float skip_below;  // a load whose maximum is below this adds nothing that matters
-    __device__ __forceinline__ void prepare(float block_max, float c, float inv_c) {
+    float skip_below;  // loads whose maximum is not above this are left out (set by the caller)
+    __device__ __forceinline__ void prepare(float block_max, float c) {
         if (__ballot(__builtin_fmaf(block_max, c, -ref) > 60.0f) != 0ull) {
             const float nref = fmaxf(ref, wave_max_f(block_max * c));
             s *= __builtin_amdgcn_exp2f(ref - nref);
             ref = nref;
         }
-        skip_below = (ref - 41.0f) * inv_c;
     }
     template <int DT>
     __device__ __forceinline__ void add_prepared(const u32x4& q, float m, float c, bool active);
@@ -1568,6 +1568,8 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     float lane_max = NEG_INF;
     float T = F32_LOWEST;       // the block's bound, the same in every thread
     float ref_s = 0.0f;         // reference of the double sums
+    float row_max = NEG_INF;    // largest value seen by the workgroup up to the last refresh
+    float skip_b = NEG_INF;     // the block's cut: chunks whose maximum is not above it are not summed
     uint32_t wq = 0;            // this wave's queue fill
     WaveLse wl;
     wl.init();
@@ -1580,13 +1582,13 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t P = wave_kth_key16(key16, kw);
         const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
         float wm = 0.0f;
-        if (first) {
+        if (first || want_lse) {
             wm = wave_max_f(lane_max);
         }
         if (lane == 0) {
             sh.bound[parity][w] = mine;
-            if (first) {
-                sh.red_f[w] = wm;
+            if (first || want_lse) {
+                sh.wmax[parity][w] = wm;
             }
         }
         __syncthreads();
@@ -1594,16 +1596,19 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         for (int i = 1; i < NWAVE; ++i) {
             t = fminf(t, sh.bound[parity][i]);
         }
-        parity ^= 1u;
         T = fmaxf(T, lower_by_slack(t));
-        if (first) {
-            float m = sh.red_f[0];
+        if (first || want_lse) {
+            float m = sh.wmax[parity][0];
             for (int i = 1; i < NWAVE; ++i) {
-                m = fmaxf(m, sh.red_f[i]);
+                m = fmaxf(m, sh.wmax[parity][i]);
             }
-            // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
-            ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
+            row_max = m;  // the largest raw value seen so far (listed ids at their raw value)
+            if (first) {
+                // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
+                ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
+            }
         }
+        parity ^= 1u;
     };
 
     struct Listed {
@@ -1634,7 +1639,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (cnt == 4095u) {
             cnt = gload(a.counts + id);
         }
-        const bool queued = chunk_max<DT>(r.chunk) >= T;  // the owner's test, on the same bits
+        const float cm = chunk_max<DT>(r.chunk);
+        const bool queued = cm >= T;  // the owner's tests, on the same bits
+        const bool summed = !queued && cm > skip_b;
         float t = r.raw;
         for (uint32_t j = 0; j < n_bias; ++j) {
             if (L.bias_id[j] == id) {
@@ -1647,7 +1654,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         if (want_lse) {
             acc_t += term_d(t, c2, ref_s);
-            if (!queued) {
+            if (summed) {
                 acc_r += term_d(r.raw, c2, ref_s);
             }
         }
@@ -1668,12 +1675,16 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // Block b + 1 is requested before block b is worked on (two register buffers that swap
     // roles), so the arithmetic - eight exponentials per chunk when a log-probability is
     // wanted - runs under the loads.
-    const float inv_c2 = a.temperature * 0.6931471805599453f;
+    const float lse_cut = (log2f((float)g.vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
+    Listed ahead;  // this thread's listed id of the next block, requested a block early
+    ahead.ent = NONE;
+    if (listed_row && nblocks > 0) {
+        listed_fetch(ahead, 0, 0);
+    }
     auto work = [&](const u32x4 (&cur)[U], uint32_t b) {
-        Listed lcur;
-        lcur.ent = NONE;
-        if (listed_row) {
-            listed_fetch(lcur, b, 0);
+        const Listed lcur = ahead;
+        if (listed_row && b + 1 < nblocks) {
+            listed_fetch(ahead, b + 1, 0);
         }
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
@@ -1687,7 +1698,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             sum_max = max2_raw(sum_max, m8[u] >= T_prev ? NEG_INF : m8[u]);
         }
         if (LSE && want_lse) {
-            wl.prepare(sum_max, c2, inv_c2);
+            // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
+            // sum by more than 2^-21 of it, even with every element of the row at that level:
+            // such chunks are left out, by a rule every thread of the block can evaluate.
+            skip_b = row_max - lse_cut;
+            wl.skip_below = skip_b;
+            wl.prepare(sum_max, c2);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 wl.template add_prepared<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
@@ -1717,7 +1733,8 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 // At or above the previous bound but below the new one: not queued after all.
                 const bool late = m8[u] >= T_prev && !pass;
                 if (__ballot(late) != 0ull) {
-                    wl.template add_chunk<DT>(cur[u], m8[u], c2, late);
+                    wl.prepare(late ? m8[u] : NEG_INF, c2);
+                    wl.template add_prepared<DT>(cur[u], m8[u], c2, late);
                 }
             }
         }
