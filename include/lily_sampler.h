@@ -113,9 +113,11 @@ int lily_sampler_synchronize(lily_sampler_t* s);
 /* Per-kernel profile transport of the reference (LILY_KERNEL_PROFILE, src/metal.rs:30-33,
  * :140-198) at a finer grain: while trace_dev is set, thread 0 of every workgroup of the row
  * kernels stores the 100 MHz device wall clock at up to 16 phase boundaries into
- * trace_dev[(row * slices + slice) * 16 + phase] (u64; phases: 0 start, 1 bitmap built,
- * 2 scan done, 3 specials done, 4 slice top-k done, 5 ticket taken, 6 merge done, 7 row
- * done; 8-15 finer marks inside phase 3).  capacity_words bounds rows * slices * 16; larger launches run untraced.  NULL stops. */
+ * trace_dev[(row * slices + slice) * 16 + phase] (u64; 0 start, 1 listed ids bucketed / bitmap
+ * built, 2 scan done, 3 sums merged, 4 slice top-k done, 5 ticket taken, 6 slices merged, 7 row
+ * done; 8-15 finer marks: 8 queue expanded, 9 edge ids done, 10-11 sum merge, 12 candidates
+ * ranked, 13-15 inside phase 1).  capacity_words bounds rows * slices * 16; larger launches run
+ * untraced.  NULL stops. */
 int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_t capacity_words);
 /* Diagnostics with no counterpart in the reference: while stats_dev (device, u32[4], cleared by
  * the caller) is set, every workgroup of a sampled row adds 1 to [0] when the streaming select

@@ -92,7 +92,6 @@ struct LaunchCfg {
     uint32_t step_delta;    // added to every row's step
     uint32_t ws_k;          // candidate slots per (row, slice) in ws_cand
     uint64_t* ws_cand;      // [rows][slices][ws_k] (value key << 32 | ~id)
-    uint32_t* ws_n;         // [rows][slices] candidates written
     double* ws_lse;         // [rows][slices][2] log2-domain reference, sum of 2^(x - reference)
     uint32_t* ws_ticket;    // [rows] arrival counter, left at 0
     uint32_t path;          // 0 = automatic, 1 = exhaustive select only, 2 = two-pass select only,

@@ -54,7 +54,6 @@ struct lily_sampler {
     int device = 0;
     hipStream_t stream = nullptr;
     uint64_t* ws_cand = nullptr;
-    uint32_t* ws_n = nullptr;
     double* ws_lse = nullptr;
     uint32_t* ws_ticket = nullptr;
     // Row table of lily_sample_rows batches above INLINE_ROWS.
@@ -271,7 +270,6 @@ void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t sl
     cfg->step_delta = step_delta;
     cfg->ws_k = kmax ? kmax : 1;
     cfg->ws_cand = s->ws_cand;
-    cfg->ws_n = s->ws_n;
     cfg->ws_lse = s->ws_lse;
     cfg->ws_ticket = s->ws_ticket;
     cfg->path = s->force_path;
@@ -594,7 +592,6 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     const size_t slots = (size_t)WS_ROWS * MAX_SLICES;
     hipError_t err = hipMalloc(reinterpret_cast<void**>(&s->ws_cand),
                                (size_t)WS_SLOTS * sizeof(uint64_t));
-    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_n), slots * 4);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 16);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
     if (err == hipSuccess) err = hipMemset(s->ws_ticket, 0, WS_ROWS * 4);
@@ -616,7 +613,6 @@ void lily_sampler_destroy(lily_sampler_t* s) {
     (void)hipSetDevice(s->device);
     (void)hipStreamSynchronize(s->stream);
     (void)hipFree(s->ws_cand);
-    (void)hipFree(s->ws_n);
     (void)hipFree(s->ws_lse);
     (void)hipFree(s->ws_ticket);
     (void)hipFree(s->table_dev);

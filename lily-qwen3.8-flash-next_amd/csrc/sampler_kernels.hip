@@ -135,6 +135,25 @@ __device__ __forceinline__ float wave_max_f(float v) {
     }
     return v;
 }
+// The wave's maximum in every lane, without LDS traffic: an inclusive running maximum inside
+// each row of 16 lanes by DPP row shifts (a lane whose source lies outside the row keeps its
+// own value), then the four row results read from lanes 15, 31, 47 and 63.
+__device__ __forceinline__ float wave_max_dpp(float v) {
+#define LILY_ROW_SHR_MAX(n)                                                                \
+    v = fmaxf(v, lilym_bits_f32((uint32_t)__builtin_amdgcn_update_dpp(                       \
+                     (int)lilym_f32_bits(v), (int)lilym_f32_bits(v), 0x110 + (n), 0xf, 0xf, false)))
+    LILY_ROW_SHR_MAX(1);
+    LILY_ROW_SHR_MAX(2);
+    LILY_ROW_SHR_MAX(4);
+    LILY_ROW_SHR_MAX(8);
+#undef LILY_ROW_SHR_MAX
+    const int b = (int)lilym_f32_bits(v);
+    const float r0 = lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(b, 15));
+    const float r1 = lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(b, 31));
+    const float r2 = lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(b, 47));
+    const float r3 = lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(b, 63));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
 __device__ __forceinline__ double wave_sum_d(double v) {
     for (int o = 32; o > 0; o >>= 1) {
         v += __shfl_xor(v, o);
@@ -632,7 +651,7 @@ struct WaveLse {
     float skip_below;  // loads whose maximum is not above this are left out (set by the caller)
     __device__ __forceinline__ void prepare(float block_max, float c) {
         if (__ballot(__builtin_fmaf(block_max, c, -ref) > 60.0f) != 0ull) {
-            const float nref = fmaxf(ref, wave_max_f(block_max * c));
+            const float nref = fmaxf(ref, wave_max_dpp(block_max * c));
             s *= __builtin_amdgcn_exp2f(ref - nref);
             ref = nref;
         }
@@ -1188,10 +1207,6 @@ __device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, 
                 rest = s_s - s_r * exp2(m_r - m_s);
                 bad = !(rest > 0.05 * s_s);  // cancellation: the streamed sum is too coarse
             }
-            if (cfg.phase_trace != nullptr && tid == 0) {  // DEBUG
-                uint64_t* t = cfg.phase_trace + ((size_t)blockIdx.y * cfg.slices + blockIdx.x) * PHASE_SLOTS;
-                __builtin_memcpy(&t[13], &s_s, 8); __builtin_memcpy(&t[14], &s_r, 8); double dd = m_r - m_s; __builtin_memcpy(&t[15], &dd, 8);
-            }
             if (bad) {
                 phase(cfg, 12);
                 // Rare: penalised ids held nearly all the raw mass.  Redo the sum exactly.
@@ -1583,7 +1598,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
         float wm = 0.0f;
         if (first || want_lse) {
-            wm = wave_max_f(lane_max);
+            wm = wave_max_dpp(lane_max);
         }
         if (lane == 0) {
             sh.bound[parity][w] = mine;
@@ -1690,20 +1705,20 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         // the previous bound cannot be queued: their terms are summed right away.
         const float T_prev = T;
         float m8[U];
-        float sum_max = NEG_INF;
+        float block_max = NEG_INF;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             m8[u] = chunk_max<DT>(cur[u]);
-            lane_max = max2_raw(lane_max, m8[u]);
-            sum_max = max2_raw(sum_max, m8[u] >= T_prev ? NEG_INF : m8[u]);
+            block_max = max2_raw(block_max, m8[u]);
         }
+        lane_max = max2_raw(lane_max, block_max);
         if (LSE && want_lse) {
             // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
             // sum by more than 2^-21 of it, even with every element of the row at that level:
             // such chunks are left out, by a rule every thread of the block can evaluate.
             skip_b = row_max - lse_cut;
             wl.skip_below = skip_b;
-            wl.prepare(sum_max, c2);
+            wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 wl.template add_prepared<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
@@ -2112,22 +2127,6 @@ __device__ __forceinline__ uint32_t pick_sequential(const float* prefix, uint32_
 
 // log p(id) = (u*c2 - mc - log2 s) * ln 2, with the id's exponent u*c2 formed exactly as
 // the row sum formed its terms, so the two cancel when the id carries all the mass.
-template <int DT>
-__device__ __forceinline__ void write_logprob(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
-    if (a.out_logprob == nullptr) {
-        return;
-    }
-    float lp = NEG_INF;
-    if (id < vocab) {
-        const float u = pre_temperature_of<DT>(a, id);
-        if (u > NEG_INF) {
-            const double e = (double)u * (double)a.c2 - sh.lse_mc - log2(sh.lse_s);
-            lp = fminf((float)(e * 0.6931471805599453), 0.0f);  // the sum is approximate: clamp
-        }
-    }
-    *a.out_logprob = lp;
-}
-
 // Emits `id` and, when asked, its log-probability, with the memory operations of both in one
 // round trip: the count's atomic increment returns the count the penalties used, the bitmap's
 // atomic OR tells whether the id is listed already, and the logit and the list position load
