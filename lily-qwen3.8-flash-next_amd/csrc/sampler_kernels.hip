@@ -218,7 +218,9 @@ struct Shared {
     double lse_s;    // sum of 2^(x * log2e / T - lse_mc) over the row
     // streaming select
     float bound[2][NWAVE];   // each wave's lower bound of its share of the k-th largest (two parities)
-    float wmax[2][NWAVE];    // each wave's largest value so far
+    float wmax[2][3][NWAVE];  // each wave's largest raw value, largest raw and largest true value
+                              // of listed ids so far
+    uint32_t dense_listed;    // some block holds more listed ids than the workgroup has threads
     uint32_t qfill[NWAVE];   // chunks each wave queued
     uint32_t n_fc;           // final candidates
     uint32_t n_drop;         // listed ids found inside queued chunks
@@ -1467,6 +1469,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         sh.n_fc = 0;
         sh.n_drop = 0;
         sh.fail = 0;
+        sh.dense_listed = 0;
     }
     for (uint32_t i = tid; i < n_bias; i += NT) {
         L.bias_id[i] = gload(&a.bias[i].id);
@@ -1555,6 +1558,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 phase(cfg, 14);
                 if (tid < 64) {  // counts -> exclusive offsets, total in bkt[MAX_BUCKETS]
                     const uint32_t cnt = L.bkt[tid];
+                    const uint64_t big = __ballot(cnt > (uint32_t)NT);
+                    if (tid == 0) {
+                        sh.dense_listed = big != 0ull ? 1u : 0u;
+                    }
                     uint32_t incl = cnt;
                     for (int o = 1; o < 64; o <<= 1) {
                         const uint32_t t = __shfl_up(incl, o);
@@ -1583,7 +1590,8 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     float lane_max = NEG_INF;
     float T = F32_LOWEST;       // the block's bound, the same in every thread
     float ref_s = 0.0f;         // reference of the double sums
-    float row_max = NEG_INF;    // largest value seen by the workgroup up to the last refresh
+    float row_max = NEG_INF;    // lower bound of the row's largest true value, as of the last refresh
+    float listed_raw_max = NEG_INF, listed_true_max = NEG_INF;  // this thread's listed ids so far
     float skip_b = NEG_INF;     // the block's cut: chunks whose maximum is not above it are not summed
     uint32_t wq = 0;            // this wave's queue fill
     WaveLse wl;
@@ -1596,14 +1604,20 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t key16 = lane_max > NEG_INF ? (lilym_order_key(lane_max) >> 16) : 0u;
         const uint32_t P = wave_kth_key16(key16, kw);
         const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
-        float wm = 0.0f;
+        float wm[3] = {0.0f, 0.0f, 0.0f};
         if (first || want_lse) {
-            wm = wave_max_dpp(lane_max);
+            wm[0] = wave_max_dpp(lane_max);
+            if (want_lse && listed_row) {
+                wm[1] = wave_max_dpp(listed_raw_max);
+                wm[2] = wave_max_dpp(listed_true_max);
+            }
         }
         if (lane == 0) {
             sh.bound[parity][w] = mine;
             if (first || want_lse) {
-                sh.wmax[parity][w] = wm;
+                for (int q = 0; q < 3; ++q) {
+                    sh.wmax[parity][q][w] = wm[q];
+                }
             }
         }
         __syncthreads();
@@ -1613,14 +1627,28 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         T = fmaxf(T, lower_by_slack(t));
         if (first || want_lse) {
-            float m = sh.wmax[parity][0];
-            for (int i = 1; i < NWAVE; ++i) {
-                m = fmaxf(m, sh.wmax[parity][i]);
+            float m[3];
+            for (int q = 0; q < 3; ++q) {
+                m[q] = sh.wmax[parity][q][0];
+                for (int i = 1; i < NWAVE; ++i) {
+                    m[q] = fmaxf(m[q], sh.wmax[parity][q][i]);
+                }
             }
-            row_max = m;  // the largest raw value seen so far (listed ids at their raw value)
+            // A lower bound of the row's largest TRUE value: the largest raw value when it
+            // exceeds every listed id's raw value (then it belongs to an id that keeps its
+            // value), and the largest true value of the listed ids in any case.  All three
+            // maxima cover the same blocks.  A block with more listed ids than threads breaks
+            // that (its later rounds lag), so such rows skip nothing.
+            if (!listed_row) {
+                row_max = m[0];
+            } else if (sh.dense_listed != 0u) {
+                row_max = NEG_INF;
+            } else {
+                row_max = m[0] > m[1] ? fmaxf(m[0], m[2]) : m[2];
+            }
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
-                ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
+                ref_s = m[0] > NEG_INF ? fminf(fmaxf(m[0] * c2, -1.0e30f), 1.0e30f) : 0.0f;
             }
         }
         parity ^= 1u;
@@ -1645,18 +1673,17 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             r.raw = load_logit<DT>(a.logits, id);
         }
     };
-    auto listed_process = [&](const Listed& r) {
+    // A listed id's true value before the temperature (bias in list order, then penalties);
+    // also feeds the thread's maxima of listed raw and true values.
+    auto listed_value = [&](const Listed& r) -> float {
         if (r.ent == NONE) {
-            return;
+            return NEG_INF;
         }
         const uint32_t id = r.ent & ID_MASK;
         uint32_t cnt = r.ent >> SPEC_ID_BITS;
         if (cnt == 4095u) {
             cnt = gload(a.counts + id);
         }
-        const float cm = chunk_max<DT>(r.chunk);
-        const bool queued = cm >= T;  // the owner's tests, on the same bits
-        const bool summed = !queued && cm > skip_b;
         float t = r.raw;
         for (uint32_t j = 0; j < n_bias; ++j) {
             if (L.bias_id[j] == id) {
@@ -1667,8 +1694,24 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             t = t > 0.0f ? t / a.repetition : t * a.repetition;
             t -= a.presence + a.frequency * (float)cnt;
         }
+        listed_raw_max = fmaxf(listed_raw_max, r.raw);
+        listed_true_max = fmaxf(listed_true_max, t);
+        return t;
+    };
+    // After the block's bound is known: was the id's chunk queued or summed by its owner (the
+    // owner's tests on the same bits), the id's terms, and the id as a candidate.
+    auto listed_finish = [&](const Listed& r, float t) {
+        if (r.ent == NONE) {
+            return;
+        }
+        const uint32_t id = r.ent & ID_MASK;
+        const float cm = chunk_max<DT>(r.chunk);
+        const bool queued = cm >= T;
+        const bool summed = !queued && cm > skip_b;
         if (want_lse) {
-            acc_t += term_d(t, c2, ref_s);
+            if (t > skip_b) {  // the same cut as for streamed terms
+                acc_t += term_d(t, c2, ref_s);
+            }
             if (summed) {
                 acc_r += term_d(r.raw, c2, ref_s);
             }
@@ -1701,6 +1744,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (listed_row && b + 1 < nblocks) {
             listed_fetch(ahead, b + 1, 0);
         }
+        const float lcur_t = listed_row ? listed_value(lcur) : NEG_INF;
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
         const float T_prev = T;
@@ -1744,7 +1788,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 }
                 wq += (uint32_t)__popcll(mask);
             }
-            if (LSE && want_lse) {
+            if (LSE && want_lse && T != T_prev) {
                 // At or above the previous bound but below the new one: not queued after all.
                 const bool late = m8[u] >= T_prev && !pass;
                 if (__ballot(late) != 0ull) {
@@ -1754,12 +1798,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
         if (listed_row) {
-            listed_process(lcur);
+            listed_finish(lcur, lcur_t);
             const uint32_t n_b = L.bkt[b + 1] - L.bkt[b];
             for (uint32_t round = 1; round * NT < n_b; ++round) {
                 Listed extra;
                 listed_fetch(extra, b, round);
-                listed_process(extra);
+                listed_finish(extra, listed_value(extra));
             }
         }
     };

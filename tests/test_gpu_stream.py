@@ -248,6 +248,33 @@ def test_log_probabilities_of_peaked_and_flat_rows(sampler):
         s_.close()
 
 
+def test_skipped_terms_are_measured_against_the_largest_true_value(sampler):
+    """The largest raw value belongs to a heavily penalised id: terms may only be skipped
+    relative to what that id is worth after the penalties, or the mass of the values in between
+    would be lost."""
+    rng = np.random.default_rng(21)
+    vocab, rows = 151_936, 3
+    x = rng.normal(0, 2, (rows, vocab)).astype(np.float32)
+    hist = []
+    for r in range(rows):
+        x[r, 4000 + r] = 150.0                                   # worth 150 / 2.5 - 41 = 19 after penalties
+        x[r, rng.choice(vocab, 3000, replace=False)] = 18.0      # real mass just below it
+        hist.append(np.concatenate([np.full(40, 4000 + r), rng.integers(0, vocab, 1000)]))
+    x[2, 9000] = 60.0                                            # row 2: a plain id above everything
+    xs = W.to_bf16_bits(x)
+    sc, counts = _scratches(sampler, hist, vocab)
+    kw = [dict(temperature=0.8, top_k=64, top_p=0.9, seed=r, repetition_penalty=2.5,
+               presence_penalty=1.0, frequency_penalty=1.0) for r in range(rows)]
+    for step in range(2):
+        r = run_rows(sampler, xs, kw, [step] * rows, scratch=sc, logprobs=True)
+        for i in range(rows):
+            d = O.sample(xs[i], counts[i], o_params(**kw[i]), step, want_logprob=True)
+            check_row_against_oracle(r, i, d)
+            _check_logprob(r, i, d, ("true max", step))
+    for s_ in sc:
+        s_.close()
+
+
 def test_a_batch_replays(sampler):
     """The same batch from the same counts: identical ids, log-probabilities equal to 2e-6
     (the listed ids' terms are summed in the order their bucket slots were taken)."""
