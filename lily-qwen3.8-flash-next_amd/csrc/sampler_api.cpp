@@ -245,11 +245,29 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
 }
 
 // Workgroups per row for a batch of `rows` whose largest candidate count is kmax.
-uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab) {
+// The longest scratch list among `rows` (the host's bound, as packed into the rows).
+uint32_t longest_list(const RowArgs* rows, uint32_t n) {
+    uint32_t longest = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        if ((rows[i].flags & F_PEN) && rows[i].pairs_hint > longest) {
+            longest = rows[i].pairs_hint;
+        }
+    }
+    return longest;
+}
+
+// `listed`: the longest list of penalised ids among the rows (0 = none): a workgroup buckets
+// at most SPEC_CAP of them, so long lists are spread over more slices.
+uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab,
+                       uint32_t listed = 0) {
     if (rows > WS_ROWS) {
         return 1;
     }
     uint32_t sl = s->force_slices ? s->force_slices : (TARGET_GROUPS + rows - 1) / rows;
+    if (!s->force_slices) {
+        const uint32_t by_list = (listed + 64 + (SPEC_CAP * 2) / 3 - 1) / ((SPEC_CAP * 2) / 3);
+        sl = sl < by_list ? by_list : sl;
+    }
     sl = sl < 1 ? 1 : sl;
     sl = sl > MAX_SLICES ? MAX_SLICES : sl;
     const uint32_t by_k = MERGE_CAP / (kmax ? kmax : 1);
@@ -356,7 +374,7 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     HIP_TRY(hipSetDevice(s->device));
     const uint32_t kmax = max_k(rows.r, n);
     LaunchCfg cfg;
-    const uint32_t slices = choose_slices(s, n, kmax, vocab);
+    const uint32_t slices = choose_slices(s, n, kmax, vocab, longest_list(rows.r, n));
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
     attach_trace(s, &cfg, n);
     const LaunchShape shp = shape_of(s, rows.r, n, dtype, vocab, slices, kmax);
@@ -996,7 +1014,8 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     s->stage_used[slot] = true;
     const uint32_t kmax = max_k(s->stage[slot], b->rows);
     LaunchCfg cfg;
-    const uint32_t slices = choose_slices(s, b->rows, kmax, b->vocab);
+    const uint32_t slices =
+        choose_slices(s, b->rows, kmax, b->vocab, longest_list(s->stage[slot], b->rows));
     fill_cfg(s, &cfg, b->vocab, slices, kmax, 0, s->table_dev);
     attach_trace(s, &cfg, b->rows);
     const LaunchShape shp =
@@ -1060,7 +1079,9 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->vocab = b->vocab;
     p->dtype = b->dtype;
     p->ws_k = max_k(table.data(), b->rows);
-    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab);
+    // Room for the lists to grow by the draws of about a thousand runs of the plan.
+    const uint32_t listed = longest_list(table.data(), b->rows);
+    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab, listed ? listed + 1024 : 0);
     const LaunchShape shp = shape_of(p->s, table.data(), b->rows, (int)b->dtype, b->vocab,
                                      p->slices, p->ws_k);
     p->kind = shp.kind();

@@ -172,6 +172,32 @@ def test_lists_beyond_the_workgroup_and_the_scratch(sampler):
         s_.close()
 
 
+def test_long_lists_are_spread_over_more_slices():
+    """6 000 listed ids per row: the launch takes enough slices for every workgroup to bucket
+    its share, so the streaming select still serves every slice."""
+    s = LS.Sampler(0)
+    rng = np.random.default_rng(15)
+    vocab, rows = 151_936, 300
+    x = W.to_bf16_bits(rng.normal(0, 2, (rows, vocab)).astype(np.float32))
+    hist = [rng.choice(vocab, 6000, replace=False) for _ in range(rows)]
+    sc, counts = _scratches(s, hist, vocab)
+    kw = [dict(temperature=0.7, top_k=40, top_p=0.9, seed=r, repetition_penalty=1.1,
+               presence_penalty=0.2, frequency_penalty=0.1) for r in range(rows)]
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    s.set_path_stats(stats)
+    r = run_rows(s, x, kw, [0] * rows, scratch=sc, logprobs=True)
+    s.set_path_stats(None)
+    st = stats.cpu().tolist()
+    assert st[0] > rows and st[1] == 0 and st[2] == 0, st
+    for i in range(0, rows, 7):
+        d = O.sample(x[i], counts[i], o_params(**kw[i]), 0, want_logprob=True)
+        check_row_against_oracle(r, i, d)
+        _check_logprob(r, i, d, "long lists")
+    for s_ in sc:
+        s_.close()
+    s.close()
+
+
 def test_the_list_follows_every_scratch_operation(sampler):
     """Draws after uncount (to zero and back), reset, copy and a dense rewrite of the counts
     see exactly the counts the reference's histogram would hold (the oracle's draw adds the
