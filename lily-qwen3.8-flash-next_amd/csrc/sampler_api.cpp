@@ -107,6 +107,7 @@ struct lily_plan {
     uint32_t excl_words = 0;
     bool old_layout = false;
     uint32_t cand_cap = 0;
+    uint32_t listed = 0;                     // longest scratch list when the table was packed
     uint32_t runs = 0;                       // launches since the table was packed
     std::vector<lily_scratch*> penalised;    // scratches whose rows count their draws
 };
@@ -256,6 +257,13 @@ uint32_t longest_list(const RowArgs* rows, uint32_t n) {
     return longest;
 }
 
+// Slices that leave every workgroup about a tenth of its bucket capacity free when a list
+// of `listed` ids is spread evenly over the vocabulary.
+uint32_t slices_for_list(uint32_t listed) {
+    const uint32_t room = SPEC_CAP - SPEC_CAP / 10;
+    return (listed + room - 1) / room;
+}
+
 // `listed`: the longest list of penalised ids among the rows (0 = none): a workgroup buckets
 // at most SPEC_CAP of them, so long lists are spread over more slices.
 uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab,
@@ -265,7 +273,7 @@ uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint
     }
     uint32_t sl = s->force_slices ? s->force_slices : (TARGET_GROUPS + rows - 1) / rows;
     if (!s->force_slices) {
-        const uint32_t by_list = (listed + 64 + (SPEC_CAP * 2) / 3 - 1) / ((SPEC_CAP * 2) / 3);
+        const uint32_t by_list = slices_for_list(listed);
         sl = sl < by_list ? by_list : sl;
     }
     sl = sl < 1 ? 1 : sl;
@@ -1079,9 +1087,8 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->vocab = b->vocab;
     p->dtype = b->dtype;
     p->ws_k = max_k(table.data(), b->rows);
-    // Room for the lists to grow by the draws of about a thousand runs of the plan.
-    const uint32_t listed = longest_list(table.data(), b->rows);
-    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab, listed ? listed + 1024 : 0);
+    p->listed = longest_list(table.data(), b->rows);
+    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab, p->listed);
     const LaunchShape shp = shape_of(p->s, table.data(), b->rows, (int)b->dtype, b->vocab,
                                      p->slices, p->ws_k);
     p->kind = shp.kind();
@@ -1105,6 +1112,19 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
         return fail(LILY_ERR_INVALID_ARG, "plan is null or not set");
     }
     HIP_TRY(hipSetDevice(p->s->device));
+    if (p->listed != 0 && p->kind == 2 && p->rows <= WS_ROWS) {
+        // The lists grow by one id per run at most: take more slices before a workgroup's
+        // buckets overflow (only the merge's share of dynamic LDS depends on the slices).
+        const uint32_t need = slices_for_list(p->listed + p->runs + 1);
+        const uint64_t by_ws = (uint64_t)WS_SLOTS / ((uint64_t)p->rows * (p->ws_k ? p->ws_k : 1));
+        if (need > p->slices && need <= MAX_SLICES && need <= by_ws) {
+            p->slices = need;
+            const size_t merge = (size_t)need * p->ws_k * 8;
+            if (merge > p->dyn_bytes) {
+                p->dyn_bytes = merge;
+            }
+        }
+    }
     LaunchCfg cfg;
     fill_cfg(p->s, &cfg, p->vocab, p->slices, p->ws_k, step_delta, p->table_dev);
     attach_trace(p->s, &cfg, p->rows);
