@@ -741,12 +741,14 @@ template <int DT>
 __device__ __forceinline__ void WaveLse::add_prepared(const u32x4& q, float m, float c, bool active) {
     constexpr int E = DT == LILY_BF16 ? 8 : 4;
     active = active && m > skip_below;
-    if (__ballot(active) == 0ull) {
-        return;
-    }
     if (active) {
+        // The raw bits pass through an empty asm so that this unpack is not merged with the
+        // one that fed the chunk maximum: merged, 8 values per chunk stay live across the
+        // whole block for a path that rows with a dominant value never take.
+        u32x4 r = q;
+        asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
         float v[E];
-        unpack<DT>(q, v);
+        unpack<DT>(r, v);
 #pragma unroll
         for (int j = 0; j < E; ++j) {
             s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], c, -ref));
@@ -1734,16 +1736,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // roles), so the arithmetic - eight exponentials per chunk when a log-probability is
     // wanted - runs under the loads.
     const float lse_cut = (log2f((float)g.vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
-    Listed ahead;  // this thread's listed id of the next block, requested a block early
-    ahead.ent = NONE;
-    if (listed_row && nblocks > 0) {
-        listed_fetch(ahead, 0, 0);
-    }
-    auto work = [&](const u32x4 (&cur)[U], uint32_t b) {
-        const Listed lcur = ahead;
-        if (listed_row && b + 1 < nblocks) {
-            listed_fetch(ahead, b + 1, 0);
-        }
+    // Memory operations of a wave complete in the order they were issued: a block's listed
+    // gathers are requested BEFORE the next stream block, so using them never waits for it.
+    Listed lst_a, lst_b;
+    lst_a.ent = NONE;
+    lst_b.ent = NONE;
+    auto work = [&](const u32x4 (&cur)[U], const Listed& lcur, uint32_t b) {
         const float lcur_t = listed_row ? listed_value(lcur) : NEG_INF;
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
@@ -1809,17 +1807,25 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     };
     if (nblocks == 0) {
         refresh_bound(true);  // the same barriers in every workgroup
+    } else if (listed_row) {
+        listed_fetch(lst_a, 0, 0);
     }
     for (uint32_t b = 0; b < nblocks; b += 2) {
         if (b + 1 < nblocks) {
+            if (listed_row) {
+                listed_fetch(lst_b, b + 1, 0);
+            }
             fetch(buf_b, b + 1);
         }
-        work(buf_a, b);
+        work(buf_a, lst_a, b);
         if (b + 1 < nblocks) {
             if (b + 2 < nblocks) {
+                if (listed_row) {
+                    listed_fetch(lst_a, b + 2, 0);
+                }
                 fetch(buf_a, b + 2);
             }
-            work(buf_b, b + 1);
+            work(buf_b, lst_b, b + 1);
         }
     }
     phase(cfg, 2);
