@@ -1520,15 +1520,19 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                             (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS);
             }
         }
+        // Entries held in registers take their place inside the bucket with the first pass's
+        // atomic (counted in bfill); everything else is counted in bkt and placed behind them
+        // by a second atomic in the second pass.
+        uint32_t place[PREG];
         for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
             for (int q = 0; q < PREG; ++q) {
                 if (packed[q] != NONE) {
                     const uint32_t b = block_of(packed[q] & ID_MASK);
                     if (pass == 0) {
-                        atomicAdd(&L.bkt[b], 1u);
+                        place[q] = atomicAdd(&L.bfill[b], 1u);
                     } else {
-                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = packed[q];
+                        L.spec[L.bkt[b] + place[q]] = packed[q];
                     }
                 }
             }
@@ -1559,7 +1563,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             if (pass == 0) {
                 phase(cfg, 14);
                 if (tid < 64) {  // counts -> exclusive offsets, total in bkt[MAX_BUCKETS]
-                    const uint32_t cnt = L.bkt[tid];
+                    const uint32_t cnt = L.bkt[tid] + L.bfill[tid];
                     const uint64_t big = __ballot(cnt > (uint32_t)NT);
                     if (tid == 0) {
                         sh.dense_listed = big != 0ull ? 1u : 0u;
