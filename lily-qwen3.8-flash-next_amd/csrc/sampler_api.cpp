@@ -44,7 +44,7 @@ int hip_fail(hipError_t e, const char* what) {
     } while (0)
 
 constexpr uint32_t WS_ROWS = 4096;      // rows that may span several workgroups
-constexpr uint32_t WS_SLOTS = 1u << 20; // candidate slots of the workspace (rows x slices x k)
+constexpr uint32_t WS_SLOTS = 1u << 22; // candidate slots of the workspace (rows x slices x k)
 constexpr uint32_t STAGE_SLOTS = 4;
 constexpr uint32_t TARGET_GROUPS = 512;  // workgroups a small batch is spread over
 
@@ -114,7 +114,7 @@ struct lily_plan {
 
 namespace {
 
-constexpr uint32_t PAIRS_CAP = 16384;  // listed ids a scratch keeps (more: the list is not used)
+constexpr uint32_t PAIRS_CAP = 65536;  // listed ids a scratch keeps (more: the list is not used)
 
 ScratchView view_of(const lily_scratch* sc) {
     ScratchView v;

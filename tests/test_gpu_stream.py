@@ -153,18 +153,19 @@ def test_rows_that_defeat_the_bound(sampler):
 
 
 def test_lists_beyond_the_workgroup_and_the_scratch(sampler):
-    """4 000 listed ids (more than a workgroup buckets) and 20 000 (more than a scratch lists):
-    the draw falls back and still agrees; later draws keep agreeing."""
+    """4 000 listed ids (more than a workgroup buckets), 20 000 (spread over slices) and
+    70 000 (more than a scratch lists): the draws agree whichever select serves them, and
+    later draws keep agreeing."""
     rng = np.random.default_rng(5)
-    vocab = 40_961
-    x = W.to_bf16_bits(rng.normal(0, 2, (2, vocab)).astype(np.float32))
-    hist = [rng.choice(vocab, 4000, replace=False), rng.choice(vocab, 20_000, replace=False)]
+    vocab = 90_001
+    x = W.to_bf16_bits(rng.normal(0, 2, (3, vocab)).astype(np.float32))
+    hist = [rng.choice(vocab, n, replace=False) for n in (4000, 20_000, 70_000)]
     sc, counts = _scratches(sampler, hist, vocab)
     for step in range(3):
         kw = [dict(temperature=0.7, top_k=40, top_p=0.9, seed=r, repetition_penalty=1.1,
-                   presence_penalty=0.2, frequency_penalty=0.1) for r in range(2)]
-        r = run_rows(sampler, x, kw, [step] * 2, scratch=sc, logprobs=True)
-        for i in range(2):
+                   presence_penalty=0.2, frequency_penalty=0.1) for r in range(3)]
+        r = run_rows(sampler, x, kw, [step] * 3, scratch=sc, logprobs=True)
+        for i in range(3):
             d = O.sample(x[i], counts[i], o_params(**kw[i]), step, want_logprob=True)
             check_row_against_oracle(r, i, d)
             _check_logprob(r, i, d, ("long", step))
