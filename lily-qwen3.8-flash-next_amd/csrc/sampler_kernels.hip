@@ -737,6 +737,28 @@ __device__ __forceinline__ float chunk_max(const u32x4& q) {
     return max2_raw(max3_raw(v[0], v[1], v[2]), v[3]);
 }
 
+// Signed 16-bit maximum of both halves of a and b.  bf16 patterns of values that are not
+// negative order like the values; every negative one is below all of them.
+__device__ __forceinline__ uint32_t pk_max_i16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_max_i16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
+// The largest element of one 16-byte chunk when that element is not negative, +0 otherwise:
+// exact wherever the result is compared with a positive bound, an upper bound elsewhere.
+// Half the instructions of chunk_max() for bf16 (no unpacking); the same for f32.
+template <int DT>
+__device__ __forceinline__ float chunk_max_nonneg(const u32x4& q) {
+    if (DT == LILY_BF16) {
+        const uint32_t r = pk_max_i16(pk_max_i16(q.x, q.y), pk_max_i16(q.z, q.w));
+        uint32_t m;
+        asm("v_max3_i32 %0, %1, %2, 0" : "=v"(m) : "v"(r << 16), "v"(r & 0xffff0000u));
+        return lilym_bits_f32(m);
+    }
+    return chunk_max<DT>(q);
+}
+
 template <int DT>
 __device__ __forceinline__ void WaveLse::add_prepared(const u32x4& q, float m, float c, bool active) {
     constexpr int E = DT == LILY_BF16 ? 8 : 4;
@@ -1454,7 +1476,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             early[q] = p < loaded ? gload(reinterpret_cast<const uint64_t*>(a.pairs) + p) : ~0ull;
         }
     }
-    u32x4 buf_a[U], buf_b[U];
+    u32x4 buf_a[U], buf_b[U], buf_c[U];
     if (nblocks > 0) {
         fetch(buf_a, 0);
     }
@@ -1509,7 +1531,47 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         return b;
     };
-    if (listed_row) {
+    if (listed_row && nblocks == 1u) {
+        // One block: its bucket starts at slot 0, so a single atomic places each entry and
+        // there is nothing to count first.
+        auto put = [&](uint32_t entry) {
+            const uint32_t at = atomicAdd(&L.bfill[0], 1u);
+            if (at < SPEC_CAP) {
+                L.spec[at] = entry;
+            }
+        };
+#pragma unroll
+        for (int q = 0; q < PREG; ++q) {
+            const uint32_t p = (uint32_t)q * NT + tid;
+            if (p < n_pairs && p < loaded && block_of((uint32_t)early[q]) != NONE) {
+                put((uint32_t)early[q] | (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS));
+            }
+        }
+        for (uint32_t p = loaded + tid; p < n_pairs; p += NT) {
+            const uint64_t e = gload(reinterpret_cast<const uint64_t*>(a.pairs) + p);
+            if (block_of((uint32_t)e) != NONE) {
+                put((uint32_t)e | (min((uint32_t)(e >> 32), 4095u) << SPEC_ID_BITS));
+            }
+        }
+        for (uint32_t i = tid; i < n_bias; i += NT) {
+            if (bias_block(i) != NONE) {
+                put(L.bias_id[i]);
+            }
+        }
+        __syncthreads();
+        const uint32_t total = L.bfill[0];
+        if (total > SPEC_CAP) {
+            return stream_fail(cfg, 3u);
+        }
+        // Every wave writes the bucket's end for its own later reads (the same value).
+        if (lane == 0) {
+            L.bkt[1] = total;
+            L.bkt[MAX_BUCKETS] = total;
+            if (total > (uint32_t)NT) {
+                sh.dense_listed = 1u;
+            }
+        }
+    } else if (listed_row) {
         uint32_t packed[PREG];  // id | min(count, 4095) << 20, NONE when not of this slice
 #pragma unroll
         for (int q = 0; q < PREG; ++q) {
@@ -1606,12 +1668,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     uint32_t parity = 0;
 
     // Brings T up to date with everything the lanes have seen, the current block included.
-    auto refresh_bound = [&](bool first) {
+    auto refresh_bound = [&](bool first, bool maxima) {
         const uint32_t key16 = lane_max > NEG_INF ? (lilym_order_key(lane_max) >> 16) : 0u;
         const uint32_t P = wave_kth_key16(key16, kw);
         const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
         float wm[3] = {0.0f, 0.0f, 0.0f};
-        if (first || want_lse) {
+        if (maxima) {
             wm[0] = wave_max_dpp(lane_max);
             if (want_lse && listed_row) {
                 wm[1] = wave_max_dpp(listed_raw_max);
@@ -1620,7 +1682,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         if (lane == 0) {
             sh.bound[parity][w] = mine;
-            if (first || want_lse) {
+            if (maxima) {
                 for (int q = 0; q < 3; ++q) {
                     sh.wmax[parity][q][w] = wm[q];
                 }
@@ -1632,7 +1694,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             t = fminf(t, sh.bound[parity][i]);
         }
         T = fmaxf(T, lower_by_slack(t));
-        if (first || want_lse) {
+        if (maxima) {
             float m[3];
             for (int q = 0; q < 3; ++q) {
                 m[q] = sh.wmax[parity][q][0];
@@ -1706,12 +1768,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     };
     // After the block's bound is known: was the id's chunk queued or summed by its owner (the
     // owner's tests on the same bits), the id's terms, and the id as a candidate.
-    auto listed_finish = [&](const Listed& r, float t) {
+    auto listed_finish = [&](const Listed& r, float t, bool nonneg) {
         if (r.ent == NONE) {
             return;
         }
         const uint32_t id = r.ent & ID_MASK;
-        const float cm = chunk_max<DT>(r.chunk);
+        const float cm = nonneg ? chunk_max_nonneg<DT>(r.chunk) : chunk_max<DT>(r.chunk);
         const bool queued = cm >= T;
         const bool summed = !queued && cm > skip_b;
         if (want_lse) {
@@ -1736,26 +1798,40 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
     };
 
-    // Block b + 1 is requested before block b is worked on (two register buffers that swap
-    // roles), so the arithmetic - eight exponentials per chunk when a log-probability is
-    // wanted - runs under the loads.
+    // Blocks b + 1 and b + 2 are on their way while block b is worked on (three register
+    // buffers that swap roles): one block in flight per wave leaves the memory idle whenever
+    // a wave's arithmetic outlasts its load.
     const float lse_cut = (log2f((float)g.vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
     // Memory operations of a wave complete in the order they were issued: a block's listed
     // gathers are requested BEFORE the next stream block, so using them never waits for it.
-    Listed lst_a, lst_b;
+    Listed lst_a, lst_b, lst_c;
     lst_a.ent = NONE;
     lst_b.ent = NONE;
+    lst_c.ent = NONE;
     auto work = [&](const u32x4 (&cur)[U], const Listed& lcur, uint32_t b) {
         const float lcur_t = listed_row ? listed_value(lcur) : NEG_INF;
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
         const float T_prev = T;
+        // Once the bound is positive only chunks with a positive element can matter to it:
+        // their maximum comes from the cheaper form, which reports +0 for all others (the sum
+        // then takes such a chunk unless the cut is positive too, and the lanes' maxima are
+        // only overstated up to 0, below the bound they could move).
+        const bool nonneg = DT == LILY_BF16 && __builtin_amdgcn_readfirstlane((int)(T_prev > 0.0f)) != 0;
         float m8[U];
         float block_max = NEG_INF;
+        if (nonneg) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            m8[u] = chunk_max<DT>(cur[u]);
-            block_max = max2_raw(block_max, m8[u]);
+            for (int u = 0; u < U; ++u) {
+                m8[u] = chunk_max_nonneg<DT>(cur[u]);
+                block_max = max2_raw(block_max, m8[u]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                m8[u] = chunk_max<DT>(cur[u]);
+                block_max = max2_raw(block_max, m8[u]);
+            }
         }
         lane_max = max2_raw(lane_max, block_max);
         if (LSE && want_lse) {
@@ -1764,17 +1840,23 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // such chunks are left out, by a rule every thread of the block can evaluate.
             skip_b = row_max - lse_cut;
             wl.skip_below = skip_b;
-            wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
+            // Rows with a dominant value skip nearly every block as a whole.
+            if (__ballot(block_max > skip_b) != 0ull) {
+                wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                wl.template add_prepared<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
+                for (int u = 0; u < U; ++u) {
+                    wl.template add_prepared<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
+                }
             }
         }
         // The bound moves most in the first blocks: refresh it for each of them, then for
-        // every fourth block (each refresh is a ballot search and a barrier).
+        // every fourth block (each refresh is a ballot search and a barrier).  The row's
+        // maxima behind the sum's cut follow with every other of those.
         if (b < 4u || (b & 3u) == 0u) {
-            refresh_bound(b == 0);
+            refresh_bound(b == 0, b == 0 || (LSE && want_lse && (b < 4u || (b & 7u) == 0u)));
         }
+        const bool any_late = LSE && want_lse && T != T_prev &&
+                              __ballot(block_max >= T_prev && block_max > skip_b) != 0ull;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t c = g.cb + (b * U + u) * NT + tid;
@@ -1790,7 +1872,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 }
                 wq += (uint32_t)__popcll(mask);
             }
-            if (LSE && want_lse && T != T_prev) {
+            if (any_late) {
                 // At or above the previous bound but below the new one: not queued after all.
                 const bool late = m8[u] >= T_prev && !pass;
                 if (__ballot(late) != 0ull) {
@@ -1800,36 +1882,39 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
         if (listed_row) {
-            listed_finish(lcur, lcur_t);
+            listed_finish(lcur, lcur_t, nonneg);
             const uint32_t n_b = L.bkt[b + 1] - L.bkt[b];
             for (uint32_t round = 1; round * NT < n_b; ++round) {
                 Listed extra;
                 listed_fetch(extra, b, round);
-                listed_finish(extra, listed_value(extra));
+                listed_finish(extra, listed_value(extra), nonneg);
             }
         }
     };
     if (nblocks == 0) {
-        refresh_bound(true);  // the same barriers in every workgroup
+        refresh_bound(true, true);  // the same barriers in every workgroup
     } else if (listed_row) {
         listed_fetch(lst_a, 0, 0);
     }
-    for (uint32_t b = 0; b < nblocks; b += 2) {
-        if (b + 1 < nblocks) {
+    auto request = [&](u32x4 (&dst)[U], Listed& ldst, uint32_t b) {
+        if (b < nblocks) {
             if (listed_row) {
-                listed_fetch(lst_b, b + 1, 0);
+                listed_fetch(ldst, b, 0);
             }
-            fetch(buf_b, b + 1);
+            fetch(dst, b);
         }
+    };
+    request(buf_b, lst_b, 1);
+    for (uint32_t b = 0; b < nblocks; b += 3) {
+        request(buf_c, lst_c, b + 2);
         work(buf_a, lst_a, b);
         if (b + 1 < nblocks) {
-            if (b + 2 < nblocks) {
-                if (listed_row) {
-                    listed_fetch(lst_a, b + 2, 0);
-                }
-                fetch(buf_a, b + 2);
-            }
+            request(buf_a, lst_a, b + 3);
             work(buf_b, lst_b, b + 1);
+            if (b + 2 < nblocks) {
+                request(buf_b, lst_b, b + 4);
+                work(buf_c, lst_c, b + 2);
+            }
         }
     }
     phase(cfg, 2);
