@@ -193,7 +193,8 @@ int lily_copy_row_u32(lily_sampler_t* s, const uint32_t* src_dev, uint32_t rows,
 /* The verify pass's draws (src/qwen4exp/model.rs:3008-3040) followed by spec_accept
  * (src/qwen4exp/spec.rs:414-424): rows j < m-1 are speculative draws against dists slot j
  * and proposal ids_dev[j+1] at step0+j, the last row a plain draw; row j sees the counts
- * of rows before it.  verify_tokens_dev[m] receives the draws, ctrl_dev the control block. */
+ * of rows before it (one launch per row under penalties, one launch for all rows without).
+ * verify_tokens_dev[m] receives the draws, ctrl_dev the control block. */
 int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype, uint32_t vocab,
                      uint64_t row_stride, uint32_t m, lily_scratch_t* scratch,
                      const lily_sampling_params* params, uint32_t step0,

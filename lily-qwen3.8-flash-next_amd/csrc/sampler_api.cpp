@@ -960,10 +960,13 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
         return fail(LILY_ERR_RANGE, "verify needs %u draft distribution slots", m - 1);
     }
     const size_t es = dtype == LILY_BF16 ? 2 : 4;
-    // One launch per row: row j must see the counts of rows before it.
+    // Under penalties row j must see the counts of the rows before it: one launch per row.
+    // Without them the rows are independent and share one launch.
+    static_assert(LILY_MAX_VERIFY_ROWS <= (uint32_t)INLINE_ROWS, "verify rows travel inline");
+    const bool chained = lily_params_uses_penalties(params) != 0;
+    InlineRows rows;
     for (uint32_t j = 0; j < m; ++j) {
         const char* row = static_cast<const char*>(logits_dev) + (size_t)j * row_stride * es;
-        InlineRows rows;
         RowExtras x;
         lily_draft_dist slot;
         const bool spec = j + 1 < m && sampled;
@@ -972,12 +975,19 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
                 return rc;
             }
         }
-        if (int rc = pack_row(&rows.r[0], row, vocab, scratch, params, step0 + j,
+        if (int rc = pack_row(&rows.r[chained ? 0 : j], row, vocab, scratch, params, step0 + j,
                               spec ? MODE_SPEC : MODE_PLAIN, verify_tokens_dev + j,
                               spec ? &slot : nullptr, spec ? ids_dev + j + 1 : nullptr, x)) {
             return rc;
         }
-        if (int rc = launch_inline(s, dtype, vocab, rows, 1)) {
+        if (chained) {
+            if (int rc = launch_inline(s, dtype, vocab, rows, 1)) {
+                return rc;
+            }
+        }
+    }
+    if (!chained) {
+        if (int rc = launch_inline(s, dtype, vocab, rows, m)) {
             return rc;
         }
     }
