@@ -739,10 +739,10 @@ __device__ __forceinline__ float chunk_max(const u32x4& q) {
 
 // Signed 16-bit maximum of both halves of a and b.  bf16 patterns of values that are not
 // negative order like the values; every negative one is below all of them.
+typedef short s16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pk_max_i16(uint32_t a, uint32_t b) {
-    uint32_t r;
-    asm("v_pk_max_i16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return r;
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2, a),
+                                                                   __builtin_bit_cast(s16x2, b)));
 }
 
 // The largest element of one 16-byte chunk when that element is not negative, +0 otherwise:
@@ -752,9 +752,8 @@ template <int DT>
 __device__ __forceinline__ float chunk_max_nonneg(const u32x4& q) {
     if (DT == LILY_BF16) {
         const uint32_t r = pk_max_i16(pk_max_i16(q.x, q.y), pk_max_i16(q.z, q.w));
-        uint32_t m;
-        asm("v_max3_i32 %0, %1, %2, 0" : "=v"(m) : "v"(r << 16), "v"(r & 0xffff0000u));
-        return lilym_bits_f32(m);
+        const int m = max(max((int)(r << 16), (int)(r & 0xffff0000u)), 0);
+        return lilym_bits_f32((uint32_t)m);
     }
     return chunk_max<DT>(q);
 }
@@ -1821,19 +1820,24 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         float m8[U];
         float block_max = NEG_INF;
         if (nonneg) {
+            // No value here is below +0: their bit patterns order like integers, and such a
+            // pattern exceeds that of any negative value the lane's maximum may still hold.
+            int bm = 0;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 m8[u] = chunk_max_nonneg<DT>(cur[u]);
-                block_max = max2_raw(block_max, m8[u]);
+                bm = max(bm, (int)lilym_f32_bits(m8[u]));
             }
+            block_max = lilym_bits_f32((uint32_t)bm);
+            lane_max = lilym_bits_f32((uint32_t)max((int)lilym_f32_bits(lane_max), bm));
         } else {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 m8[u] = chunk_max<DT>(cur[u]);
                 block_max = max2_raw(block_max, m8[u]);
             }
+            lane_max = max2_raw(lane_max, block_max);
         }
-        lane_max = max2_raw(lane_max, block_max);
         if (LSE && want_lse) {
             // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
             // sum by more than 2^-21 of it, even with every element of the row at that level:
