@@ -1317,6 +1317,84 @@ __device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, 
 }
 
 
+// ------------------------------------------------------------------ sparse select
+//
+// Rows whose allow-mask admits few ids: the slice's allowed ids are listed from the mask
+// (two passes over its words: count, then place by an exclusive scan of the threads'
+// counts, so the order is the same in every run), each is evaluated exactly (bias,
+// penalties), adds its term to the row sum and becomes a candidate.  Nothing of the row is
+// streamed: the mask's words and one logit per allowed id are all that is read.  Returns
+// false, with nothing changed, when the slice admits more ids than `cap` candidates.
+template <int DT, bool LSE>
+__device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g, uint32_t k, uint64_t* cand,
+                                              uint32_t cap, Shared& sh, bool& sorted) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    const bool pen = (a.flags & F_PEN) != 0;
+    const uint32_t w_lo = g.id_lo >> 5, w_hi = (g.id_hi + 31u) >> 5;
+    auto word = [&](uint32_t i) -> uint32_t {
+        return gload(a.allow + i) & range32_at(g.id_lo, g.id_hi, (int64_t)i * 32);
+    };
+    uint32_t mine = 0;
+    for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
+        mine += (uint32_t)__popc(word(i));
+    }
+    // Exclusive scan of the threads' counts: inside the wave, then over the waves.
+    uint32_t incl = mine;
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t t = __shfl_up(incl, o);
+        if ((int)lane >= o) {
+            incl += t;
+        }
+    }
+    if (lane == 63u) {
+        sh.red_i[w] = incl;
+    }
+    __syncthreads();
+    uint32_t base = incl - mine, total = 0;
+    for (int i = 0; i < NWAVE; ++i) {
+        const uint32_t c = sh.red_i[i];
+        base += (uint32_t)i < w ? c : 0u;
+        total += c;
+    }
+    __syncthreads();
+    if (total > cap) {
+        return false;
+    }
+    for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
+        uint32_t bits = word(i);
+        while (bits != 0u) {
+            cand[base++] = (uint64_t)(i * 32u + (uint32_t)__builtin_ctz(bits));
+            bits &= bits - 1u;
+        }
+    }
+    __syncthreads();
+    LseAcc lse;
+    lse.init();
+    for (uint32_t i = tid; i < total; i += NT) {
+        const uint32_t id = (uint32_t)cand[i];
+        const float l = load_logit<DT>(a.logits, id);
+        const uint32_t c = pen ? gload(a.counts + id) : 0u;
+        const float u = finish_pre_temperature(a, id, l, c, true);
+        if (want_lse) {
+            lse.add_one(u, a.c2);
+        }
+        cand[i] = composite_of(u / a.temperature, id);  // 0 for -inf: dropped by the select
+    }
+    if (want_lse) {
+        lse_reduce(sh, lse);
+    } else {
+        __syncthreads();
+    }
+    sorted = false;
+    const uint32_t n = select_topk(cand, total, k, sh, sorted);
+    if (tid == 0) {
+        sh.n_cand = n;
+    }
+    __syncthreads();
+    return true;
+}
+
 // ------------------------------------------------------------------ streaming select
 //
 // The select of rows with k <= STREAM_K_MAX and no allow-mask.  One pass, one barrier per
@@ -2413,36 +2491,71 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         }
     }
     __syncthreads();
-    if (tid == 0) {
-        float total = 0.0f;
-        for (uint32_t i = 0; i < k; ++i) {
-            total += sh.prob[i];
-        }
-        const float limit = a.top_p * total;
-        float cum = 0.0f;
-        uint32_t kept = 0;
-        for (uint32_t rank = 0; rank < k; ++rank) {
-            const float p = sh.prob[rank];
-            if (rank > 0 && !(cum < limit && p >= a.min_p)) {
-                break;
+    // The reference's left-to-right f32 sums: one wave runs the chain of additions (64
+    // candidates at a time, a candidate per lane, every lane the same chain on values read
+    // lane by lane) and keeps every prefix.  The row total is the last prefix, and the sum
+    // the reference holds before rank r is the prefix of rank r - 1: the cut by top-p and
+    // min-p and the inverse-CDF pick then are searches every thread takes part in.
+    if (tid < 64u) {
+        float run = 0.0f;
+        for (uint32_t r0 = 0; r0 < k; r0 += 64u) {
+            const uint32_t i = r0 + tid;
+            const int pbits = (int)lilym_f32_bits(i < k ? sh.prob[i] : 0.0f);
+            float mine = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 64; ++j) {
+                run += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, j));
+                mine = tid == (uint32_t)j ? run : mine;
             }
-            cum += p;
-            sh.cum[rank] = cum;
-            ++kept;
-        }
-        sh.n_keep = kept;
-        sh.mass = cum;
-        sh.p_d = 0.0f;
-        sh.q_d = 0.0f;
-        if (a.dbg_counts) {
-            a.dbg_counts[0] = k;
-            a.dbg_counts[1] = kept;
+            if (i < k) {
+                sh.cum[i] = mine;
+            }
         }
     }
     __syncthreads();
-    const uint32_t n_keep = sh.n_keep;
-    const float mass = sh.mass;
+    auto first_of = [&](uint32_t mine_first) -> uint32_t {  // the lowest index any thread found
+        mine_first = wave_min_u32(mine_first);
+        if ((tid & 63u) == 0) {
+            sh.red_i[tid >> 6] = mine_first;
+        }
+        __syncthreads();
+        uint32_t r = sh.red_i[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            r = min(r, sh.red_i[i]);
+        }
+        __syncthreads();
+        return r;
+    };
+    const float limit = a.top_p * sh.cum[k - 1];
+    uint32_t stop = k;
+    for (uint32_t r = 1 + tid; r < k; r += NT) {
+        if (!(sh.cum[r - 1] < limit && sh.prob[r] >= a.min_p)) {
+            stop = min(stop, r);
+        }
+    }
+    if (tid == 0) {
+        sh.p_d = 0.0f;
+        sh.q_d = 0.0f;
+    }
+    const uint32_t n_keep = first_of(stop);
+    const float mass = sh.cum[n_keep - 1];
     const float u1 = (a.flags & F_UNIFORM) ? a.uniform : lilym_uniform_for(a.seed, step);
+    if (tid == 0) {
+        if (a.dbg_counts) {
+            a.dbg_counts[0] = k;
+            a.dbg_counts[1] = n_keep;
+        }
+    }
+    // First slot of cum[0..n) whose value exceeds target, else the last slot.
+    auto pick = [&](const float* prefix, uint32_t n, float target) -> uint32_t {
+        uint32_t hit = n - 1u;
+        for (uint32_t i = tid; i < n; i += NT) {
+            if (target < prefix[i]) {
+                hit = min(hit, i);
+            }
+        }
+        return first_of(hit);
+    };
 
     if (a.mode == MODE_DRAFT) {
         for (uint32_t i = tid; i < n_keep; i += NT) {
@@ -2455,8 +2568,8 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     }
 
     if (a.mode != MODE_SPEC) {
+        const uint32_t slot = pick(sh.cum, n_keep, u1 * mass);
         if (tid == 0) {
-            const uint32_t slot = pick_sequential(sh.cum, n_keep, u1 * mass);
             const uint32_t id = composite_id(cand[slot]);
             finish_token<DT>(a, sh, id, vocab);
         }
@@ -2610,19 +2723,9 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
     bool sorted = false;
     if (argmax) {
         best = slice_argmax<DT>(a, g, sh);
-    } else if (a.flags & F_FORCED) {
-        // Only the row's log-sum-exp is needed.
-        LseAcc lse;
-        lse.init();
-        for (uint32_t id = g.id_lo + tid; id < g.id_hi; id += NT) {
-            lse.add_one(pre_temperature_of<DT>(a, id), a.c2);
-        }
-        lse_reduce(sh, lse);
-        if (tid == 0) {
-            sh.n_cand = 0;
-        }
-        __syncthreads();
     } else {
+        // A forced row with a log-probability needs the row sum only: it takes the same
+        // selects (their sums are the fast ones) and its candidates are dropped below.
         bool done = false;
         uint32_t took = 2;
         if (cfg.path == 0u && (a.flags & F_STREAM)) {
@@ -2631,6 +2734,10 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
             if (!done) {
                 __syncthreads();
             }
+        }
+        if (KIND == 1 && !done && cfg.path == 0u && a.allow != nullptr) {
+            done = select_sparse<DT, LSE>(a, g, a.k, cand, min(cfg.dyn_slots, MERGE_CAP), sh, sorted);
+            took = done ? 1u : took;
         }
         if (KIND != 2 && !done && cfg.path != 1u && cfg.old_layout != 0u) {
             const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
@@ -2651,7 +2758,8 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         }
     }
 
-    uint32_t n = argmax ? 0u : min(sh.n_cand, cfg.cand_cap);
+    const bool forced = (a.flags & F_FORCED) != 0;
+    uint32_t n = (argmax || forced) ? 0u : min(sh.n_cand, cfg.cand_cap);
     phase(cfg, 4);
     if (S > 1) {
         const size_t slot = (size_t)row * S + s;
@@ -2663,7 +2771,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
             }
         } else {
             // Every slot is written (0 = no candidate), so the merge needs no counts.
-            for (uint32_t i = tid; i < cfg.ws_k; i += NT) {
+            for (uint32_t i = tid; !forced && i < cfg.ws_k; i += NT) {
                 store_through(&cfg.ws_cand[slot * cfg.ws_k + i], i < n ? cand[i] : (uint64_t)0);
             }
             if (tid == 0) {
@@ -2711,7 +2819,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
 #pragma unroll
             for (int q = 0; q < PER; ++q) {
                 const uint32_t j = tid + (uint32_t)q * NT;
-                mine[q] = j < slots ? load_through(&cfg.ws_cand[base * cfg.ws_k + j]) : 0ull;
+                mine[q] = (!forced && j < slots) ? load_through(&cfg.ws_cand[base * cfg.ws_k + j]) : 0ull;
             }
             if (want_lse && tid < 64) {
                 double mt = -__builtin_huge_val(), st = 0.0;
@@ -2958,7 +3066,9 @@ static hipError_t launch_variant(hipStream_t stream, uint32_t rows, const Launch
 }
 
 hipError_t launch_rows(hipStream_t stream, int dtype, int kind, bool lse, uint32_t rows,
-                       const LaunchCfg& cfg, const InlineRows* inline_rows, size_t dyn_bytes) {
+                       const LaunchCfg& cfg_in, const InlineRows* inline_rows, size_t dyn_bytes) {
+    LaunchCfg cfg = cfg_in;
+    cfg.dyn_slots = (uint32_t)(dyn_bytes / 8);
 #define LILY_DISPATCH(DT)                                                                     \
     switch (kind) {                                                                           \
         case 0:                                                                               \
