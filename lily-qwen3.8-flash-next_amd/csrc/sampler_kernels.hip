@@ -2258,8 +2258,78 @@ __device__ __forceinline__ void select_exhaustive(const RowArgs& a, uint32_t e0,
 
 // ------------------------------------------------------------------ sort
 
-// Descending sort of cand[0..n).  Up to 64 entries: one wave, in registers.
-// More: bitonic in LDS over the next power of two (the buffer holds it).
+// Descending bitonic sort of cand[0..n), n <= 4 * NT, four entries per thread (entry
+// 4 * tid + r in register r; absent entries are 0, the smallest).  Exchanges at distance
+// 1 and 2 stay inside a thread, 4 .. 128 are lane shuffles inside a wave, and only the
+// three at distance 256 and 512 go through LDS with a barrier.
+__device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
+    static_assert(NT == 256, "four entries per thread cover 1024");
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    uint64_t v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t i = tid * 4u + (uint32_t)r;
+        v[r] = i < n ? cand[i] : 0ull;
+    }
+    __syncthreads();
+    auto exchange = [](uint64_t& lo, uint64_t& hi, bool desc) {  // lo sits at the lower index
+        const bool swap = desc ? lo < hi : lo > hi;
+        const uint64_t t = lo;
+        lo = swap ? hi : lo;
+        hi = swap ? t : hi;
+    };
+    for (uint32_t size = 2; size <= 4u * NT; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            if (stride >= 4u * 64u) {
+                const uint32_t other = tid ^ (stride >> 2);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    cand[tid * 4u + (uint32_t)r] = v[r];
+                }
+                __syncthreads();
+                const bool desc = ((tid * 4u) & size) == 0;
+                const bool take_max = ((tid & (stride >> 2)) == 0) == desc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint64_t o = cand[other * 4u + (uint32_t)r];
+                    v[r] = take_max ? (o > v[r] ? o : v[r]) : (o < v[r] ? o : v[r]);
+                }
+                __syncthreads();
+            } else if (stride >= 4u) {
+                const uint32_t m = stride >> 2;
+                const bool desc = ((tid * 4u) & size) == 0;
+                const bool take_max = ((lane & m) == 0) == desc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint64_t o = shfl_xor_u64(v[r], (int)m);
+                    v[r] = take_max ? (o > v[r] ? o : v[r]) : (o < v[r] ? o : v[r]);
+                }
+            } else if (stride == 2u) {
+                const bool desc = ((tid * 4u) & size) == 0;  // size >= 4 here
+                exchange(v[0], v[2], desc);
+                exchange(v[1], v[3], desc);
+            } else {
+                if (size == 2u) {
+                    exchange(v[0], v[1], true);   // index bit 1 clear: descending
+                    exchange(v[2], v[3], false);  // set: ascending
+                } else {
+                    const bool desc = ((tid * 4u) & size) == 0;
+                    exchange(v[0], v[1], desc);
+                    exchange(v[2], v[3], desc);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        cand[tid * 4u + (uint32_t)r] = v[r];
+    }
+    __syncthreads();
+}
+
+// Descending sort of cand[0..n).  Up to 64 entries: one wave, in registers.  Up to 4 * NT:
+// four per thread in registers.  More: bitonic in LDS over the next power of two (the
+// buffer holds it).
 __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
     if (n <= 64) {
         if (threadIdx.x < 64) {
@@ -2277,6 +2347,10 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
             cand[lane] = c;
         }
         __syncthreads();
+        return;
+    }
+    if (n <= 4u * NT) {
+        sort_desc_regs(cand, n);
         return;
     }
     uint32_t p = 128;
@@ -2398,7 +2472,12 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
 // cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
 template <int DT>
 __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
-                     uint64_t* cand, Shared& sh) {
+                     uint64_t* cand, Shared& sh, const LaunchCfg& cfg) {
+#ifdef LILY_TAIL_TRACE
+#define TAIL_MARK(i) phase(cfg, i)
+#else
+#define TAIL_MARK(i)
+#endif
     const uint32_t tid = threadIdx.x;
     if (n == 0) {
         // No finite value anywhere: the oracle's order then starts at id 0.
@@ -2420,6 +2499,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     if (!sorted) {
         sort_desc(cand, n);
     }
+    TAIL_MARK(8);
     const uint32_t k = min(a.k, n);
     const float top = composite_value(cand[0]);
     if (k <= 64u && a.mode != MODE_SPEC) {
@@ -2491,28 +2571,36 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         }
     }
     __syncthreads();
-    // The reference's left-to-right f32 sums: one wave runs the chain of additions (64
-    // candidates at a time, a candidate per lane, every lane the same chain on values read
-    // lane by lane) and keeps every prefix.  The row total is the last prefix, and the sum
-    // the reference holds before rank r is the prefix of rank r - 1: the cut by top-p and
-    // min-p and the inverse-CDF pick then are searches every thread takes part in.
+    TAIL_MARK(9);
+    // The reference's left-to-right f32 sums: one wave runs the chain of additions, 64
+    // candidates at a time with a candidate per lane, and keeps every prefix.  Each step adds
+    // the lane's value to the running sum of the lane below (a shift by one lane across the
+    // whole wave; lane 0 has no lane below and keeps what it has): after step j the lanes up
+    // to j hold their final prefix, which further steps only reproduce.  The row total is
+    // the last prefix, and the sum the reference holds before rank r is the prefix of rank
+    // r - 1: the cut by top-p and min-p and the inverse-CDF pick then are searches every
+    // thread takes part in.
     if (tid < 64u) {
-        float run = 0.0f;
+        float carry = 0.0f;
         for (uint32_t r0 = 0; r0 < k; r0 += 64u) {
             const uint32_t i = r0 + tid;
-            const int pbits = (int)lilym_f32_bits(i < k ? sh.prob[i] : 0.0f);
-            float mine = 0.0f;
+            const float p = i < k ? sh.prob[i] : 0.0f;
+            float run = carry + p;  // final in lane 0
 #pragma unroll
-            for (int j = 0; j < 64; ++j) {
-                run += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, j));
-                mine = tid == (uint32_t)j ? run : mine;
+            for (int j = 1; j < 64; ++j) {
+                // Two idle cycles between a lane's write and the neighbour's read of it.
+                asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %1 wave_shr:1 row_mask:0xf bank_mask:0xf"
+                             : "+v"(run)
+                             : "v"(p));
             }
             if (i < k) {
-                sh.cum[i] = mine;
+                sh.cum[i] = run;
             }
+            carry = lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane((int)lilym_f32_bits(run), 63));
         }
     }
     __syncthreads();
+    TAIL_MARK(10);
     auto first_of = [&](uint32_t mine_first) -> uint32_t {  // the lowest index any thread found
         mine_first = wave_min_u32(mine_first);
         if ((tid & 63u) == 0) {
@@ -2539,6 +2627,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     }
     const uint32_t n_keep = first_of(stop);
     const float mass = sh.cum[n_keep - 1];
+    TAIL_MARK(11);
     const float u1 = (a.flags & F_UNIFORM) ? a.uniform : lilym_uniform_for(a.seed, step);
     if (tid == 0) {
         if (a.dbg_counts) {
@@ -2569,6 +2658,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
 
     if (a.mode != MODE_SPEC) {
         const uint32_t slot = pick(sh.cum, n_keep, u1 * mass);
+        TAIL_MARK(12);
         if (tid == 0) {
             const uint32_t id = composite_id(cand[slot]);
             finish_token<DT>(a, sh, id, vocab);
@@ -2888,7 +2978,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         }
         return;
     }
-    tail<DT>(a, vocab, step, n, sorted, cand, sh);
+    tail<DT>(a, vocab, step, n, sorted, cand, sh, cfg);
     phase(cfg, 7);
 }
 
