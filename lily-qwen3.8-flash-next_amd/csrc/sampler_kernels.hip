@@ -2273,7 +2273,7 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
     }
     __syncthreads();
     auto exchange = [](uint64_t& lo, uint64_t& hi, bool desc) {  // lo sits at the lower index
-        const bool swap = desc ? lo < hi : lo > hi;
+        const bool swap = (lo < hi) == desc;  // equal entries may swap: nothing changes
         const uint64_t t = lo;
         lo = swap ? hi : lo;
         hi = swap ? t : hi;
@@ -2292,7 +2292,7 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const uint64_t o = cand[other * 4u + (uint32_t)r];
-                    v[r] = take_max ? (o > v[r] ? o : v[r]) : (o < v[r] ? o : v[r]);
+                    v[r] = ((o > v[r]) == take_max) ? o : v[r];
                 }
                 __syncthreads();
             } else if (stride >= 4u) {
@@ -2302,7 +2302,7 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const uint64_t o = shfl_xor_u64(v[r], (int)m);
-                    v[r] = take_max ? (o > v[r] ? o : v[r]) : (o < v[r] ? o : v[r]);
+                    v[r] = ((o > v[r]) == take_max) ? o : v[r];
                 }
             } else if (stride == 2u) {
                 const bool desc = ((tid * 4u) & size) == 0;  // size >= 4 here
