@@ -2488,7 +2488,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             emit(a, 0);
             if (a.dbg_counts) {
                 a.dbg_counts[0] = 0;
-                a.dbg_counts[1] = 0;
+                a.dbg_counts[1] = 1;  // the reference keeps rank 0 whatever its value
             }
             if (a.mode == MODE_DRAFT) {
                 *a.q_n = 0;

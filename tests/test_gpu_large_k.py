@@ -1,0 +1,177 @@
+"""Rows outside the streaming select: k above 64 (the reference's default when top_k is 0
+is 1024), allow-masks served by the sparse select, and forced rows that want a
+log-probability.
+
+Bit-exact ids, candidates, probabilities and kept counts against the oracle; the
+log-probability within 1e-5 (relative, floor 1).  The 1024-candidate tail is the part under
+test for flat rows: its prefix sums must be the reference's left-to-right f32 sums, or the
+top-p cut and the pick move.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import lily_sampler as LS
+import lily_workloads as W
+import oracle as O
+from gpu_util import check_row_against_oracle, dev, o_params, run_rows
+
+
+@pytest.fixture(scope="module")
+def sampler():
+    s = LS.Sampler(0)
+    yield s
+    s.close()
+
+
+def _check_logprob(r, i, d, what):
+    if np.isfinite(d.logprob):
+        assert abs(r.logprobs[i] - d.logprob) <= 1e-5 * max(1.0, abs(d.logprob)), (what, i)
+    else:
+        assert r.logprobs[i] == -np.inf, (what, i)
+
+
+@pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
+def test_all_1024_candidates_kept(sampler, bf16):
+    """Flat rows with top_p 1 and min_p 0: every one of the 1024 candidates is kept, so the
+    pick depends on all 1024 sequential prefix sums (several uniforms per row, among them
+    draws at both ends)."""
+    rng = np.random.default_rng(31 + bf16)
+    rows, vocab = 6, 151_936
+    x = rng.normal(0, 0.05, (rows, vocab)).astype(np.float32)
+    x[1] = rng.integers(-2, 3, vocab) / 8.0          # heavy ties across the k-th place
+    x[2, :] = 0.25                                    # constant: ids decide
+    if bf16:
+        x = W.to_bf16_bits(x)
+    for trial, u in enumerate((None, 0.0, 0.999999, 0.5)):
+        kw = [dict(temperature=1.3, top_k=0, top_p=1.0, min_p=0.0, seed=900 + r) for r in range(rows)]
+        uniforms = None if u is None else [u] * rows
+        r = run_rows(sampler, x, kw, [trial] * rows, uniforms=uniforms, logprobs=True)
+        for i in range(rows):
+            d = O.sample(x[i], None, o_params(**kw[i]), trial, want_logprob=True,
+                         uniform=None if u is None else u)
+            check_row_against_oracle(r, i, d)
+            assert r.n_kept[i] == 1024
+            _check_logprob(r, i, d, ("kept-all", trial))
+
+
+def test_top_k_between_65_and_1024(sampler):
+    """k just above the streaming select's limit, odd sizes, and k above the number of
+    finite values."""
+    rng = np.random.default_rng(32)
+    rows, vocab = 8, 50_021
+    x = rng.standard_t(4, (rows, vocab)).astype(np.float32) * 2
+    x[3, rng.random(vocab) < 0.995] = -np.inf        # ~250 finite values < k
+    for trial, k in enumerate((65, 100, 257, 513, 1000, 1023)):
+        kw = [dict(temperature=0.9, top_k=k, top_p=0.97, min_p=1e-4, seed=40 + r) for r in range(rows)]
+        r = run_rows(sampler, x, kw, [trial] * rows, logprobs=True)
+        for i in range(rows):
+            d = O.sample(x[i], None, o_params(**kw[i]), trial, want_logprob=True)
+            check_row_against_oracle(r, i, d)
+            _check_logprob(r, i, d, ("k", k))
+
+
+@pytest.mark.parametrize("slices", [0, 1], ids=["auto-slices", "one-slice"])
+def test_masks_of_every_density_report_their_select(slices):
+    """Sparse masks are served from the mask's words (no row is streamed), dense ones by the
+    bitmap select (with one workgroup per row the 5 % and 60 % masks admit more ids than the
+    workgroup holds); both agree with the oracle."""
+    old = os.environ.get("LILY_SAMPLER_SLICES")
+    os.environ["LILY_SAMPLER_SLICES"] = str(slices)
+    try:
+        s = LS.Sampler(0)
+    finally:
+        if old is None:
+            os.environ.pop("LILY_SAMPLER_SLICES", None)
+        else:
+            os.environ["LILY_SAMPLER_SLICES"] = old
+    rng = np.random.default_rng(33)
+    vocab = 151_936
+    fracs = (0.0, 0.0002, 0.02, 0.02, 0.05, 0.6)
+    rows = len(fracs)
+    x = W.to_bf16_bits(rng.normal(0, 2, (rows, vocab)).astype(np.float32))
+    masks = np.stack([W.allow_mask(rng, vocab, frac=max(f, 1e-5)) for f in fracs])
+    masks[0] = 0                                      # nothing allowed: id 0, log-probability -inf
+    bias = [[(int(i), float(d)) for i, d in zip(rng.integers(0, vocab, 32),
+                                                 rng.choice([-5.0, 5.0], 32))] for _ in range(rows)]
+    hist = rng.integers(0, vocab, (rows, 2000)).astype(np.int32)
+    sc = []
+    counts = []
+    for r_ in range(rows):
+        t = LS.SamplerScratch(s, vocab)
+        t.add_history(torch.from_numpy(hist[r_]).to(dev()))
+        sc.append(t)
+        counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    for trial, k in enumerate((0, 300, 40)):
+        kw = [dict(temperature=0.8, top_k=k, top_p=0.9, seed=60 + r_, repetition_penalty=1.1,
+                   presence_penalty=0.3, frequency_penalty=0.1) for r_ in range(rows)]
+        s.set_path_stats(stats)
+        r = run_rows(s, x, kw, [trial] * rows, scratch=sc, allow=masks, bias=bias, logprobs=True)
+        s.set_path_stats(None)
+        st = stats.cpu().tolist()
+        assert st[0] == 0, st                         # masked rows: never the streaming select
+        if slices == 0:
+            assert st[2] == 0, st                     # and with several slices never the exhaustive one
+        for i in range(rows):
+            d = O.sample(x[i], counts[i], o_params(**kw[i]), trial, allow=masks[i], bias=bias[i],
+                         want_logprob=True)
+            check_row_against_oracle(r, i, d)
+            if fracs[i] > 0:
+                assert (masks[i][r.ids[i] >> 5] >> (r.ids[i] & 31)) & 1
+            _check_logprob(r, i, d, ("mask", fracs[i], k))
+        stats.zero_()
+    for t in sc:
+        t.close()
+    s.close()
+
+
+@pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
+def test_forced_rows_with_a_log_probability(sampler, bf16):
+    """A forced id consumes no draw; its log-probability is that of the full row
+    (penalised, biased, masked), whichever select computed the row sum."""
+    rng = np.random.default_rng(34 + bf16)
+    rows, vocab = 8, 151_936
+    x = rng.normal(0, 2, (rows, vocab)).astype(np.float32)
+    if bf16:
+        x = W.to_bf16_bits(x)
+    hist = rng.integers(0, vocab, (rows, 1500)).astype(np.int32)
+    forced = [int(hist[r, 0]) if r % 2 else int(rng.integers(0, vocab)) for r in range(rows)]
+    forced[5] = None                                  # an ordinary row among them
+    masks = np.stack([W.allow_mask(rng, vocab, frac=0.03) for _ in range(rows)])
+    for variant in ("plain", "penalised", "masked"):
+        for k in (20, 0):
+            sc, counts = None, [None] * rows
+            pen = dict()
+            if variant == "penalised":
+                pen = dict(repetition_penalty=1.2, presence_penalty=0.4, frequency_penalty=0.1)
+                sc = []
+                counts = []
+                for r_ in range(rows):
+                    t = LS.SamplerScratch(sampler, vocab)
+                    t.add_history(torch.from_numpy(hist[r_]).to(dev()))
+                    sc.append(t)
+                    counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
+            allow = masks if variant == "masked" else None
+            kw = [dict(temperature=0.7, top_k=k, top_p=0.9, seed=80 + r_, **pen) for r_ in range(rows)]
+            r = run_rows(sampler, x, kw, [3] * rows, scratch=sc, allow=allow, forced=forced,
+                         logprobs=True)
+            for i in range(rows):
+                ext = dict(want_logprob=True)
+                if allow is not None:
+                    ext["allow"] = masks[i]
+                d = O.sample(x[i], counts[i], o_params(**kw[i]), 3, forced=forced[i], **ext)
+                if forced[i] is not None:
+                    assert r.ids[i] == forced[i]
+                else:
+                    check_row_against_oracle(r, i, d)
+                _check_logprob(r, i, d, (variant, k))
+            if sc is not None:
+                for i in range(rows):
+                    assert np.array_equal(sc[i].read_counts().numpy().view(np.uint32), counts[i])
+                for t in sc:
+                    t.close()
