@@ -356,8 +356,40 @@ __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, u
         prefix |= (uint64_t)sh.sel_bin << shift;
         pmask |= (uint64_t)255u << shift;
         const bool whole_bin = sh.bin_count == sh.need;
+        const uint32_t in_bin = sh.bin_count;
         need = sh.need;
         if (whole_bin) {
+            break;
+        }
+        if (in_bin <= 128u) {
+            // Few entries left (rows of bf16 logits tie by the dozen at the k-th value and
+            // would take every remaining pass to split by id): rank them against each
+            // other; the one with `need - 1` above it is the k-th entry itself.
+            uint64_t* left = reinterpret_cast<uint64_t*>(sh.hist);  // free after find_bin
+            if (tid == 0) {
+                sh.n_cand = 0;
+            }
+            __syncthreads();
+            for (uint32_t i = tid; i < n; i += NT) {
+                const uint64_t c = cand[i];
+                if (c != 0 && (c & pmask) == prefix) {
+                    left[atomicAdd(&sh.n_cand, 1u)] = c;
+                }
+            }
+            __syncthreads();
+            if (tid < in_bin) {
+                const uint64_t me = left[tid];
+                uint32_t above = 0;
+                for (uint32_t j = 0; j < in_bin; ++j) {
+                    above += left[j] > me ? 1u : 0u;
+                }
+                if (above == need - 1u) {
+                    sh.red_u[0] = me;
+                }
+            }
+            __syncthreads();
+            prefix = sh.red_u[0];
+            __syncthreads();
             break;
         }
     }
