@@ -1360,6 +1360,7 @@ __device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, 
 template <int DT, bool LSE>
 __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g, uint32_t k, uint64_t* cand,
                                               uint32_t cap, Shared& sh, bool& sorted) {
+    static_assert(STREAM_BIAS_CAP <= NT, "one thread stages one bias entry");
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const bool want_lse = LSE && a.out_logprob != nullptr;
     const bool pen = (a.flags & F_PEN) != 0;
@@ -1367,6 +1368,17 @@ __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g
     auto word = [&](uint32_t i) -> uint32_t {
         return gload(a.allow + i) & range32_at(g.id_lo, g.id_hi, (int64_t)i * 32);
     };
+    // A short bias list is kept in the last slots of the buffer (id, delta) and walked from
+    // there for every candidate; a longer one is read from memory.
+    const uint32_t n_bias = a.n_bias;
+    const bool bias_lds = n_bias != 0 && n_bias <= STREAM_BIAS_CAP && cap > 2u * STREAM_BIAS_CAP;
+    if (bias_lds) {
+        cap -= STREAM_BIAS_CAP;
+        if (tid < n_bias) {
+            cand[cap + tid] = ((uint64_t)lilym_f32_bits(gload(&a.bias[tid].delta)) << 32) |
+                              gload(&a.bias[tid].id);
+        }
+    }
     uint32_t mine = 0;
     for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
         mine += (uint32_t)__popc(word(i));
@@ -1405,9 +1417,24 @@ __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g
     lse.init();
     for (uint32_t i = tid; i < total; i += NT) {
         const uint32_t id = (uint32_t)cand[i];
-        const float l = load_logit<DT>(a.logits, id);
+        float l = load_logit<DT>(a.logits, id);
         const uint32_t c = pen ? gload(a.counts + id) : 0u;
-        const float u = finish_pre_temperature(a, id, l, c, true);
+        float u;
+        if (bias_lds) {
+            for (uint32_t j = 0; j < n_bias; ++j) {
+                const uint64_t e = cand[cap + j];
+                if ((uint32_t)e == id) {
+                    l += lilym_bits_f32((uint32_t)(e >> 32));
+                }
+            }
+            if (c > 0u) {
+                l = l > 0.0f ? l / a.repetition : l * a.repetition;
+                l -= a.presence + a.frequency * (float)c;
+            }
+            u = l;
+        } else {
+            u = finish_pre_temperature(a, id, l, c, true);
+        }
         if (want_lse) {
             lse.add_one(u, a.c2);
         }
