@@ -1874,16 +1874,26 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             const uint32_t id = r.ent & ID_MASK;
             const uint32_t c = (id + g.pad) / E;
             r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (size_t)c * 16));
-            r.raw = load_logit<DT>(a.logits, id);
         }
+    };
+    // The id's own logit out of its chunk (one gather per listed id, not two).
+    auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
+        const uint32_t j = (id + g.pad) % E;
+        const uint32_t w4 = E == 8 ? j >> 1 : j;
+        const uint32_t d = w4 == 0u ? q.x : (w4 == 1u ? q.y : (w4 == 2u ? q.z : q.w));
+        if (E == 8) {
+            return lilym_bits_f32((j & 1u) ? (d & 0xffff0000u) : (d << 16));
+        }
+        return lilym_bits_f32(d);
     };
     // A listed id's true value before the temperature (bias in list order, then penalties);
     // also feeds the thread's maxima of listed raw and true values.
-    auto listed_value = [&](const Listed& r) -> float {
+    auto listed_value = [&](Listed& r) -> float {
         if (r.ent == NONE) {
             return NEG_INF;
         }
         const uint32_t id = r.ent & ID_MASK;
+        r.raw = raw_of(r.chunk, id);
         uint32_t cnt = r.ent >> SPEC_ID_BITS;
         if (cnt == 4095u) {
             cnt = gload(a.counts + id);
@@ -1944,7 +1954,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     lst_a.ent = NONE;
     lst_b.ent = NONE;
     lst_c.ent = NONE;
-    auto work = [&](const u32x4 (&cur)[U], const Listed& lcur, uint32_t b) {
+    auto work = [&](const u32x4 (&cur)[U], Listed& lcur, uint32_t b) {
         const float lcur_t = listed_row ? listed_value(lcur) : NEG_INF;
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
