@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--rows", type=int, default=1024)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip configurations 1, 3 and 4 (profiles of the two headline launches)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device copy (a known-size kernel that counter runs "
                          "under rocprofv3 --pmc are scaled by)")
@@ -164,54 +166,55 @@ def main():
 
     # ---- the other BASELINE configurations, for the record (latency-bound launches)
     others = {}
-    n_lat, w_lat = max(a.steps, 100), max(a.warmup, 10)
-    c1 = W.config1()
-    l1 = torch.from_numpy(c1["logits"]).to(device)
-    o1 = torch.zeros(1, dtype=torch.int32, device=device)
-    for name, kw in (("config1_greedy", dict()), ("config1_sampled", c1["params"])):
+    if not a.no_others:
+        n_lat, w_lat = max(a.steps, 100), max(a.warmup, 10)
+        c1 = W.config1()
+        l1 = torch.from_numpy(c1["logits"]).to(device)
+        o1 = torch.zeros(1, dtype=torch.int32, device=device)
+        for name, kw in (("config1_greedy", dict()), ("config1_sampled", c1["params"])):
+            torch.cuda.synchronize()
+            p1 = sampler.plan(l1, [LS.SamplingParams.greedy(**kw)], [0], o1)
+            others[name] = {"us_per_step": time_steps(stream, lambda i: p1.run(i), n_lat, w_lat) * 1e3}
+            p1.close()
+        c3 = W.config3()
+        m3 = c3["target"].shape[0]
+        t3 = torch.from_numpy(c3["target"]).to(device)
+        d3 = torch.from_numpy(c3["draft"]).to(device)
+        for name, kw in (("config3_verify_greedy", dict()), ("config3_verify_sampled", c3["params"])):
+            lp3 = LS.SamplingParams.greedy(**kw)
+            sc3 = LS.SamplerScratch(sampler, vocab)
+            dists = LS.DraftDists(sampler, m3)
+            props = torch.zeros(m3, dtype=torch.int32, device=device)
+            torch.cuda.synchronize()
+            for j in range(m3 - 1):
+                sampler.sample_draft_f32(d3[j], sc3, LS.draft_params(lp3), LS.draft_step(j),
+                                         props[j:j + 1], dists.slot(j))
+            sampler.synchronize()
+            ids3 = torch.cat([torch.tensor([42], dtype=torch.int32, device=device), props[:m3 - 1]])
+            ver = torch.zeros(m3, dtype=torch.int32, device=device)
+            ctrl = torch.zeros(LS.ctrl_words(2), dtype=torch.int32, device=device)
+            torch.cuda.synchronize()
+            us = time_steps(stream, lambda i: sampler.spec_verify(t3, sc3, lp3, i, dists, ids3, ver, ctrl,
+                                                                  pos0=100, ratio=4, chain=2),
+                            n_lat, w_lat) * 1e3
+            others[name] = {"us_per_step": us, "rows": m3}
+            sampler.synchronize()
+            sc3.close()
+            dists.close()
+        c4 = W.config4(rows=64)
+        l4 = torch.from_numpy(c4["logits"].view(np.int16)).to(device).view(torch.bfloat16)
+        o4 = torch.zeros(64, dtype=torch.int32, device=device)
+        lp4 = torch.zeros(64, dtype=torch.float32, device=device)
+        allow4 = torch.from_numpy(np.ascontiguousarray(c4["allow"]).view(np.int32)).to(device)
         torch.cuda.synchronize()
-        p1 = sampler.plan(l1, [LS.SamplingParams.greedy(**kw)], [0], o1)
-        others[name] = {"us_per_step": time_steps(stream, lambda i: p1.run(i), n_lat, w_lat) * 1e3}
-        p1.close()
-    c3 = W.config3()
-    m3 = c3["target"].shape[0]
-    t3 = torch.from_numpy(c3["target"]).to(device)
-    d3 = torch.from_numpy(c3["draft"]).to(device)
-    for name, kw in (("config3_verify_greedy", dict()), ("config3_verify_sampled", c3["params"])):
-        lp3 = LS.SamplingParams.greedy(**kw)
-        sc3 = LS.SamplerScratch(sampler, vocab)
-        dists = LS.DraftDists(sampler, m3)
-        props = torch.zeros(m3, dtype=torch.int32, device=device)
-        torch.cuda.synchronize()
-        for j in range(m3 - 1):
-            sampler.sample_draft_f32(d3[j], sc3, LS.draft_params(lp3), LS.draft_step(j),
-                                     props[j:j + 1], dists.slot(j))
-        sampler.synchronize()
-        ids3 = torch.cat([torch.tensor([42], dtype=torch.int32, device=device), props[:m3 - 1]])
-        ver = torch.zeros(m3, dtype=torch.int32, device=device)
-        ctrl = torch.zeros(LS.ctrl_words(2), dtype=torch.int32, device=device)
-        torch.cuda.synchronize()
-        us = time_steps(stream, lambda i: sampler.spec_verify(t3, sc3, lp3, i, dists, ids3, ver, ctrl,
-                                                              pos0=100, ratio=4, chain=2),
-                        n_lat, w_lat) * 1e3
-        others[name] = {"us_per_step": us, "rows": m3}
-        sampler.synchronize()
-        sc3.close()
-        dists.close()
-    c4 = W.config4(rows=64)
-    l4 = torch.from_numpy(c4["logits"].view(np.int16)).to(device).view(torch.bfloat16)
-    o4 = torch.zeros(64, dtype=torch.int32, device=device)
-    lp4 = torch.zeros(64, dtype=torch.float32, device=device)
-    allow4 = torch.from_numpy(np.ascontiguousarray(c4["allow"]).view(np.int32)).to(device)
-    torch.cuda.synchronize()
-    p4 = sampler.plan(l4, [LS.SamplingParams.greedy(**kw) for kw in c4["params"]], [7] * 64, o4,
-                      allow=allow4, bias=c4["bias"], forced=c4["forced"], out_logprobs=lp4)
-    us4 = time_steps(stream, lambda i: p4.run(i), n_lat, w_lat) * 1e3
-    bytes4 = 64 * W.algorithmic_bytes_per_row(vocab, 2, mask_words=c4["allow"].shape[1], bias_pairs=32,
-                                              logprob=True)
-    others["config4_constrained"] = {"us_per_step": us4, "rows": 64,
-                                     "achieved_GBs": bytes4 / (us4 * 1e-6) / 1e9}
-    p4.close()
+        p4 = sampler.plan(l4, [LS.SamplingParams.greedy(**kw) for kw in c4["params"]], [7] * 64, o4,
+                          allow=allow4, bias=c4["bias"], forced=c4["forced"], out_logprobs=lp4)
+        us4 = time_steps(stream, lambda i: p4.run(i), n_lat, w_lat) * 1e3
+        bytes4 = 64 * W.algorithmic_bytes_per_row(vocab, 2, mask_words=c4["allow"].shape[1], bias_pairs=32,
+                                                  logprob=True)
+        others["config4_constrained"] = {"us_per_step": us4, "rows": 64,
+                                         "achieved_GBs": bytes4 / (us4 * 1e-6) / 1e9}
+        p4.close()
 
     line = {
         "metric": "rows/s and us/step at B=4 and B=1024 x151,936 vocab; achieved HBM GB/s",

@@ -2347,8 +2347,11 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
         lo = swap ? hi : lo;
         hi = swap ? t : hi;
     };
-    for (uint32_t size = 2; size <= 4u * NT; size <<= 1) {
-        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+#pragma unroll
+    for (int lsize = 1; lsize <= 10; ++lsize) {
+#pragma unroll
+        for (int lstride = lsize - 1; lstride >= 0; --lstride) {
+            const uint32_t size = 1u << lsize, stride = 1u << lstride;
             if (stride >= 4u * 64u) {
                 const uint32_t other = tid ^ (stride >> 2);
 #pragma unroll
