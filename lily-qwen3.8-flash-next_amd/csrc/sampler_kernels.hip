@@ -332,6 +332,14 @@ __device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
 // returns how many there are.
 __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
     const uint32_t tid = threadIdx.x;
+    constexpr int PER = MERGE_CAP / NT;  // n <= MERGE_CAP
+    // Every pass works on the thread's own entries, read from LDS once.
+    uint64_t mine[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const uint32_t i = tid + (uint32_t)j * NT;
+        mine[j] = i < n ? cand[i] : 0ull;
+    }
     uint64_t prefix = 0, pmask = 0;
     uint32_t need = k;
     bool all = false;
@@ -341,10 +349,10 @@ __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, u
             sh.hist[tid] = 0;
         }
         __syncthreads();
-        for (uint32_t i = tid; i < n; i += NT) {
-            const uint64_t c = cand[i];
-            if (c != 0 && (c & pmask) == prefix) {
-                atomicAdd(&sh.hist[(uint32_t)(c >> shift) & 255u], 1u);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            if (mine[j] != 0 && (mine[j] & pmask) == prefix) {
+                atomicAdd(&sh.hist[(uint32_t)(mine[j] >> shift) & 255u], 1u);
             }
         }
         __syncthreads();
@@ -370,10 +378,10 @@ __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, u
                 sh.n_cand = 0;
             }
             __syncthreads();
-            for (uint32_t i = tid; i < n; i += NT) {
-                const uint64_t c = cand[i];
-                if (c != 0 && (c & pmask) == prefix) {
-                    left[atomicAdd(&sh.n_cand, 1u)] = c;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                if (mine[j] != 0 && (mine[j] & pmask) == prefix) {
+                    left[atomicAdd(&sh.n_cand, 1u)] = mine[j];
                 }
             }
             __syncthreads();
@@ -394,16 +402,11 @@ __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, u
         }
     }
     const uint64_t floor_c = all ? 1ull : prefix;
-    constexpr int PER = MERGE_CAP / NT;  // n <= MERGE_CAP
-    uint64_t mine[PER];
-    for (int j = 0; j < PER; ++j) {
-        const uint32_t i = tid + (uint32_t)j * NT;
-        mine[j] = i < n ? cand[i] : 0ull;
-    }
     if (tid == 0) {
         sh.n_cand = 0;
     }
     __syncthreads();
+#pragma unroll
     for (int j = 0; j < PER; ++j) {
         if (mine[j] != 0 && mine[j] >= floor_c) {
             cand[atomicAdd(&sh.n_cand, 1u)] = mine[j];
