@@ -2405,6 +2405,8 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
 // Descending sort of cand[0..n).  Up to 64 entries: one wave, in registers.  Up to 4 * NT:
 // four per thread in registers.  More: bitonic in LDS over the next power of two (the
 // buffer holds it).
+// BIG = false leaves the register sort out (kernels whose rows never sort more than 64).
+template <bool BIG>
 __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
     if (n <= 64) {
         if (threadIdx.x < 64) {
@@ -2424,7 +2426,7 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
         __syncthreads();
         return;
     }
-    if (n <= 4u * NT) {
+    if (BIG && n <= 4u * NT) {
         sort_desc_regs(cand, n);
         return;
     }
@@ -2545,7 +2547,7 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
 }
 
 // cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
-template <int DT>
+template <int DT, bool BIG>
 __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
                      uint64_t* cand, Shared& sh, const LaunchCfg& cfg) {
 #ifdef LILY_TAIL_TRACE
@@ -2572,7 +2574,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         return;
     }
     if (!sorted) {
-        sort_desc(cand, n);
+        sort_desc<BIG>(cand, n);
     }
     TAIL_MARK(8);
     const uint32_t k = min(a.k, n);
@@ -3053,7 +3055,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         }
         return;
     }
-    tail<DT>(a, vocab, step, n, sorted, cand, sh, cfg);
+    tail<DT, KIND != 2>(a, vocab, step, n, sorted, cand, sh, cfg);
     phase(cfg, 7);
 }
 
