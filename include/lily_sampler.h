@@ -121,11 +121,12 @@ int lily_sampler_synchronize(lily_sampler_t* s);
 int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_t capacity_words);
 /* Diagnostics with no counterpart in the reference: while stats_dev (device, u32[4], cleared by
  * the caller) is set, every workgroup of a sampled row adds 1 to [0] when the streaming select
- * (k <= 64, no allow-mask) produced its slice, [1] for the bitmap select, [2] for the
- * exhaustive select.  NULL stops. */
+ * (k <= 64, no allow-mask) produced its slice, [1] for the selects of masked rows and of
+ * k > 64 (sparse or bitmap), [2] for the exhaustive select.  NULL stops. */
 int lily_sampler_set_path_stats(lily_sampler_t* s, uint32_t* stats_dev);
 /* Workgroups per row the next launch of `rows` rows with candidate count k would use. */
-uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab);
+uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab,
+                                 lily_dtype dtype);
 
 /* ---- SamplerScratch ------------------------------------------------------------------- */
 

@@ -267,12 +267,18 @@ uint32_t slices_for_list(uint32_t listed) {
 // `listed`: the longest list of penalised ids among the rows (0 = none): a workgroup buckets
 // at most SPEC_CAP of them, so long lists are spread over more slices.
 uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab,
-                       uint32_t listed = 0) {
+                       int dtype, uint32_t listed = 0) {
     if (rows > WS_ROWS) {
         return 1;
     }
     uint32_t sl = s->force_slices ? s->force_slices : (TARGET_GROUPS + rows - 1) / rows;
     if (!s->force_slices) {
+        // No finer than one block of 256 x 4 chunks per slice: below that a slice saves no
+        // time and every further workgroup costs the merge a partial to gather.
+        const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
+        const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
+        const uint32_t by_block = (nch + 256u * STREAM_UNROLL - 1) / (256u * STREAM_UNROLL);
+        sl = sl > by_block ? by_block : sl;
         const uint32_t by_list = slices_for_list(listed);
         sl = sl < by_list ? by_list : sl;
     }
@@ -382,7 +388,7 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     HIP_TRY(hipSetDevice(s->device));
     const uint32_t kmax = max_k(rows.r, n);
     LaunchCfg cfg;
-    const uint32_t slices = choose_slices(s, n, kmax, vocab, longest_list(rows.r, n));
+    const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype, longest_list(rows.r, n));
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
     attach_trace(s, &cfg, n);
     const LaunchShape shp = shape_of(s, rows.r, n, dtype, vocab, slices, kmax);
@@ -666,11 +672,12 @@ int lily_sampler_set_path_stats(lily_sampler_t* s, uint32_t* stats_dev) {
     return LILY_OK;
 }
 
-uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab) {
+uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab,
+                                 lily_dtype dtype) {
     if (s == nullptr || rows == 0) {
         return 0;
     }
-    return choose_slices(s, rows, k ? k : 1, vocab);
+    return choose_slices(s, rows, k ? k : 1, vocab, (int)dtype);
 }
 
 int lily_sampler_synchronize(lily_sampler_t* s) {
@@ -1033,7 +1040,7 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     const uint32_t kmax = max_k(s->stage[slot], b->rows);
     LaunchCfg cfg;
     const uint32_t slices =
-        choose_slices(s, b->rows, kmax, b->vocab, longest_list(s->stage[slot], b->rows));
+        choose_slices(s, b->rows, kmax, b->vocab, (int)b->dtype, longest_list(s->stage[slot], b->rows));
     fill_cfg(s, &cfg, b->vocab, slices, kmax, 0, s->table_dev);
     attach_trace(s, &cfg, b->rows);
     const LaunchShape shp =
@@ -1098,7 +1105,7 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->dtype = b->dtype;
     p->ws_k = max_k(table.data(), b->rows);
     p->listed = longest_list(table.data(), b->rows);
-    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab, p->listed);
+    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab, (int)b->dtype, p->listed);
     const LaunchShape shp = shape_of(p->s, table.data(), b->rows, (int)b->dtype, b->vocab,
                                      p->slices, p->ws_k);
     p->kind = shp.kind();

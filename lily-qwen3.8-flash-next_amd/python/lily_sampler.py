@@ -109,7 +109,7 @@ def _load():
         getattr(L, n).restype = C.c_uint32
         getattr(L, n).argtypes = [C.c_uint32]
     L.lily_sampler_slices_for.restype = C.c_uint32
-    L.lily_sampler_slices_for.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32]
+    L.lily_sampler_slices_for.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int]
     L.lily_scratch_vocab.restype = C.c_uint32
     L.lily_scratch_vocab.argtypes = [C.c_void_p]
     vp, u32, u64 = C.c_void_p, C.c_uint32, C.c_uint64
@@ -244,8 +244,8 @@ class Sampler:
         _check(_lib.lily_sampler_set_path_stats(
             self._h, _ptr(stats, torch.int32) if stats is not None else None))
 
-    def slices_for(self, rows, k, vocab):
-        return int(_lib.lily_sampler_slices_for(self._h, rows, k, vocab))
+    def slices_for(self, rows, k, vocab, bf16=False):
+        return int(_lib.lily_sampler_slices_for(self._h, rows, k, vocab, 1 if bf16 else 0))
 
     def synchronize(self):
         """ComputePass::commit_wait."""

@@ -67,7 +67,7 @@ def test_the_streaming_select_serves_the_throughput_shape(sampler):
     finally:
         sampler.set_path_stats(None)
     st = stats.cpu().tolist()
-    assert st[0] == 16 * sampler.slices_for(16, 64, vocab) and st[1] == 0 and st[2] == 0, st
+    assert st[0] == 16 * sampler.slices_for(16, 64, vocab, bf16=True) and st[1] == 0 and st[2] == 0, st
     for i in range(16):
         d = O.sample(c["logits"][i], counts[i], o_params(**c["params"][i]), 2, want_logprob=True)
         check_row_against_oracle(r, i, d)
