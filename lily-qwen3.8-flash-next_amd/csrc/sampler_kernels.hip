@@ -1560,7 +1560,7 @@ __device__ __forceinline__ bool stream_fail(const LaunchCfg& cfg, uint32_t why) 
 
 template <int DT, bool LSE>
 __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g, uint32_t k, Shared& sh,
-                                              const LaunchCfg& cfg, bool& sorted) {
+                                              const LaunchCfg& cfg, bool& sorted, uint64_t*& out) {
     constexpr int E = Geo<DT>::E;
     constexpr int U = STREAM_UNROLL;
     constexpr uint32_t BLOCK = NT * U;
@@ -2247,20 +2247,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             return stream_fail(cfg, 6u);
         }
     }
-    // The caller and the tail expect the candidates at the start of dynamic LDS.
-    uint64_t* cand = dyn_lds;
-    uint64_t keep[(STREAM_K_MAX + NT - 1) / NT];
-    for (uint32_t q = 0; q * NT < STREAM_K_MAX; ++q) {
-        const uint32_t i = q * NT + tid;
-        keep[q] = i < n ? L.fc[i] : 0ull;
-    }
-    __syncthreads();
-    for (uint32_t q = 0; q * NT < STREAM_K_MAX; ++q) {
-        const uint32_t i = q * NT + tid;
-        if (i < n) {
-            cand[i] = keep[q];
-        }
-    }
+    // The candidates stay where they are (the tail's arrays and the merge's buffer lie below
+    // them in dynamic LDS).
+    out = L.fc;
     if (tid == 0) {
         sh.n_cand = n;
     }
@@ -2872,6 +2861,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
     const uint32_t step = a.step + cfg.step_delta;
     const bool want_lse = LSE && a.out_logprob != nullptr;
     uint64_t* cand = dyn_lds;
+    uint64_t* found = cand;  // where the select left the slice's candidates
     uint32_t* excl = reinterpret_cast<uint32_t*>(dyn_lds + cfg.cand_cap);
 
     if ((a.flags & F_FORCED) && !want_lse) {
@@ -2896,7 +2886,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         bool done = false;
         uint32_t took = 2;
         if (cfg.path == 0u && (a.flags & F_STREAM)) {
-            done = select_stream<DT, LSE>(a, g, a.k, sh, cfg, sorted);
+            done = select_stream<DT, LSE>(a, g, a.k, sh, cfg, sorted, found);
             took = done ? 0u : took;
             if (!done) {
                 __syncthreads();
@@ -2939,7 +2929,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         } else {
             // Every slot is written (0 = no candidate), so the merge needs no counts.
             for (uint32_t i = tid; !forced && i < cfg.ws_k; i += NT) {
-                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], i < n ? cand[i] : (uint64_t)0);
+                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], i < n ? found[i] : (uint64_t)0);
             }
             if (tid == 0) {
                 store_through(&cfg.ws_lse[2 * slot], want_lse ? sh.lse_mc : 0.0);
@@ -3038,6 +3028,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
             n = sh.n_cand;
             sorted = false;
             n = select_topk(cand, n, a.k, sh, sorted);
+            found = cand;
         }
     }
 
@@ -3055,7 +3046,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         }
         return;
     }
-    tail<DT, KIND != 2>(a, vocab, step, n, sorted, cand, sh, cfg);
+    tail<DT, KIND != 2>(a, vocab, step, n, sorted, found, sh, cfg);
     phase(cfg, 7);
 }
 
