@@ -2229,19 +2229,24 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // map such a value to.
     if (filt > F32_LOWEST) {
         uint32_t lowest = 0xffffffffu;
-        for (uint32_t i = tid; i < n; i += NT) {
-            lowest = min(lowest, (uint32_t)(L.fc[i] >> 32));
+        if (sorted) {
+            // Ranked candidates are in descending order: the last one is the lowest.
+            lowest = n > 0u ? (uint32_t)(L.fc[n - 1u] >> 32) : lowest;
+        } else {
+            for (uint32_t i = tid; i < n; i += NT) {
+                lowest = min(lowest, (uint32_t)(L.fc[i] >> 32));
+            }
+            lowest = wave_min_u32(lowest);
+            if (lane == 0) {
+                sh.red_i[w] = lowest;
+            }
+            __syncthreads();
+            lowest = sh.red_i[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                lowest = min(lowest, sh.red_i[i]);
+            }
+            __syncthreads();
         }
-        lowest = wave_min_u32(lowest);
-        if (lane == 0) {
-            sh.red_i[w] = lowest;
-        }
-        __syncthreads();
-        lowest = sh.red_i[0];
-        for (int i = 1; i < NWAVE; ++i) {
-            lowest = min(lowest, sh.red_i[i]);
-        }
-        __syncthreads();
         const float below = lilym_key_value(lilym_order_key(filt) - 1u) / a.temperature;
         if (!(n >= k && lilym_order_key(below) < lowest)) {
             return stream_fail(cfg, 6u);
