@@ -636,6 +636,12 @@ __device__ __forceinline__ bool list_push(bool has, uint32_t id, uint32_t* list,
     return true;
 }
 
+// A term's exponent v*c - ref is formed in f32: its rounding error grows with its size, and
+// the terms that carry the sum are the ones above the reference.  The reference is raised
+// before any exponent exceeds this (values below 32 are at most 0.95e-6 off: a relative
+// error of 0.7e-6 in the term, well inside the log-probability's 1e-5).
+constexpr float LSE_RAISE = 24.0f;
+
 // One wave's sum of 2^(v*c - ref) with a reference that is the same in every lane.
 struct WaveLse {
     float ref;
@@ -648,7 +654,7 @@ struct WaveLse {
     // every term is below 2^-40 of the reference.
     template <int E>
     __device__ __forceinline__ void add(const float (&v)[E], float m, float c) {
-        if (__ballot(__builtin_fmaf(m, c, -ref) > 60.0f) != 0ull) {
+        if (__ballot(__builtin_fmaf(m, c, -ref) > LSE_RAISE) != 0ull) {
             // A term would dwarf the reference: raise it to the wave's maximum (rare).
             const float nref = fmaxf(ref, wave_max_f(m * c));
             s *= __builtin_amdgcn_exp2f(ref - nref);
@@ -665,7 +671,7 @@ struct WaveLse {
     template <int E>
     __device__ __forceinline__ void add_if(const float (&v)[E], float m, float c, bool active) {
         const float d = __builtin_fmaf(active ? m : NEG_INF, c, -ref);
-        if (__ballot(d > 60.0f) != 0ull) {
+        if (__ballot(d > LSE_RAISE) != 0ull) {
             const float nref = fmaxf(ref, wave_max_f(active ? m * c : NEG_INF));
             s *= __builtin_amdgcn_exp2f(ref - nref);
             ref = nref;
@@ -687,7 +693,7 @@ struct WaveLse {
     // (raises the reference when some lane's would dwarf it), then add_prepared() per load.
     float skip_below;  // loads whose maximum is not above this are left out (set by the caller)
     __device__ __forceinline__ void prepare(float block_max, float c) {
-        if (__ballot(__builtin_fmaf(block_max, c, -ref) > 60.0f) != 0ull) {
+        if (__ballot(__builtin_fmaf(block_max, c, -ref) > LSE_RAISE) != 0ull) {
             const float nref = fmaxf(ref, wave_max_dpp(block_max * c));
             s *= __builtin_amdgcn_exp2f(ref - nref);
             ref = nref;
@@ -1151,7 +1157,10 @@ __device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, 
                 const float u = finish_pre_temperature(a, id, l, cnt, true);
                 if (!lse_done) {
                     lse_true.add_one(u, c2);
-                    if (patch) {
+                    // The raw term is taken off only where the stream added it: ids of the
+                    // partial chunks at the row's ends were never streamed.
+                    const uint32_t ch = (id + g.pad) / E;
+                    if (patch && ch >= g.main_lo && ch < g.main_hi) {
                         lse_raw.add_one(l, c2);
                     }
                 }
@@ -1513,13 +1522,15 @@ struct StreamLds {
 
 // 2^(v*c - ref) as a double for any argument (0 below 2^-1000).
 __device__ __forceinline__ double term_d(float v, float c, float ref) {
-    float d = __builtin_fmaf(v, c, -ref);
-    if (!(d > -1000.0f)) {
+    // The exponent in double: a row's largest value may lie hundreds of units above the
+    // reference (fixed after the first block), where an f32 difference is good to 1e-5 only.
+    double d = (double)v * (double)c - (double)ref;
+    if (!(d > -1000.0)) {
         return 0.0;  // far below the reference, -inf, NaN
     }
-    d = fminf(d, 1000.0f);
-    const float di = __builtin_floorf(d);
-    const float fr = d - di;
+    d = d < 1000.0 ? d : 1000.0;
+    const double di = __builtin_floor(d);
+    const float fr = (float)(d - di);
     return __builtin_ldexp((double)__builtin_amdgcn_exp2f(fr), (int)di);
 }
 
@@ -2168,11 +2179,11 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         // reference, then the three sums are reduced together.
         double part[3];
         {
-            float d = wl.ref - ref_s;
-            d = fminf(fmaxf(d, -1000.0f), 1000.0f);
-            const float di = __builtin_floorf(d);
+            double d = (double)wl.ref - (double)ref_s;  // exact
+            d = d < -1000.0 ? -1000.0 : (d > 1000.0 ? 1000.0 : d);
+            const double di = __builtin_floor(d);
             part[0] = wl.s > 0.0f ? (double)wl.s * __builtin_ldexp(
-                                        (double)__builtin_amdgcn_exp2f(d - di), (int)di)
+                                        (double)__builtin_amdgcn_exp2f((float)(d - di)), (int)di)
                                   : 0.0;
         }
         part[1] = acc_r;

@@ -75,20 +75,25 @@ def test_top_k_between_65_and_1024(sampler):
             _check_logprob(r, i, d, ("k", k))
 
 
-@pytest.mark.parametrize("slices", [0, 1], ids=["auto-slices", "one-slice"])
-def test_masks_of_every_density_report_their_select(slices):
-    """Sparse masks are served from the mask's words (no row is streamed), dense ones by the
-    bitmap select (with one workgroup per row the 5 % and 60 % masks admit more ids than the
-    workgroup holds); both agree with the oracle."""
+def _sampler_with_slices(slices):
+    """A sampler whose launches use `slices` workgroups per row (0 = its own choice)."""
     old = os.environ.get("LILY_SAMPLER_SLICES")
     os.environ["LILY_SAMPLER_SLICES"] = str(slices)
     try:
-        s = LS.Sampler(0)
+        return LS.Sampler(0)
     finally:
         if old is None:
             os.environ.pop("LILY_SAMPLER_SLICES", None)
         else:
             os.environ["LILY_SAMPLER_SLICES"] = old
+
+
+@pytest.mark.parametrize("slices", [0, 1], ids=["auto-slices", "one-slice"])
+def test_masks_of_every_density_report_their_select(slices):
+    """Sparse masks are served from the mask's words (no row is streamed), dense ones by the
+    bitmap select (with one workgroup per row the 5 % and 60 % masks admit more ids than the
+    workgroup holds); both agree with the oracle."""
+    s = _sampler_with_slices(slices)
     rng = np.random.default_rng(33)
     vocab = 151_936
     fracs = (0.0, 0.0002, 0.02, 0.02, 0.05, 0.6)
@@ -175,3 +180,75 @@ def test_forced_rows_with_a_log_probability(sampler, bf16):
                     assert np.array_equal(sc[i].read_counts().numpy().view(np.uint32), counts[i])
                 for t in sc:
                     t.close()
+
+
+@pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
+def test_log_probability_when_the_largest_value_arrives_late(bf16):
+    """The row's largest values sit hundreds of units above everything the first block
+    holds (one workgroup per row, as in large batches): the exponents of their terms must
+    not be rounded to f32 relative to the first block's reference (that costs 1e-5 of the
+    log-probability)."""
+    sampler = _sampler_with_slices(1)
+    rng = np.random.default_rng(41 + bf16)
+    rows, vocab = 6, 151_936
+    x = rng.normal(0, 1, (rows, vocab)).astype(np.float32)
+    for r_ in range(rows):
+        at = vocab - 1 - 37 * r_
+        x[r_, at] = 520.0 + 24.0 * r_                # the draw, with most of the mass
+        x[r_, at - 5000] = 519.5 + 24.0 * r_         # a close second
+    if bf16:
+        x = W.to_bf16_bits(x)
+    hist = rng.integers(0, vocab, (rows, 300)).astype(np.int32)
+    for variant in ("plain", "penalised"):
+        sc, counts, pen = None, [None] * rows, dict()
+        if variant == "penalised":
+            pen = dict(repetition_penalty=1.1, presence_penalty=0.2, frequency_penalty=0.1)
+            sc, counts = [], []
+            for r_ in range(rows):
+                t = LS.SamplerScratch(sampler, vocab)
+                t.add_history(torch.from_numpy(hist[r_]).to(dev()))
+                sc.append(t)
+                counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
+        for k in (20, 300):
+            kw = [dict(temperature=1.0, top_k=k, top_p=1.0, seed=7 + r_, **pen) for r_ in range(rows)]
+            r = run_rows(sampler, x, kw, [2] * rows, scratch=sc, logprobs=True)
+            for i in range(rows):
+                d = O.sample(x[i], counts[i], o_params(**kw[i]), 2, want_logprob=True)
+                check_row_against_oracle(r, i, d)
+                _check_logprob(r, i, d, ("late maximum", variant, k))
+        if sc is not None:
+            for t in sc:
+                t.close()
+    sampler.close()
+
+
+def test_penalised_ids_in_the_partial_chunks_of_unaligned_rows(sampler):
+    """Rows of odd length start at every 16-byte phase, so their first and last ids lie in
+    partial chunks that no select streams.  With those ids penalised and k above 64 the row
+    sum must still hold each of them once."""
+    rng = np.random.default_rng(43)
+    rows, vocab = 9, 4099
+    for bf16 in (False, True):
+        x = rng.normal(0, 0.02, (rows, vocab)).astype(np.float32)
+        if bf16:
+            x = W.to_bf16_bits(x)
+        # the ids at both ends of the row and a tenth of the others
+        hist = np.stack([np.concatenate([np.arange(12), np.arange(vocab - 12, vocab),
+                                         rng.choice(np.arange(12, vocab - 12), 400, replace=False)])
+                         for _ in range(rows)]).astype(np.int32)
+        sc, counts = [], []
+        for r_ in range(rows):
+            t = LS.SamplerScratch(sampler, vocab)
+            t.add_history(torch.from_numpy(hist[r_]).to(dev()))
+            sc.append(t)
+            counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
+        for k in (300, 20):
+            kw = [dict(temperature=1.0, top_k=k, top_p=1.0, seed=3 + r_, repetition_penalty=1.3,
+                       presence_penalty=0.5, frequency_penalty=0.1) for r_ in range(rows)]
+            r = run_rows(sampler, x, kw, [5] * rows, scratch=sc, logprobs=True)
+            for i in range(rows):
+                d = O.sample(x[i], counts[i], o_params(**kw[i]), 5, want_logprob=True)
+                check_row_against_oracle(r, i, d)
+                _check_logprob(r, i, d, ("edges", bf16, k))
+        for t in sc:
+            t.close()
