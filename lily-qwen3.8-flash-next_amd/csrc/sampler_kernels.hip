@@ -1521,17 +1521,11 @@ struct StreamLds {
 };
 
 // 2^(v*c - ref) as a double for any argument (0 below 2^-1000).
-__device__ __forceinline__ double term_d(float v, float c, float ref) {
-    // The exponent in double: a row's largest value may lie hundreds of units above the
-    // reference (fixed after the first block), where an f32 difference is good to 1e-5 only.
-    double d = (double)v * (double)c - (double)ref;
-    if (!(d > -1000.0)) {
-        return 0.0;  // far below the reference, -inf, NaN
-    }
-    d = d < 1000.0 ? d : 1000.0;
+// 2^d for d in (-1000, 1000]: the fraction through the hardware exponential, the integer
+// part as a power of two.
+__device__ __forceinline__ double pow2_d(double d) {
     const double di = __builtin_floor(d);
-    const float fr = (float)(d - di);
-    return __builtin_ldexp((double)__builtin_amdgcn_exp2f(fr), (int)di);
+    return __builtin_ldexp((double)__builtin_amdgcn_exp2f((float)(d - di)), (int)di);
 }
 
 // The largest 16-bit prefix P with at least `need` lanes holding key16 >= P; 0 when fewer
@@ -1815,7 +1809,30 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     WaveLse wl;
     wl.init();
     double acc_t = 0.0, acc_r = 0.0, acc_q = 0.0;
+    int up = 0;                 // this thread's double sums are relative to ref_s + up
+    bool beyond = false;        // the streamed sums lie outside the doubles' range
     uint32_t parity = 0;
+    // One term 2^(v*c2 - ref_s - up) of a double sum.  The exponent is formed in double: a
+    // row's largest value may lie hundreds of units above the reference (fixed after the
+    // first block), where an f32 difference is good to 1e-5 only.  A term beyond 2^900 moves
+    // the thread's own reference up to it (its three sums are scaled down by the same power
+    // of two); the threads' references are brought together at the end.
+    auto term_d = [&](float v) -> double {
+        double d = (double)v * (double)c2 - (double)ref_s - (double)up;
+        if (!(d > -1000.0)) {
+            return 0.0;  // far below the reference, -inf, NaN
+        }
+        if (d > 900.0) {
+            const int step = (int)__builtin_floor(d < 1.0e6 ? d : 1.0e6);
+            acc_t = __builtin_ldexp(acc_t, -step);
+            acc_r = __builtin_ldexp(acc_r, -step);
+            acc_q = __builtin_ldexp(acc_q, -step);
+            up += step;
+            d -= (double)step;
+            d = d < 900.0 ? d : 900.0;
+        }
+        return pow2_d(d);
+    };
 
     // Brings T up to date with everything the lanes have seen, the current block included.
     auto refresh_bound = [&](bool first, bool maxima) {
@@ -1938,10 +1955,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const bool summed = !queued && cm > skip_b;
         if (want_lse) {
             if (t > skip_b) {  // the same cut as for streamed terms
-                acc_t += term_d(t, c2, ref_s);
+                acc_t += term_d(t);
             }
             if (summed) {
-                acc_r += term_d(r.raw, c2, ref_s);
+                acc_r += term_d(r.raw);
             }
         }
         if (queued) {
@@ -2153,7 +2170,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             for (int j = 0; j < E; ++j) {
                 if (!((dm >> j) & 1u)) {
                     if (want_lse) {
-                        acc_q += term_d(v[j], c2, ref_s);
+                        acc_q += term_d(v[j]);
                     }
                     offer(v[j], g.id_of(c, j));
                 }
@@ -2168,26 +2185,38 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         for (uint32_t id = lo + tid; id < hi; id += NT) {
             const float u = pre_temperature_of<DT>(a, id);
             if (want_lse) {
-                acc_q += term_d(u, c2, ref_s);
+                acc_q += term_d(u);
             }
             offer(u, id);
         }
     }
     phase(cfg, 9);
     if (want_lse) {
-        // Everything relative to ref_s: this lane's streamed sum is rescaled from its wave's
-        // reference, then the three sums are reduced together.
+        // The threads' references are brought together (the highest one), then everything is
+        // relative to ref_s + up_all: this lane's streamed sum is rescaled from its wave's
+        // reference, and the three sums are reduced together.
+        uint32_t up_all = wave_min_u32(~(uint32_t)up);
+        if (lane == 0) {
+            sh.red_i[w] = up_all;
+        }
+        __syncthreads();
+        up_all = sh.red_i[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            up_all = min(up_all, sh.red_i[i]);
+        }
+        up_all = ~up_all;
+        const int down = up - (int)up_all;  // <= 0
         double part[3];
         {
-            double d = (double)wl.ref - (double)ref_s;  // exact
+            double d = (double)wl.ref - (double)ref_s - (double)up_all;  // exact
+            if (d > 1000.0 && wl.s > 0.0f) {
+                beyond = true;
+            }
             d = d < -1000.0 ? -1000.0 : (d > 1000.0 ? 1000.0 : d);
-            const double di = __builtin_floor(d);
-            part[0] = wl.s > 0.0f ? (double)wl.s * __builtin_ldexp(
-                                        (double)__builtin_amdgcn_exp2f((float)(d - di)), (int)di)
-                                  : 0.0;
+            part[0] = wl.s > 0.0f ? (double)wl.s * pow2_d(d) : 0.0;
         }
-        part[1] = acc_r;
-        part[2] = acc_t + acc_q;
+        part[1] = __builtin_ldexp(acc_r, down);
+        part[2] = __builtin_ldexp(acc_t + acc_q, down);
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             part[i] = wave_sum_d(part[i]);
@@ -2195,7 +2224,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 sh.red3[i][w] = part[i];
             }
         }
-        __syncthreads();
+        const bool any_beyond = __syncthreads_or(beyond ? 1 : 0) != 0;
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             part[i] = 0.0;
@@ -2205,8 +2234,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         const double streamed = part[0], booked = part[1], exact = part[2];
         const double rest = streamed - booked;
-        // Listed ids held nearly all of what was streamed: the difference is too coarse.
-        const bool coarse = booked > 0.0 && !(rest > 0.05 * streamed);
+        // Listed ids held nearly all of what was streamed: the difference is too coarse.  Or
+        // the row spans more than the doubles can hold relative to the first block.
+        const bool coarse = any_beyond || (booked > 0.0 && !(rest > 0.05 * streamed));
         phase(cfg, 10);
         if (coarse) {
             phase(cfg, 11);
@@ -2222,7 +2252,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 sh.lse_s = s_e;
             }
         } else if (tid == 0) {
-            sh.lse_mc = (double)ref_s;
+            sh.lse_mc = (double)ref_s + (double)up_all;
             sh.lse_s = (rest > 0.0 ? rest : 0.0) + exact;
         }
     }

@@ -187,7 +187,8 @@ def test_log_probability_when_the_largest_value_arrives_late(bf16):
     """The row's largest values sit hundreds of units above everything the first block
     holds (one workgroup per row, as in large batches): the exponents of their terms must
     not be rounded to f32 relative to the first block's reference (that costs 1e-5 of the
-    log-probability)."""
+    log-probability), and at temperature 0.5 they lie beyond 2^1000 times that reference,
+    outside the range of the doubles the sum is kept in."""
     sampler = _sampler_with_slices(1)
     rng = np.random.default_rng(41 + bf16)
     rows, vocab = 6, 151_936
@@ -209,13 +210,14 @@ def test_log_probability_when_the_largest_value_arrives_late(bf16):
                 t.add_history(torch.from_numpy(hist[r_]).to(dev()))
                 sc.append(t)
                 counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
-        for k in (20, 300):
-            kw = [dict(temperature=1.0, top_k=k, top_p=1.0, seed=7 + r_, **pen) for r_ in range(rows)]
+        for k, temperature in ((20, 1.0), (300, 1.0), (20, 0.5)):
+            kw = [dict(temperature=temperature, top_k=k, top_p=1.0, seed=7 + r_, **pen)
+                  for r_ in range(rows)]
             r = run_rows(sampler, x, kw, [2] * rows, scratch=sc, logprobs=True)
             for i in range(rows):
                 d = O.sample(x[i], counts[i], o_params(**kw[i]), 2, want_logprob=True)
                 check_row_against_oracle(r, i, d)
-                _check_logprob(r, i, d, ("late maximum", variant, k))
+                _check_logprob(r, i, d, ("late maximum", variant, k, temperature))
         if sc is not None:
             for t in sc:
                 t.close()
