@@ -2945,9 +2945,20 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         if (KIND != 2 && !done && cfg.path != 1u && cfg.old_layout != 0u) {
             const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
             if (EXCL || !special) {
-                const bool two_pass = a.k > 64u || cfg.path == 2u;
-                done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh, cfg,
-                                                  sorted);
+                // A single pass whose running bound let too many candidates in is repeated
+                // as two passes (bound first, then collect) before the exhaustive select.
+#pragma nounroll
+                for (int attempt = 0; attempt < 2 && !done; ++attempt) {
+                    const bool two_pass = a.k > 64u || cfg.path == 2u || attempt == 1;
+                    if (attempt == 1) {
+                        __syncthreads();
+                    }
+                    done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh,
+                                                      cfg, sorted);
+                    if (a.k > 64u || cfg.path == 2u) {
+                        break;  // it was two passes already
+                    }
+                }
                 took = done ? 1u : took;
             }
         }
