@@ -238,8 +238,8 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
     out->presence = params->presence_penalty;
     out->frequency = params->frequency_penalty;
     out->repetition = params->repetition_penalty;
-    if (mode != MODE_ARGMAX && k <= STREAM_K_MAX && x.allow == nullptr &&
-        out->n_bias <= STREAM_BIAS_CAP && vocab <= (1u << SPEC_ID_BITS)) {
+    if (mode != MODE_ARGMAX && k <= STREAM_K_MAX && out->n_bias <= STREAM_BIAS_CAP &&
+        vocab <= (1u << SPEC_ID_BITS)) {
         out->flags |= F_STREAM;
     }
     return LILY_OK;
@@ -343,7 +343,8 @@ LaunchShape shape_of(const lily_sampler* s, const RowArgs* rows, uint32_t n, int
         }
         const bool stream = (rows[i].flags & F_STREAM) && s->force_path == 0;
         any_stream = any_stream || stream;
-        any_old = any_old || !stream;
+        // A masked row may be streamed (dense masks), but decides that on the device.
+        any_old = any_old || !stream || rows[i].allow != nullptr;
         masked = masked || rows[i].allow != nullptr;
     }
     // Rows outside the streaming select need the candidate buffer, the id list and (rows with

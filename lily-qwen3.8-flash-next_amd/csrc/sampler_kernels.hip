@@ -1563,7 +1563,7 @@ __device__ __forceinline__ bool stream_fail(const LaunchCfg& cfg, uint32_t why) 
     return false;
 }
 
-template <int DT, bool LSE>
+template <int DT, bool LSE, bool MASKS>
 __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g, uint32_t k, Shared& sh,
                                               const LaunchCfg& cfg, bool& sorted, uint64_t*& out) {
     constexpr int E = Geo<DT>::E;
@@ -1648,7 +1648,36 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     if (n_pairs > a.pairs_cap) {
         return stream_fail(cfg, 2u);  // the list overflowed: the bitmap and the counts hold the truth
     }
-    const bool listed_row = n_pairs != 0 || n_bias != 0;
+    // A row with an allow-mask is streamed when the mask is dense: its disallowed ids join the
+    // listed ids (true value -inf).  Otherwise the row is left to the selects made for masks.
+    // (MASKS is false in kernels whose launches hold no masked row.)
+    const bool masked = MASKS && a.allow != nullptr;
+    const uint32_t w_lo = g.id_lo >> 5, w_hi = (g.id_hi + 31u) >> 5;
+    auto barred = [&](uint32_t i) -> uint32_t {  // disallowed ids of mask word i inside the slice
+        return ~gload(a.allow + i) & range32_at(g.id_lo, g.id_hi, (int64_t)i * 32);
+    };
+    uint32_t n_barred = 0;
+    if (masked) {
+        uint32_t mine = 0;
+        for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
+            mine += (uint32_t)__popc(barred(i));
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            mine += __shfl_xor(mine, o);
+        }
+        if (lane == 0) {
+            sh.red_i[w] = mine;
+        }
+        __syncthreads();
+        for (int i = 0; i < NWAVE; ++i) {
+            n_barred += sh.red_i[i];
+        }
+        __syncthreads();
+        if ((uint64_t)n_barred + n_pairs + n_bias > SPEC_CAP - SPEC_CAP / 10u) {
+            return false;  // not a failure: the mask is not dense enough for this select
+        }
+    }
+    const bool listed_row = n_pairs != 0 || n_bias != 0 || n_barred != 0;
     // Block of a streamed id of this slice, NONE for ids outside it or in a partial chunk.
     auto block_of = [&](uint32_t id) -> uint32_t {
         if (id >= g.vocab) {
@@ -1674,6 +1703,28 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             return NONE;
         }
         return b;
+    };
+    // The disallowed ids that open a bucket slot of their own: streamed ones that neither
+    // the scratch's list nor the bias list covers already.
+    auto each_barred = [&](auto&& fn) {
+        if (n_barred == 0u) {
+            return;
+        }
+        for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
+            uint32_t bits = barred(i);
+            while (bits != 0u) {
+                const uint32_t id = i * 32u + (uint32_t)__builtin_ctz(bits);
+                bits &= bits - 1u;
+                const uint32_t b = block_of(id);
+                bool open = b != NONE && !(pen && bit_of(a.touched, id));
+                for (uint32_t j = 0; open && j < n_bias; ++j) {
+                    open = L.bias_id[j] != id;
+                }
+                if (open) {
+                    fn(id, b);
+                }
+            }
+        }
     };
     if (listed_row && nblocks == 1u) {
         // One block: its bucket starts at slot 0, so a single atomic places each entry and
@@ -1702,6 +1753,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 put(L.bias_id[i]);
             }
         }
+        each_barred([&](uint32_t id, uint32_t) { put(id); });
         __syncthreads();
         const uint32_t total = L.bfill[0];
         if (total > SPEC_CAP) {
@@ -1765,6 +1817,13 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     }
                 }
             }
+            each_barred([&](uint32_t id, uint32_t b) {
+                if (pass == 0) {
+                    atomicAdd(&L.bkt[b], 1u);
+                } else {
+                    L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = id;
+                }
+            });
             __syncthreads();
             if (pass == 0) {
                 phase(cfg, 14);
@@ -1809,27 +1868,39 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     WaveLse wl;
     wl.init();
     double acc_t = 0.0, acc_r = 0.0, acc_q = 0.0;
-    int up = 0;                 // this thread's double sums are relative to ref_s + up
-    bool beyond = false;        // the streamed sums lie outside the doubles' range
+    constexpr int UP_UNSET = INT_MIN;
+    int up = UP_UNSET;          // this thread's double sums are relative to ref_s + up
     uint32_t parity = 0;
     // One term 2^(v*c2 - ref_s - up) of a double sum.  The exponent is formed in double: a
     // row's largest value may lie hundreds of units above the reference (fixed after the
-    // first block), where an f32 difference is good to 1e-5 only.  A term beyond 2^900 moves
-    // the thread's own reference up to it (its three sums are scaled down by the same power
-    // of two); the threads' references are brought together at the end.
+    // first block), where an f32 difference is good to 1e-5 only.  The thread's own
+    // reference ref_s + up starts at its first term and moves up (its three sums scaled down
+    // by the same power of two) when a term lies beyond 2^900 of it, so what a thread drops
+    // as too small is small against something it holds - the row's raw maximum, which ref_s
+    // comes from, may belong to an id that a mask or a bias takes out.  The threads'
+    // references are brought together at the end.
+    double base = -1.0e300;     // ref_s + up; far below anything while up is unset
+    const double c2d = (double)c2;
     auto term_d = [&](float v) -> double {
-        double d = (double)v * (double)c2 - (double)ref_s - (double)up;
-        if (!(d > -1000.0)) {
-            return 0.0;  // far below the reference, -inf, NaN
-        }
+        double d = __builtin_fma((double)v, c2d, -base);
         if (d > 900.0) {
-            const int step = (int)__builtin_floor(d < 1.0e6 ? d : 1.0e6);
-            acc_t = __builtin_ldexp(acc_t, -step);
-            acc_r = __builtin_ldexp(acc_r, -step);
-            acc_q = __builtin_ldexp(acc_q, -step);
-            up += step;
-            d -= (double)step;
-            d = d < 900.0 ? d : 900.0;
+            // The thread's first term, or one beyond 2^900 of its reference: the reference
+            // moves to the term (the three sums, if any, scaled down by the same power of two).
+            double e = (double)v * c2d - (double)ref_s;
+            e = e < 1.0e9 ? (e > -1.0e9 ? e : -1.0e9) : 1.0e9;
+            const int now = (int)__builtin_floor(e);
+            if (up != UP_UNSET) {
+                const int step = now - up;
+                acc_t = __builtin_ldexp(acc_t, -step);
+                acc_r = __builtin_ldexp(acc_r, -step);
+                acc_q = __builtin_ldexp(acc_q, -step);
+            }
+            up = now;
+            base = (double)ref_s + (double)up;
+            d = e - (double)up;
+        }
+        if (!(d > -1000.0)) {
+            return 0.0;  // -inf, NaN, or nothing against what the thread already holds
         }
         return pow2_d(d);
     };
@@ -1938,6 +2009,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (cnt > 0u) {
             t = t > 0.0f ? t / a.repetition : t * a.repetition;
             t -= a.presence + a.frequency * (float)cnt;
+        }
+        if (masked && !bit_of(a.allow, id)) {
+            t = NEG_INF;
         }
         listed_raw_max = fmaxf(listed_raw_max, r.raw);
         listed_true_max = fmaxf(listed_true_max, t);
@@ -2192,27 +2266,23 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     }
     phase(cfg, 9);
     if (want_lse) {
-        // The threads' references are brought together (the highest one), then everything is
-        // relative to ref_s + up_all: this lane's streamed sum is rescaled from its wave's
-        // reference, and the three sums are reduced together.
-        uint32_t up_all = wave_min_u32(~(uint32_t)up);
-        if (lane == 0) {
-            sh.red_i[w] = up_all;
+        // Each wave brings its sums to one reference of its own: the highest of its threads'
+        // references and of the streamed sums' (wave-uniform) reference.  The waves' partial
+        // sums and references meet in LDS and are brought together after one barrier.
+        int ref_w = up;
+        for (int o = 32; o > 0; o >>= 1) {
+            ref_w = max(ref_w, __shfl_xor(ref_w, o));
         }
-        __syncthreads();
-        up_all = sh.red_i[0];
-        for (int i = 1; i < NWAVE; ++i) {
-            up_all = min(up_all, sh.red_i[i]);
+        const double stream_at = (double)wl.ref - (double)ref_s;  // exact
+        if (__ballot(wl.s > 0.0f) != 0ull) {
+            const double e = stream_at < 1.0e9 ? (stream_at > -1.0e9 ? stream_at : -1.0e9) : 1.0e9;
+            ref_w = max(ref_w, (int)__builtin_floor(e));
         }
-        up_all = ~up_all;
-        const int down = up - (int)up_all;  // <= 0
+        const int down = up == UP_UNSET ? 0 : up - ref_w;  // <= 0
         double part[3];
         {
-            double d = (double)wl.ref - (double)ref_s - (double)up_all;  // exact
-            if (d > 1000.0 && wl.s > 0.0f) {
-                beyond = true;
-            }
-            d = d < -1000.0 ? -1000.0 : (d > 1000.0 ? 1000.0 : d);
+            double d = stream_at - (double)ref_w;  // <= 1 where there is a sum
+            d = d < -1000.0 ? -1000.0 : d;
             part[0] = wl.s > 0.0f ? (double)wl.s * pow2_d(d) : 0.0;
         }
         part[1] = __builtin_ldexp(acc_r, down);
@@ -2224,19 +2294,29 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 sh.red3[i][w] = part[i];
             }
         }
-        const bool any_beyond = __syncthreads_or(beyond ? 1 : 0) != 0;
+        if (lane == 0) {
+            sh.red_i[w] = (uint32_t)ref_w;
+        }
+        __syncthreads();
+        int ref_all = (int)sh.red_i[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            ref_all = max(ref_all, (int)sh.red_i[i]);
+        }
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             part[i] = 0.0;
             for (int ww = 0; ww < NWAVE; ++ww) {
-                part[i] += sh.red3[i][ww];
+                const int at = (int)sh.red_i[ww];
+                part[i] += at == UP_UNSET ? 0.0 : __builtin_ldexp(sh.red3[i][ww], at - ref_all);
             }
+        }
+        if (ref_all == UP_UNSET) {
+            ref_all = 0;  // no term anywhere: the sums are zero
         }
         const double streamed = part[0], booked = part[1], exact = part[2];
         const double rest = streamed - booked;
-        // Listed ids held nearly all of what was streamed: the difference is too coarse.  Or
-        // the row spans more than the doubles can hold relative to the first block.
-        const bool coarse = any_beyond || (booked > 0.0 && !(rest > 0.05 * streamed));
+        // Listed ids held nearly all of what was streamed: the difference is too coarse.
+        const bool coarse = booked > 0.0 && !(rest > 0.05 * streamed);
         phase(cfg, 10);
         if (coarse) {
             phase(cfg, 11);
@@ -2252,7 +2332,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 sh.lse_s = s_e;
             }
         } else if (tid == 0) {
-            sh.lse_mc = (double)ref_s + (double)up_all;
+            sh.lse_mc = (double)ref_s + (double)ref_all;
             sh.lse_s = (rest > 0.0 ? rest : 0.0) + exact;
         }
     }
@@ -2932,7 +3012,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         bool done = false;
         uint32_t took = 2;
         if (cfg.path == 0u && (a.flags & F_STREAM)) {
-            done = select_stream<DT, LSE>(a, g, a.k, sh, cfg, sorted, found);
+            done = select_stream<DT, LSE, KIND != 2>(a, g, a.k, sh, cfg, sorted, found);
             took = done ? 0u : took;
             if (!done) {
                 __syncthreads();
