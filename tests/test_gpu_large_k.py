@@ -254,3 +254,56 @@ def test_penalised_ids_in_the_partial_chunks_of_unaligned_rows(sampler):
                 _check_logprob(r, i, d, ("edges", bf16, k))
         for t in sc:
             t.close()
+
+
+@pytest.mark.parametrize("slices", [0, 1], ids=["auto-slices", "one-slice"])
+def test_dense_masks_are_streamed(slices):
+    """A mask that bars a few hundred ids - among them the row's best ones, as a list of
+    banned tokens would - is served by the streaming select: the barred ids join the listed
+    ids with a true value of -inf.  Penalties and a bias list on top; the row's largest raw
+    value is barred, so the row sum must not be measured against it."""
+    s = _sampler_with_slices(slices)
+    rng = np.random.default_rng(51)
+    rows, vocab = 7, 151_936
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    for bf16 in (False, True):
+        x = rng.normal(0, 2, (rows, vocab)).astype(np.float32)
+        x[3, 70_000] = 400.0                              # far above everything, and barred
+        masks = np.full((rows, (vocab + 31) // 32), 0xFFFFFFFF, np.uint32)
+        masks[:, -1] = (1 << (vocab % 32)) - 1 if vocab % 32 else 0xFFFFFFFF
+        for r_ in range(rows):
+            barred = np.concatenate([np.argsort(x[r_])[::-1][:5 + 3 * r_],          # the best ones
+                                     rng.choice(vocab, 300, replace=False),
+                                     np.arange(0, 9), np.arange(vocab - 9, vocab)])   # both ends
+            for id_ in barred:
+                masks[r_, id_ >> 5] &= ~np.uint32(1 << (id_ & 31))
+        xs = W.to_bf16_bits(x) if bf16 else x
+        bias = [[(int(i), float(d)) for i, d in zip(rng.integers(0, vocab, 20),
+                                                     rng.choice([-4.0, 6.0], 20))] for _ in range(rows)]
+        hist = rng.integers(0, vocab, (rows, 1500)).astype(np.int32)
+        sc, counts = [], []
+        for r_ in range(rows):
+            t = LS.SamplerScratch(s, vocab)
+            t.add_history(torch.from_numpy(hist[r_]).to(dev()))
+            sc.append(t)
+            counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
+        for trial, k in enumerate((64, 20)):
+            kw = [dict(temperature=0.8, top_k=k, top_p=0.95, seed=90 + r_, repetition_penalty=1.15,
+                       presence_penalty=0.3, frequency_penalty=0.1) for r_ in range(rows)]
+            stats.zero_()
+            s.set_path_stats(stats)
+            r = run_rows(s, xs, kw, [trial] * rows, scratch=sc, allow=masks, bias=bias, logprobs=True)
+            s.set_path_stats(None)
+            st = stats.cpu().tolist()
+            # With one workgroup per row the rows that bar more of their best ids than the
+            # bound's slack covers fail the streaming select's check and take the bitmap one.
+            assert st[0] > 0 and st[2] == 0 and (slices == 1 or st[1] == 0), st
+            for i in range(rows):
+                d = O.sample(xs[i], counts[i], o_params(**kw[i]), trial, allow=masks[i], bias=bias[i],
+                             want_logprob=True)
+                check_row_against_oracle(r, i, d)
+                assert (masks[i][r.ids[i] >> 5] >> (r.ids[i] & 31)) & 1
+                _check_logprob(r, i, d, ("dense mask", bf16, k))
+        for t in sc:
+            t.close()
+    s.close()
