@@ -3209,7 +3209,7 @@ __device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowAr
 }
 
 template <int DT, int KIND, bool LSE>
-__global__ __launch_bounds__(NT, 4) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
+__global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
     __shared__ Shared sh;
     // `rows` is the first kernel argument: index it in the kernel-argument segment itself
     // (indexing the by-value copy would move all of it to scratch memory).
@@ -3225,7 +3225,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_inline(InlineRows rows, LaunchCf
 }
 
 template <int DT, int KIND, bool LSE>
-__global__ __launch_bounds__(NT, 4) void k_rows_table(LaunchCfg cfg) {
+__global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_table(LaunchCfg cfg) {
     __shared__ Shared sh;
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
     RowArgs a;
