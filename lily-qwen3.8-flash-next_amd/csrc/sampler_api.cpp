@@ -11,6 +11,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <algorithm>
 #include <vector>
 
 #include "../../include/lily_sampler.h"
@@ -92,13 +93,10 @@ struct lily_draft_dists {
     uint32_t* counts = nullptr;
 };
 
-struct lily_plan {
-    lily_sampler* s = nullptr;
-    uint32_t max_rows = 0;
-    RowArgs* table_dev = nullptr;
+// One launch over consecutive rows of a packed table.
+struct LaunchPart {
+    uint32_t first = 0;
     uint32_t rows = 0;
-    uint32_t vocab = 0;
-    uint32_t dtype = 0;
     uint32_t slices = 1;
     uint32_t ws_k = 0;
     int kind = 0;
@@ -108,6 +106,17 @@ struct lily_plan {
     bool old_layout = false;
     uint32_t cand_cap = 0;
     uint32_t listed = 0;                     // longest scratch list when the table was packed
+};
+
+struct lily_plan {
+    lily_sampler* s = nullptr;
+    uint32_t max_rows = 0;
+    RowArgs* table_dev = nullptr;
+    uint32_t rows = 0;
+    uint32_t vocab = 0;
+    uint32_t dtype = 0;
+    LaunchPart parts[2];                     // the batch's one or two launches
+    uint32_t n_parts = 0;
     uint32_t runs = 0;                       // launches since the table was packed
     std::vector<lily_scratch*> penalised;    // scratches whose rows count their draws
 };
@@ -383,6 +392,66 @@ uint32_t max_k(const RowArgs* rows, uint32_t n) {
         }
     }
     return k;
+}
+
+// Rows that need the kernel holding every select: not streamable, or carrying an allow-mask.
+bool heavy_row(const lily_sampler* s, const RowArgs& r) {
+    if (r.mode == MODE_ARGMAX) {
+        return false;
+    }
+    return s->force_path != 0 || !(r.flags & F_STREAM) || r.allow != nullptr;
+}
+
+constexpr uint32_t SPLIT_MIN_LIGHT = 64;  // streamable rows worth a launch of their own
+
+// Describes the launch(es) of a packed table.  A few rows that need the kernel with every
+// select would drag a large batch of streamable rows into it (three workgroups per compute
+// unit, more LDS each): the table is then reordered - every row carries its own output
+// pointers - and launched in two parts, streamable rows first.
+uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dtype, uint32_t vocab,
+                    LaunchPart* parts) {
+    uint32_t heavy = 0;
+    for (uint32_t i = 0; i < rows; ++i) {
+        heavy += heavy_row(s, table[i]) ? 1u : 0u;
+    }
+    const bool split = heavy != 0 && rows - heavy >= SPLIT_MIN_LIGHT;
+    if (split) {
+        std::stable_partition(table, table + rows,
+                              [s](const RowArgs& r) { return !heavy_row(s, r); });
+    }
+    const uint32_t n_parts = split ? 2u : 1u;
+    for (uint32_t q = 0; q < n_parts; ++q) {
+        LaunchPart& part = parts[q];
+        part.first = q == 0 ? 0u : rows - heavy;
+        part.rows = !split ? rows : (q == 0 ? rows - heavy : heavy);
+        const RowArgs* sub = table + part.first;
+        part.ws_k = max_k(sub, part.rows);
+        part.listed = longest_list(sub, part.rows);
+        part.slices = choose_slices(s, part.rows, part.ws_k, vocab, dtype, part.listed);
+        const LaunchShape shp = shape_of(s, sub, part.rows, dtype, vocab, part.slices, part.ws_k);
+        part.kind = shp.kind();
+        part.lse = shp.lse;
+        part.dyn_bytes = shp.dyn_bytes;
+        part.excl_words = shp.excl_words;
+        part.old_layout = shp.old_layout;
+        part.cand_cap = shp.cand_cap;
+    }
+    return n_parts;
+}
+
+int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_dev, int dtype,
+                uint32_t vocab, uint32_t step_delta, uint32_t hint_growth, bool traced) {
+    LaunchCfg cfg;
+    fill_cfg(s, &cfg, vocab, part.slices, part.ws_k, step_delta, table_dev + part.first);
+    if (traced) {
+        attach_trace(s, &cfg, part.rows);
+    }
+    cfg.excl_words = part.excl_words;
+    cfg.old_layout = part.old_layout ? 1u : 0u;
+    cfg.cand_cap = part.cand_cap;
+    cfg.hint_growth = hint_growth;
+    HIP_TRY(launch_rows(s->stream, dtype, part.kind, part.lse, part.rows, cfg, nullptr, part.dyn_bytes));
+    return LILY_OK;
 }
 
 int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n) {
@@ -1034,23 +1103,17 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     if (int rc = pack_batch(b, s->stage[slot])) {
         return rc;
     }
+    LaunchPart parts[2];
+    const uint32_t n_parts = plan_parts(s, s->stage[slot], b->rows, (int)b->dtype, b->vocab, parts);
     HIP_TRY(hipMemcpyAsync(s->table_dev, s->stage[slot], (size_t)b->rows * sizeof(RowArgs),
                            hipMemcpyHostToDevice, s->stream));
     HIP_TRY(hipEventRecord(s->stage_done[slot], s->stream));
     s->stage_used[slot] = true;
-    const uint32_t kmax = max_k(s->stage[slot], b->rows);
-    LaunchCfg cfg;
-    const uint32_t slices =
-        choose_slices(s, b->rows, kmax, b->vocab, (int)b->dtype, longest_list(s->stage[slot], b->rows));
-    fill_cfg(s, &cfg, b->vocab, slices, kmax, 0, s->table_dev);
-    attach_trace(s, &cfg, b->rows);
-    const LaunchShape shp =
-        shape_of(s, s->stage[slot], b->rows, (int)b->dtype, b->vocab, slices, kmax);
-    cfg.excl_words = shp.excl_words;
-    cfg.old_layout = shp.old_layout ? 1u : 0u;
-    cfg.cand_cap = shp.cand_cap;
-    HIP_TRY(launch_rows(s->stream, (int)b->dtype, shp.kind(), shp.lse, b->rows, cfg, nullptr,
-                        shp.dyn_bytes));
+    for (uint32_t q = 0; q < n_parts; ++q) {
+        if (int rc = launch_part(s, parts[q], s->table_dev, (int)b->dtype, b->vocab, 0, 0, q == 0)) {
+            return rc;
+        }
+    }
     return LILY_OK;
 }
 
@@ -1097,6 +1160,7 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     if (int rc = pack_batch(b, table.data())) {
         return rc;
     }
+    p->n_parts = plan_parts(p->s, table.data(), b->rows, (int)b->dtype, b->vocab, p->parts);
     HIP_TRY(hipSetDevice(p->s->device));
     HIP_TRY(hipStreamSynchronize(p->s->stream));
     HIP_TRY(hipMemcpy(p->table_dev, table.data(), (size_t)b->rows * sizeof(RowArgs),
@@ -1104,21 +1168,12 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->rows = b->rows;
     p->vocab = b->vocab;
     p->dtype = b->dtype;
-    p->ws_k = max_k(table.data(), b->rows);
-    p->listed = longest_list(table.data(), b->rows);
-    p->slices = choose_slices(p->s, b->rows, p->ws_k, b->vocab, (int)b->dtype, p->listed);
-    const LaunchShape shp = shape_of(p->s, table.data(), b->rows, (int)b->dtype, b->vocab,
-                                     p->slices, p->ws_k);
-    p->kind = shp.kind();
-    p->lse = shp.lse;
-    p->dyn_bytes = shp.dyn_bytes;
-    p->excl_words = shp.excl_words;
-    p->old_layout = shp.old_layout;
-    p->cand_cap = shp.cand_cap;
     p->runs = 0;
     p->penalised.clear();
     for (uint32_t r = 0; r < b->rows; ++r) {
-        if (b->scratch != nullptr && b->scratch[r] != nullptr && (table[r].flags & F_PEN)) {
+        // (the table may be reordered: the batch's own arrays tell which scratches count)
+        if (b->scratch != nullptr && b->scratch[r] != nullptr &&
+            lily_params_uses_penalties(&b->params[r]) != 0) {
             p->penalised.push_back(b->scratch[r]);
         }
     }
@@ -1130,32 +1185,31 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
         return fail(LILY_ERR_INVALID_ARG, "plan is null or not set");
     }
     HIP_TRY(hipSetDevice(p->s->device));
-    if (p->listed != 0 && p->kind == 2 && p->rows <= WS_ROWS) {
-        // The lists grow by one id per run at most: take more slices before a workgroup's
-        // buckets overflow (only the merge's share of dynamic LDS depends on the slices).
-        const uint32_t need = slices_for_list(p->listed + p->runs + 1);
-        const uint64_t by_ws = (uint64_t)WS_SLOTS / ((uint64_t)p->rows * (p->ws_k ? p->ws_k : 1));
-        if (need > p->slices && need <= MAX_SLICES && need <= by_ws) {
-            p->slices = need;
-            const size_t merge = (size_t)need * p->ws_k * 8;
-            if (merge > p->dyn_bytes) {
-                p->dyn_bytes = merge;
+    for (uint32_t q = 0; q < p->n_parts; ++q) {
+        LaunchPart& part = p->parts[q];
+        if (part.listed != 0 && part.kind == 2 && part.rows <= WS_ROWS) {
+            // The lists grow by one id per run at most: take more slices before a workgroup's
+            // buckets overflow (only the merge's share of dynamic LDS depends on the slices).
+            const uint32_t need = slices_for_list(part.listed + p->runs + 1);
+            const uint64_t by_ws =
+                (uint64_t)WS_SLOTS / ((uint64_t)part.rows * (part.ws_k ? part.ws_k : 1));
+            if (need > part.slices && need <= MAX_SLICES && need <= by_ws) {
+                part.slices = need;
+                const size_t merge = (size_t)need * part.ws_k * 8;
+                if (merge > part.dyn_bytes) {
+                    part.dyn_bytes = merge;
+                }
             }
         }
+        if (int rc = launch_part(p->s, part, p->table_dev, (int)p->dtype, p->vocab, step_delta, p->runs,
+                                 q == 0)) {
+            return rc;
+        }
     }
-    LaunchCfg cfg;
-    fill_cfg(p->s, &cfg, p->vocab, p->slices, p->ws_k, step_delta, p->table_dev);
-    attach_trace(p->s, &cfg, p->rows);
-    cfg.excl_words = p->excl_words;
-    cfg.old_layout = p->old_layout ? 1u : 0u;
-    cfg.cand_cap = p->cand_cap;
-    cfg.hint_growth = p->runs;
     p->runs += 1;
     for (lily_scratch* sc : p->penalised) {
         sc->listed_bound += 1;
     }
-    HIP_TRY(launch_rows(p->s->stream, (int)p->dtype, p->kind, p->lse, p->rows, cfg, nullptr,
-                        p->dyn_bytes));
     return LILY_OK;
 }
 

@@ -307,3 +307,44 @@ def test_dense_masks_are_streamed(slices):
         for t in sc:
             t.close()
     s.close()
+
+
+@pytest.mark.parametrize("use_plan", [False, True], ids=["direct", "plan"])
+def test_mixed_batches_run_as_two_launches(sampler, use_plan):
+    """A batch of mostly streamable rows with a few that need the other selects (k above
+    64, a long bias list) is reordered and launched in two parts; every row still writes its
+    own outputs and its own scratch, step after step."""
+    rng = np.random.default_rng(61)
+    rows, vocab = 150, 30_011
+    x = W.to_bf16_bits(rng.normal(0, 2, (rows, vocab)).astype(np.float32))
+    ks = rng.choice([20, 64, 300, 0, 1], rows, p=[0.5, 0.3, 0.08, 0.07, 0.05])
+    bias = [[(int(i), float(d)) for i, d in zip(rng.integers(0, vocab, 100 if r_ % 17 == 0 else 5),
+                                                 rng.choice([-3.0, 4.0], 100 if r_ % 17 == 0 else 5))]
+            for r_ in range(rows)]
+    hist = rng.integers(0, vocab, (rows, 400)).astype(np.int32)
+    sc, counts = [], []
+    for r_ in range(rows):
+        t = LS.SamplerScratch(sampler, vocab)
+        t.add_history(torch.from_numpy(hist[r_]).to(dev()))
+        sc.append(t)
+        counts.append(np.bincount(hist[r_], minlength=vocab).astype(np.uint32))
+    kw = [dict(temperature=0.0 if ks[r_] == 1 else 0.9, top_k=int(ks[r_]), top_p=0.92, seed=300 + r_,
+               repetition_penalty=1.1, presence_penalty=0.2, frequency_penalty=0.05)
+          for r_ in range(rows)]
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    for step in range(3):
+        stats.zero_()
+        sampler.set_path_stats(stats)
+        r = run_rows(sampler, x, kw, [step] * rows, scratch=sc, bias=bias, logprobs=True,
+                     use_plan=use_plan)
+        sampler.set_path_stats(None)
+        st = stats.cpu().tolist()
+        assert st[0] > 0 and st[1] > 0 and st[2] == 0, st
+        for i in range(rows):
+            d = O.sample(x[i], counts[i], o_params(**kw[i]), step, bias=bias[i], want_logprob=True)
+            check_row_against_oracle(r, i, d)
+            _check_logprob(r, i, d, ("mixed", step, int(ks[i])))
+        for i in range(0, rows, 11):
+            assert np.array_equal(sc[i].read_counts().numpy().view(np.uint32), counts[i]), i
+    for t in sc:
+        t.close()
