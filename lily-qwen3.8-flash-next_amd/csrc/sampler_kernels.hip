@@ -129,6 +129,33 @@ __device__ __forceinline__ float adjusted_of(const RowArgs& a, uint32_t id) {
     return pre_temperature_of<DT>(a, id) / a.temperature;
 }
 
+// The exact terms of ids [lo, hi), a thread's share sixteen at a time so that their loads
+// are in flight together (the loop is a chain of memory round trips otherwise).  The slow way
+// to a row sum, for the rare slices whose fast sum cancels.
+template <int DT, typename Acc>
+__device__ __forceinline__ void exact_terms(const RowArgs& a, uint32_t lo, uint32_t hi, float c2, Acc& acc) {
+    constexpr int DEPTH = 16;
+    const bool pen = (a.flags & F_PEN) != 0;
+    for (uint32_t id0 = lo + threadIdx.x; id0 < hi; id0 += (uint32_t)DEPTH * NT) {
+        float l[DEPTH];
+        uint32_t c[DEPTH];
+#pragma unroll
+        for (int q = 0; q < DEPTH; ++q) {
+            const uint32_t id = id0 + (uint32_t)q * NT;
+            l[q] = id < hi ? load_logit<DT>(a.logits, id) : 0.0f;
+            c[q] = (id < hi && pen) ? gload(a.counts + id) : 0u;
+        }
+#pragma unroll
+        for (int q = 0; q < DEPTH; ++q) {
+            const uint32_t id = id0 + (uint32_t)q * NT;
+            if (id < hi) {
+                const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
+                acc.add_one(finish_pre_temperature(a, id, l[q], c[q], allowed), c2);
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ float wave_max_f(float v) {
     for (int o = 32; o > 0; o >>= 1) {
         v = fmaxf(v, __shfl_xor(v, o));
@@ -1281,9 +1308,7 @@ __device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, 
                 // Rare: penalised ids held nearly all the raw mass.  Redo the sum exactly.
                 LseAcc exact;
                 exact.init();
-                for (uint32_t id = g.id_lo + tid; id < g.id_hi; id += NT) {
-                    exact.add_one(pre_temperature_of<DT>(a, id), c2);
-                }
+                exact_terms<DT>(a, g.id_lo, g.id_hi, c2, exact);
                 double m_e, s_e;
                 wg_merge_lse(sh, exact.mc, exact.s, m_e, s_e);
                 if (tid == 0) {
@@ -2322,9 +2347,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             phase(cfg, 11);
             LseAcc all;
             all.init();
-            for (uint32_t id = g.id_lo + tid; id < g.id_hi; id += NT) {
-                all.add_one(pre_temperature_of<DT>(a, id), c2);
-            }
+            exact_terms<DT>(a, g.id_lo, g.id_hi, c2, all);
             double m_e, s_e;
             wg_merge_lse(sh, all.mc, all.s, m_e, s_e);
             if (tid == 0) {
