@@ -140,6 +140,14 @@ uint32_t lily_scratch_vocab(const lily_scratch_t* sc);
 int lily_scratch_reset_counts(lily_scratch_t* sc);
 /* SamplerScratch::uncount (sample.rs:147-157): saturating, out-of-range ignored; stream-ordered. */
 int lily_scratch_uncount(lily_scratch_t* sc, uint32_t token);
+/* The rollback of a verify step's rejected draws (finish_speculation,
+ * src/qwen4exp/spec.rs:213-217: `for token in sampled[accepted + 1..] { uncount(token) }`)
+ * without the host reading the accepted row: a = min(accepted_dev[0], accepted_cap) and
+ * draws_dev[a + 1 .. m) are un-counted in order.  accepted_dev is typically the control
+ * block's LILY_SLOT_ACCEPTED word; accepted_cap is where the engine stopped earlier (a stop
+ * token among the accepted rows), UINT32_MAX when it did not.  Stream-ordered. */
+int lily_scratch_uncount_after(lily_scratch_t* sc, const uint32_t* draws_dev, uint32_t m,
+                               const uint32_t* accepted_dev, uint32_t accepted_cap);
 /* SamplerScratch::copy_counts_from (sample.rs:168-174): LILY_ERR_VOCAB on a size mismatch. */
 int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src);
 /* No counterpart in the reference (its histogram only ever grows by the kernel's own

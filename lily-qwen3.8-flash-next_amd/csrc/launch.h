@@ -16,6 +16,8 @@ hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t
 hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const uint32_t* ids,
                               uint32_t n);
 hipError_t launch_uncount(hipStream_t stream, const ScratchView& sc, uint32_t token);
+hipError_t launch_uncount_after(hipStream_t stream, const ScratchView& sc, const uint32_t* draws,
+                                uint32_t m, const uint32_t* accepted, uint32_t cap);
 hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc);
 hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const uint32_t* ids,
                               uint32_t* ctrl, uint32_t m, uint32_t pos0, uint32_t ratio,

@@ -834,6 +834,22 @@ int lily_scratch_uncount(lily_scratch_t* sc, uint32_t token) {
     return LILY_OK;
 }
 
+int lily_scratch_uncount_after(lily_scratch_t* sc, const uint32_t* draws_dev, uint32_t m,
+                               const uint32_t* accepted_dev, uint32_t accepted_cap) {
+    if (sc == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "scratch is null");
+    }
+    if (draws_dev == nullptr || accepted_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "draws or accepted row is null");
+    }
+    if (m == 0 || m > LILY_MAX_VERIFY_ROWS) {
+        return fail(LILY_ERR_RANGE, "rollback over %u rows (1..%u)", m, (unsigned)LILY_MAX_VERIFY_ROWS);
+    }
+    HIP_TRY(hipSetDevice(sc->s->device));
+    HIP_TRY(launch_uncount_after(sc->s->stream, view_of(sc), draws_dev, m, accepted_dev, accepted_cap));
+    return LILY_OK;
+}
+
 int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src) {
     if (dst == nullptr || src == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "scratch is null");

@@ -3300,16 +3300,39 @@ __global__ void k_refresh_pairs(ScratchView sc) {
 }
 
 // Saturating decrement; the id stays listed (with a count that may now be 0).
-__global__ void k_uncount(ScratchView sc, uint32_t token) {
-    if (blockIdx.x == 0 && threadIdx.x == 0 && token < sc.vocab) {
-        const uint32_t c = sc.counts[token];
-        if (c > 0u) {
-            sc.counts[token] = c - 1u;
-            const uint32_t p = sc.pos[token];
-            if (((sc.touched[token >> 5] >> (token & 31u)) & 1u) && p < sc.pairs_cap) {
-                sc.pairs[p].count = c - 1u;
-            }
+__device__ __forceinline__ void uncount_one(const ScratchView& sc, uint32_t token) {
+    if (token >= sc.vocab) {
+        return;
+    }
+    const uint32_t c = sc.counts[token];
+    if (c > 0u) {
+        sc.counts[token] = c - 1u;
+        const uint32_t p = sc.pos[token];
+        if (((sc.touched[token >> 5] >> (token & 31u)) & 1u) && p < sc.pairs_cap) {
+            sc.pairs[p].count = c - 1u;
         }
+    }
+}
+
+__global__ void k_uncount(ScratchView sc, uint32_t token) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        uncount_one(sc, token);
+    }
+}
+
+// The rollback of the rejected rows' draws (src/qwen4exp/spec.rs:213-217) with the accepted
+// row read on the device: draws[a + 1 .. m) are un-counted in order, a = min(accepted[0], cap).
+__global__ void k_uncount_after(ScratchView sc, const uint32_t* draws, uint32_t m,
+                                const uint32_t* accepted, uint32_t cap) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) {
+        return;
+    }
+    const uint32_t a = min(accepted[0], cap);
+    if (a >= m) {
+        return;
+    }
+    for (uint32_t j = a + 1u; j < m; ++j) {
+        uncount_one(sc, draws[j]);
     }
 }
 
@@ -3426,6 +3449,12 @@ hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const u
 
 hipError_t launch_uncount(hipStream_t stream, const ScratchView& sc, uint32_t token) {
     hipLaunchKernelGGL(k_uncount, dim3(1), dim3(64), 0, stream, sc, token);
+    return hipGetLastError();
+}
+
+hipError_t launch_uncount_after(hipStream_t stream, const ScratchView& sc, const uint32_t* draws,
+                                uint32_t m, const uint32_t* accepted, uint32_t cap) {
+    hipLaunchKernelGGL(k_uncount_after, dim3(1), dim3(64), 0, stream, sc, draws, m, accepted, cap);
     return hipGetLastError();
 }
 

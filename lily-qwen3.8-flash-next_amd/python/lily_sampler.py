@@ -122,6 +122,7 @@ def _load():
         "lily_scratch_create": [vp, u32, C.POINTER(vp)],
         "lily_scratch_reset_counts": [vp],
         "lily_scratch_uncount": [vp, u32],
+        "lily_scratch_uncount_after": [vp, vp, u32, vp, u32],
         "lily_scratch_copy_counts_from": [vp, vp],
         "lily_scratch_add_history": [vp, vp, u32],
         "lily_scratch_write_counts": [vp, vp],
@@ -423,6 +424,12 @@ class SamplerScratch:
 
     def uncount(self, token):
         _check(_lib.lily_scratch_uncount(self._h, token))
+
+    def uncount_after(self, draws, accepted, accepted_cap=0xFFFFFFFF):
+        """Un-counts draws[a + 1:], a = min(accepted[0], accepted_cap), read on the device
+        (`draws`, `accepted`: int32 device tensors)."""
+        _check(_lib.lily_scratch_uncount_after(self._h, draws.data_ptr(), draws.numel(),
+                                               accepted.data_ptr(), accepted_cap))
 
     def reset_counts(self):
         _check(_lib.lily_scratch_reset_counts(self._h))

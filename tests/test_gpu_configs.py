@@ -151,6 +151,55 @@ def test_config3_speculative_verify(sampler):
         dists.close()
 
 
+def test_rollback_of_rejected_draws_on_the_device(sampler):
+    """finish_speculation's rollback (src/qwen4exp/spec.rs:213-217) with the accepted row read
+    from the control block on the device: the counts equal the oracle's uncount over
+    sampled[accepted + 1:], the list the draws read stays consistent with them (a further
+    penalised draw agrees with the oracle), and an earlier stop of the engine caps the row."""
+    rng = np.random.default_rng(77)
+    vocab = 151_936
+    x = rng.normal(0, 3, (2, vocab)).astype(np.float32)
+    kw = dict(temperature=0.7, top_k=20, top_p=0.95, seed=5, repetition_penalty=1.3,
+              presence_penalty=0.5, frequency_penalty=0.25)
+    hist = rng.integers(0, vocab, 600).astype(np.int32)
+    top = np.argsort(-x[0])[:6].astype(np.int32)          # ids a penalised draw looks at
+    hist[:12] = np.repeat(top[:4], 3)
+    cases = [
+        # draws, accepted word, cap
+        ([int(top[0]), int(top[1]), int(top[1]), int(top[2])], 1, 0xFFFFFFFF),
+        ([int(top[0]), int(top[1]), int(top[2]), int(top[3])], 3, 0xFFFFFFFF),   # all accepted
+        ([int(top[0]), int(top[1]), int(top[2]), int(top[3])], 3, 0),            # engine stopped at row 0
+        ([int(top[3]), vocab + 9, 12345, int(top[3])], 0, 0xFFFFFFFF),           # out of range, never counted
+        ([int(top[0])], 0, 0xFFFFFFFF),                                          # one row: nothing after it
+        ([int(top[5])] * 8, 2, 5),                                               # saturates at 0
+    ]
+    for draws, acc, cap in cases:
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(hist).to(dev()))
+        counts = np.bincount(hist, minlength=vocab).astype(np.uint32)
+        m = len(draws)
+        t_draws = torch.from_numpy(np.array(draws, dtype=np.uint32).view(np.int32)).to(dev())
+        ctrl = torch.zeros(LS.ctrl_words(2), dtype=torch.int32, device=dev())
+        ctrl[LS.SLOT_ACCEPTED * LS.CTRL_STRIDE] = acc
+        sc.uncount_after(t_draws, ctrl[LS.SLOT_ACCEPTED * LS.CTRL_STRIDE:], cap)
+        for t in draws[min(acc, cap) + 1:]:
+            O.lib().lo_uncount(counts.ctypes.data, vocab, t)
+        assert np.array_equal(sc.read_counts().numpy().view(np.uint32), counts), (draws, acc, cap)
+        for step in (3, 4):
+            r = run_rows(sampler, x[:1], [kw], [step], scratch=[sc])
+            d = O.sample(x[0], counts, o_params(**kw), step)   # bumps counts[chosen] like the kernel
+            check_row_against_oracle(r, 0, d)
+        assert np.array_equal(sc.read_counts().numpy().view(np.uint32), counts)
+        sc.close()
+    with pytest.raises(LS.SamplerError):
+        sc2 = LS.SamplerScratch(sampler, vocab)
+        try:
+            sc2.uncount_after(torch.zeros(9, dtype=torch.int32, device=dev()),
+                              torch.zeros(1, dtype=torch.int32, device=dev()))
+        finally:
+            sc2.close()
+
+
 def test_config4_constrained_bf16(sampler):
     c = W.config4(rows=64)
     x = c["logits"]
