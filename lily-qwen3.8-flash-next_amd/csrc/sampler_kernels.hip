@@ -615,6 +615,10 @@ __device__ __forceinline__ void phase(const LaunchCfg& cfg, uint32_t i) {
     if (cfg.phase_trace != nullptr && threadIdx.x == 0) {
         cfg.phase_trace[((size_t)blockIdx.y * cfg.slices + blockIdx.x) * PHASE_SLOTS + i] =
             wall_clock64();
+        // The store is waited for here, where it is rare: a store still in flight next to
+        // loads makes every later wait for a load drain all loads in flight (stores and
+        // loads share one counter and complete in no fixed order).
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     }
 }
 
@@ -1611,21 +1615,23 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     StreamLds L;
     L.init();
 
-    // Blocks lying wholly inside the streamed chunks are loaded without per-load checks.
+    // Every load of a block is issued whatever its chunk: a conditional load makes the wait
+    // for its result drain every load in flight, the blocks requested ahead included.  Chunks
+    // past the slice's end read its last chunk instead (every chunk of the slice holds an
+    // element of the row, so the 16 bytes are readable); chunks that are not streamed are
+    // replaced by -inf when the block is worked on (`full_block`).
+    const uint32_t c_last = g.ce - 1u;  // nblocks > 0 wherever a block is fetched
     auto fetch = [&](u32x4 (&dst)[U], uint32_t b) {
-        const uint32_t c0 = g.cb + b * BLOCK;
-        if (c0 >= g.main_lo && c0 + BLOCK <= g.main_hi) {
-            const uint32_t off = (c0 + tid) << 4;  // the stream path's rows are below 4 GiB
+        const uint32_t c0 = g.cb + b * BLOCK + tid;
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                dst[u] = gload(reinterpret_cast<const u32x4*>(g.base + (off + (uint32_t)u * NT * 16u)));
-            }
-        } else {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                dst[u] = g.load_raw(c0 + (uint32_t)u * NT + tid);
-            }
+        for (int u = 0; u < U; ++u) {
+            const uint32_t c = min(c0 + (uint32_t)u * NT, c_last);
+            dst[u] = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));  // rows are below 4 GiB
         }
+    };
+    auto full_block = [&](uint32_t b) -> bool {
+        const uint32_t c0 = g.cb + b * BLOCK;
+        return c0 >= g.main_lo && c0 + BLOCK <= g.main_hi;
     };
     // ---- the slice's listed ids, bucketed by block
     // The first PREG x NT list entries are requested together with the list's length (the
@@ -1990,18 +1996,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         float raw;
         u32x4 chunk;
     };
+    // Unconditional as well: a thread without an entry reads the slice's last chunk.
     auto listed_fetch = [&](Listed& r, uint32_t b, uint32_t round) {
-        r.ent = NONE;
         r.raw = 0.0f;
-        r.chunk = u32x4{0u, 0u, 0u, 0u};
         const uint32_t lo = L.bkt[b], hi = L.bkt[b + 1];
         const uint32_t e = lo + round * NT + ((tid + NT - ((b * 64u) % NT)) % NT);
-        if (e < hi) {
-            r.ent = L.spec[e];
-            const uint32_t id = r.ent & ID_MASK;
-            const uint32_t c = (id + g.pad) / E;
-            r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (size_t)c * 16));
-        }
+        r.ent = e < hi ? L.spec[min(e, SPEC_CAP - 1u)] : NONE;
+        const uint32_t c = min(((r.ent & ID_MASK) + g.pad) / E, c_last);
+        r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
     };
     // The id's own logit out of its chunk (one gather per listed id, not two).
     auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
@@ -2024,6 +2026,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         uint32_t cnt = r.ent >> SPEC_ID_BITS;
         if (cnt == 4095u) {
             cnt = gload(a.counts + id);
+            // The value is waited for here, inside the branch: waiting after it would make
+            // every thread drain the loads it has in flight.
+            asm volatile("" : "+v"(cnt));
         }
         float t = r.raw;
         for (uint32_t j = 0; j < n_bias; ++j) {
@@ -2084,7 +2089,17 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     lst_a.ent = NONE;
     lst_b.ent = NONE;
     lst_c.ent = NONE;
-    auto work = [&](const u32x4 (&cur)[U], Listed& lcur, uint32_t b) {
+    auto work = [&](u32x4 (&cur)[U], Listed& lcur, uint32_t b) {
+        if (!full_block(b)) {
+            const uint32_t ninf = DT == LILY_BF16 ? 0xff80ff80u : 0xff800000u;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t c = g.cb + (b * U + u) * NT + tid;
+                if (c < g.main_lo || c >= g.main_hi) {
+                    cur[u] = u32x4{ninf, ninf, ninf, ninf};
+                }
+            }
+        }
         const float lcur_t = listed_row ? listed_value(lcur) : NEG_INF;
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
@@ -2172,29 +2187,34 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
     };
+    // A request past the last block asks for the last block again (its lines are in the
+    // cache and nothing uses the result): with the same loads in flight on every path the
+    // wait for a block's data leaves the blocks requested after it in flight, where a request
+    // that may be skipped makes that wait count as if it had been.
+    auto request = [&](u32x4 (&dst)[U], Listed& ldst, uint32_t b) {
+        const uint32_t bb = min(b, nblocks - 1u);
+        if (listed_row) {
+            listed_fetch(ldst, bb, 0);
+        }
+        fetch(dst, bb);
+    };
     if (nblocks == 0) {
         refresh_bound(true, true);  // the same barriers in every workgroup
-    } else if (listed_row) {
-        listed_fetch(lst_a, 0, 0);
-    }
-    auto request = [&](u32x4 (&dst)[U], Listed& ldst, uint32_t b) {
-        if (b < nblocks) {
-            if (listed_row) {
-                listed_fetch(ldst, b, 0);
-            }
-            fetch(dst, b);
+    } else {
+        if (listed_row) {
+            listed_fetch(lst_a, 0, 0);
         }
-    };
-    request(buf_b, lst_b, 1);
-    for (uint32_t b = 0; b < nblocks; b += 3) {
-        request(buf_c, lst_c, b + 2);
-        work(buf_a, lst_a, b);
-        if (b + 1 < nblocks) {
-            request(buf_a, lst_a, b + 3);
-            work(buf_b, lst_b, b + 1);
-            if (b + 2 < nblocks) {
-                request(buf_b, lst_b, b + 4);
-                work(buf_c, lst_c, b + 2);
+        request(buf_b, lst_b, 1);
+        for (uint32_t b = 0; b < nblocks; b += 3) {
+            request(buf_c, lst_c, b + 2);
+            work(buf_a, lst_a, b);
+            if (b + 1 < nblocks) {
+                request(buf_a, lst_a, b + 3);
+                work(buf_b, lst_b, b + 1);
+                if (b + 2 < nblocks) {
+                    request(buf_b, lst_b, b + 4);
+                    work(buf_c, lst_c, b + 2);
+                }
             }
         }
     }
@@ -2953,9 +2973,12 @@ __device__ __forceinline__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>
     float bv = NEG_INF;
     uint32_t bi = 0xffffffffu;
     for (uint32_t c0 = g.cb; c0 < g.ce; c0 += NT * UNROLL) {
+        // Unconditional loads (chunks past the slice's end read its last chunk; `inside`
+        // below discards them): a load that may be skipped is waited for as the last one issued.
         u32x4 raw[UNROLL];
         for (int u = 0; u < UNROLL; ++u) {
-            raw[u] = g.load_raw(c0 + u * NT + tid);
+            const uint32_t c = min(c0 + u * NT + tid, g.ce - 1u);
+            raw[u] = gload(reinterpret_cast<const u32x4*>(g.base + (size_t)c * 16));
         }
         for (int u = 0; u < UNROLL; ++u) {
             const uint32_t c = c0 + u * NT + tid;
