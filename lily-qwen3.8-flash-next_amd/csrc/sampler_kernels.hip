@@ -2089,7 +2089,24 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     lst_a.ent = NONE;
     lst_b.ent = NONE;
     lst_c.ent = NONE;
+    // The waves of a compute unit's oldest workgroup win the issue slots and its youngest
+    // finishes last, alone.  Rows that carry both listed ids and a row sum (the most
+    // instructions per block) lower their waves' priority as they advance, so a workgroup
+    // that fell behind catches up; lighter rows lose by it and leave the priority alone.
+    const bool paced = listed_row && want_lse;
     auto work = [&](u32x4 (&cur)[U], Listed& lcur, uint32_t b) {
+        if (paced) {
+            const uint32_t q = b * 4u / nblocks;
+            if (q == 0u) {
+                __builtin_amdgcn_s_setprio(3);
+            } else if (q == 1u) {
+                __builtin_amdgcn_s_setprio(2);
+            } else if (q == 2u) {
+                __builtin_amdgcn_s_setprio(1);
+            } else {
+                __builtin_amdgcn_s_setprio(0);
+            }
+        }
         if (!full_block(b)) {
             const uint32_t ninf = DT == LILY_BF16 ? 0xff80ff80u : 0xff800000u;
 #pragma unroll
@@ -3433,6 +3450,14 @@ hipError_t launch_rows(hipStream_t stream, int dtype, int kind, bool lse, uint32
                        const LaunchCfg& cfg_in, const InlineRows* inline_rows, size_t dyn_bytes) {
     LaunchCfg cfg = cfg_in;
     cfg.dyn_slots = (uint32_t)(dyn_bytes / 8);
+#ifdef LILY_ONE_VARIANT
+    // For looking at one kernel's generated code (seconds instead of minutes): only the
+    // bf16 streaming kernels with a row sum are instantiated.  Never defined in a build that runs.
+    (void)dtype;
+    (void)kind;
+    (void)lse;
+    return launch_variant<LILY_BF16, 2, true>(stream, rows, cfg, inline_rows, dyn_bytes);
+#else
 #define LILY_DISPATCH(DT)                                                                     \
     switch (kind) {                                                                           \
         case 0:                                                                               \
@@ -3450,6 +3475,7 @@ hipError_t launch_rows(hipStream_t stream, int dtype, int kind, bool lse, uint32
     }
     LILY_DISPATCH(LILY_F32)
 #undef LILY_DISPATCH
+#endif
 }
 
 hipError_t launch_fill_u32(hipStream_t stream, uint32_t* p, uint32_t n, uint32_t v) {
