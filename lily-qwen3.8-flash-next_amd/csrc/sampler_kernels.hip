@@ -1640,7 +1640,11 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     uint32_t n_pairs = 0, loaded = 0;
     uint64_t early[PREG];
     if (pen) {
-        n_pairs = gload(a.n_pairs);
+        // The list's length comes through the scalar path (nothing writes it while the
+        // slices of its row still read it): a vector load of a value that is the same in
+        // every lane is moved to a scalar register at once, and that move would hold the
+        // list's loads below back until the length had arrived.
+        n_pairs = *(const LILY_CONST uint32_t*)a.n_pairs;
         // The host's bound of the length says how much to request; a longer list is still
         // read completely (by the loop further down), a shorter one costs idle loads.
         const uint64_t want = ((uint64_t)a.pairs_hint + cfg.hint_growth + NT - 1) / NT * NT;
