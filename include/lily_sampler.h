@@ -167,7 +167,11 @@ int lily_draft_dists_slot(const lily_draft_dists_t* d, uint32_t i, lily_draft_di
 
 /* ---- single-row draws (the reference's call signature) --------------------------------- */
 
-/* sample_f32 (sample.rs:373-387): one draw from logits_dev[vocab] into out_dev[0].
+/* Logits are read in whole 16-byte aligned blocks: up to 15 bytes before a row's first and
+ * after its last element are read and discarded (never beyond the aligned blocks the row
+ * itself occupies).
+ *
+ * sample_f32 (sample.rs:373-387): one draw from logits_dev[vocab] into out_dev[0].
  * Greedy without penalties is the exact first-max argmax; otherwise penalties,
  * temperature, top-k, top-p/min-p and the inverse-CDF draw on uniform_for(seed, step).
  * Under penalties counts[out] += 1.  `scratch` may be NULL when params use no penalties. */
