@@ -2239,6 +2239,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
     }
+    if (paced) {
+        __builtin_amdgcn_s_setprio(0);  // a row of fewer than four blocks never reached it
+    }
     phase(cfg, 2);
 
     // ---- after the scan
