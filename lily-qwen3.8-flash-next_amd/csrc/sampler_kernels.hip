@@ -2312,7 +2312,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
 #pragma unroll
             for (int j = 0; j < E; ++j) {
                 if (!((dm >> j) & 1u)) {
-                    if (want_lse) {
+                    if (want_lse && v[j] > skip_b) {  // the cut of the streamed terms
                         acc_q += term_d(v[j]);
                     }
                     offer(v[j], g.id_of(c, j));
