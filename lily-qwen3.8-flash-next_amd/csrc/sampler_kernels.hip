@@ -2011,13 +2011,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     };
     // The id's own logit out of its chunk (one gather per listed id, not two).
     auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
+        // One compare picks the 8-byte half, one 64-bit shift the element inside it.
         const uint32_t j = (id + g.pad) % E;
-        const uint32_t w4 = E == 8 ? j >> 1 : j;
-        const uint32_t d = w4 == 0u ? q.x : (w4 == 1u ? q.y : (w4 == 2u ? q.z : q.w));
+        const bool upper = (j & (uint32_t)(E / 2)) != 0u;
+        const uint64_t half = upper ? (((uint64_t)q.w << 32) | q.z) : (((uint64_t)q.y << 32) | q.x);
         if (E == 8) {
-            return lilym_bits_f32((j & 1u) ? (d & 0xffff0000u) : (d << 16));
+            return lilym_bits_f32((uint32_t)(half >> ((j & 3u) * 16u)) << 16);
         }
-        return lilym_bits_f32(d);
+        return lilym_bits_f32((uint32_t)(half >> ((j & 1u) * 32u)));
     };
     // A listed id's true value before the temperature (bias in list order, then penalties);
     // also feeds the thread's maxima of listed raw and true values.
