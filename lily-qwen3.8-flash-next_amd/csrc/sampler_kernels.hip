@@ -2010,15 +2010,17 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
     };
     // The id's own logit out of its chunk (one gather per listed id, not two).
-    auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
-        // One compare picks the 8-byte half, one 64-bit shift the element inside it.
-        const uint32_t j = (id + g.pad) % E;
+    // Element j of a chunk: one compare picks the 8-byte half, one 64-bit shift the element.
+    auto elem_of = [&](const u32x4& q, uint32_t j) -> float {
         const bool upper = (j & (uint32_t)(E / 2)) != 0u;
         const uint64_t half = upper ? (((uint64_t)q.w << 32) | q.z) : (((uint64_t)q.y << 32) | q.x);
         if (E == 8) {
             return lilym_bits_f32((uint32_t)(half >> ((j & 3u) * 16u)) << 16);
         }
         return lilym_bits_f32((uint32_t)(half >> ((j & 1u) * 32u)));
+    };
+    auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
+        return elem_of(q, (id + g.pad) % E);
     };
     // A listed id's true value before the temperature (bias in list order, then penalties);
     // also feeds the thread's maxima of listed raw and true values.
@@ -2310,14 +2312,25 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             const uint32_t dm = (L.dmask[slot >> 2] >> ((slot & 3u) * 8u)) & 0xffu;
             float v[E];
             unpack<DT>(q, v);
+            // Few elements of a queued chunk matter (usually the one that got it queued):
+            // they are marked first and then taken one at a time, in ascending order, instead
+            // of eight branches that some lane of the wave enters every time.
+            uint32_t todo = 0;
 #pragma unroll
             for (int j = 0; j < E; ++j) {
-                if (!((dm >> j) & 1u)) {
-                    if (want_lse && v[j] > skip_b) {  // the cut of the streamed terms
-                        acc_q += term_d(v[j]);
-                    }
-                    offer(v[j], g.id_of(c, j));
+                const bool term = want_lse && v[j] > skip_b;  // the cut of the streamed terms
+                const bool cand = v[j] >= filt && v[j] > NEG_INF;
+                todo |= (term || cand) ? 1u << j : 0u;
+            }
+            todo &= ~dm;
+            while (todo != 0u) {
+                const uint32_t j = (uint32_t)__builtin_ctz(todo);
+                todo &= todo - 1u;
+                const float x = elem_of(q, j);
+                if (want_lse && x > skip_b) {
+                    acc_q += term_d(x);
                 }
+                offer(x, g.id_of(c, (int)j));
             }
         }
     }
