@@ -23,7 +23,7 @@ sys.path.insert(0, os.path.join(ROOT, "lily-qwen3.8-flash-next_amd", "python"))
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per 1024-row launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised
 # in profiles/k_rows_table_bf16_config5_b1024.md (valid for --rows 1024 only).
-MEASURED_TRAFFIC_BYTES = 333.9e6
+MEASURED_TRAFFIC_BYTES = 333.7e6
 
 
 def parse():
