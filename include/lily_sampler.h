@@ -189,6 +189,14 @@ int lily_sample_spec_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vo
                          lily_scratch_t* scratch, const lily_sampling_params* params,
                          uint32_t step, const lily_draft_dist* dist, const uint32_t* draft_dev,
                          uint32_t* out_dev);
+/* As lily_sample_spec_f32 with the two draws given instead of seeded: u1 stands in for
+ * uniform_for(seed, step) (the accept test and, for a greedy-free plain row, the draw) and u2
+ * for the residual draw's uniform_for(seed, step | 0x80000000) (sample.metal:626-651; the host
+ * twin uniform_for exists "for tests and replay", sample.rs:434-441).  Both in [0, 1). */
+int lily_sample_spec_f32_uniforms(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                                  lily_scratch_t* scratch, const lily_sampling_params* params,
+                                  uint32_t step, const lily_draft_dist* dist,
+                                  const uint32_t* draft_dev, uint32_t* out_dev, float u1, float u2);
 /* argmax_f32 (src/kernels/elementwise.rs:297-308): first max, lowest index on ties. */
 int lily_argmax_f32(lily_sampler_t* s, const float* x_dev, uint32_t n, uint32_t* out_dev);
 
@@ -207,13 +215,16 @@ int lily_copy_row_u32(lily_sampler_t* s, const uint32_t* src_dev, uint32_t rows,
  * (src/qwen4exp/spec.rs:414-424): rows j < m-1 are speculative draws against dists slot j
  * and proposal ids_dev[j+1] at step0+j, the last row a plain draw; row j sees the counts
  * of rows before it (one launch per row under penalties, one launch for all rows without).
- * verify_tokens_dev[m] receives the draws, ctrl_dev the control block. */
+ * verify_tokens_dev[m] receives the draws, ctrl_dev the control block (NULL: no spec_accept).
+ * uniforms: NULL, or host [m][2] = (u1, u2) per row replacing the seeded draws (the last
+ * row, a plain draw, uses its u1 only).  Every argument is validated before the first row is
+ * enqueued, so an error return leaves the counts untouched. */
 int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype, uint32_t vocab,
                      uint64_t row_stride, uint32_t m, lily_scratch_t* scratch,
                      const lily_sampling_params* params, uint32_t step0,
                      const lily_draft_dists_t* dists, const uint32_t* ids_dev,
                      uint32_t* verify_tokens_dev, uint32_t* ctrl_dev, uint32_t ctrl_words,
-                     uint32_t pos0, uint32_t ratio, uint32_t chain);
+                     uint32_t pos0, uint32_t ratio, uint32_t chain, const float* uniforms);
 
 /* ---- batched rows ---------------------------------------------------------------------- */
 

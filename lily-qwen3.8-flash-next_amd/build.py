@@ -1,35 +1,60 @@
 """Builds liblily_sampler_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
 
     python lily-qwen3.8-flash-next_amd/build.py
+
+The row kernel is compiled once per (logits type, kernel kind) pair from rows_variant.hip, in
+parallel; the objects are linked with the small kernels and the C-ABI layer.
 """
+import concurrent.futures
 import os
 import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "liblily_sampler_hip.so")
-SOURCES = ["sampler_kernels.hip", "sampler_api.cpp"]
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # Token ids depend on exact f32 arithmetic: no contraction into FMAs, IEEE division
     # (hipcc's default), denormals kept (hipcc's default).
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
 ]
+VARIANTS = [(dt, kind) for dt in (0, 1) for kind in (0, 1, 2)]
+NOISE = "is not a recognized feature for this target"
 
 
-def build(verbose=False):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
+def units():
+    """(source, object, extra flags) of every translation unit."""
+    out = [("rows_variant.hip", f"rows_dt{dt}_kind{kind}.o", [f"-DLILY_DT={dt}", f"-DLILY_KIND={kind}"])
+           for dt, kind in VARIANTS]
+    out.append(("scratch_kernels.hip", "scratch_kernels.o", []))
+    out.append(("sampler_api.cpp", "sampler_api.o", []))
+    return out
+
+
+def _run(cmd):
     res = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
-    if verbose or res.returncode != 0:
-        sys.stderr.write(err + "\n")
+    err = "\n".join(l for l in res.stderr.splitlines() if NOISE not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + err)
+        raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + err)
+    return err
+
+
+def build(verbose=False, jobs=None):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    cmds = [[hipcc] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ, obj)]
+            for src, obj, extra in units()]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        for err in pool.map(_run, cmds):
+            if verbose and err.strip():
+                sys.stderr.write(err + "\n")
+    objs = [os.path.join(OBJ, obj) for _, obj, _ in units()]
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB])
     return LIB
 
 

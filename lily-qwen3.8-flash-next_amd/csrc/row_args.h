@@ -100,7 +100,7 @@ struct LaunchCfg {
     uint64_t* phase_trace;  // null, or [rows][slices][PHASE_SLOTS] 100 MHz timestamps
     uint32_t excl_words;    // words reserved for the slice bitmap (the specials' id list follows)
     uint32_t list_cap;      // ids the specials' list holds
-    uint32_t old_layout;    // dynamic LDS holds cand_cap candidates + the bitmap + the id list
+    uint32_t bitmap_layout;    // dynamic LDS holds cand_cap candidates + the bitmap + the id list
     uint32_t hint_growth;   // added to every row's pairs_hint (draws since the table was packed)
     uint32_t dyn_slots;     // 64-bit slots of dynamic LDS in all
     uint32_t* path_stats;   // null, or [4] counters: slices finished by the streaming select, the

@@ -1,0 +1,351 @@
+// row_kernel.h - the row kernel: one launch serves a batch of logits rows.  Row r is scanned
+// by `slices` workgroups of 256 threads (grid = slices x rows).  Each workgroup finds the exact
+// top-k of its slice; with several slices the last workgroup to arrive (an atomic ticket,
+// nobody waits) merges them.  That workgroup then runs the tail.
+#pragma once
+
+#include "device_common.h"
+#include "select_bitmap.h"
+#include "select_exhaustive.h"
+#include "select_sparse.h"
+#include "select_stream.h"
+#include "tail.h"
+
+namespace lily {
+
+// ------------------------------------------------------------------ argmax
+
+// First maximum under float comparison (NaN never wins, -0 == +0), lowest id on
+// ties: elementwise.metal:145-150.  Result: the best (value, id) of the slice as a
+// composite; id bits all zero when no element qualified.
+template <int DT>
+__device__ __forceinline__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>& g, Shared& sh) {
+    constexpr int E = Geo<DT>::E;
+    const uint32_t tid = threadIdx.x;
+    float bv = NEG_INF;
+    uint32_t bi = 0xffffffffu;
+    for (uint32_t c0 = g.cb; c0 < g.ce; c0 += NT * UNROLL) {
+        // Unconditional loads (chunks past the slice's end read its last chunk; `inside`
+        // below discards them): a load that may be skipped is waited for as the last one issued.
+        u32x4 raw[UNROLL];
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t c = min(c0 + u * NT + tid, g.ce - 1u);
+            raw[u] = gload(reinterpret_cast<const u32x4*>(g.base + (size_t)c * 16));
+        }
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t c = c0 + u * NT + tid;
+            float v[E];
+            unpack<DT>(raw[u], v);
+            for (int j = 0; j < E; ++j) {
+                const uint32_t id = g.id_of(c, j);
+                const bool inside = c >= g.main_lo && c < g.main_hi;
+                const float x = v[j];
+                if (inside && (x > bv || (x == bv && id < bi))) {
+                    bv = x;
+                    bi = id;
+                }
+            }
+        }
+    }
+    for (int side = 0; side < 2; ++side) {
+        const uint32_t lo = side == 0 ? g.id_lo : g.edge_hi_begin;
+        const uint32_t hi = side == 0 ? g.edge_lo_end : g.id_hi;
+        for (uint32_t id = lo + tid; id < hi; id += NT) {
+            const float x = load_logit<DT>(a.logits, id);
+            if (x > bv || (x == bv && id < bi)) {
+                bv = x;
+                bi = id;
+            }
+        }
+    }
+    uint64_t best = ((uint64_t)lilym_order_key(bv + 0.0f) << 32) | (uint32_t)(~bi);
+    best = wave_max_u64(best);
+    if ((tid & 63u) == 0) {
+        sh.red_u[tid >> 6] = best;
+    }
+    __syncthreads();
+    best = sh.red_u[0];
+    for (int i = 1; i < NWAVE; ++i) {
+        best = sh.red_u[i] > best ? sh.red_u[i] : best;
+    }
+    __syncthreads();
+    return best;
+}
+
+// ------------------------------------------------------------------ the row kernel
+
+template <int DT, int KIND, bool LSE>
+__device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
+    // KIND: 0 = rows without masks, penalties or bias lists, 1 = rows with any of them (the
+    // bitmap select is compiled for them), 2 = streaming rows only (no bitmap select at all).
+    constexpr bool EXCL = KIND == 1;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t s = blockIdx.x, row = blockIdx.y, S = cfg.slices;
+    const uint32_t vocab = cfg.vocab;
+    const uint32_t step = a.step + cfg.step_delta;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    uint64_t* cand = dyn_lds;
+    uint64_t* found = cand;  // where the select left the slice's candidates
+    uint32_t* excl = reinterpret_cast<uint32_t*>(dyn_lds + cfg.cand_cap);
+
+    if ((a.flags & F_FORCED) && !want_lse) {
+        if (s == 0 && tid == 0) {
+            emit(a, a.forced);
+        }
+        return;
+    }
+
+    Geo<DT> g;
+    g.init(a.logits, vocab, s, S);
+    phase(cfg, 0);
+
+    const bool argmax = a.mode == MODE_ARGMAX;
+    uint64_t best = 0;
+    bool sorted = false;
+    if (argmax) {
+        best = slice_argmax<DT>(a, g, sh);
+    } else {
+        // A forced row with a log-probability needs the row sum only: it takes the same
+        // selects (their sums are the fast ones) and its candidates are dropped below.
+        bool done = false;
+        uint32_t took = 2;
+        if (cfg.path == 0u && (a.flags & F_STREAM)) {
+            done = select_stream<DT, LSE, KIND != 2>(a, g, a.k, sh, cfg, sorted, found);
+            took = done ? 0u : took;
+            if (!done) {
+                __syncthreads();
+            }
+        }
+        if (KIND == 1 && !done && cfg.path == 0u && a.allow != nullptr) {
+            done = select_sparse<DT, LSE>(a, g, a.k, cand, min(cfg.dyn_slots, MERGE_CAP), sh, sorted);
+            took = done ? 1u : took;
+        }
+        if (KIND != 2 && !done && cfg.path != 1u && cfg.bitmap_layout != 0u) {
+            const bool special = a.allow != nullptr || (a.flags & F_PEN) || a.n_bias != 0;
+            if (EXCL || !special) {
+                // A single pass whose running bound let too many candidates in is repeated
+                // as two passes (bound first, then collect) before the exhaustive select.
+#pragma nounroll
+                for (int attempt = 0; attempt < 2 && !done; ++attempt) {
+                    const bool two_pass = a.k > 64u || cfg.path == 2u || attempt == 1;
+                    if (attempt == 1) {
+                        __syncthreads();
+                    }
+                    done = select_fast<DT, EXCL, LSE>(a, g, a.k, two_pass, cand, cfg.cand_cap, excl, sh,
+                                                      cfg, sorted);
+                    if (a.k > 64u || cfg.path == 2u) {
+                        break;  // it was two passes already
+                    }
+                }
+                took = done ? 1u : took;
+            }
+        }
+        if (cfg.path_stats != nullptr && tid == 0) {
+            atomicAdd(&cfg.path_stats[took], 1u);
+        }
+        if (!done) {
+            __syncthreads();
+            sorted = false;
+            select_exhaustive<DT>(a, g.id_lo, g.id_hi, a.k, want_lse, cand, cfg.cand_cap, sh);
+        }
+    }
+
+    const bool forced = (a.flags & F_FORCED) != 0;
+    uint32_t n = (argmax || forced) ? 0u : min(sh.n_cand, cfg.cand_cap);
+    phase(cfg, 4);
+    if (S > 1) {
+        const size_t slot = (size_t)row * S + s;
+        // Partials go through to memory (no dirty L2 lines to write back), the wave waits
+        // for its stores, the workgroup meets, and one thread takes the row's ticket.
+        if (argmax) {
+            if (tid == 0) {
+                store_through(&cfg.ws_cand[slot * cfg.ws_k], best);
+            }
+        } else {
+            // Every slot is written (0 = no candidate), so the merge needs no counts.
+            for (uint32_t i = tid; !forced && i < cfg.ws_k; i += NT) {
+                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], i < n ? found[i] : (uint64_t)0);
+            }
+            if (tid == 0) {
+                store_through(&cfg.ws_lse[2 * slot], want_lse ? sh.lse_mc : 0.0);
+                store_through(&cfg.ws_lse[2 * slot + 1], want_lse ? sh.lse_s : 0.0);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+            sh.last = (t == S - 1) ? 1u : 0u;
+        }
+        __syncthreads();
+        phase(cfg, 5);
+        if (sh.last == 0u) {
+            return;
+        }
+        if (tid == 0) {
+            store_through(&cfg.ws_ticket[row], 0u);
+        }
+        const size_t base = (size_t)row * S;
+        if (argmax) {
+            best = 0;
+            for (uint32_t t = tid; t < S; t += NT) {
+                const uint64_t c = load_through(&cfg.ws_cand[(base + t) * cfg.ws_k]);
+                best = c > best ? c : best;
+            }
+            best = wave_max_u64(best);
+            if ((tid & 63u) == 0) {
+                sh.red_u[tid >> 6] = best;
+            }
+            __syncthreads();
+            best = sh.red_u[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                best = sh.red_u[i] > best ? sh.red_u[i] : best;
+            }
+        } else {
+            // Gather every slice's candidates (0 = no candidate) and the log-sum-exp partials
+            // in one round trip.
+            constexpr int PER = MERGE_CAP / NT;
+            const uint32_t slots = S * cfg.ws_k;
+            uint64_t mine[PER];
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const uint32_t j = tid + (uint32_t)q * NT;
+                mine[q] = (!forced && j < slots) ? load_through(&cfg.ws_cand[base * cfg.ws_k + j]) : 0ull;
+            }
+            if (want_lse && tid < 64) {
+                double mt = -__builtin_huge_val(), st = 0.0;
+                if (tid < S) {
+                    mt = load_through(&cfg.ws_lse[2 * (base + tid)]);
+                    st = load_through(&cfg.ws_lse[2 * (base + tid) + 1]);
+                    if (!(st > 0.0)) {
+                        mt = -__builtin_huge_val();
+                    }
+                }
+                double m = mt;
+                for (int o = 32; o > 0; o >>= 1) {
+                    m = fmax(m, __shfl_xor(m, o));
+                }
+                const double sum = wave_sum_d(st > 0.0 ? st * exp2(mt - m) : 0.0);
+                if (tid == 0) {
+                    sh.lse_mc = m;
+                    sh.lse_s = sum;
+                }
+            }
+            // A bound of the k-th largest from the lanes' best entries (as in the streaming
+            // select: each wave's ceil(k / NWAVE)-th largest lane maximum, the minimum over the
+            // waves), then only entries at or above it are ranked.
+            uint64_t best_mine = 0;
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                best_mine = mine[q] > best_mine ? mine[q] : best_mine;
+            }
+            const uint32_t kw = (a.k + NWAVE - 1) / NWAVE;
+            const uint32_t P = kw <= 64u ? wave_kth_key16((uint32_t)(best_mine >> 48), kw) : 0u;
+            if ((tid & 63u) == 0) {
+                sh.red_i[tid >> 6] = P;
+            }
+            if (tid == 0) {
+                sh.n_cand = 0;
+            }
+            __syncthreads();
+            uint32_t bound = sh.red_i[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                bound = min(bound, sh.red_i[i]);
+            }
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                if (mine[q] != 0ull && (uint32_t)(mine[q] >> 48) >= bound) {
+                    cand[atomicAdd(&sh.n_cand, 1u)] = mine[q];
+                }
+            }
+            __syncthreads();
+            n = sh.n_cand;
+            sorted = false;
+            n = select_topk(cand, n, a.k, sh, sorted);
+            found = cand;
+        }
+    }
+
+    phase(cfg, 6);
+    if (argmax) {
+        if (tid == 0) {
+            const uint32_t id = composite_id(best);
+            *a.out_id = id == 0xffffffffu ? 0u : id;
+        }
+        return;
+    }
+    if (a.flags & F_FORCED) {
+        if (tid == 0) {
+            finish_token<DT>(a, sh, a.forced, vocab);
+        }
+        return;
+    }
+    tail<DT, KIND != 2>(a, vocab, step, n, sorted, found, sh, cfg);
+    phase(cfg, 7);
+}
+
+// Dynamic LDS: [0, cand_cap) candidates while scanning, then the bitmap.  In the tail the
+// first K_CAP slots hold the sorted candidates and the three float arrays follow them
+// (the launcher sizes the region for at least K_CAP * 8 + 3 * K_CAP * 4 bytes).
+__device__ __forceinline__ void tail_arrays(Shared& sh) {
+    float* f = reinterpret_cast<float*>(dyn_lds + K_CAP);
+    sh.prob = f;
+    sh.cum = f + K_CAP;
+    sh.res = f + 2 * K_CAP;
+}
+
+// The row's arguments are the same for every thread: read through the constant address
+// space they arrive by scalar loads and stay in scalar registers.
+__device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowArgs* src) {
+    static_assert(sizeof(RowArgs) % 16 == 0, "RowArgs is copied in 16-byte pieces");
+    const LILY_CONST u32x4* from = (const LILY_CONST u32x4*)src;
+    u32x4* to = reinterpret_cast<u32x4*>(&a);
+    for (unsigned i = 0; i < sizeof(RowArgs) / 16; ++i) {
+        to[i] = from[i];
+    }
+}
+
+template <int DT, int KIND, bool LSE>
+__global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
+    __shared__ Shared sh;
+    // `rows` is the first kernel argument: index it in the kernel-argument segment itself
+    // (indexing the by-value copy would move all of it to scratch memory).
+    const LILY_CONST RowArgs* table =
+        (const LILY_CONST RowArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+    RowArgs a;
+    load_row_args(a, table + blockIdx.y);
+    if (threadIdx.x == 0) {
+        tail_arrays(sh);
+    }
+    __syncthreads();
+    row_body<DT, KIND, LSE>(a, cfg, sh);
+}
+
+template <int DT, int KIND, bool LSE>
+__global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_table(LaunchCfg cfg) {
+    __shared__ Shared sh;
+    const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
+    RowArgs a;
+    load_row_args(a, table + blockIdx.y);
+    if (threadIdx.x == 0) {
+        tail_arrays(sh);
+    }
+    __syncthreads();
+    row_body<DT, KIND, LSE>(a, cfg, sh);
+}
+
+template <int DT, int KIND, bool LSE>
+static hipError_t launch_variant(hipStream_t stream, uint32_t rows, const LaunchCfg& cfg,
+                                 const InlineRows* inline_rows, size_t dyn_bytes) {
+    const dim3 grid(cfg.slices, rows), block(NT);
+    if (inline_rows != nullptr) {
+        hipLaunchKernelGGL((k_rows_inline<DT, KIND, LSE>), grid, block, dyn_bytes, stream,
+                           *inline_rows, cfg);
+    } else {
+        hipLaunchKernelGGL((k_rows_table<DT, KIND, LSE>), grid, block, dyn_bytes, stream, cfg);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace lily

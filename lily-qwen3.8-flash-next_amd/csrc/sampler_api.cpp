@@ -103,7 +103,7 @@ struct LaunchPart {
     bool lse = false;
     size_t dyn_bytes = 0;
     uint32_t excl_words = 0;
-    bool old_layout = false;
+    bool bitmap_layout = false;
     uint32_t cand_cap = 0;
     uint32_t listed = 0;                     // longest scratch list when the table was packed
 };
@@ -333,11 +333,11 @@ void attach_trace(const lily_sampler* s, LaunchCfg* cfg, uint32_t rows) {
 struct LaunchShape {
     bool excl = false;
     bool lse = false;
-    bool old_layout = false;
+    bool bitmap_layout = false;
     size_t dyn_bytes = 0;
     uint32_t excl_words = 0;
     uint32_t cand_cap = 0;
-    int kind() const { return old_layout ? (excl ? 1 : 0) : 2; }
+    int kind() const { return bitmap_layout ? (excl ? 1 : 0) : 2; }
 };
 
 LaunchShape shape_of(const lily_sampler* s, const RowArgs* rows, uint32_t n, int dtype,
@@ -359,7 +359,7 @@ LaunchShape shape_of(const lily_sampler* s, const RowArgs* rows, uint32_t n, int
     // Rows outside the streaming select need the candidate buffer, the id list and (rows with
     // an allow-mask) the slice bitmap; a launch of streaming rows only falls back to the
     // exhaustive select.
-    sh.old_layout = any_old;
+    sh.bitmap_layout = any_old;
     if (any_old) {
         const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
         const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
@@ -433,7 +433,7 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
         part.lse = shp.lse;
         part.dyn_bytes = shp.dyn_bytes;
         part.excl_words = shp.excl_words;
-        part.old_layout = shp.old_layout;
+        part.bitmap_layout = shp.bitmap_layout;
         part.cand_cap = shp.cand_cap;
     }
     return n_parts;
@@ -447,7 +447,7 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
         attach_trace(s, &cfg, part.rows);
     }
     cfg.excl_words = part.excl_words;
-    cfg.old_layout = part.old_layout ? 1u : 0u;
+    cfg.bitmap_layout = part.bitmap_layout ? 1u : 0u;
     cfg.cand_cap = part.cand_cap;
     cfg.hint_growth = hint_growth;
     HIP_TRY(launch_rows(s->stream, dtype, part.kind, part.lse, part.rows, cfg, nullptr, part.dyn_bytes));
@@ -463,7 +463,7 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     attach_trace(s, &cfg, n);
     const LaunchShape shp = shape_of(s, rows.r, n, dtype, vocab, slices, kmax);
     cfg.excl_words = shp.excl_words;
-    cfg.old_layout = shp.old_layout ? 1u : 0u;
+    cfg.bitmap_layout = shp.bitmap_layout ? 1u : 0u;
     cfg.cand_cap = shp.cand_cap;
     HIP_TRY(launch_rows(s->stream, dtype, shp.kind(), shp.lse, n, cfg, &rows, shp.dyn_bytes));
     return LILY_OK;
@@ -471,12 +471,11 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
 
 int one_row(lily_sampler* s, const void* logits, int dtype, uint32_t vocab, lily_scratch* scratch,
             const lily_sampling_params* params, uint32_t step, uint32_t mode, uint32_t* out,
-            const lily_draft_dist* dist, const uint32_t* draft) {
+            const lily_draft_dist* dist, const uint32_t* draft, const RowExtras& x = RowExtras()) {
     if (s == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "sampler is null");
     }
     InlineRows rows;
-    RowExtras x;
     if (int rc = pack_row(&rows.r[0], logits, vocab, scratch, params, step, mode, out, dist, draft, x)) {
         return rc;
     }
@@ -983,6 +982,32 @@ int lily_sample_spec_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vo
                    draft_dev);
 }
 
+// A draw's uniforms lie in [0, 1) like uniform_for's (sample.rs:435-441).
+static int check_uniform(float u, const char* name) {
+    if (!(u >= 0.0f && u < 1.0f)) {
+        return fail(LILY_ERR_INVALID_ARG, "%s must lie in [0, 1)", name);
+    }
+    return LILY_OK;
+}
+
+int lily_sample_spec_f32_uniforms(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                                  lily_scratch_t* scratch, const lily_sampling_params* params,
+                                  uint32_t step, const lily_draft_dist* dist,
+                                  const uint32_t* draft_dev, uint32_t* out_dev, float u1, float u2) {
+    if (int rc = check_uniform(u1, "u1")) {
+        return rc;
+    }
+    if (int rc = check_uniform(u2, "u2")) {
+        return rc;
+    }
+    RowExtras x;
+    x.has_uniform = true;
+    x.uniform = u1;
+    x.uniform2 = u2;
+    return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step, MODE_SPEC, out_dev, dist,
+                   draft_dev, x);
+}
+
 int lily_argmax_f32(lily_sampler_t* s, const float* x_dev, uint32_t n, uint32_t* out_dev) {
     lily_sampling_params g;
     lily_params_greedy(&g);
@@ -1032,7 +1057,7 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
                      const lily_sampling_params* params, uint32_t step0,
                      const lily_draft_dists_t* dists, const uint32_t* ids_dev,
                      uint32_t* verify_tokens_dev, uint32_t* ctrl_dev, uint32_t ctrl_words,
-                     uint32_t pos0, uint32_t ratio, uint32_t chain) {
+                     uint32_t pos0, uint32_t ratio, uint32_t chain, const float* uniforms) {
     if (s == nullptr || logits_dev == nullptr || ids_dev == nullptr || verify_tokens_dev == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "verify needs logits, ids and verify_tokens");
     }
@@ -1052,6 +1077,20 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
     if (sampled && m > 1 && (dists == nullptr || dists->slots < m - 1)) {
         return fail(LILY_ERR_RANGE, "verify needs %u draft distribution slots", m - 1);
     }
+    // Everything is validated before the first row is enqueued: an error leaves no draw counted.
+    if (ctrl_dev != nullptr) {
+        if (ctrl_words < lily_ctrl_words(chain)) {
+            return fail(LILY_ERR_RANGE, "control block too small for %u chain rows", chain);
+        }
+        if (ratio == 0) {
+            return fail(LILY_ERR_INVALID_ARG, "indexer block ratio must be nonzero");
+        }
+    }
+    for (uint32_t j = 0; uniforms != nullptr && j < 2 * m; ++j) {
+        if (int rc = check_uniform(uniforms[j], "verify uniforms")) {
+            return rc;
+        }
+    }
     const size_t es = dtype == LILY_BF16 ? 2 : 4;
     // Under penalties row j must see the counts of the rows before it: one launch per row.
     // Without them the rows are independent and share one launch.
@@ -1061,6 +1100,11 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
     for (uint32_t j = 0; j < m; ++j) {
         const char* row = static_cast<const char*>(logits_dev) + (size_t)j * row_stride * es;
         RowExtras x;
+        if (uniforms != nullptr) {
+            x.has_uniform = true;
+            x.uniform = uniforms[2 * j];
+            x.uniform2 = uniforms[2 * j + 1];
+        }
         lily_draft_dist slot;
         const bool spec = j + 1 < m && sampled;
         if (spec) {

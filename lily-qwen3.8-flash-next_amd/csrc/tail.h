@@ -1,0 +1,486 @@
+// tail.h - from a row's candidates to its token: sort, softmax over the candidates, the
+// sequential top-p / min-p prefix, the draw, the draft export and the speculative accept /
+// residual draw, and the bookkeeping of the emitted id.
+#pragma once
+
+#include "device_common.h"
+
+namespace lily {
+
+// ------------------------------------------------------------------ sort
+
+// Descending bitonic sort of cand[0..n), n <= 4 * NT, four entries per thread (entry
+// 4 * tid + r in register r; absent entries are 0, the smallest).  Exchanges at distance
+// 1 and 2 stay inside a thread, 4 .. 128 are lane shuffles inside a wave, and only the
+// three at distance 256 and 512 go through LDS with a barrier.
+__device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
+    static_assert(NT == 256, "four entries per thread cover 1024");
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    uint64_t v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t i = tid * 4u + (uint32_t)r;
+        v[r] = i < n ? cand[i] : 0ull;
+    }
+    __syncthreads();
+    auto exchange = [](uint64_t& lo, uint64_t& hi, bool desc) {  // lo sits at the lower index
+        const bool swap = (lo < hi) == desc;  // equal entries may swap: nothing changes
+        const uint64_t t = lo;
+        lo = swap ? hi : lo;
+        hi = swap ? t : hi;
+    };
+#pragma unroll
+    for (int lsize = 1; lsize <= 10; ++lsize) {
+#pragma unroll
+        for (int lstride = lsize - 1; lstride >= 0; --lstride) {
+            const uint32_t size = 1u << lsize, stride = 1u << lstride;
+            if (stride >= 4u * 64u) {
+                const uint32_t other = tid ^ (stride >> 2);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    cand[tid * 4u + (uint32_t)r] = v[r];
+                }
+                __syncthreads();
+                const bool desc = ((tid * 4u) & size) == 0;
+                const bool take_max = ((tid & (stride >> 2)) == 0) == desc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint64_t o = cand[other * 4u + (uint32_t)r];
+                    v[r] = ((o > v[r]) == take_max) ? o : v[r];
+                }
+                __syncthreads();
+            } else if (stride >= 4u) {
+                const uint32_t m = stride >> 2;
+                const bool desc = ((tid * 4u) & size) == 0;
+                const bool take_max = ((lane & m) == 0) == desc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint64_t o = shfl_xor_u64(v[r], (int)m);
+                    v[r] = ((o > v[r]) == take_max) ? o : v[r];
+                }
+            } else if (stride == 2u) {
+                const bool desc = ((tid * 4u) & size) == 0;  // size >= 4 here
+                exchange(v[0], v[2], desc);
+                exchange(v[1], v[3], desc);
+            } else {
+                if (size == 2u) {
+                    exchange(v[0], v[1], true);   // index bit 1 clear: descending
+                    exchange(v[2], v[3], false);  // set: ascending
+                } else {
+                    const bool desc = ((tid * 4u) & size) == 0;
+                    exchange(v[0], v[1], desc);
+                    exchange(v[2], v[3], desc);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        cand[tid * 4u + (uint32_t)r] = v[r];
+    }
+    __syncthreads();
+}
+
+// Descending sort of cand[0..n).  Up to 64 entries: one wave, in registers.  Up to 4 * NT:
+// four per thread in registers.  More: bitonic in LDS over the next power of two (the
+// buffer holds it).
+// BIG = false leaves the register sort out (kernels whose rows never sort more than 64).
+template <bool BIG>
+__device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
+    if (n <= 64) {
+        if (threadIdx.x < 64) {
+            const uint32_t lane = threadIdx.x;
+            uint64_t c = lane < n ? cand[lane] : 0ull;
+            for (uint32_t size = 2; size <= 64; size <<= 1) {
+                for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+                    const uint64_t o = shfl_xor_u64(c, (int)stride);
+                    const bool desc = (lane & size) == 0;
+                    const bool lower = (lane & stride) == 0;
+                    const bool take_max = lower == desc;
+                    c = take_max ? (o > c ? o : c) : (o < c ? o : c);
+                }
+            }
+            cand[lane] = c;
+        }
+        __syncthreads();
+        return;
+    }
+    if (BIG && n <= 4u * NT) {
+        sort_desc_regs(cand, n);
+        return;
+    }
+    uint32_t p = 128;
+    while (p < n) {
+        p <<= 1;
+    }
+    for (uint32_t i = n + threadIdx.x; i < p; i += NT) {
+        cand[i] = 0;
+    }
+    __syncthreads();
+    for (uint32_t size = 2; size <= p; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for (uint32_t i = threadIdx.x; i < (p >> 1); i += NT) {
+                const uint32_t pos = ((i / stride) * (stride << 1)) + (i % stride);
+                const uint32_t partner = pos + stride;
+                const bool desc = (pos & size) == 0;
+                const uint64_t x = cand[pos], y = cand[partner];
+                if (desc ? x < y : x > y) {
+                    cand[pos] = y;
+                    cand[partner] = x;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// ------------------------------------------------------------------ tail
+
+// Counts one emission of `id` in a scratch: the dense count, and the id's entry in the list
+// (appended with the first count; `touched` marks the listed ids).
+__device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched, CountPair* pairs,
+                                            uint32_t* n_pairs, uint32_t* pos, uint32_t pairs_cap,
+                                            uint32_t id) {
+    const uint32_t before = atomicAdd(&counts[id], 1u);
+    const uint32_t bit = 1u << (id & 31u);
+    const uint32_t bits = atomicOr(&touched[id >> 5], bit);
+    if ((bits & bit) == 0u) {
+        const uint32_t p = atomicAdd(n_pairs, 1u);
+        if (p < pairs_cap) {
+            pairs[p].id = id;
+            pairs[p].count = before + 1u;
+        }
+        pos[id] = p < pairs_cap ? p : 0xffffffffu;  // listed ids always have a meaningful pos
+    } else {
+        const uint32_t p = pos[id];
+        if (p < pairs_cap) {
+            pairs[p].count = before + 1u;
+        }
+    }
+}
+
+__device__ __forceinline__ void emit(const RowArgs& a, uint32_t id) {
+    *a.out_id = id;
+    if (a.flags & F_PEN) {
+        count_token(a.counts, a.touched, a.pairs, a.n_pairs, a.pos, a.pairs_cap, id);
+    }
+}
+
+// First slot of prefix[0..n) whose value exceeds target, else the last slot.
+__device__ __forceinline__ uint32_t pick_sequential(const float* prefix, uint32_t n, float target) {
+    for (uint32_t i = 0; i < n; ++i) {
+        if (target < prefix[i]) {
+            return i;
+        }
+    }
+    return n - 1;
+}
+
+// log p(id) = (u*c2 - mc - log2 s) * ln 2, with the id's exponent u*c2 formed exactly as
+// the row sum formed its terms, so the two cancel when the id carries all the mass.
+// Emits `id` and, when asked, its log-probability, with the memory operations of both in one
+// round trip: the count's atomic increment returns the count the penalties used, the bitmap's
+// atomic OR tells whether the id is listed already, and the logit and the list position load
+// beside them.
+template <int DT>
+__device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
+    *a.out_id = id;
+    const bool pen = (a.flags & F_PEN) != 0;
+    const bool want = a.out_logprob != nullptr;
+    if (id >= vocab) {
+        if (want) {
+            *a.out_logprob = NEG_INF;
+        }
+        return;
+    }
+    uint32_t before = 0, bits = 0, p = 0xffffffffu;
+    const uint32_t bit = 1u << (id & 31u);
+    if (pen) {
+        before = atomicAdd(&a.counts[id], 1u);
+        bits = atomicOr(&a.touched[id >> 5], bit);
+        p = gload(a.pos + id);
+    }
+    if (want) {
+        const float l = load_logit<DT>(a.logits, id);
+        const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
+        const float u = finish_pre_temperature(a, id, l, before, allowed);
+        float lp = NEG_INF;
+        if (u > NEG_INF) {
+            const double e = (double)u * (double)a.c2 - sh.lse_mc - log2(sh.lse_s);
+            lp = fminf((float)(e * 0.6931471805599453), 0.0f);  // the sum is approximate: clamp
+        }
+        *a.out_logprob = lp;
+    }
+    if (pen) {
+        if ((bits & bit) == 0u) {
+            const uint32_t at = atomicAdd(a.n_pairs, 1u);
+            if (at < a.pairs_cap) {
+                a.pairs[at].id = id;
+                a.pairs[at].count = before + 1u;
+            }
+            a.pos[id] = at < a.pairs_cap ? at : 0xffffffffu;
+        } else if (p < a.pairs_cap) {
+            a.pairs[p].count = before + 1u;
+        }
+    }
+}
+
+// cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
+template <int DT, bool BIG>
+__device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
+                     uint64_t* cand, Shared& sh, const LaunchCfg& cfg) {
+#ifdef LILY_TAIL_TRACE
+#define TAIL_MARK(i) phase(cfg, i)
+#else
+#define TAIL_MARK(i)
+#endif
+    const uint32_t tid = threadIdx.x;
+    if (n == 0) {
+        // No finite value anywhere: the oracle's order then starts at id 0.
+        if (tid == 0) {
+            if (a.out_logprob) {
+                *a.out_logprob = NEG_INF;
+            }
+            emit(a, 0);
+            if (a.dbg_counts) {
+                a.dbg_counts[0] = 0;
+                a.dbg_counts[1] = 1;  // the reference keeps rank 0 whatever its value
+            }
+            if (a.mode == MODE_DRAFT) {
+                *a.q_n = 0;
+            }
+        }
+        return;
+    }
+    if (!sorted) {
+        sort_desc<BIG>(cand, n);
+    }
+    TAIL_MARK(8);
+    const uint32_t k = min(a.k, n);
+    const float top = composite_value(cand[0]);
+    if (k <= 64u && a.mode != MODE_SPEC) {
+        // One wave, a candidate per lane.  The sums keep the reference's left-to-right f32
+        // order: every lane runs the same chain of 64 additions on values read lane by lane
+        // (lanes past k hold 0, which changes nothing), so nothing waits on LDS.
+        if (tid >= 64u) {
+            return;
+        }
+        const uint32_t lane = tid;
+        const uint64_t c = lane < k ? cand[lane] : 0ull;
+        const float p = lane < k ? lilym_expf(composite_value(c) - top) : 0.0f;
+        if (lane < k) {
+            if (a.dbg_ids) {
+                a.dbg_ids[lane] = composite_id(c);
+            }
+            if (a.dbg_probs) {
+                a.dbg_probs[lane] = p;
+            }
+        }
+        const int pbits = (int)lilym_f32_bits(p);
+        float total = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 64; ++i) {
+            total += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, i));
+        }
+        const float limit = a.top_p * total;
+        float cum = 0.0f, before = 0.0f, mine = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 64; ++i) {
+            before = lane == (uint32_t)i ? cum : before;
+            cum += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, i));
+            mine = lane == (uint32_t)i ? cum : mine;
+        }
+        const bool stop = lane >= 1u && lane < k && !(before < limit && p >= a.min_p);
+        const uint64_t stops = __ballot(stop);
+        const uint32_t kept = stops != 0ull ? (uint32_t)__builtin_ctzll(stops) : k;
+        const float mass = __shfl(mine, (int)kept - 1);
+        if (lane == 0 && a.dbg_counts) {
+            a.dbg_counts[0] = k;
+            a.dbg_counts[1] = kept;
+        }
+        if (a.mode == MODE_DRAFT) {
+            if (lane < kept) {
+                a.q_ids[lane] = composite_id(c);
+                a.q_probs[lane] = p / mass;
+            }
+            if (lane == 0) {
+                *a.q_n = kept;
+            }
+        }
+        const float u1 = (a.flags & F_UNIFORM) ? a.uniform : lilym_uniform_for(a.seed, step);
+        const uint64_t hits = __ballot(lane < kept && u1 * mass < mine);
+        const uint32_t slot = hits != 0ull ? (uint32_t)__builtin_ctzll(hits) : kept - 1u;
+        const uint32_t id = ~(uint32_t)__shfl((int)(uint32_t)c, (int)slot);
+        if (lane == 0) {
+            finish_token<DT>(a, sh, id, vocab);
+        }
+        return;
+    }
+    for (uint32_t i = tid; i < k; i += NT) {
+        const float p = lilym_expf(composite_value(cand[i]) - top);
+        sh.prob[i] = p;
+        if (a.dbg_ids) {
+            a.dbg_ids[i] = composite_id(cand[i]);
+        }
+        if (a.dbg_probs) {
+            a.dbg_probs[i] = p;
+        }
+    }
+    __syncthreads();
+    TAIL_MARK(9);
+    // The reference's left-to-right f32 sums: one wave runs the chain of additions, 64
+    // candidates at a time with a candidate per lane, and keeps every prefix.  Each step adds
+    // the lane's value to the running sum of the lane below (a shift by one lane across the
+    // whole wave; lane 0 has no lane below and keeps what it has): after step j the lanes up
+    // to j hold their final prefix, which further steps only reproduce.  The row total is
+    // the last prefix, and the sum the reference holds before rank r is the prefix of rank
+    // r - 1: the cut by top-p and min-p and the inverse-CDF pick then are searches every
+    // thread takes part in.
+    if (tid < 64u) {
+        float carry = 0.0f;
+        for (uint32_t r0 = 0; r0 < k; r0 += 64u) {
+            const uint32_t i = r0 + tid;
+            const float p = i < k ? sh.prob[i] : 0.0f;
+            float run = carry + p;  // final in lane 0
+#pragma unroll
+            for (int j = 1; j < 64; ++j) {
+                // Two idle cycles between a lane's write and the neighbour's read of it.
+                asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %1 wave_shr:1 row_mask:0xf bank_mask:0xf"
+                             : "+v"(run)
+                             : "v"(p));
+            }
+            if (i < k) {
+                sh.cum[i] = run;
+            }
+            carry = lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane((int)lilym_f32_bits(run), 63));
+        }
+    }
+    __syncthreads();
+    TAIL_MARK(10);
+    auto first_of = [&](uint32_t mine_first) -> uint32_t {  // the lowest index any thread found
+        mine_first = wave_min_u32(mine_first);
+        if ((tid & 63u) == 0) {
+            sh.red_i[tid >> 6] = mine_first;
+        }
+        __syncthreads();
+        uint32_t r = sh.red_i[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            r = min(r, sh.red_i[i]);
+        }
+        __syncthreads();
+        return r;
+    };
+    const float limit = a.top_p * sh.cum[k - 1];
+    uint32_t stop = k;
+    for (uint32_t r = 1 + tid; r < k; r += NT) {
+        if (!(sh.cum[r - 1] < limit && sh.prob[r] >= a.min_p)) {
+            stop = min(stop, r);
+        }
+    }
+    if (tid == 0) {
+        sh.p_d = 0.0f;
+        sh.q_d = 0.0f;
+    }
+    const uint32_t n_keep = first_of(stop);
+    const float mass = sh.cum[n_keep - 1];
+    TAIL_MARK(11);
+    const float u1 = (a.flags & F_UNIFORM) ? a.uniform : lilym_uniform_for(a.seed, step);
+    if (tid == 0) {
+        if (a.dbg_counts) {
+            a.dbg_counts[0] = k;
+            a.dbg_counts[1] = n_keep;
+        }
+    }
+    // First slot of cum[0..n) whose value exceeds target, else the last slot.
+    auto pick = [&](const float* prefix, uint32_t n, float target) -> uint32_t {
+        uint32_t hit = n - 1u;
+        for (uint32_t i = tid; i < n; i += NT) {
+            if (target < prefix[i]) {
+                hit = min(hit, i);
+            }
+        }
+        return first_of(hit);
+    };
+
+    if (a.mode == MODE_DRAFT) {
+        for (uint32_t i = tid; i < n_keep; i += NT) {
+            a.q_ids[i] = composite_id(cand[i]);
+            a.q_probs[i] = sh.prob[i] / mass;
+        }
+        if (tid == 0) {
+            *a.q_n = n_keep;
+        }
+    }
+
+    if (a.mode != MODE_SPEC) {
+        const uint32_t slot = pick(sh.cum, n_keep, u1 * mass);
+        TAIL_MARK(12);
+        if (tid == 0) {
+            const uint32_t id = composite_id(cand[slot]);
+            finish_token<DT>(a, sh, id, vocab);
+        }
+        return;
+    }
+
+    // Speculative draw (sample.metal:596-658, cpu_spec at tests/unit/kernels/sample.rs:264-283).
+    const uint32_t d = *a.draft;
+    const uint32_t qn = min(*a.q_n, K_CAP);
+    for (uint32_t i = tid; i < n_keep; i += NT) {
+        if (composite_id(cand[i]) == d) {
+            sh.p_d = sh.prob[i] / mass;
+        }
+    }
+    for (uint32_t j = tid; j < qn; j += NT) {
+        if (a.q_ids[j] == d) {
+            sh.q_d = a.q_probs[j];
+        }
+    }
+    __syncthreads();
+    if (u1 * sh.q_d < sh.p_d) {
+        if (tid == 0) {
+            finish_token<DT>(a, sh, d, vocab);
+        }
+        return;
+    }
+    for (uint32_t i = tid; i < n_keep; i += NT) {
+        const uint32_t id = composite_id(cand[i]);
+        float q_i = 0.0f;
+        for (uint32_t j = 0; j < qn; ++j) {
+            if (a.q_ids[j] == id) {
+                q_i = a.q_probs[j];
+                break;
+            }
+        }
+        sh.res[i] = fmaxf(sh.prob[i] / mass - q_i, 0.0f);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const float u2 = (a.flags & F_UNIFORM) ? a.uniform2
+                                               : lilym_uniform_for(a.seed, lilym_residual_step(step));
+        float total = 0.0f;
+        for (uint32_t i = 0; i < n_keep; ++i) {
+            total += sh.res[i];
+        }
+        uint32_t slot;
+        if (total > 0.0f) {
+            const float target = u2 * total;
+            float cum = 0.0f;
+            slot = n_keep - 1;
+            for (uint32_t i = 0; i < n_keep; ++i) {
+                cum += sh.res[i];
+                if (target < cum) {
+                    slot = i;
+                    break;
+                }
+            }
+        } else {
+            // Only rounding gives a rejected proposal a massless residual: draw from p.
+            slot = pick_sequential(sh.cum, n_keep, u2 * mass);
+        }
+        const uint32_t id = composite_id(cand[slot]);
+        finish_token<DT>(a, sh, id, vocab);
+    }
+}
+
+
+}  // namespace lily

@@ -136,7 +136,9 @@ def _load():
         "lily_spec_accept": [vp, vp, vp, u32, vp, u32, u32, u32, u32],
         "lily_copy_row_u32": [vp, vp, u32, u32, vp, vp],
         "lily_spec_verify": [vp, vp, C.c_int, u32, u64, u32, vp, P, u32, vp, vp, vp, vp, u32, u32,
-                             u32, u32],
+                             u32, u32, C.POINTER(C.c_float)],
+        "lily_sample_spec_f32_uniforms": [vp, vp, u32, vp, P, u32, C.POINTER(DraftDist), vp, vp,
+                                          C.c_float, C.c_float],
         "lily_sample_rows": [vp, C.POINTER(_Rows)],
         "lily_plan_create": [vp, u32, C.POINTER(vp)],
         "lily_plan_set": [vp, C.POINTER(_Rows)],
@@ -263,7 +265,15 @@ class Sampler:
                                           scratch._h if scratch else None, C.byref(params), step,
                                           _ptr(out, torch.int32), C.byref(dist)))
 
-    def sample_spec_f32(self, logits, scratch, params, step, dist, draft, out):
+    def sample_spec_f32(self, logits, scratch, params, step, dist, draft, out, uniforms=None):
+        """uniforms: None (seeded draws) or (u1, u2) for the accept test and the residual draw."""
+        if uniforms is not None:
+            _check(_lib.lily_sample_spec_f32_uniforms(
+                self._h, _ptr(logits, torch.float32), logits.numel(),
+                scratch._h if scratch else None, C.byref(params), step, C.byref(dist),
+                _ptr(draft, torch.int32), _ptr(out, torch.int32), float(uniforms[0]),
+                float(uniforms[1])))
+            return
         _check(_lib.lily_sample_spec_f32(self._h, _ptr(logits, torch.float32), logits.numel(),
                                          scratch._h if scratch else None, C.byref(params), step,
                                          C.byref(dist), _ptr(draft, torch.int32),
@@ -291,15 +301,22 @@ class Sampler:
                                       _ptr(row, torch.int32), _ptr(dst, torch.int32)))
 
     def spec_verify(self, logits, scratch, params, step0, dists, ids, verify_tokens, ctrl=None,
-                    pos0=0, ratio=1, chain=0):
+                    pos0=0, ratio=1, chain=0, uniforms=None):
+        """uniforms: None or [m][2] host values (u1, u2) per row replacing the seeded draws."""
         m, vocab = logits.shape
         dtype = BF16 if logits.dtype == torch.bfloat16 else F32
+        uarr = None
+        if uniforms is not None:
+            flat = [float(u) for pair in uniforms for u in pair]
+            if len(flat) != 2 * m:
+                raise SamplerError(-1, "uniforms must hold (u1, u2) per verify row")
+            uarr = (C.c_float * (2 * m))(*flat)
         _check(_lib.lily_spec_verify(
             self._h, _ptr(logits), dtype, vocab, logits.stride(0) if m > 1 else vocab, m,
             scratch._h if scratch else None, C.byref(params), step0,
             dists._h if dists else None, _ptr(ids, torch.int32), _ptr(verify_tokens, torch.int32),
             _ptr(ctrl, torch.int32) if ctrl is not None else None,
-            ctrl.numel() if ctrl is not None else 0, pos0, ratio, chain))
+            ctrl.numel() if ctrl is not None else 0, pos0, ratio, chain, uarr))
 
     # -- batched rows, src/qwen4exp/batch.rs:583-593
     def _rows(self, logits, params, steps, out_ids, scratch=None, allow=None, bias=None,
@@ -479,6 +496,22 @@ class DraftDists:
         _check(_lib.lily_draft_dists_slot(self._h, i, C.byref(d)))
         return d
 
+    def write(self, i, ids, probs):
+        """Overwrites slot i with a hand-made distribution (numpy uint32 ids, float32 probs);
+        synchronises.  For tests of cases no real draft head produces."""
+        d = self.slot(i)
+        self._s.synchronize()
+        k = len(ids)
+        if k > SAMPLE_K_CAP or len(probs) != k:
+            raise SamplerError(-6, "a slot holds at most 1024 (id, prob) pairs")
+        t_ids = torch.tensor([int(x) for x in ids], dtype=torch.int64).to(torch.int32)
+        t_pr = torch.tensor([float(x) for x in probs], dtype=torch.float32)
+        t_n = torch.tensor([k], dtype=torch.int32)
+        if k:
+            _hip_copy_to_device(d.ids_dev, t_ids, 4 * k)
+            _hip_copy_to_device(d.probs_dev, t_pr, 4 * k)
+        _hip_copy_to_device(d.count_dev, t_n, 4)
+
     def read(self, i):
         """(ids, probs) of slot i on the host; synchronises."""
         d = self.slot(i)
@@ -497,13 +530,22 @@ class DraftDists:
 _hip = None
 
 
-def _hip_copy(dst_cpu, src_dev, nbytes):
-    """Device -> host copy of raw library-owned memory (tests read the draft export)."""
+def _hip_memcpy(dst, src, nbytes, kind):
     global _hip
     if _hip is None:
         _hip = C.CDLL("libamdhip64.so.7")  # the SONAME torch already loaded
         _hip.hipMemcpy.restype = C.c_int
         _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-    rc = _hip.hipMemcpy(C.c_void_p(dst_cpu.data_ptr()), C.c_void_p(src_dev), nbytes, 2)
+    rc = _hip.hipMemcpy(C.c_void_p(dst), C.c_void_p(src), nbytes, kind)
     if rc != 0:
         raise SamplerError(-4, f"hipMemcpy failed with {rc}")
+
+
+def _hip_copy(dst_cpu, src_dev, nbytes):
+    """Device -> host copy of raw library-owned memory (tests read the draft export)."""
+    _hip_memcpy(dst_cpu.data_ptr(), src_dev, nbytes, 2)
+
+
+def _hip_copy_to_device(dst_dev, src_cpu, nbytes):
+    """Host -> device copy into raw library-owned memory (tests write a draft export)."""
+    _hip_memcpy(dst_dev, src_cpu.data_ptr(), nbytes, 1)

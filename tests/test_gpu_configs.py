@@ -94,8 +94,12 @@ def test_config2_batch_of_four_with_penalties(sampler, use_plan):
         s.close()
 
 
-def test_config3_speculative_verify(sampler):
+@pytest.mark.parametrize("given", [False, True])
+def test_config3_speculative_verify(sampler, given):
+    """given: the configuration's fixed (u1, u2) per position replace the seeded draws
+    (accept test and plain draw on u1, residual draw on u2: sample.metal:626-651)."""
     c = W.config3()
+    us = c["u"] if given else None
     target, draft = c["target"], c["draft"]
     m, vocab = target.shape
     t_target = torch.from_numpy(target).to(dev())
@@ -119,7 +123,7 @@ def test_config3_speculative_verify(sampler):
         verify = torch.zeros(m, dtype=torch.int32, device=dev())
         ctrl = torch.zeros(LS.ctrl_words(2), dtype=torch.int32, device=dev())
         sampler.spec_verify(t_target, scratch, lp, step0, dists, ids, verify, ctrl, pos0=100,
-                            ratio=4, chain=2)
+                            ratio=4, chain=2, uniforms=us)
         sampler.synchronize()
         got = verify.cpu().numpy()
         # oracle: the same sequence with the counts flowing from row to row
@@ -132,7 +136,9 @@ def test_config3_speculative_verify(sampler):
                 assert dd.chosen == props[j]
                 trunk = O.sample(target[j], counts.copy(), op, step0 + j)
                 tok, acc, zero, gap = O.spec(trunk.kept_ids, trunk.kept_q, dd.kept_ids, dd.kept_q,
-                                             int(props[j]), op.seed, step0 + j)
+                                             int(props[j]), op.seed, step0 + j,
+                                             u1=float(us[j, 0]) if given else None,
+                                             u2=float(us[j, 1]) if given else None)
                 if zero:
                     tok = int(got[j])
                 if O.lib().lo_uses_penalties(op):
@@ -140,7 +146,8 @@ def test_config3_speculative_verify(sampler):
             else:
                 if j + 1 < m:
                     assert props[j] == O.argmax(draft[j])
-                tok = O.sample(target[j], counts, op, step0 + j).chosen
+                ukw = dict(uniform=float(us[j, 0])) if given and O.lib().lo_samples(op) else {}
+                tok = O.sample(target[j], counts, op, step0 + j, **ukw).chosen
             want.append(tok)
         assert list(got) == want, (kw, got, want)
         if O.lib().lo_uses_penalties(op):

@@ -211,6 +211,92 @@ def test_speculative_draw_matches_the_cpu_reference(sampler):
     dists.close()
 
 
+def test_speculative_draw_with_given_uniforms(sampler):
+    """The two draws given instead of seeded (accept test on u1, residual draw on u2,
+    sample.metal:626-651): every pair agrees with cpu_spec, including the corners u1 = 0
+    (accepts whenever p(d) > 0) and u2 just below 1 (the last residual entry)."""
+    rng = np.random.default_rng(29)
+    v = 4099
+    head = rng.normal(0, 2.5, v).astype(np.float32)
+    trunk = (head + rng.normal(0, 0.6, v)).astype(np.float32)
+    kw = dict(temperature=1.0, top_k=20, top_p=0.95, seed=3)
+    lp, op = both_params(**kw)
+    p_ids, p_pr = O.kept(trunk, op)
+    q_ids, q_pr = O.kept(head, O.draft_params(op))
+    t_trunk = torch.from_numpy(trunk).to(dev())
+    t_head = torch.from_numpy(head).to(dev())
+    scratch = LS.SamplerScratch(sampler, v)
+    dists = LS.DraftDists(sampler, 1)
+    dist = dists.slot(0)
+    drafted = torch.zeros(1, dtype=torch.int32, device=dev())
+    out = torch.zeros(1, dtype=torch.int32, device=dev())
+    # a draft step whose proposal the trunk keeps with p(d) < q(d): both outcomes occur
+    pd, qd = dict(zip(p_ids.tolist(), p_pr.tolist())), dict(zip(q_ids.tolist(), q_pr.tolist()))
+    def proposal(t):
+        return O.sample(head, None, O.draft_params(op), O.lib().lo_draft_step(t)).chosen
+
+    dstep = next(t for t in range(200) if 0.0 < pd.get(proposal(t), 0.0) < 0.7 * qd[proposal(t)])
+    sampler.sample_draft_f32(t_head, scratch, LS.draft_params(lp), LS.draft_step(dstep), drafted,
+                             dist)
+    sampler.synchronize()
+    d = int(drafted.item())
+    pairs = [(0.0, 0.0), (0.0, 0.99999994), (0.99999994, 0.0), (0.99999994, 0.99999994)]
+    pairs += [(float(a), float(b)) for a, b in rng.random((60, 2)).astype(np.float32)]
+    outcomes = set()
+    for u1, u2 in pairs:
+        sampler.sample_spec_f32(t_trunk, scratch, lp, 5, dist, drafted, out, uniforms=(u1, u2))
+        sampler.synchronize()
+        want, acc, zero, gap = O.spec(p_ids, p_pr, q_ids, q_pr, d, op.seed, 5, u1=u1, u2=u2)
+        assert not zero
+        assert int(out.item()) == want, (u1, u2, int(out.item()), want)
+        outcomes.add(acc)
+    assert outcomes == {True, False}
+    for bad in ((1.0, 0.5), (0.5, -0.1), (float("nan"), 0.5)):
+        with pytest.raises(LS.SamplerError):
+            sampler.sample_spec_f32(t_trunk, scratch, lp, 5, dist, drafted, out, uniforms=bad)
+    scratch.close()
+    dists.close()
+
+
+def test_massless_residual_draws_from_the_trunk_on_the_second_uniform(sampler):
+    """A rejected proposal whose residual has no mass: the kernel draws from p on the second
+    uniform (sample.metal:650-651) where the CPU test takes p's last entry
+    (tests/unit/kernels/sample.rs:282).  Exact arithmetic never gets there (p <= q on p's
+    support with sum 1 forces q == p, which always accepts), so the exported distribution is
+    written by hand: q == p except q(d) = 2 p(d), and u1 = 0.75 rejects.  The oracle reports
+    the case; the draw must be the plain inverse-CDF pick of u2 over the trunk's kept set."""
+    rng = np.random.default_rng(31)
+    v = 2048
+    row = rng.uniform(-4, 4, v).astype(np.float32)
+    kw = dict(temperature=1.0, top_k=12, top_p=1.0, seed=9)
+    lp, op = both_params(**kw)
+    t_row = torch.from_numpy(row).to(dev())
+    scratch = LS.SamplerScratch(sampler, v)
+    dists = LS.DraftDists(sampler, 1)
+    dist = dists.slot(0)
+    out = torch.zeros(1, dtype=torch.int32, device=dev())
+    p_ids, p_pr = O.kept(row, op)
+    for which in (0, 5, len(p_ids) - 1):
+        d = int(p_ids[which])
+        q_pr = p_pr.copy()
+        q_pr[which] = np.float32(2.0) * p_pr[which]
+        dists.write(0, p_ids, q_pr)
+        drafted = torch.tensor([d], dtype=torch.int32, device=dev())
+        for u2 in (0.0, 0.3, 0.77, 0.99999994):
+            sampler.sample_spec_f32(t_row, scratch, lp, 0, dist, drafted, out, uniforms=(0.75, u2))
+            sampler.synchronize()
+            want, acc, zero, gap = O.spec(p_ids, p_pr, p_ids, q_pr, d, op.seed, 0, u1=0.75, u2=u2)
+            assert zero and not acc
+            plain = O.sample(row, None, op, 0, uniform=u2)
+            assert int(out.item()) == plain.chosen, (which, u2, int(out.item()), plain.chosen)
+        # the same hand-written q accepts below one half
+        sampler.sample_spec_f32(t_row, scratch, lp, 0, dist, drafted, out, uniforms=(0.25, 0.5))
+        sampler.synchronize()
+        assert int(out.item()) == d
+    scratch.close()
+    dists.close()
+
+
 def test_speculative_draw_is_distributed_as_the_trunk(sampler):
     rng = np.random.default_rng(25)
     v = 48
