@@ -197,6 +197,19 @@ int lily_sample_spec_f32_uniforms(lily_sampler_t* s, const float* logits_dev, ui
                                   lily_scratch_t* scratch, const lily_sampling_params* params,
                                   uint32_t step, const lily_draft_dist* dist,
                                   const uint32_t* draft_dev, uint32_t* out_dev, float u1, float u2);
+/* No counterpart in the reference.  lily_sample_f32 for callers that cannot allocate device
+ * memory or own a sampler object: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  The draw is enqueued on `hip_stream` of the CURRENT device; the memory
+ * a row spread over several workgroups needs (slices' candidates, partial sums, the arrival
+ * ticket: 34 048 bytes) lives in a device array inside the library, one copy per GPU, kept
+ * until the process ends.  The call allocates and frees nothing and does not synchronise.
+ * Same results as lily_sample_f32.  Limits: one row of at most LILY_STATIC_MAX_VOCAB logits
+ * (LILY_ERR_RANGE beyond); every call on a GPU shares that GPU's array, so two calls that may
+ * overlap on one GPU (different streams, or graphs replayed concurrently) race - order them. */
+#define LILY_STATIC_MAX_VOCAB 1048576u
+int lily_sample_f32_static(void* hip_stream, const float* logits_dev, uint32_t vocab,
+                           lily_scratch_t* scratch, const lily_sampling_params* params,
+                           uint32_t step, uint32_t* out_dev);
 /* argmax_f32 (src/kernels/elementwise.rs:297-308): first max, lowest index on ties. */
 int lily_argmax_f32(lily_sampler_t* s, const float* x_dev, uint32_t n, uint32_t* out_dev);
 

@@ -31,6 +31,7 @@ def units():
     out = [("rows_variant.hip", f"rows_dt{dt}_kind{kind}.o", [f"-DLILY_DT={dt}", f"-DLILY_KIND={kind}"])
            for dt, kind in VARIANTS]
     out.append(("scratch_kernels.hip", "scratch_kernels.o", []))
+    out.append(("static_entry.hip", "static_entry.o", []))
     out.append(("sampler_api.cpp", "sampler_api.o", []))
     return out
 

@@ -16,6 +16,7 @@
 
 #include "../../include/lily_sampler.h"
 #include "../../include/lily_sampler_math.h"
+#include "api_internal.h"
 #include "launch.h"
 
 using namespace lily;
@@ -57,6 +58,8 @@ struct lily_sampler {
     uint64_t* ws_cand = nullptr;
     double* ws_lse = nullptr;
     uint32_t* ws_ticket = nullptr;
+    uint32_t ws_rows = WS_ROWS;    // rows that may span several workgroups
+    uint32_t ws_slots = WS_SLOTS;  // candidate slots behind ws_cand
     // Row table of lily_sample_rows batches above INLINE_ROWS.
     RowArgs* table_dev = nullptr;
     uint32_t table_cap = 0;
@@ -277,7 +280,7 @@ uint32_t slices_for_list(uint32_t listed) {
 // at most SPEC_CAP of them, so long lists are spread over more slices.
 uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab,
                        int dtype, uint32_t listed = 0) {
-    if (rows > WS_ROWS) {
+    if (rows > s->ws_rows) {
         return 1;
     }
     uint32_t sl = s->force_slices ? s->force_slices : (TARGET_GROUPS + rows - 1) / rows;
@@ -297,7 +300,7 @@ uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint
     sl = sl > by_k ? by_k : sl;
     const uint32_t by_len = (vocab + 2047u) / 2048u;
     sl = sl > by_len ? by_len : sl;
-    const uint64_t by_ws = (uint64_t)WS_SLOTS / ((uint64_t)rows * (kmax ? kmax : 1));
+    const uint64_t by_ws = (uint64_t)s->ws_slots / ((uint64_t)rows * (kmax ? kmax : 1));
     sl = sl > by_ws ? (uint32_t)by_ws : sl;
     return sl < 1 ? 1 : sl;
 }
@@ -591,6 +594,35 @@ int ensure_table(lily_sampler* s, uint32_t rows) {
 
 }  // namespace
 
+namespace lily {
+
+int api_fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int scratch_device(const lily_scratch_t* sc) { return sc->s->device; }
+
+int sample_row_with_workspace(int device, hipStream_t stream, const Workspace& ws, const float* logits,
+                              uint32_t vocab, lily_scratch_t* scratch,
+                              const lily_sampling_params* params, uint32_t step, uint32_t* out) {
+    lily_sampler s;  // a view for this one launch: owns nothing, is never destroyed
+    s.device = device;
+    s.stream = stream;
+    s.ws_cand = ws.cand;
+    s.ws_lse = ws.lse;
+    s.ws_ticket = ws.ticket;
+    s.ws_rows = ws.rows;
+    s.ws_slots = ws.slots;
+    return one_row(&s, logits, LILY_F32, vocab, scratch, params, step, MODE_PLAIN, out, nullptr,
+                   nullptr);
+}
+
+}  // namespace lily
+
 extern "C" {
 
 const char* lily_last_error(void) { return g_error; }
@@ -702,6 +734,10 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     if (err != hipSuccess) {
         lily_sampler_destroy(s);
         return hip_fail(err, "sampler workspace");
+    }
+    if (int rc = static_scratch_init(device)) {
+        lily_sampler_destroy(s);
+        return rc;
     }
     *out = s;
     return LILY_OK;
@@ -1247,12 +1283,12 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     HIP_TRY(hipSetDevice(p->s->device));
     for (uint32_t q = 0; q < p->n_parts; ++q) {
         LaunchPart& part = p->parts[q];
-        if (part.listed != 0 && part.kind == 2 && part.rows <= WS_ROWS) {
+        if (part.listed != 0 && part.kind == 2 && part.rows <= p->s->ws_rows) {
             // The lists grow by one id per run at most: take more slices before a workgroup's
             // buckets overflow (only the merge's share of dynamic LDS depends on the slices).
             const uint32_t need = slices_for_list(part.listed + p->runs + 1);
             const uint64_t by_ws =
-                (uint64_t)WS_SLOTS / ((uint64_t)part.rows * (part.ws_k ? part.ws_k : 1));
+                (uint64_t)p->s->ws_slots / ((uint64_t)part.rows * (part.ws_k ? part.ws_k : 1));
             if (need > part.slices && need <= MAX_SLICES && need <= by_ws) {
                 part.slices = need;
                 const size_t merge = (size_t)need * part.ws_k * 8;

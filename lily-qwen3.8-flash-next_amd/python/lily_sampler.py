@@ -133,6 +133,7 @@ def _load():
         "lily_sample_draft_f32": [vp, vp, u32, vp, P, u32, vp, C.POINTER(DraftDist)],
         "lily_sample_spec_f32": [vp, vp, u32, vp, P, u32, C.POINTER(DraftDist), vp, vp],
         "lily_argmax_f32": [vp, vp, u32, vp],
+        "lily_sample_f32_static": [vp, vp, u32, vp, P, u32, vp],
         "lily_spec_accept": [vp, vp, vp, u32, vp, u32, u32, u32, u32],
         "lily_copy_row_u32": [vp, vp, u32, u32, vp, vp],
         "lily_spec_verify": [vp, vp, C.c_int, u32, u64, u32, vp, P, u32, vp, vp, vp, vp, u32, u32,
@@ -173,6 +174,14 @@ def _ptr(t, dtype=None):
     if not t.is_contiguous():
         raise SamplerError(-1, "tensor must be contiguous")
     return C.c_void_p(t.data_ptr())
+
+
+def sample_f32_static(stream, logits, scratch, params, step, out):
+    """lily_sample_f32_static: the draw that needs no sampler object and allocates nothing,
+    enqueued on `stream` (a torch.cuda.Stream) of the current device."""
+    _check(_lib.lily_sample_f32_static(C.c_void_p(stream.cuda_stream), _ptr(logits, torch.float32),
+                                       logits.numel(), scratch._h if scratch else None,
+                                       C.byref(params), step, _ptr(out, torch.int32)))
 
 
 def uniform_for(seed, step):
