@@ -83,9 +83,11 @@ struct lily_scratch {
     uint32_t* counts = nullptr;   // [vocab]; the one allocation, the rest follows it
     uint32_t* pos = nullptr;      // [vocab] pairs index of a listed id
     uint32_t* touched = nullptr;  // [words + 4] bit per listed id
-    CountPair* pairs = nullptr;   // [pairs_cap] listed ids with their counts
-    uint32_t* n_pairs = nullptr;  // [1]
-    uint64_t listed_bound = 0;    // host's upper bound of *n_pairs (ids added + draws enqueued)
+    ListEntry* pairs = nullptr;   // [pairs_cap] listed ids with their counts
+    uint32_t* list_hdr = nullptr; // [LIST_HDR_WORDS + buckets + 1] lengths, then the bucket starts
+    uint32_t buckets = 0;
+    uint32_t tail_bound = 0;      // host's upper bound of the unsorted tail's length (draws
+                                  // enqueued since the list was last sorted)
 };
 
 struct lily_draft_dists {
@@ -108,7 +110,7 @@ struct LaunchPart {
     uint32_t excl_words = 0;
     bool bitmap_layout = false;
     uint32_t cand_cap = 0;
-    uint32_t listed = 0;                     // longest scratch list when the table was packed
+    bool sort_first = false;                 // some row's list is sorted before the launch
 };
 
 struct lily_plan {
@@ -121,6 +123,10 @@ struct lily_plan {
     LaunchPart parts[2];                     // the batch's one or two launches
     uint32_t n_parts = 0;
     uint32_t runs = 0;                       // launches since the table was packed
+    bool sort_on_first_run = false;          // a row's list was due for sorting when it was packed
+    bool sorted = false;                     // the lists were sorted by a run of this plan, so
+    uint32_t since_sort = 0;                 // the tails hold at most this many ids
+    uint32_t longest_tail = 0;               // largest bound of a tail among the scratches
     std::vector<lily_scratch*> penalised;    // scratches whose rows count their draws
 };
 
@@ -133,7 +139,7 @@ ScratchView view_of(const lily_scratch* sc) {
     v.counts = sc->counts;
     v.touched = sc->touched;
     v.pairs = sc->pairs;
-    v.n_pairs = sc->n_pairs;
+    v.list_hdr = sc->list_hdr;
     v.pos = sc->pos;
     v.vocab = sc->vocab;
     v.pairs_cap = sc->pairs_cap;
@@ -217,12 +223,15 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
         out->counts = scratch->counts;
         out->touched = scratch->touched;
         out->pairs = scratch->pairs;
-        out->n_pairs = scratch->n_pairs;
+        out->list_hdr = scratch->list_hdr;
         out->pos = scratch->pos;
         out->pairs_cap = scratch->pairs_cap;
-        out->pairs_hint = (uint32_t)(scratch->listed_bound < scratch->pairs_cap
-                                         ? scratch->listed_bound : scratch->pairs_cap);
-        scratch->listed_bound += 1;  // this draw may list one more id
+        if (scratch->tail_bound >= TAIL_SORT_AT) {
+            out->flags |= F_SORT_FIRST;  // the launch is preceded by a sort of this row's list
+            scratch->tail_bound = 0;
+        }
+        out->tail_hint = scratch->tail_bound;
+        scratch->tail_bound += 1;  // this draw may list one more id
         out->flags |= F_PEN;
     }
     if (x.has_uniform) {
@@ -258,28 +267,8 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
 }
 
 // Workgroups per row for a batch of `rows` whose largest candidate count is kmax.
-// The longest scratch list among `rows` (the host's bound, as packed into the rows).
-uint32_t longest_list(const RowArgs* rows, uint32_t n) {
-    uint32_t longest = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        if ((rows[i].flags & F_PEN) && rows[i].pairs_hint > longest) {
-            longest = rows[i].pairs_hint;
-        }
-    }
-    return longest;
-}
-
-// Slices that leave every workgroup about a tenth of its bucket capacity free when a list
-// of `listed` ids is spread evenly over the vocabulary.
-uint32_t slices_for_list(uint32_t listed) {
-    const uint32_t room = SPEC_CAP - SPEC_CAP / 10;
-    return (listed + room - 1) / room;
-}
-
-// `listed`: the longest list of penalised ids among the rows (0 = none): a workgroup buckets
-// at most SPEC_CAP of them, so long lists are spread over more slices.
 uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint32_t vocab,
-                       int dtype, uint32_t listed = 0) {
+                       int dtype) {
     if (rows > s->ws_rows) {
         return 1;
     }
@@ -291,8 +280,6 @@ uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint
         const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
         const uint32_t by_block = (nch + 256u * STREAM_UNROLL - 1) / (256u * STREAM_UNROLL);
         sl = sl > by_block ? by_block : sl;
-        const uint32_t by_list = slices_for_list(listed);
-        sl = sl < by_list ? by_list : sl;
     }
     sl = sl < 1 ? 1 : sl;
     sl = sl > MAX_SLICES ? MAX_SLICES : sl;
@@ -429,8 +416,11 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
         part.rows = !split ? rows : (q == 0 ? rows - heavy : heavy);
         const RowArgs* sub = table + part.first;
         part.ws_k = max_k(sub, part.rows);
-        part.listed = longest_list(sub, part.rows);
-        part.slices = choose_slices(s, part.rows, part.ws_k, vocab, dtype, part.listed);
+        part.slices = choose_slices(s, part.rows, part.ws_k, vocab, dtype);
+        part.sort_first = false;
+        for (uint32_t i = 0; i < part.rows; ++i) {
+            part.sort_first = part.sort_first || (sub[i].flags & F_SORT_FIRST) != 0;
+        }
         const LaunchShape shp = shape_of(s, sub, part.rows, dtype, vocab, part.slices, part.ws_k);
         part.kind = shp.kind();
         part.lse = shp.lse;
@@ -443,7 +433,8 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
 }
 
 int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_dev, int dtype,
-                uint32_t vocab, uint32_t step_delta, uint32_t hint_growth, bool traced) {
+                uint32_t vocab, uint32_t step_delta, uint32_t hint_growth, bool hint_replace,
+                bool traced) {
     LaunchCfg cfg;
     fill_cfg(s, &cfg, vocab, part.slices, part.ws_k, step_delta, table_dev + part.first);
     if (traced) {
@@ -453,6 +444,7 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
     cfg.bitmap_layout = part.bitmap_layout ? 1u : 0u;
     cfg.cand_cap = part.cand_cap;
     cfg.hint_growth = hint_growth;
+    cfg.hint_replace = hint_replace ? 1u : 0u;
     HIP_TRY(launch_rows(s->stream, dtype, part.kind, part.lse, part.rows, cfg, nullptr, part.dyn_bytes));
     return LILY_OK;
 }
@@ -460,8 +452,15 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
 int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n) {
     HIP_TRY(hipSetDevice(s->device));
     const uint32_t kmax = max_k(rows.r, n);
+    bool sort_first = false;
+    for (uint32_t i = 0; i < n; ++i) {
+        sort_first = sort_first || (rows.r[i].flags & F_SORT_FIRST) != 0;
+    }
+    if (sort_first) {
+        HIP_TRY(launch_sort_lists(s->stream, nullptr, &rows, n, vocab, true));
+    }
     LaunchCfg cfg;
-    const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype, longest_list(rows.r, n));
+    const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
     attach_trace(s, &cfg, n);
     const LaunchShape shp = shape_of(s, rows.r, n, dtype, vocab, slices, kmax);
@@ -809,11 +808,14 @@ int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out)
     sc->vocab = vocab;
     sc->words = (vocab + 31u) / 32u;
     sc->pairs_cap = vocab < PAIRS_CAP ? vocab : PAIRS_CAP;
-    // One allocation: counts, pos, the bitmap, the list, its length (each 16-byte aligned).
+    sc->buckets = (vocab + (1u << SORT_SHIFT) - 1u) >> SORT_SHIFT;
+    // One allocation: counts, pos, the bitmap, the list, its lengths and bucket starts (each
+    // 16-byte aligned).
     const size_t dense = (((size_t)vocab * 4) + 15) & ~(size_t)15;
     const size_t bitmap = (((size_t)(sc->words + 4) * 4) + 15) & ~(size_t)15;
-    const size_t list = (size_t)sc->pairs_cap * sizeof(CountPair);
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts), 2 * dense + bitmap + list + 16);
+    const size_t list = (size_t)sc->pairs_cap * sizeof(ListEntry);
+    const size_t header = (((size_t)(LIST_HDR_WORDS + sc->buckets + 1) * 4) + 15) & ~(size_t)15;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts), 2 * dense + bitmap + list + header);
     if (e != hipSuccess) {
         delete sc;
         return hip_fail(e, "scratch allocation");
@@ -821,8 +823,8 @@ int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out)
     char* base = reinterpret_cast<char*>(sc->counts);
     sc->pos = reinterpret_cast<uint32_t*>(base + dense);
     sc->touched = reinterpret_cast<uint32_t*>(base + 2 * dense);
-    sc->pairs = reinterpret_cast<CountPair*>(base + 2 * dense + bitmap);
-    sc->n_pairs = reinterpret_cast<uint32_t*>(base + 2 * dense + bitmap + list);
+    sc->pairs = reinterpret_cast<ListEntry*>(base + 2 * dense + bitmap);
+    sc->list_hdr = reinterpret_cast<uint32_t*>(base + 2 * dense + bitmap + list);
     e = hipMemsetAsync(sc->pos, 0, dense, s->stream);  // never read before written; defined anyway
     if (e != hipSuccess) {
         (void)hipFree(sc->counts);
@@ -852,8 +854,8 @@ int lily_scratch_reset_counts(lily_scratch_t* sc) {
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->counts, sc->vocab, 0));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->touched, sc->words + 4, 0));
-    HIP_TRY(launch_fill_u32(sc->s->stream, sc->n_pairs, 1, 0));
-    sc->listed_bound = 0;
+    HIP_TRY(launch_fill_u32(sc->s->stream, sc->list_hdr, LIST_HDR_WORDS + sc->buckets + 1, 0));
+    sc->tail_bound = 0;
     return LILY_OK;
 }
 
@@ -897,12 +899,9 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
                            dst->s->stream));
     HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)src->words * 4,
                            hipMemcpyDeviceToDevice, dst->s->stream));
-    HIP_TRY(hipMemcpyAsync(dst->pos, src->pos, (size_t)src->vocab * 4, hipMemcpyDeviceToDevice,
-                           dst->s->stream));
-    HIP_TRY(hipMemcpyAsync(dst->pairs, src->pairs, (size_t)src->pairs_cap * sizeof(CountPair),
-                           hipMemcpyDeviceToDevice, dst->s->stream));
-    HIP_TRY(hipMemcpyAsync(dst->n_pairs, src->n_pairs, 4, hipMemcpyDeviceToDevice, dst->s->stream));
-    dst->listed_bound = src->listed_bound;
+    // The list is a function of the counts and the bitmap: rebuilt here instead of copied.
+    HIP_TRY(launch_sort_list(dst->s->stream, view_of(dst)));
+    dst->tail_bound = 0;
     return LILY_OK;
 }
 
@@ -912,7 +911,7 @@ int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32
     }
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(launch_add_history(sc->s->stream, view_of(sc), ids_dev, n));
-    sc->listed_bound += n;
+    sc->tail_bound = 0;  // the list was sorted afresh
     return LILY_OK;
 }
 
@@ -924,7 +923,7 @@ int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts) {
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     HIP_TRY(hipMemcpy(sc->counts, host_counts, (size_t)sc->vocab * 4, hipMemcpyHostToDevice));
     HIP_TRY(launch_rebuild_listed(sc->s->stream, view_of(sc)));
-    sc->listed_bound = sc->vocab;
+    sc->tail_bound = 0;
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     return LILY_OK;
 }
@@ -1205,8 +1204,12 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
                            hipMemcpyHostToDevice, s->stream));
     HIP_TRY(hipEventRecord(s->stage_done[slot], s->stream));
     s->stage_used[slot] = true;
+    if (parts[0].sort_first || (n_parts > 1 && parts[1].sort_first)) {
+        HIP_TRY(launch_sort_lists(s->stream, s->table_dev, nullptr, b->rows, b->vocab, true));
+    }
     for (uint32_t q = 0; q < n_parts; ++q) {
-        if (int rc = launch_part(s, parts[q], s->table_dev, (int)b->dtype, b->vocab, 0, 0, q == 0)) {
+        if (int rc = launch_part(s, parts[q], s->table_dev, (int)b->dtype, b->vocab, 0, 0, false,
+                                 q == 0)) {
             return rc;
         }
     }
@@ -1265,6 +1268,10 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->vocab = b->vocab;
     p->dtype = b->dtype;
     p->runs = 0;
+    p->sorted = false;
+    p->since_sort = 0;
+    p->longest_tail = 0;
+    p->sort_on_first_run = p->parts[0].sort_first || (p->n_parts > 1 && p->parts[1].sort_first);
     p->penalised.clear();
     for (uint32_t r = 0; r < b->rows; ++r) {
         // (the table may be reordered: the batch's own arrays tell which scratches count)
@@ -1281,30 +1288,29 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
         return fail(LILY_ERR_INVALID_ARG, "plan is null or not set");
     }
     HIP_TRY(hipSetDevice(p->s->device));
-    for (uint32_t q = 0; q < p->n_parts; ++q) {
-        LaunchPart& part = p->parts[q];
-        if (part.listed != 0 && part.kind == 2 && part.rows <= p->s->ws_rows) {
-            // The lists grow by one id per run at most: take more slices before a workgroup's
-            // buckets overflow (only the merge's share of dynamic LDS depends on the slices).
-            const uint32_t need = slices_for_list(part.listed + p->runs + 1);
-            const uint64_t by_ws =
-                (uint64_t)p->s->ws_slots / ((uint64_t)part.rows * (part.ws_k ? part.ws_k : 1));
-            if (need > part.slices && need <= MAX_SLICES && need <= by_ws) {
-                part.slices = need;
-                const size_t merge = (size_t)need * part.ws_k * 8;
-                if (merge > part.dyn_bytes) {
-                    part.dyn_bytes = merge;
-                }
-            }
+    if (p->longest_tail >= TAIL_SORT_AT || (p->runs == 0 && p->sort_on_first_run)) {
+        // The draws append the ids they count for the first time to their lists' unsorted
+        // tails: one launch sorts every penalised row's list again.
+        HIP_TRY(launch_sort_lists(p->s->stream, p->table_dev, nullptr, p->rows, p->vocab, false));
+        for (lily_scratch* sc : p->penalised) {
+            sc->tail_bound = 0;
         }
-        if (int rc = launch_part(p->s, part, p->table_dev, (int)p->dtype, p->vocab, step_delta, p->runs,
-                                 q == 0)) {
+        p->sorted = true;
+        p->since_sort = 0;
+    }
+    for (uint32_t q = 0; q < p->n_parts; ++q) {
+        const LaunchPart& part = p->parts[q];
+        if (int rc = launch_part(p->s, part, p->table_dev, (int)p->dtype, p->vocab, step_delta,
+                                 p->sorted ? p->since_sort : p->runs, p->sorted, q == 0)) {
             return rc;
         }
     }
     p->runs += 1;
+    p->since_sort += 1;
+    p->longest_tail = 0;
     for (lily_scratch* sc : p->penalised) {
-        sc->listed_bound += 1;
+        sc->tail_bound += 1;
+        p->longest_tail = sc->tail_bound > p->longest_tail ? sc->tail_bound : p->longest_tail;
     }
     return LILY_OK;
 }

@@ -42,6 +42,7 @@ struct StreamLds {
     uint32_t* dmask;   // per queue slot, a byte: bit j set = element j is a listed id
     uint32_t* bkt;
     uint32_t* bfill;
+    uint2* hseg;
     uint32_t* bias_id;
     float* bias_delta;
     __device__ __forceinline__ void init() {
@@ -56,6 +57,7 @@ struct StreamLds {
         bfill = reinterpret_cast<uint32_t*>(b + OFF_BFILL);
         bias_id = reinterpret_cast<uint32_t*>(b + OFF_BIAS);
         bias_delta = reinterpret_cast<float*>(b + OFF_BIAS + STREAM_BIAS_CAP * 4);
+        hseg = reinterpret_cast<uint2*>(b + OFF_HSEG);
     }
 };
 
@@ -111,7 +113,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     constexpr uint32_t QSEG = Q_CAP / NWAVE;
     constexpr uint32_t NONE = 0xffffffffu;
     constexpr uint32_t ID_MASK = (1u << SPEC_ID_BITS) - 1u;
-    constexpr int PREG = 12;  // listed ids a thread keeps in registers between the two bucket passes
+    constexpr int PREG = 2;   // tail entries a thread keeps in registers between the two bucket passes
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const uint32_t nchunks = g.ce - g.cb;
     const uint32_t nblocks = (nchunks + BLOCK - 1) / BLOCK;
@@ -143,26 +145,47 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t c0 = g.cb + b * BLOCK;
         return c0 >= g.main_lo && c0 + BLOCK <= g.main_hi;
     };
-    // ---- the slice's listed ids, bucketed by block
-    // The first PREG x NT list entries are requested together with the list's length (the
-    // list's memory is valid up to pairs_cap whatever the length turns out to be), ahead of
-    // the first block of the row, which is then in flight while the ids are bucketed.
-    uint32_t n_pairs = 0, loaded = 0;
-    uint64_t early[PREG];
+    // ---- the slice's listed ids
+    // The scratch's list comes in two parts.  Its sorted part (ascending ids, indexed by
+    // buckets of 1 << SORT_SHIFT ids) is read straight from memory while the row streams:
+    // block b's entries lie between two bucket starts, requested here by thread b.  Its tail
+    // (the ids first counted since the list was last sorted: a few, the host has the list
+    // sorted again before there are many) is bucketed by block in LDS below, together with
+    // the bias list's ids and a dense mask's barred ids.  The tail's first PREG x NT entries
+    // are requested together with the two lengths (the tail grows downwards from the end of
+    // the list's memory, so their addresses depend on nothing), ahead of the first block of
+    // the row, which is then in flight while they are bucketed.
+    uint32_t n_sorted = 0, n_tail = 0, loaded = 0;
+    uint32_t seg_s = 0, seg_e = 0;   // thread b: block b's entries of the sorted part
+    uint32_t early[PREG];
+    const ListEntry* list = a.pairs;
     if (pen) {
-        // The list's length comes through the scalar path (nothing writes it while the
-        // slices of its row still read it): a vector load of a value that is the same in
-        // every lane is moved to a scalar register at once, and that move would hold the
-        // list's loads below back until the length had arrived.
-        n_pairs = *(const LILY_CONST uint32_t*)a.n_pairs;
-        // The host's bound of the length says how much to request; a longer list is still
-        // read completely (by the loop further down), a shorter one costs idle loads.
-        const uint64_t want = ((uint64_t)a.pairs_hint + cfg.hint_growth + NT - 1) / NT * NT;
+        // The lengths come through the scalar path (nothing writes them while the slices of
+        // their row still read them): a vector load of a value that is the same in every lane
+        // is moved to a scalar register at once, and that move would hold the loads below
+        // back until the lengths had arrived.
+        const LILY_CONST uint32_t* hdr = (const LILY_CONST uint32_t*)a.list_hdr;
+        n_sorted = hdr[HDR_SORTED];
+        n_tail = hdr[HDR_TAIL];
+        if (tid < nblocks) {
+            const uint32_t c0 = max(g.cb + tid * BLOCK, g.main_lo);
+            const uint32_t c1 = min(g.cb + (tid + 1u) * BLOCK, g.main_hi);
+            if (c1 > c0) {
+                const uint32_t id_first = c0 * E - g.pad, id_last = c1 * E - g.pad - 1u;
+                const uint32_t* start = a.list_hdr + LIST_HDR_WORDS;
+                seg_s = gload(start + (id_first >> SORT_SHIFT));
+                seg_e = gload(start + (id_last >> SORT_SHIFT) + 1u);
+            }
+        }
+        // The host's bound of the tail's length says how much to request; a longer tail is
+        // still read completely (by the loop further down), a shorter one costs idle loads.
+        const uint64_t hint = (cfg.hint_replace != 0u ? 0u : a.tail_hint) + (uint64_t)cfg.hint_growth;
+        const uint64_t want = (hint + NT - 1) / NT * NT;
         loaded = (uint32_t)min(want, (uint64_t)min(a.pairs_cap, (uint32_t)(PREG * NT)));
 #pragma unroll
         for (int q = 0; q < PREG; ++q) {
             const uint32_t p = (uint32_t)q * NT + tid;
-            early[q] = p < loaded ? gload(reinterpret_cast<const uint64_t*>(a.pairs) + p) : ~0ull;
+            early[q] = p < loaded ? gload(list + (a.pairs_cap - 1u - p)) : NONE;
         }
     }
     u32x4 buf_a[U], buf_b[U], buf_c[U];
@@ -178,11 +201,22 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     if (tid < Q_CAP / 4) {
         L.dmask[tid] = 0;
     }
+    if (tid < MAX_BUCKETS) {
+        // A list that does not fit its memory is not used (checked below); its bucket starts
+        // then mean nothing, and a start is never taken beyond the sorted part.
+        seg_e = min(seg_e, n_sorted);
+        seg_s = min(seg_s, seg_e);
+        L.hseg[tid] = uint2{seg_s, seg_e};
+        // A block with more listed ids than the workgroup has threads (see row_max below).
+        const uint64_t big = __ballot(seg_e - seg_s > (uint32_t)NT);
+        if (tid == 0) {
+            sh.dense_listed = big != 0ull ? 1u : 0u;
+        }
+    }
     if (tid == 0) {
         sh.n_fc = 0;
         sh.n_drop = 0;
         sh.fail = 0;
-        sh.dense_listed = 0;
     }
     for (uint32_t i = tid; i < n_bias; i += NT) {
         L.bias_id[i] = gload(&a.bias[i].id);
@@ -190,7 +224,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     }
     __syncthreads();
     phase(cfg, 13);
-    if (n_pairs > a.pairs_cap) {
+    if ((uint64_t)n_sorted + n_tail > a.pairs_cap) {
         return stream_fail(cfg, 2u);  // the list overflowed: the bitmap and the counts hold the truth
     }
     // A row with an allow-mask is streamed when the mask is dense: its disallowed ids join the
@@ -218,11 +252,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             n_barred += sh.red_i[i];
         }
         __syncthreads();
-        if ((uint64_t)n_barred + n_pairs + n_bias > SPEC_CAP - SPEC_CAP / 10u) {
+        if ((uint64_t)n_barred + n_tail + n_bias > SPEC_CAP - SPEC_CAP / 10u) {
             return false;  // not a failure: the mask is not dense enough for this select
         }
     }
-    const bool listed_row = n_pairs != 0 || n_bias != 0 || n_barred != 0;
+    // `bucketed`: some listed ids reach the scan through the LDS buckets; `listed_row`: the row
+    // has listed ids at all (the sorted part included).
+    const bool bucketed = n_tail != 0 || n_bias != 0 || n_barred != 0;
+    const bool listed_row = bucketed || n_sorted != 0;
     // Block of a streamed id of this slice, NONE for ids outside it or in a partial chunk.
     auto block_of = [&](uint32_t id) -> uint32_t {
         if (id >= g.vocab) {
@@ -271,7 +308,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
     };
-    if (listed_row && nblocks == 1u) {
+    if (bucketed && nblocks == 1u) {
         // One block: its bucket starts at slot 0, so a single atomic places each entry and
         // there is nothing to count first.
         auto put = [&](uint32_t entry) {
@@ -283,14 +320,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
 #pragma unroll
         for (int q = 0; q < PREG; ++q) {
             const uint32_t p = (uint32_t)q * NT + tid;
-            if (p < n_pairs && p < loaded && block_of((uint32_t)early[q]) != NONE) {
-                put((uint32_t)early[q] | (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS));
+            if (p < n_tail && p < loaded && block_of(early[q] & ID_MASK) != NONE) {
+                put(early[q]);
             }
         }
-        for (uint32_t p = loaded + tid; p < n_pairs; p += NT) {
-            const uint64_t e = gload(reinterpret_cast<const uint64_t*>(a.pairs) + p);
-            if (block_of((uint32_t)e) != NONE) {
-                put((uint32_t)e | (min((uint32_t)(e >> 32), 4095u) << SPEC_ID_BITS));
+        for (uint32_t p = loaded + tid; p < n_tail; p += NT) {
+            const uint32_t e = gload(list + (a.pairs_cap - 1u - p));
+            if (block_of(e & ID_MASK) != NONE) {
+                put(e);
             }
         }
         for (uint32_t i = tid; i < n_bias; i += NT) {
@@ -308,19 +345,18 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (lane == 0) {
             L.bkt[1] = total;
             L.bkt[MAX_BUCKETS] = total;
-            if (total > (uint32_t)NT) {
+            if (total + (L.hseg[0].y - L.hseg[0].x) > (uint32_t)NT) {
                 sh.dense_listed = 1u;
             }
         }
-    } else if (listed_row) {
+    } else if (bucketed) {
         uint32_t packed[PREG];  // id | min(count, 4095) << 20, NONE when not of this slice
 #pragma unroll
         for (int q = 0; q < PREG; ++q) {
             const uint32_t p = (uint32_t)q * NT + tid;
             packed[q] = NONE;
-            if (p < n_pairs && p < loaded && block_of((uint32_t)early[q]) != NONE) {
-                packed[q] = (uint32_t)early[q] |
-                            (min((uint32_t)(early[q] >> 32), 4095u) << SPEC_ID_BITS);
+            if (p < n_tail && p < loaded && block_of(early[q] & ID_MASK) != NONE) {
+                packed[q] = early[q];
             }
         }
         // Entries held in registers take their place inside the bucket with the first pass's
@@ -339,16 +375,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     }
                 }
             }
-            for (uint32_t p = loaded + tid; p < n_pairs; p += NT) {  // what the registers do not hold
-                const uint64_t e = gload(reinterpret_cast<const uint64_t*>(a.pairs) + p);
-                const uint32_t id = (uint32_t)e;
-                const uint32_t b = block_of(id);
+            for (uint32_t p = loaded + tid; p < n_tail; p += NT) {  // what the registers do not hold
+                const uint32_t e = gload(list + (a.pairs_cap - 1u - p));
+                const uint32_t b = block_of(e & ID_MASK);
                 if (b != NONE) {
                     if (pass == 0) {
                         atomicAdd(&L.bkt[b], 1u);
                     } else {
-                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] =
-                            id | (min((uint32_t)(e >> 32), 4095u) << SPEC_ID_BITS);
+                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = e;
                     }
                 }
             }
@@ -374,9 +408,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 phase(cfg, 14);
                 if (tid < 64) {  // counts -> exclusive offsets, total in bkt[MAX_BUCKETS]
                     const uint32_t cnt = L.bkt[tid] + L.bfill[tid];
-                    const uint64_t big = __ballot(cnt > (uint32_t)NT);
-                    if (tid == 0) {
-                        sh.dense_listed = big != 0ull ? 1u : 0u;
+                    const uint64_t big =
+                        __ballot(cnt + (L.hseg[tid].y - L.hseg[tid].x) > (uint32_t)NT);
+                    if (tid == 0 && big != 0ull) {
+                        sh.dense_listed = 1u;
                     }
                     uint32_t incl = cnt;
                     for (int o = 1; o < 64; o <<= 1) {
@@ -507,16 +542,39 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
 
     struct Listed {
         uint32_t ent;
-        float raw;
         u32x4 chunk;
     };
-    // Unconditional as well: a thread without an entry reads the slice's last chunk.
-    auto listed_fetch = [&](Listed& r, uint32_t b, uint32_t round) {
-        r.raw = 0.0f;
-        const uint32_t lo = L.bkt[b], hi = L.bkt[b + 1];
-        const uint32_t e = lo + round * NT + ((tid + NT - ((b * 64u) % NT)) % NT);
-        r.ent = e < hi ? L.spec[min(e, SPEC_CAP - 1u)] : NONE;
-        const uint32_t c = min(((r.ent & ID_MASK) + g.pad) / E, c_last);
+    // A thread's place among block b's listed ids in round `round` (rotated from block to
+    // block so that the same threads do not serve every block's first entries).
+    auto slot_of = [&](uint32_t b, uint32_t round) -> uint32_t {
+        return round * NT + ((tid + NT - ((b * 64u) % NT)) % NT);
+    };
+    // Block b's entries are those of the sorted part between its two bucket starts (ids of
+    // the neighbouring blocks at either end are dropped when the entry is used), then those
+    // of its LDS bucket.  The load is unconditional as well: a thread without an entry reads
+    // some entry of the list (rows without a list read the row's first bytes).
+    const ListEntry* ent_base = pen ? list : reinterpret_cast<const ListEntry*>(g.base);
+    const uint32_t ent_last = pen ? a.pairs_cap - 1u : 0u;
+    auto entry_load = [&](uint32_t b, uint32_t round) -> uint32_t {
+        return gload(ent_base + min(L.hseg[b].x + slot_of(b, round), ent_last));
+    };
+    // `pre`: what entry_load(b, round) returned.  Issues the gather of the entry's chunk; a
+    // thread without an entry reads the slice's last chunk.
+    auto listed_fetch = [&](Listed& r, uint32_t pre, uint32_t b, uint32_t round) {
+        const uint2 seg = L.hseg[b];
+        const uint32_t nh = seg.y - seg.x;
+        const uint32_t lo = L.bkt[b], nl = L.bkt[b + 1] - lo;
+        const uint32_t j = slot_of(b, round);
+        uint32_t ent = NONE;
+        if (j < nh) {
+            if (block_of(pre & ID_MASK) == b) {
+                ent = pre;
+            }
+        } else if (j - nh < nl) {
+            ent = L.spec[min(lo + (j - nh), SPEC_CAP - 1u)];
+        }
+        r.ent = ent;
+        const uint32_t c = min(((ent & ID_MASK) + g.pad) / E, c_last);
         r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
     };
     // The id's own logit out of its chunk (one gather per listed id, not two).
@@ -532,14 +590,23 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
         return elem_of(q, (id + g.pad) % E);
     };
-    // A listed id's true value before the temperature (bias in list order, then penalties);
-    // also feeds the thread's maxima of listed raw and true values.
-    auto listed_value = [&](Listed& r) -> float {
-        if (r.ent == NONE) {
-            return NEG_INF;
+    // Penalties with a repetition factor of at least 1 and non-negative presence and frequency
+    // terms can only lower a value, and a barred id's value is -inf: without a bias list a
+    // listed id's true value never exceeds its raw one.
+    const bool lowering = n_bias == 0u && a.repetition >= 1.0f && a.presence >= 0.0f &&
+                          a.frequency >= 0.0f;
+    // A listed id's raw value, into the thread's maximum of listed raw values (which must
+    // cover every listed id: see row_max).
+    auto listed_raw = [&](const Listed& r) {
+        if (r.ent != NONE) {
+            listed_raw_max = fmaxf(listed_raw_max, raw_of(r.chunk, r.ent & ID_MASK));
         }
+    };
+    // A listed id's true value before the temperature (bias in list order, then penalties);
+    // also feeds the thread's maximum of listed true values (a lower bound of the row's largest
+    // true value whichever ids it covers).
+    auto listed_true = [&](const Listed& r, float raw) -> float {
         const uint32_t id = r.ent & ID_MASK;
-        r.raw = raw_of(r.chunk, id);
         uint32_t cnt = r.ent >> SPEC_ID_BITS;
         if (cnt == 4095u) {
             cnt = gload(a.counts + id);
@@ -547,7 +614,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // every thread drain the loads it has in flight.
             asm volatile("" : "+v"(cnt));
         }
-        float t = r.raw;
+        float t = raw;
         for (uint32_t j = 0; j < n_bias; ++j) {
             if (L.bias_id[j] == id) {
                 t += L.bias_delta[j];
@@ -560,26 +627,31 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (masked && !bit_of(a.allow, id)) {
             t = NEG_INF;
         }
-        listed_raw_max = fmaxf(listed_raw_max, r.raw);
         listed_true_max = fmaxf(listed_true_max, t);
         return t;
     };
     // After the block's bound is known: was the id's chunk queued or summed by its owner (the
-    // owner's tests on the same bits), the id's terms, and the id as a candidate.
-    auto listed_finish = [&](const Listed& r, float t, bool nonneg) {
-        if (r.ent == NONE) {
+    // owner's tests on the same bits), the id's terms, and the id as a candidate.  When values
+    // can only be lowered, an id whose chunk was neither queued nor summed is below the bound
+    // and below the sum's cut with its true value too: nothing of it is evaluated (most blocks
+    // of most rows hold no other kind, and their waves skip all of this).
+    auto listed_finish = [&](const Listed& r, bool nonneg) {
+        const bool has = r.ent != NONE;
+        const float cm = nonneg ? chunk_max_nonneg<DT>(r.chunk) : chunk_max<DT>(r.chunk);
+        const bool queued = cm >= T;
+        const bool summed = !queued && cm > skip_b;  // the cut is -inf without a row sum
+        if (!has || (lowering && !queued && !(want_lse && summed))) {
             return;
         }
         const uint32_t id = r.ent & ID_MASK;
-        const float cm = nonneg ? chunk_max_nonneg<DT>(r.chunk) : chunk_max<DT>(r.chunk);
-        const bool queued = cm >= T;
-        const bool summed = !queued && cm > skip_b;
+        const float raw = raw_of(r.chunk, id);
+        const float t = listed_true(r, raw);
         if (want_lse) {
             if (t > skip_b) {  // the same cut as for streamed terms
                 acc_t += term_d(t);
             }
             if (summed) {
-                acc_r += term_d(r.raw);
+                acc_r += term_d(raw);
             }
         }
         if (queued) {
@@ -634,7 +706,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 }
             }
         }
-        const float lcur_t = listed_row ? listed_value(lcur) : NEG_INF;
+        if (listed_row) {
+            listed_raw(lcur);
+        }
         // The block's own maxima enter the bound before the block is filtered.  Chunks below
         // the previous bound cannot be queued: their terms are summed right away.
         const float T_prev = T;
@@ -712,12 +786,20 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
         if (listed_row) {
-            listed_finish(lcur, lcur_t, nonneg);
-            const uint32_t n_b = L.bkt[b + 1] - L.bkt[b];
+            listed_finish(lcur, nonneg);
+            const uint32_t n_b = (L.hseg[b].y - L.hseg[b].x) + (L.bkt[b + 1] - L.bkt[b]);
             for (uint32_t round = 1; round * NT < n_b; ++round) {
+                // Rare (a block with more listed ids than threads).  Both loads are waited for
+                // right here, inside the loop: left to the first use, their waits would be
+                // placed where every path meets and drain the blocks requested ahead.
                 Listed extra;
-                listed_fetch(extra, b, round);
-                listed_finish(extra, listed_value(extra), nonneg);
+                uint32_t e = entry_load(b, round);
+                asm volatile("" : "+v"(e));
+                listed_fetch(extra, e, b, round);
+                asm volatile("" : "+v"(extra.chunk.x), "+v"(extra.chunk.y), "+v"(extra.chunk.z),
+                             "+v"(extra.chunk.w));
+                listed_raw(extra);
+                listed_finish(extra, nonneg);
             }
         }
     };
@@ -725,28 +807,36 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // cache and nothing uses the result): with the same loads in flight on every path the
     // wait for a block's data leaves the blocks requested after it in flight, where a request
     // that may be skipped makes that wait count as if it had been.
-    auto request = [&](u32x4 (&dst)[U], Listed& ldst, uint32_t b) {
+    // A block's entry of the sorted part is requested two requests ahead of its gather, which
+    // therefore never waits for anything younger than the block the next `work` needs anyway:
+    // `pre` is this block's entry, `ahead` receives the one of the block after next.
+    auto request = [&](u32x4 (&dst)[U], Listed& ldst, uint32_t pre, uint32_t& ahead, uint32_t b) {
         const uint32_t bb = min(b, nblocks - 1u);
         if (listed_row) {
-            listed_fetch(ldst, bb, 0);
+            listed_fetch(ldst, pre, bb, 0);
+            ahead = entry_load(min(b + 2u, nblocks - 1u), 0);
         }
         fetch(dst, bb);
     };
     if (nblocks == 0) {
         refresh_bound(true, true);  // the same barriers in every workgroup
     } else {
+        uint32_t pre_a = 0, pre_b = 0, pre_c = 0;
         if (listed_row) {
-            listed_fetch(lst_a, 0, 0);
+            pre_a = entry_load(0, 0);
+            pre_b = entry_load(min(1u, nblocks - 1u), 0);
+            pre_c = entry_load(min(2u, nblocks - 1u), 0);
+            listed_fetch(lst_a, pre_a, 0, 0);
         }
-        request(buf_b, lst_b, 1);
+        request(buf_b, lst_b, pre_b, pre_a, 1);
         for (uint32_t b = 0; b < nblocks; b += 3) {
-            request(buf_c, lst_c, b + 2);
+            request(buf_c, lst_c, pre_c, pre_b, b + 2);
             work(buf_a, lst_a, b);
             if (b + 1 < nblocks) {
-                request(buf_a, lst_a, b + 3);
+                request(buf_a, lst_a, pre_a, pre_c, b + 3);
                 work(buf_b, lst_b, b + 1);
                 if (b + 2 < nblocks) {
-                    request(buf_b, lst_b, b + 4);
+                    request(buf_b, lst_b, pre_b, pre_a, b + 4);
                     work(buf_c, lst_c, b + 2);
                 }
             }

@@ -136,25 +136,35 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
 
 // ------------------------------------------------------------------ tail
 
+// Lists an id that has just been counted for the first time: it joins the tail, which grows
+// downwards from the end of the list's memory (the sorted part grows upwards from its start;
+// when the two would meet the id stays unlisted and the lengths tell that the list is unusable).
+__device__ __forceinline__ void list_new_id(ListEntry* pairs, uint32_t* list_hdr, uint32_t* pos,
+                                            uint32_t pairs_cap, uint32_t id, uint32_t count) {
+    const uint32_t t = atomicAdd(&list_hdr[HDR_TAIL], 1u);
+    const uint32_t n_sorted = list_hdr[HDR_SORTED];
+    const bool fits = (uint64_t)n_sorted + t < pairs_cap;
+    const uint32_t at = fits ? pairs_cap - 1u - t : 0xffffffffu;
+    if (fits) {
+        pairs[at] = list_entry(id, count);
+    }
+    pos[id] = at;  // listed ids always have a meaningful pos
+}
+
 // Counts one emission of `id` in a scratch: the dense count, and the id's entry in the list
-// (appended with the first count; `touched` marks the listed ids).
-__device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched, CountPair* pairs,
-                                            uint32_t* n_pairs, uint32_t* pos, uint32_t pairs_cap,
+// (`touched` marks the listed ids).
+__device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched, ListEntry* pairs,
+                                            uint32_t* list_hdr, uint32_t* pos, uint32_t pairs_cap,
                                             uint32_t id) {
     const uint32_t before = atomicAdd(&counts[id], 1u);
     const uint32_t bit = 1u << (id & 31u);
     const uint32_t bits = atomicOr(&touched[id >> 5], bit);
     if ((bits & bit) == 0u) {
-        const uint32_t p = atomicAdd(n_pairs, 1u);
-        if (p < pairs_cap) {
-            pairs[p].id = id;
-            pairs[p].count = before + 1u;
-        }
-        pos[id] = p < pairs_cap ? p : 0xffffffffu;  // listed ids always have a meaningful pos
+        list_new_id(pairs, list_hdr, pos, pairs_cap, id, before + 1u);
     } else {
         const uint32_t p = pos[id];
         if (p < pairs_cap) {
-            pairs[p].count = before + 1u;
+            pairs[p] = list_entry(id, before + 1u);
         }
     }
 }
@@ -162,7 +172,7 @@ __device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched,
 __device__ __forceinline__ void emit(const RowArgs& a, uint32_t id) {
     *a.out_id = id;
     if (a.flags & F_PEN) {
-        count_token(a.counts, a.touched, a.pairs, a.n_pairs, a.pos, a.pairs_cap, id);
+        count_token(a.counts, a.touched, a.pairs, a.list_hdr, a.pos, a.pairs_cap, id);
     }
 }
 
@@ -213,14 +223,9 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
     }
     if (pen) {
         if ((bits & bit) == 0u) {
-            const uint32_t at = atomicAdd(a.n_pairs, 1u);
-            if (at < a.pairs_cap) {
-                a.pairs[at].id = id;
-                a.pairs[at].count = before + 1u;
-            }
-            a.pos[id] = at < a.pairs_cap ? at : 0xffffffffu;
+            list_new_id(a.pairs, a.list_hdr, a.pos, a.pairs_cap, id, before + 1u);
         } else if (p < a.pairs_cap) {
-            a.pairs[p].count = before + 1u;
+            a.pairs[p] = list_entry(id, before + 1u);
         }
     }
 }

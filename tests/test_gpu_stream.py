@@ -173,9 +173,10 @@ def test_lists_beyond_the_workgroup_and_the_scratch(sampler):
         s_.close()
 
 
-def test_long_lists_are_spread_over_more_slices():
-    """6 000 listed ids per row: the launch takes enough slices for every workgroup to bucket
-    its share, so the streaming select still serves every slice."""
+def test_long_lists_are_read_in_place():
+    """6 000 listed ids per row, far more than a workgroup could bucket in LDS: the sorted list
+    is read from memory block by block, so the streaming select serves every slice at the
+    slice count the batch size alone asks for."""
     s = LS.Sampler(0)
     rng = np.random.default_rng(15)
     vocab, rows = 151_936, 300
@@ -189,7 +190,7 @@ def test_long_lists_are_spread_over_more_slices():
     r = run_rows(s, x, kw, [0] * rows, scratch=sc, logprobs=True)
     s.set_path_stats(None)
     st = stats.cpu().tolist()
-    assert st[0] > rows and st[1] == 0 and st[2] == 0, st
+    assert st[0] == rows * s.slices_for(rows, 40, vocab, bf16=True) and st[1] == 0 and st[2] == 0, st
     for i in range(0, rows, 7):
         d = O.sample(x[i], counts[i], o_params(**kw[i]), 0, want_logprob=True)
         check_row_against_oracle(r, i, d)
