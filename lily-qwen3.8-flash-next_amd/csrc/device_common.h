@@ -222,14 +222,12 @@ struct Shared {
     double lse_s;    // sum of 2^(x * log2e / T - lse_mc) over the row
     // streaming select
     float bound[2][NWAVE];   // each wave's lower bound of its share of the k-th largest (two parities)
-    float wmax[2][3][NWAVE];  // each wave's largest raw value, largest raw and largest true value
-                              // of listed ids so far
-    uint32_t dense_listed;    // some block holds more listed ids than the workgroup has threads
+    float wmax[2][2][NWAVE];  // each wave's largest raw value, and its largest among chunks without a
+                              // listed id
     uint32_t qfill[NWAVE];   // chunks each wave queued
     uint32_t n_fc;           // final candidates
-    uint32_t n_drop;         // listed ids found inside queued chunks
     uint32_t fail;
-    double red3[3][NWAVE];
+    double red3[4][NWAVE];
 };
 
 // Running sum of 2^(v*c - mc) of one thread with its own reference mc.
@@ -654,9 +652,11 @@ constexpr float LSE_RAISE = 24.0f;
 struct WaveLse {
     float ref;
     float s;
+    float booked;   // what the caller took off `s` again, kept relative to the same reference
     __device__ __forceinline__ void init() {
         ref = F32_LOWEST;
         s = 0.0f;
+        booked = 0.0f;
     }
     // Adds the E terms of one load whose lane maximum is m; skipped by the whole wave when
     // every term is below 2^-40 of the reference.
@@ -665,7 +665,9 @@ struct WaveLse {
         if (__ballot(__builtin_fmaf(m, c, -ref) > LSE_RAISE) != 0ull) {
             // A term would dwarf the reference: raise it to the wave's maximum (rare).
             const float nref = fmaxf(ref, wave_max_f(m * c));
-            s *= __builtin_amdgcn_exp2f(ref - nref);
+            const float down = __builtin_amdgcn_exp2f(ref - nref);
+            s *= down;
+            booked *= down;
             ref = nref;
         }
         if (__ballot(__builtin_fmaf(m, c, -ref) > -40.0f) == 0ull) {
@@ -681,7 +683,9 @@ struct WaveLse {
         const float d = __builtin_fmaf(active ? m : NEG_INF, c, -ref);
         if (__ballot(d > LSE_RAISE) != 0ull) {
             const float nref = fmaxf(ref, wave_max_f(active ? m * c : NEG_INF));
-            s *= __builtin_amdgcn_exp2f(ref - nref);
+            const float down = __builtin_amdgcn_exp2f(ref - nref);
+            s *= down;
+            booked *= down;
             ref = nref;
         } else if (__ballot(d > -40.0f) == 0ull) {
             return;
@@ -703,7 +707,9 @@ struct WaveLse {
     __device__ __forceinline__ void prepare(float block_max, float c) {
         if (__ballot(__builtin_fmaf(block_max, c, -ref) > LSE_RAISE) != 0ull) {
             const float nref = fmaxf(ref, wave_max_dpp(block_max * c));
-            s *= __builtin_amdgcn_exp2f(ref - nref);
+            const float down = __builtin_amdgcn_exp2f(ref - nref);
+            s *= down;
+            booked *= down;
             ref = nref;
         }
     }

@@ -18,14 +18,8 @@ hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const u
 hipError_t launch_uncount(hipStream_t stream, const ScratchView& sc, uint32_t token);
 hipError_t launch_uncount_after(hipStream_t stream, const ScratchView& sc, const uint32_t* draws,
                                 uint32_t m, const uint32_t* accepted, uint32_t cap);
-// touched = the ids with a non-zero count, then the list sorted afresh.
+// touched = the ids with a non-zero count.
 hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc);
-// A scratch's list rebuilt in ascending id order from its bitmap and counts (tail emptied).
-hipError_t launch_sort_list(hipStream_t stream, const ScratchView& sc);
-// The same for the penalised rows of a packed table (device) or of inline rows (host): those
-// marked F_SORT_FIRST, or all of them.
-hipError_t launch_sort_lists(hipStream_t stream, const RowArgs* table_dev, const InlineRows* inline_rows,
-                             uint32_t rows, uint32_t vocab, bool flagged_only);
 hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const uint32_t* ids,
                               uint32_t* ctrl, uint32_t m, uint32_t pos0, uint32_t ratio,
                               uint32_t chain);

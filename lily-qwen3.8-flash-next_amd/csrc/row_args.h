@@ -20,32 +20,14 @@ enum : uint32_t {
     F_UNIFORM = 2u,  // use `uniform` (and `uniform2`) instead of the seeded draws
     F_FORCED = 4u,   // emit `forced`
     F_STREAM = 8u,   // eligible for the streaming select (k <= 64, no allow-mask, short bias list)
-    F_SORT_FIRST = 16u,  // host only: this row's list is due for sorting before the launch
 };
-
-// One entry of a scratch's list of the ids that were ever counted: the id in the low
-// LIST_ID_BITS bits, min(count, LIST_COUNT_MAX) above them (a saturated entry sends the reader
-// to the dense counts).
-typedef uint32_t ListEntry;
-constexpr uint32_t LIST_ID_BITS = 20;
-constexpr uint32_t LIST_COUNT_MAX = 4095;
-__host__ __device__ inline ListEntry list_entry(uint32_t id, uint32_t count) {
-    return id | ((count < LIST_COUNT_MAX ? count : LIST_COUNT_MAX) << LIST_ID_BITS);
-}
 
 struct alignas(16) RowArgs {
     const void* logits;        // this row's first element
     const uint32_t* allow;     // packed allow bits or null
     uint32_t* counts;          // dense emission histogram or null
-    uint32_t* touched;         // bit per id that is in `pairs` (set with the first count), or null
-    ListEntry* pairs;          // the listed ids with their counts (a count may have gone back to 0):
-                               // [0, n_sorted) in ascending id order, and the ids first counted
-                               // since the list was last sorted at [pairs_cap - n_tail, pairs_cap),
-                               // newest lowest
-    uint32_t* list_hdr;        // [LIST_HDR_WORDS + buckets + 1]: n_sorted, n_tail, two spare words,
-                               // then start[b] = entries of the sorted part whose id is below
-                               // b << SORT_SHIFT (n_sorted + n_tail above pairs_cap: the list is unusable)
-    uint32_t* pos;             // [vocab] pairs index of a listed id
+    uint32_t* touched;         // bit per id that was ever counted (a count may have gone back to
+                               // 0), or null
     const lily_bias* bias;     // n_bias pairs or null
     uint32_t* out_id;
     float* out_logprob;        // or null
@@ -72,29 +54,15 @@ struct alignas(16) RowArgs {
     float repetition;
     float uniform;
     float uniform2;
-    uint32_t pairs_cap;
-    uint32_t tail_hint;        // host's upper bound of n_tail when the row was packed (saves loads only)
-    uint32_t pad;
+    uint32_t pad[3];
 };
-static_assert(sizeof(RowArgs) == 224, "RowArgs layout");
-
-// The sorted part of a scratch's list is indexed by buckets of 1 << SORT_SHIFT ids.
-constexpr uint32_t SORT_SHIFT = 8;
-constexpr uint32_t LIST_HDR_WORDS = 4;   // n_sorted, n_tail, two spare words; the bucket starts follow
-constexpr uint32_t HDR_SORTED = 0, HDR_TAIL = 1;
-// Draws append to the unsorted tail; the host has the list sorted again (one launch over the
-// batch's scratches) before its bound of the tail's length passes this.
-constexpr uint32_t TAIL_SORT_AT = 256;
+static_assert(sizeof(RowArgs) == 192, "RowArgs layout");
 
 // A scratch's device state as the small maintenance kernels take it.
 struct ScratchView {
     uint32_t* counts;    // [vocab]
     uint32_t* touched;   // [ceil(vocab / 32) + 4]
-    ListEntry* pairs;    // [pairs_cap]
-    uint32_t* list_hdr;  // [LIST_HDR_WORDS + ceil(vocab >> SORT_SHIFT) + 1]
-    uint32_t* pos;       // [vocab]
     uint32_t vocab;
-    uint32_t pairs_cap;
 };
 
 constexpr int INLINE_ROWS = 8;
@@ -119,8 +87,6 @@ struct LaunchCfg {
     uint32_t excl_words;    // words reserved for the slice bitmap (the specials' id list follows)
     uint32_t list_cap;      // ids the specials' list holds
     uint32_t bitmap_layout;    // dynamic LDS holds cand_cap candidates + the bitmap + the id list
-    uint32_t hint_growth;   // added to every row's tail_hint (draws since the table was packed)
-    uint32_t hint_replace;  // the lists were sorted since: hint_growth alone bounds the tails
     uint32_t dyn_slots;     // 64-bit slots of dynamic LDS in all
     uint32_t* path_stats;   // null, or [4] counters: slices finished by the streaming select, the
                             // bitmap select, the exhaustive select; [3] unused
@@ -133,28 +99,29 @@ constexpr uint32_t MERGE_CAP = 4096;  // candidates the merging workgroup gather
 constexpr uint32_t MAX_SLICES = 64;
 constexpr uint32_t SPECIAL_LIST_CAP = 2048;  // ids of penalised / biased tokens gathered per batch
 
-// Streaming select (k <= STREAM_K_MAX, no allow-mask): dynamic LDS layout in bytes.
+// Streaming select (k <= STREAM_K_MAX): dynamic LDS layout in bytes.
 constexpr uint32_t STREAM_K_MAX = 64;
 constexpr uint32_t STREAM_UNROLL = 4;      // 16-byte chunks per thread per block
 constexpr uint32_t Q_CAP = 768;            // queued chunks (those holding a value at or above the bound)
-constexpr uint32_t SPEC_CAP = 3072;        // penalised / biased ids of one slice
 constexpr uint32_t FC_CAP = 1024;          // final candidates
-constexpr uint32_t DROP_CAP = 128;         // penalised / biased ids found inside queued chunks
-constexpr uint32_t MAX_BUCKETS = 64;       // blocks of one slice
+constexpr uint32_t MAX_BLOCKS = 64;        // blocks of one slice
 constexpr uint32_t STREAM_BIAS_CAP = 64;   // bias pairs kept in LDS
-constexpr uint32_t SPEC_ID_BITS = LIST_ID_BITS;  // an LDS bucket entry has the list's own format
+// A wave's window into a bitmap of the row's ids (listed ids, barred ids): for each of the block's
+// four loads the words that hold the bits of the wave's 64 chunks, one more for rows whose chunks
+// do not start on a word of the bitmap.
+constexpr uint32_t WIN_PIECE_MAX = 64 * 8 / 32 + 1;           // bf16: 64 chunks of 8 ids
+constexpr uint32_t WIN_WORDS = STREAM_UNROLL * WIN_PIECE_MAX; // per wave and bitmap
 constexpr uint32_t OFF_QRAW = 0;
 constexpr uint32_t OFF_QIDX = OFF_QRAW + Q_CAP * 16;
-constexpr uint32_t OFF_SPEC = OFF_QIDX + Q_CAP * 4;
-constexpr uint32_t OFF_FC = OFF_SPEC + SPEC_CAP * 4;
-constexpr uint32_t OFF_DROP = OFF_FC + FC_CAP * 8;
-constexpr uint32_t OFF_DMASK = OFF_DROP + DROP_CAP * 4;       // a byte per queue slot
-constexpr uint32_t OFF_BKT = OFF_DMASK + Q_CAP;               // [MAX_BUCKETS + 1] offsets
-constexpr uint32_t OFF_BFILL = OFF_BKT + (MAX_BUCKETS + 4) * 4;   // [MAX_BUCKETS] fill counters
-constexpr uint32_t OFF_BIAS = OFF_BFILL + MAX_BUCKETS * 4;    // ids then deltas
-constexpr uint32_t OFF_HSEG = OFF_BIAS + STREAM_BIAS_CAP * 8; // [MAX_BUCKETS] (first, end) of each block's
-                                                              // entries in the sorted part of the list
-constexpr uint32_t STREAM_LDS_BYTES = OFF_HSEG + MAX_BUCKETS * 8;
-static_assert(OFF_FC % 8 == 0 && STREAM_LDS_BYTES % 16 == 0, "stream LDS layout");
+constexpr uint32_t OFF_QBITS = OFF_QIDX + Q_CAP * 4;          // a byte per queue slot: its listed elements
+constexpr uint32_t OFF_WIN = OFF_QBITS + Q_CAP;               // [4 waves][2 bitmaps][WIN_WORDS]
+constexpr uint32_t OFF_BLK = OFF_WIN + 4 * 2 * WIN_WORDS * 4; // [MAX_BLOCKS] x (bound, cut, flags)
+constexpr uint32_t OFF_BIAS = OFF_BLK + MAX_BLOCKS * 12;      // ids then deltas
+// The final candidates lie above everything the tail and the merge use (the sorted candidates
+// and the tail's three float arrays: K_CAP * 8 + 3 * K_CAP * 4 bytes from the start).
+constexpr uint32_t OFF_FC = 20480;
+constexpr uint32_t STREAM_LDS_BYTES = OFF_FC + FC_CAP * 8;
+static_assert(OFF_BIAS + STREAM_BIAS_CAP * 8 <= OFF_FC, "stream LDS layout");
+static_assert(OFF_FC % 8 == 0 && OFF_WIN % 4 == 0 && STREAM_LDS_BYTES % 16 == 0, "stream LDS layout");
 
 }  // namespace lily

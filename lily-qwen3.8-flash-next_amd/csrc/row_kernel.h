@@ -74,8 +74,21 @@ __device__ __forceinline__ uint64_t slice_argmax(const RowArgs& a, const Geo<DT>
 
 // ------------------------------------------------------------------ the row kernel
 
+// The row's arguments are the same for every thread: read through the constant address
+// space they arrive by scalar loads and stay in scalar registers.
+__device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowArgs* src) {
+    static_assert(sizeof(RowArgs) % 16 == 0, "RowArgs is copied in 16-byte pieces");
+    const LILY_CONST u32x4* from = (const LILY_CONST u32x4*)src;
+    u32x4* to = reinterpret_cast<u32x4*>(&a);
+    for (unsigned i = 0; i < sizeof(RowArgs) / 16; ++i) {
+        to[i] = from[i];
+    }
+}
+
 template <int DT, int KIND, bool LSE>
-__device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg, Shared& sh) {
+__device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const LaunchCfg& cfg, Shared& sh) {
+    RowArgs a;
+    load_row_args(a, src);
     // KIND: 0 = rows without masks, penalties or bias lists, 1 = rows with any of them (the
     // bitmap select is compiled for them), 2 = streaming rows only (no bitmap select at all).
     constexpr bool EXCL = KIND == 1;
@@ -150,7 +163,16 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
         }
     }
 
-    const bool forced = (a.flags & F_FORCED) != 0;
+    // What follows reads the row's arguments afresh (scalar loads, served by the scalar cache):
+    // kept in registers across the scan, the fields that only the merge and the tail use
+    // crowd the scan's own values out of the scalar registers.
+    RowArgs t;
+    {
+        const LILY_CONST RowArgs* again = src;
+        asm volatile("" : "+s"(again));
+        load_row_args(t, again);
+    }
+    const bool forced = (t.flags & F_FORCED) != 0;
     uint32_t n = (argmax || forced) ? 0u : min(sh.n_cand, cfg.cand_cap);
     phase(cfg, 4);
     if (S > 1) {
@@ -240,7 +262,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
             for (int q = 0; q < PER; ++q) {
                 best_mine = mine[q] > best_mine ? mine[q] : best_mine;
             }
-            const uint32_t kw = (a.k + NWAVE - 1) / NWAVE;
+            const uint32_t kw = (t.k + NWAVE - 1) / NWAVE;
             const uint32_t P = kw <= 64u ? wave_kth_key16((uint32_t)(best_mine >> 48), kw) : 0u;
             if ((tid & 63u) == 0) {
                 sh.red_i[tid >> 6] = P;
@@ -262,7 +284,7 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
             __syncthreads();
             n = sh.n_cand;
             sorted = false;
-            n = select_topk(cand, n, a.k, sh, sorted);
+            n = select_topk(cand, n, t.k, sh, sorted);
             found = cand;
         }
     }
@@ -271,17 +293,17 @@ __device__ __forceinline__ void row_body(const RowArgs& a, const LaunchCfg& cfg,
     if (argmax) {
         if (tid == 0) {
             const uint32_t id = composite_id(best);
-            *a.out_id = id == 0xffffffffu ? 0u : id;
+            *t.out_id = id == 0xffffffffu ? 0u : id;
         }
         return;
     }
-    if (a.flags & F_FORCED) {
+    if (t.flags & F_FORCED) {
         if (tid == 0) {
-            finish_token<DT>(a, sh, a.forced, vocab);
+            finish_token<DT>(t, sh, t.forced, vocab);
         }
         return;
     }
-    tail<DT, KIND != 2>(a, vocab, step, n, sorted, found, sh, cfg);
+    tail<DT, KIND != 2>(t, vocab, step, n, sorted, found, sh, cfg);
     phase(cfg, 7);
 }
 
@@ -295,17 +317,6 @@ __device__ __forceinline__ void tail_arrays(Shared& sh) {
     sh.res = f + 2 * K_CAP;
 }
 
-// The row's arguments are the same for every thread: read through the constant address
-// space they arrive by scalar loads and stay in scalar registers.
-__device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowArgs* src) {
-    static_assert(sizeof(RowArgs) % 16 == 0, "RowArgs is copied in 16-byte pieces");
-    const LILY_CONST u32x4* from = (const LILY_CONST u32x4*)src;
-    u32x4* to = reinterpret_cast<u32x4*>(&a);
-    for (unsigned i = 0; i < sizeof(RowArgs) / 16; ++i) {
-        to[i] = from[i];
-    }
-}
-
 template <int DT, int KIND, bool LSE>
 __global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_inline(InlineRows rows, LaunchCfg cfg) {
     __shared__ Shared sh;
@@ -313,26 +324,22 @@ __global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_inline(InlineRow
     // (indexing the by-value copy would move all of it to scratch memory).
     const LILY_CONST RowArgs* table =
         (const LILY_CONST RowArgs*)__builtin_amdgcn_kernarg_segment_ptr();
-    RowArgs a;
-    load_row_args(a, table + blockIdx.y);
     if (threadIdx.x == 0) {
         tail_arrays(sh);
     }
     __syncthreads();
-    row_body<DT, KIND, LSE>(a, cfg, sh);
+    row_body<DT, KIND, LSE>(table + blockIdx.y, cfg, sh);
 }
 
 template <int DT, int KIND, bool LSE>
 __global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_table(LaunchCfg cfg) {
     __shared__ Shared sh;
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
-    RowArgs a;
-    load_row_args(a, table + blockIdx.y);
     if (threadIdx.x == 0) {
         tail_arrays(sh);
     }
     __syncthreads();
-    row_body<DT, KIND, LSE>(a, cfg, sh);
+    row_body<DT, KIND, LSE>(table + blockIdx.y, cfg, sh);
 }
 
 template <int DT, int KIND, bool LSE>

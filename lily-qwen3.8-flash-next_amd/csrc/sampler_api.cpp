@@ -79,15 +79,8 @@ struct lily_scratch {
     lily_sampler* s = nullptr;
     uint32_t vocab = 0;
     uint32_t words = 0;
-    uint32_t pairs_cap = 0;
-    uint32_t* counts = nullptr;   // [vocab]; the one allocation, the rest follows it
-    uint32_t* pos = nullptr;      // [vocab] pairs index of a listed id
-    uint32_t* touched = nullptr;  // [words + 4] bit per listed id
-    ListEntry* pairs = nullptr;   // [pairs_cap] listed ids with their counts
-    uint32_t* list_hdr = nullptr; // [LIST_HDR_WORDS + buckets + 1] lengths, then the bucket starts
-    uint32_t buckets = 0;
-    uint32_t tail_bound = 0;      // host's upper bound of the unsorted tail's length (draws
-                                  // enqueued since the list was last sorted)
+    uint32_t* counts = nullptr;   // [vocab]; the one allocation, the bitmap follows it
+    uint32_t* touched = nullptr;  // [words + 4] bit per id that was ever counted
 };
 
 struct lily_draft_dists {
@@ -110,7 +103,6 @@ struct LaunchPart {
     uint32_t excl_words = 0;
     bool bitmap_layout = false;
     uint32_t cand_cap = 0;
-    bool sort_first = false;                 // some row's list is sorted before the launch
 };
 
 struct lily_plan {
@@ -123,26 +115,15 @@ struct lily_plan {
     LaunchPart parts[2];                     // the batch's one or two launches
     uint32_t n_parts = 0;
     uint32_t runs = 0;                       // launches since the table was packed
-    bool sort_on_first_run = false;          // a row's list was due for sorting when it was packed
-    bool sorted = false;                     // the lists were sorted by a run of this plan, so
-    uint32_t since_sort = 0;                 // the tails hold at most this many ids
-    uint32_t longest_tail = 0;               // largest bound of a tail among the scratches
-    std::vector<lily_scratch*> penalised;    // scratches whose rows count their draws
 };
 
 namespace {
-
-constexpr uint32_t PAIRS_CAP = 65536;  // listed ids a scratch keeps (more: the list is not used)
 
 ScratchView view_of(const lily_scratch* sc) {
     ScratchView v;
     v.counts = sc->counts;
     v.touched = sc->touched;
-    v.pairs = sc->pairs;
-    v.list_hdr = sc->list_hdr;
-    v.pos = sc->pos;
     v.vocab = sc->vocab;
-    v.pairs_cap = sc->pairs_cap;
     return v;
 }
 
@@ -222,16 +203,6 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
     if (pen) {
         out->counts = scratch->counts;
         out->touched = scratch->touched;
-        out->pairs = scratch->pairs;
-        out->list_hdr = scratch->list_hdr;
-        out->pos = scratch->pos;
-        out->pairs_cap = scratch->pairs_cap;
-        if (scratch->tail_bound >= TAIL_SORT_AT) {
-            out->flags |= F_SORT_FIRST;  // the launch is preceded by a sort of this row's list
-            scratch->tail_bound = 0;
-        }
-        out->tail_hint = scratch->tail_bound;
-        scratch->tail_bound += 1;  // this draw may list one more id
         out->flags |= F_PEN;
     }
     if (x.has_uniform) {
@@ -259,8 +230,7 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
     out->presence = params->presence_penalty;
     out->frequency = params->frequency_penalty;
     out->repetition = params->repetition_penalty;
-    if (mode != MODE_ARGMAX && k <= STREAM_K_MAX && out->n_bias <= STREAM_BIAS_CAP &&
-        vocab <= (1u << SPEC_ID_BITS)) {
+    if (mode != MODE_ARGMAX && k <= STREAM_K_MAX && out->n_bias <= STREAM_BIAS_CAP) {
         out->flags |= F_STREAM;
     }
     return LILY_OK;
@@ -417,10 +387,6 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
         const RowArgs* sub = table + part.first;
         part.ws_k = max_k(sub, part.rows);
         part.slices = choose_slices(s, part.rows, part.ws_k, vocab, dtype);
-        part.sort_first = false;
-        for (uint32_t i = 0; i < part.rows; ++i) {
-            part.sort_first = part.sort_first || (sub[i].flags & F_SORT_FIRST) != 0;
-        }
         const LaunchShape shp = shape_of(s, sub, part.rows, dtype, vocab, part.slices, part.ws_k);
         part.kind = shp.kind();
         part.lse = shp.lse;
@@ -433,8 +399,7 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
 }
 
 int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_dev, int dtype,
-                uint32_t vocab, uint32_t step_delta, uint32_t hint_growth, bool hint_replace,
-                bool traced) {
+                uint32_t vocab, uint32_t step_delta, bool traced) {
     LaunchCfg cfg;
     fill_cfg(s, &cfg, vocab, part.slices, part.ws_k, step_delta, table_dev + part.first);
     if (traced) {
@@ -443,8 +408,6 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
     cfg.excl_words = part.excl_words;
     cfg.bitmap_layout = part.bitmap_layout ? 1u : 0u;
     cfg.cand_cap = part.cand_cap;
-    cfg.hint_growth = hint_growth;
-    cfg.hint_replace = hint_replace ? 1u : 0u;
     HIP_TRY(launch_rows(s->stream, dtype, part.kind, part.lse, part.rows, cfg, nullptr, part.dyn_bytes));
     return LILY_OK;
 }
@@ -452,13 +415,6 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
 int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n) {
     HIP_TRY(hipSetDevice(s->device));
     const uint32_t kmax = max_k(rows.r, n);
-    bool sort_first = false;
-    for (uint32_t i = 0; i < n; ++i) {
-        sort_first = sort_first || (rows.r[i].flags & F_SORT_FIRST) != 0;
-    }
-    if (sort_first) {
-        HIP_TRY(launch_sort_lists(s->stream, nullptr, &rows, n, vocab, true));
-    }
     LaunchCfg cfg;
     const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
@@ -807,30 +763,15 @@ int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out)
     sc->s = s;
     sc->vocab = vocab;
     sc->words = (vocab + 31u) / 32u;
-    sc->pairs_cap = vocab < PAIRS_CAP ? vocab : PAIRS_CAP;
-    sc->buckets = (vocab + (1u << SORT_SHIFT) - 1u) >> SORT_SHIFT;
-    // One allocation: counts, pos, the bitmap, the list, its lengths and bucket starts (each
-    // 16-byte aligned).
+    // One allocation: the counts, then the bitmap (16-byte aligned, four spare words).
     const size_t dense = (((size_t)vocab * 4) + 15) & ~(size_t)15;
     const size_t bitmap = (((size_t)(sc->words + 4) * 4) + 15) & ~(size_t)15;
-    const size_t list = (size_t)sc->pairs_cap * sizeof(ListEntry);
-    const size_t header = (((size_t)(LIST_HDR_WORDS + sc->buckets + 1) * 4) + 15) & ~(size_t)15;
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts), 2 * dense + bitmap + list + header);
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&sc->counts), dense + bitmap);
     if (e != hipSuccess) {
         delete sc;
         return hip_fail(e, "scratch allocation");
     }
-    char* base = reinterpret_cast<char*>(sc->counts);
-    sc->pos = reinterpret_cast<uint32_t*>(base + dense);
-    sc->touched = reinterpret_cast<uint32_t*>(base + 2 * dense);
-    sc->pairs = reinterpret_cast<ListEntry*>(base + 2 * dense + bitmap);
-    sc->list_hdr = reinterpret_cast<uint32_t*>(base + 2 * dense + bitmap + list);
-    e = hipMemsetAsync(sc->pos, 0, dense, s->stream);  // never read before written; defined anyway
-    if (e != hipSuccess) {
-        (void)hipFree(sc->counts);
-        delete sc;
-        return hip_fail(e, "scratch clear");
-    }
+    sc->touched = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(sc->counts) + dense);
     *out = sc;
     return lily_scratch_reset_counts(sc);
 }
@@ -854,8 +795,6 @@ int lily_scratch_reset_counts(lily_scratch_t* sc) {
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->counts, sc->vocab, 0));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->touched, sc->words + 4, 0));
-    HIP_TRY(launch_fill_u32(sc->s->stream, sc->list_hdr, LIST_HDR_WORDS + sc->buckets + 1, 0));
-    sc->tail_bound = 0;
     return LILY_OK;
 }
 
@@ -899,9 +838,6 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
                            dst->s->stream));
     HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)src->words * 4,
                            hipMemcpyDeviceToDevice, dst->s->stream));
-    // The list is a function of the counts and the bitmap: rebuilt here instead of copied.
-    HIP_TRY(launch_sort_list(dst->s->stream, view_of(dst)));
-    dst->tail_bound = 0;
     return LILY_OK;
 }
 
@@ -911,7 +847,6 @@ int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32
     }
     HIP_TRY(hipSetDevice(sc->s->device));
     HIP_TRY(launch_add_history(sc->s->stream, view_of(sc), ids_dev, n));
-    sc->tail_bound = 0;  // the list was sorted afresh
     return LILY_OK;
 }
 
@@ -923,7 +858,6 @@ int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts) {
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     HIP_TRY(hipMemcpy(sc->counts, host_counts, (size_t)sc->vocab * 4, hipMemcpyHostToDevice));
     HIP_TRY(launch_rebuild_listed(sc->s->stream, view_of(sc)));
-    sc->tail_bound = 0;
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     return LILY_OK;
 }
@@ -1204,12 +1138,8 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
                            hipMemcpyHostToDevice, s->stream));
     HIP_TRY(hipEventRecord(s->stage_done[slot], s->stream));
     s->stage_used[slot] = true;
-    if (parts[0].sort_first || (n_parts > 1 && parts[1].sort_first)) {
-        HIP_TRY(launch_sort_lists(s->stream, s->table_dev, nullptr, b->rows, b->vocab, true));
-    }
     for (uint32_t q = 0; q < n_parts; ++q) {
-        if (int rc = launch_part(s, parts[q], s->table_dev, (int)b->dtype, b->vocab, 0, 0, false,
-                                 q == 0)) {
+        if (int rc = launch_part(s, parts[q], s->table_dev, (int)b->dtype, b->vocab, 0, q == 0)) {
             return rc;
         }
     }
@@ -1268,18 +1198,6 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
     p->vocab = b->vocab;
     p->dtype = b->dtype;
     p->runs = 0;
-    p->sorted = false;
-    p->since_sort = 0;
-    p->longest_tail = 0;
-    p->sort_on_first_run = p->parts[0].sort_first || (p->n_parts > 1 && p->parts[1].sort_first);
-    p->penalised.clear();
-    for (uint32_t r = 0; r < b->rows; ++r) {
-        // (the table may be reordered: the batch's own arrays tell which scratches count)
-        if (b->scratch != nullptr && b->scratch[r] != nullptr &&
-            lily_params_uses_penalties(&b->params[r]) != 0) {
-            p->penalised.push_back(b->scratch[r]);
-        }
-    }
     return LILY_OK;
 }
 
@@ -1288,30 +1206,13 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
         return fail(LILY_ERR_INVALID_ARG, "plan is null or not set");
     }
     HIP_TRY(hipSetDevice(p->s->device));
-    if (p->longest_tail >= TAIL_SORT_AT || (p->runs == 0 && p->sort_on_first_run)) {
-        // The draws append the ids they count for the first time to their lists' unsorted
-        // tails: one launch sorts every penalised row's list again.
-        HIP_TRY(launch_sort_lists(p->s->stream, p->table_dev, nullptr, p->rows, p->vocab, false));
-        for (lily_scratch* sc : p->penalised) {
-            sc->tail_bound = 0;
-        }
-        p->sorted = true;
-        p->since_sort = 0;
-    }
     for (uint32_t q = 0; q < p->n_parts; ++q) {
-        const LaunchPart& part = p->parts[q];
-        if (int rc = launch_part(p->s, part, p->table_dev, (int)p->dtype, p->vocab, step_delta,
-                                 p->sorted ? p->since_sort : p->runs, p->sorted, q == 0)) {
+        if (int rc = launch_part(p->s, p->parts[q], p->table_dev, (int)p->dtype, p->vocab, step_delta,
+                                 q == 0)) {
             return rc;
         }
     }
     p->runs += 1;
-    p->since_sort += 1;
-    p->longest_tail = 0;
-    for (lily_scratch* sc : p->penalised) {
-        sc->tail_bound += 1;
-        p->longest_tail = sc->tail_bound > p->longest_tail ? sc->tail_bound : p->longest_tail;
-    }
     return LILY_OK;
 }
 

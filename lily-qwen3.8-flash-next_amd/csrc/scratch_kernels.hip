@@ -15,8 +15,7 @@ __global__ void k_fill_u32(uint32_t* p, uint32_t n, uint32_t v) {
     }
 }
 
-// counts[id] += 1 per occurrence and the id's bit in `touched`; the list is sorted afresh
-// afterwards (sort_list), which lists the new ids.
+// counts[id] += 1 per occurrence, and the id's bit in `touched`.
 __global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
@@ -28,102 +27,7 @@ __global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
     }
 }
 
-// One workgroup rebuilds a scratch's list from its bitmap of listed ids and its counts: every
-// listed id with its count in ascending id order (the tail is emptied), every id's position, and
-// the bucket starts.  Ids whose count went back to 0 stay listed.  With more listed ids than the
-// list's memory holds the lengths say so and the draws do not use the list.
-__device__ __forceinline__ void sort_list(const ScratchView& sc) {
-    __shared__ uint32_t wave_total[4];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    const uint32_t words = (sc.vocab + 31u) / 32u;
-    uint32_t* start = sc.list_hdr + LIST_HDR_WORDS;
-    uint32_t base = 0;  // listed ids below this round's words
-    for (uint32_t w0 = 0; w0 < words; w0 += 256u) {
-        const uint32_t wi = w0 + tid;
-        uint32_t bits = wi < words ? sc.touched[wi] : 0u;
-        const uint32_t mine = (uint32_t)__popc(bits);
-        uint32_t incl = mine;
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t t = __shfl_up(incl, o);
-            if ((int)lane >= o) {
-                incl += t;
-            }
-        }
-        if (lane == 63u) {
-            wave_total[w] = incl;
-        }
-        __syncthreads();
-        uint32_t before = base + incl - mine, round_total = 0;
-        for (uint32_t i = 0; i < 4u; ++i) {
-            before += i < w ? wave_total[i] : 0u;
-            round_total += wave_total[i];
-        }
-        __syncthreads();
-        // A bucket is 1 << SORT_SHIFT ids = 8 words: the thread at its first word knows its start.
-        if (wi < words && (wi & ((1u << (SORT_SHIFT - 5u)) - 1u)) == 0u) {
-            start[wi >> (SORT_SHIFT - 5u)] = before;
-        }
-        uint32_t at = before;
-        while (bits != 0u) {
-            const uint32_t id = wi * 32u + (uint32_t)__builtin_ctz(bits);
-            bits &= bits - 1u;
-            if (at < sc.pairs_cap) {
-                sc.pairs[at] = list_entry(id, sc.counts[id]);
-            }
-            sc.pos[id] = at < sc.pairs_cap ? at : 0xffffffffu;
-            ++at;
-        }
-        base += round_total;
-    }
-    if (tid == 0) {
-        const uint32_t buckets = (sc.vocab + (1u << SORT_SHIFT) - 1u) >> SORT_SHIFT;
-        start[buckets] = base;
-        sc.list_hdr[HDR_SORTED] = base;
-        sc.list_hdr[HDR_TAIL] = 0;
-    }
-}
-
-__global__ __launch_bounds__(256) void k_sort_list(ScratchView sc) { sort_list(sc); }
-
-// The same for every penalised row of a batch (one workgroup per row; rows without penalties
-// have no scratch to sort).
-__device__ __forceinline__ ScratchView view_of_row(const RowArgs& r, uint32_t vocab) {
-    ScratchView sc;
-    sc.counts = r.counts;
-    sc.touched = r.touched;
-    sc.pairs = r.pairs;
-    sc.list_hdr = r.list_hdr;
-    sc.pos = r.pos;
-    sc.vocab = vocab;
-    sc.pairs_cap = r.pairs_cap;
-    return sc;
-}
-
-// `flagged_only`: rows marked F_SORT_FIRST; otherwise every penalised row.
-__device__ __forceinline__ bool wants_sort(const RowArgs& r, uint32_t flagged_only) {
-    return (r.flags & F_PEN) != 0u && (flagged_only == 0u || (r.flags & F_SORT_FIRST) != 0u);
-}
-
-__global__ __launch_bounds__(256) void k_sort_lists_table(const RowArgs* table, uint32_t vocab,
-                                                          uint32_t flagged_only) {
-    const RowArgs& r = table[blockIdx.x];
-    if (wants_sort(r, flagged_only)) {
-        sort_list(view_of_row(r, vocab));
-    }
-}
-
-__global__ __launch_bounds__(256) void k_sort_lists_inline(InlineRows rows, uint32_t vocab,
-                                                           uint32_t flagged_only) {
-    // `rows` is the first kernel argument: read the row in the kernel-argument segment itself
-    // (indexing the by-value copy would move all of it to scratch memory).
-    const RowArgs* table = (const RowArgs*)__builtin_amdgcn_kernarg_segment_ptr();
-    const RowArgs r = table[blockIdx.x];
-    if (wants_sort(r, flagged_only)) {
-        sort_list(view_of_row(r, vocab));
-    }
-}
-
-// Saturating decrement; the id stays listed (with a count that may now be 0).
+// Saturating decrement; the id stays on the bitmap (with a count that may now be 0).
 __device__ __forceinline__ void uncount_one(const ScratchView& sc, uint32_t token) {
     if (token >= sc.vocab) {
         return;
@@ -131,10 +35,6 @@ __device__ __forceinline__ void uncount_one(const ScratchView& sc, uint32_t toke
     const uint32_t c = sc.counts[token];
     if (c > 0u) {
         sc.counts[token] = c - 1u;
-        const uint32_t p = sc.pos[token];
-        if (((sc.touched[token >> 5] >> (token & 31u)) & 1u) && p < sc.pairs_cap) {
-            sc.pairs[p] = list_entry(token, c - 1u);
-        }
     }
 }
 
@@ -160,8 +60,7 @@ __global__ void k_uncount_after(ScratchView sc, const uint32_t* draws, uint32_t 
     }
 }
 
-// After counts were written whole: touched[w] = bits of the non-zero counts in word w (the
-// list is sorted afresh afterwards).
+// After counts were written whole: touched[w] = bits of the non-zero counts in word w.
 __global__ void k_touch_from_counts(ScratchView sc) {
     const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t words = (sc.vocab + 31u) / 32u;
@@ -255,7 +154,6 @@ hipError_t launch_add_history(hipStream_t stream, const ScratchView& sc, const u
         return hipSuccess;
     }
     hipLaunchKernelGGL(k_add_history, dim3((n + 255) / 256), dim3(256), 0, stream, sc, ids, n);
-    hipLaunchKernelGGL(k_sort_list, dim3(1), dim3(256), 0, stream, sc);
     return hipGetLastError();
 }
 
@@ -273,23 +171,6 @@ hipError_t launch_uncount_after(hipStream_t stream, const ScratchView& sc, const
 hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc) {
     const uint32_t words = (sc.vocab + 31u) / 32u;
     hipLaunchKernelGGL(k_touch_from_counts, dim3((words + 255) / 256), dim3(256), 0, stream, sc);
-    hipLaunchKernelGGL(k_sort_list, dim3(1), dim3(256), 0, stream, sc);
-    return hipGetLastError();
-}
-
-hipError_t launch_sort_list(hipStream_t stream, const ScratchView& sc) {
-    hipLaunchKernelGGL(k_sort_list, dim3(1), dim3(256), 0, stream, sc);
-    return hipGetLastError();
-}
-
-hipError_t launch_sort_lists(hipStream_t stream, const RowArgs* table_dev, const InlineRows* inline_rows,
-                             uint32_t rows, uint32_t vocab, bool flagged_only) {
-    const uint32_t f = flagged_only ? 1u : 0u;
-    if (inline_rows != nullptr) {
-        hipLaunchKernelGGL(k_sort_lists_inline, dim3(rows), dim3(256), 0, stream, *inline_rows, vocab, f);
-    } else {
-        hipLaunchKernelGGL(k_sort_lists_table, dim3(rows), dim3(256), 0, stream, table_dev, vocab, f);
-    }
     return hipGetLastError();
 }
 

@@ -1,63 +1,68 @@
 // select_stream.h - the one-pass streaming select (k <= 64).
 #pragma once
 
+#include <type_traits>
+
 #include "device_common.h"
 
 namespace lily {
 
 // ------------------------------------------------------------------ streaming select
 //
-// The select of rows with k <= STREAM_K_MAX and no allow-mask.  One pass, one barrier per
-// block of NT x STREAM_UNROLL chunks, every 16-byte chunk read from memory once:
+// The select of rows with k <= STREAM_K_MAX.  One pass, every 16-byte chunk read from memory
+// once, a barrier every fourth block of NT x STREAM_UNROLL chunks:
 //
 //   * Bound.  Each lane keeps the maximum of what it has seen; each wave takes the kw-th
 //     largest of its 64 lane maxima (kw = ceil(k' / NWAVE), a 16-step ballot search on the
 //     top half of the order key).  At least k' distinct elements are at or above the
 //     minimum of the waves' values, so that minimum is a lower bound of the k'-th largest
-//     value; it is refreshed after every block and is the same in every wave while a
-//     block is processed, which makes the run reproducible.
+//     value; it is the same in every wave while a block is processed, which makes the run
+//     reproducible.
 //   * Owner side.  A lane whose chunk holds a value at or above the bound appends the whole
 //     chunk (16 raw bytes + its index) to its wave's queue and leaves it out of the running
 //     sum of exponentials; all other chunks only feed the lane maximum and the sum.
-//   * Listed ids (penalised: the scratch's (id, count) list; biased: the row's bias list)
-//     are sorted into per-block buckets in LDS before the scan.  While block b streams,
-//     thread t also loads the chunk of "its" listed id of block b (the same cache lines
-//     the owners are loading), evaluates the id exactly, offers it as a candidate, adds its
-//     true term to the sum and - when the chunk was not queued, which it can tell from the
-//     chunk's maximum and the block's bound - books the raw term the owner added, to be
-//     taken off at the end.  Listed ids inside queued chunks go to a short drop list.
-//   * After the scan the queued chunks are expanded: elements that are not on the drop list
-//     add their term and, at or above the final bound, become candidates.
+//   * Listed ids (ids a scratch ever counted: their true value differs from the raw one) are
+//     bits of the scratch's bitmap.  Each wave reads the words that cover its own chunks of a
+//     block (64 bytes per load of 64 bf16 chunks), so a lane knows which of its elements are
+//     listed without anybody gathering anything.  When penalties can only lower a value, a
+//     listed element matters only if its chunk is queued (it is then evaluated exactly when the
+//     queue is expanded, its count gathered from the dense histogram) or summed (its raw term
+//     is booked and its true term added on the spot); otherwise every listed element is
+//     evaluated on the spot.  Barred ids of a masked row are bits of the same kind and are
+//     replaced by -inf as the chunk arrives.
+//   * The bias list's ids (at most STREAM_BIAS_CAP) are streamed as they are; after the scan
+//     one thread per id looks its chunk up again, redoes the owner's tests with the bound and
+//     the cut its block was scanned with, books the raw term and offers the true value.
+//   * After the scan the queued chunks are expanded: their elements add their term and, at or
+//     above the final bound, become candidates.
 //
 // Values are compared before the division by the temperature; candidates are divided
-// exactly and the caller's check (k-th candidate strictly above anything a value below
-// the bound can map to) decides whether the result stands.  Any overflow returns false.
+// exactly and the final check (k-th candidate strictly above anything a value below the
+// bound can map to) decides whether the result stands.  Any overflow returns false.
 
 struct StreamLds {
     u32x4* qraw;
     uint32_t* qidx;
-    uint32_t* spec;
-    uint64_t* fc;
-    uint32_t* drop;
-    uint32_t* dmask;   // per queue slot, a byte: bit j set = element j is a listed id
-    uint32_t* bkt;
-    uint32_t* bfill;
-    uint2* hseg;
+    uint8_t* qbits;     // per queue slot: bit j set = element j is a listed id
+    uint32_t* win;      // [NWAVE][2][WIN_WORDS]
+    float* blk_bound;   // [MAX_BLOCKS] the bound block b was filtered with
+    float* blk_cut;     // [MAX_BLOCKS] the sum's cut of block b
+    uint32_t* blk_flag; // [MAX_BLOCKS] 1 = chunk maxima of block b were the non-negative kind
     uint32_t* bias_id;
     float* bias_delta;
+    uint64_t* fc;
     __device__ __forceinline__ void init() {
         char* b = reinterpret_cast<char*>(dyn_lds);
         qraw = reinterpret_cast<u32x4*>(b + OFF_QRAW);
         qidx = reinterpret_cast<uint32_t*>(b + OFF_QIDX);
-        spec = reinterpret_cast<uint32_t*>(b + OFF_SPEC);
-        fc = reinterpret_cast<uint64_t*>(b + OFF_FC);
-        drop = reinterpret_cast<uint32_t*>(b + OFF_DROP);
-        dmask = reinterpret_cast<uint32_t*>(b + OFF_DMASK);
-        bkt = reinterpret_cast<uint32_t*>(b + OFF_BKT);
-        bfill = reinterpret_cast<uint32_t*>(b + OFF_BFILL);
+        qbits = reinterpret_cast<uint8_t*>(b + OFF_QBITS);
+        win = reinterpret_cast<uint32_t*>(b + OFF_WIN);
+        blk_bound = reinterpret_cast<float*>(b + OFF_BLK);
+        blk_cut = reinterpret_cast<float*>(b + OFF_BLK + MAX_BLOCKS * 4);
+        blk_flag = reinterpret_cast<uint32_t*>(b + OFF_BLK + MAX_BLOCKS * 8);
         bias_id = reinterpret_cast<uint32_t*>(b + OFF_BIAS);
         bias_delta = reinterpret_cast<float*>(b + OFF_BIAS + STREAM_BIAS_CAP * 4);
-        hseg = reinterpret_cast<uint2*>(b + OFF_HSEG);
+        fc = reinterpret_cast<uint64_t*>(b + OFF_FC);
     }
 };
 
@@ -112,16 +117,20 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     constexpr uint32_t BLOCK = NT * U;
     constexpr uint32_t QSEG = Q_CAP / NWAVE;
     constexpr uint32_t NONE = 0xffffffffu;
-    constexpr uint32_t ID_MASK = (1u << SPEC_ID_BITS) - 1u;
-    constexpr int PREG = 2;   // tail entries a thread keeps in registers between the two bucket passes
+    constexpr uint32_t EMASK = (1u << E) - 1u;
+    constexpr uint32_t WPP = 64u * E / 32u;   // bitmap words that hold the bits of a wave's 64 chunks
+    constexpr uint32_t PIECE = WPP + 1u;      // + one for rows whose chunks start inside a word
+    static_assert(PIECE <= WIN_PIECE_MAX && U == 4, "window layout");
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const uint32_t nchunks = g.ce - g.cb;
     const uint32_t nblocks = (nchunks + BLOCK - 1) / BLOCK;
     const bool pen = (a.flags & F_PEN) != 0;
+    const bool masked = MASKS && a.allow != nullptr;
     const uint32_t n_bias = a.n_bias;
     const bool want_lse = LSE && a.out_logprob != nullptr;
     const float c2 = a.c2;
-    if (nblocks > MAX_BUCKETS || n_bias > STREAM_BIAS_CAP || g.vocab > (1u << SPEC_ID_BITS)) {
+    const uint32_t row_words = (g.vocab + 31u) / 32u;
+    if (nblocks > MAX_BLOCKS || n_bias > STREAM_BIAS_CAP) {
         return stream_fail(cfg, 1u);
     }
     StreamLds L;
@@ -145,77 +154,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t c0 = g.cb + b * BLOCK;
         return c0 >= g.main_lo && c0 + BLOCK <= g.main_hi;
     };
-    // ---- the slice's listed ids
-    // The scratch's list comes in two parts.  Its sorted part (ascending ids, indexed by
-    // buckets of 1 << SORT_SHIFT ids) is read straight from memory while the row streams:
-    // block b's entries lie between two bucket starts, requested here by thread b.  Its tail
-    // (the ids first counted since the list was last sorted: a few, the host has the list
-    // sorted again before there are many) is bucketed by block in LDS below, together with
-    // the bias list's ids and a dense mask's barred ids.  The tail's first PREG x NT entries
-    // are requested together with the two lengths (the tail grows downwards from the end of
-    // the list's memory, so their addresses depend on nothing), ahead of the first block of
-    // the row, which is then in flight while they are bucketed.
-    uint32_t n_sorted = 0, n_tail = 0, loaded = 0;
-    uint32_t seg_s = 0, seg_e = 0;   // thread b: block b's entries of the sorted part
-    uint32_t early[PREG];
-    const ListEntry* list = a.pairs;
-    if (pen) {
-        // The lengths come through the scalar path (nothing writes them while the slices of
-        // their row still read them): a vector load of a value that is the same in every lane
-        // is moved to a scalar register at once, and that move would hold the loads below
-        // back until the lengths had arrived.
-        const LILY_CONST uint32_t* hdr = (const LILY_CONST uint32_t*)a.list_hdr;
-        n_sorted = hdr[HDR_SORTED];
-        n_tail = hdr[HDR_TAIL];
-        if (tid < nblocks) {
-            const uint32_t c0 = max(g.cb + tid * BLOCK, g.main_lo);
-            const uint32_t c1 = min(g.cb + (tid + 1u) * BLOCK, g.main_hi);
-            if (c1 > c0) {
-                const uint32_t id_first = c0 * E - g.pad, id_last = c1 * E - g.pad - 1u;
-                const uint32_t* start = a.list_hdr + LIST_HDR_WORDS;
-                seg_s = gload(start + (id_first >> SORT_SHIFT));
-                seg_e = gload(start + (id_last >> SORT_SHIFT) + 1u);
-            }
-        }
-        // The host's bound of the tail's length says how much to request; a longer tail is
-        // still read completely (by the loop further down), a shorter one costs idle loads.
-        const uint64_t hint = (cfg.hint_replace != 0u ? 0u : a.tail_hint) + (uint64_t)cfg.hint_growth;
-        const uint64_t want = (hint + NT - 1) / NT * NT;
-        loaded = (uint32_t)min(want, (uint64_t)min(a.pairs_cap, (uint32_t)(PREG * NT)));
-#pragma unroll
-        for (int q = 0; q < PREG; ++q) {
-            const uint32_t p = (uint32_t)q * NT + tid;
-            early[q] = p < loaded ? gload(list + (a.pairs_cap - 1u - p)) : NONE;
-        }
-    }
     u32x4 buf_a[U], buf_b[U], buf_c[U];
     if (nblocks > 0) {
         fetch(buf_a, 0);
     }
-    if (tid <= MAX_BUCKETS) {
-        L.bkt[tid] = 0;
-    }
-    if (tid < MAX_BUCKETS) {
-        L.bfill[tid] = 0;
-    }
-    if (tid < Q_CAP / 4) {
-        L.dmask[tid] = 0;
-    }
-    if (tid < MAX_BUCKETS) {
-        // A list that does not fit its memory is not used (checked below); its bucket starts
-        // then mean nothing, and a start is never taken beyond the sorted part.
-        seg_e = min(seg_e, n_sorted);
-        seg_s = min(seg_s, seg_e);
-        L.hseg[tid] = uint2{seg_s, seg_e};
-        // A block with more listed ids than the workgroup has threads (see row_max below).
-        const uint64_t big = __ballot(seg_e - seg_s > (uint32_t)NT);
-        if (tid == 0) {
-            sh.dense_listed = big != 0ull ? 1u : 0u;
-        }
-    }
     if (tid == 0) {
         sh.n_fc = 0;
-        sh.n_drop = 0;
         sh.fail = 0;
     }
     for (uint32_t i = tid; i < n_bias; i += NT) {
@@ -224,22 +168,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     }
     __syncthreads();
     phase(cfg, 13);
-    if ((uint64_t)n_sorted + n_tail > a.pairs_cap) {
-        return stream_fail(cfg, 2u);  // the list overflowed: the bitmap and the counts hold the truth
-    }
-    // A row with an allow-mask is streamed when the mask is dense: its disallowed ids join the
-    // listed ids (true value -inf).  Otherwise the row is left to the selects made for masks.
-    // (MASKS is false in kernels whose launches hold no masked row.)
-    const bool masked = MASKS && a.allow != nullptr;
-    const uint32_t w_lo = g.id_lo >> 5, w_hi = (g.id_hi + 31u) >> 5;
-    auto barred = [&](uint32_t i) -> uint32_t {  // disallowed ids of mask word i inside the slice
-        return ~gload(a.allow + i) & range32_at(g.id_lo, g.id_hi, (int64_t)i * 32);
-    };
-    uint32_t n_barred = 0;
     if (masked) {
+        // A row whose mask admits few ids is left to the select that reads only those.
+        const uint32_t w_lo = g.id_lo >> 5, w_hi = (g.id_hi + 31u) >> 5;
         uint32_t mine = 0;
         for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
-            mine += (uint32_t)__popc(barred(i));
+            mine += (uint32_t)__popc(gload(a.allow + i) & range32_at(g.id_lo, g.id_hi, (int64_t)i * 32));
         }
         for (int o = 32; o > 0; o >>= 1) {
             mine += __shfl_xor(mine, o);
@@ -248,213 +182,73 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             sh.red_i[w] = mine;
         }
         __syncthreads();
+        uint32_t n_allowed = 0;
         for (int i = 0; i < NWAVE; ++i) {
-            n_barred += sh.red_i[i];
+            n_allowed += sh.red_i[i];
         }
         __syncthreads();
-        if ((uint64_t)n_barred + n_tail + n_bias > SPEC_CAP - SPEC_CAP / 10u) {
-            return false;  // not a failure: the mask is not dense enough for this select
+        if (n_allowed <= min(cfg.dyn_slots, MERGE_CAP)) {
+            return false;  // not a failure: the sparse select takes the row
         }
     }
-    // `bucketed`: some listed ids reach the scan through the LDS buckets; `listed_row`: the row
-    // has listed ids at all (the sorted part included).
-    const bool bucketed = n_tail != 0 || n_bias != 0 || n_barred != 0;
-    const bool listed_row = bucketed || n_sorted != 0;
-    // Block of a streamed id of this slice, NONE for ids outside it or in a partial chunk.
-    auto block_of = [&](uint32_t id) -> uint32_t {
-        if (id >= g.vocab) {
-            return NONE;
+    // Penalties with a repetition factor of at least 1 and non-negative presence and frequency
+    // terms can only lower a value.  `lowering`: no listed id's true value exceeds its raw one
+    // (ids the bias list names are dealt with apart, after the scan, listed or not).
+    const bool special = pen || masked;   // the row's chunks come with bits
+    const bool lowering = a.repetition >= 1.0f && a.presence >= 0.0f && a.frequency >= 0.0f;
+    // Whether id is named by the bias list (its true value then comes from the pass after the scan).
+    auto biased = [&](uint32_t id) -> bool {
+        bool hit = false;
+        for (uint32_t j = 0; j < n_bias; ++j) {
+            hit = hit || L.bias_id[j] == id;
         }
-        const uint32_t c = (id + g.pad) / E;
-        if (c < g.main_lo || c >= g.main_hi) {
-            return NONE;
-        }
-        return (c - g.cb) / BLOCK;
+        return hit;
     };
-    // The bias entry i opens a bucket slot when it is the first of its id and the id is
-    // not on the scratch's list (that entry covers it).
-    auto bias_block = [&](uint32_t i) -> uint32_t {
-        const uint32_t id = L.bias_id[i];
-        for (uint32_t j = 0; j < i; ++j) {
+    // A listed id's true value before the temperature from its raw one: bias in list order,
+    // then penalties with the count gathered from the dense histogram.  (A barred id never
+    // gets here: its raw value was replaced by -inf when its chunk arrived.)
+    auto true_value = [&](uint32_t id, float raw) -> float {
+        uint32_t cnt = 0;
+        if (pen) {
+            cnt = gload(a.counts + id);
+            // The value is waited for here, inside the branch: waiting after it would make
+            // every thread drain the loads it has in flight.
+            asm volatile("" : "+v"(cnt));
+        }
+        float t = raw;
+        for (uint32_t j = 0; j < n_bias; ++j) {
             if (L.bias_id[j] == id) {
-                return NONE;
+                t += L.bias_delta[j];
             }
         }
-        const uint32_t b = block_of(id);
-        if (b != NONE && pen && bit_of(a.touched, id)) {
-            return NONE;
+        if (cnt > 0u) {
+            t = t > 0.0f ? t / a.repetition : t * a.repetition;
+            t -= a.presence + a.frequency * (float)cnt;
         }
-        return b;
+        return t;
     };
-    // The disallowed ids that open a bucket slot of their own: streamed ones that neither
-    // the scratch's list nor the bias list covers already.
-    auto each_barred = [&](auto&& fn) {
-        if (n_barred == 0u) {
-            return;
-        }
-        for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
-            uint32_t bits = barred(i);
-            while (bits != 0u) {
-                const uint32_t id = i * 32u + (uint32_t)__builtin_ctz(bits);
-                bits &= bits - 1u;
-                const uint32_t b = block_of(id);
-                bool open = b != NONE && !(pen && bit_of(a.touched, id));
-                for (uint32_t j = 0; open && j < n_bias; ++j) {
-                    open = L.bias_id[j] != id;
-                }
-                if (open) {
-                    fn(id, b);
-                }
-            }
-        }
-    };
-    if (bucketed && nblocks == 1u) {
-        // One block: its bucket starts at slot 0, so a single atomic places each entry and
-        // there is nothing to count first.
-        auto put = [&](uint32_t entry) {
-            const uint32_t at = atomicAdd(&L.bfill[0], 1u);
-            if (at < SPEC_CAP) {
-                L.spec[at] = entry;
-            }
-        };
-#pragma unroll
-        for (int q = 0; q < PREG; ++q) {
-            const uint32_t p = (uint32_t)q * NT + tid;
-            if (p < n_tail && p < loaded && block_of(early[q] & ID_MASK) != NONE) {
-                put(early[q]);
-            }
-        }
-        for (uint32_t p = loaded + tid; p < n_tail; p += NT) {
-            const uint32_t e = gload(list + (a.pairs_cap - 1u - p));
-            if (block_of(e & ID_MASK) != NONE) {
-                put(e);
-            }
-        }
-        for (uint32_t i = tid; i < n_bias; i += NT) {
-            if (bias_block(i) != NONE) {
-                put(L.bias_id[i]);
-            }
-        }
-        each_barred([&](uint32_t id, uint32_t) { put(id); });
-        __syncthreads();
-        const uint32_t total = L.bfill[0];
-        if (total > SPEC_CAP) {
-            return stream_fail(cfg, 3u);
-        }
-        // Every wave writes the bucket's end for its own later reads (the same value).
-        if (lane == 0) {
-            L.bkt[1] = total;
-            L.bkt[MAX_BUCKETS] = total;
-            if (total + (L.hseg[0].y - L.hseg[0].x) > (uint32_t)NT) {
-                sh.dense_listed = 1u;
-            }
-        }
-    } else if (bucketed) {
-        uint32_t packed[PREG];  // id | min(count, 4095) << 20, NONE when not of this slice
-#pragma unroll
-        for (int q = 0; q < PREG; ++q) {
-            const uint32_t p = (uint32_t)q * NT + tid;
-            packed[q] = NONE;
-            if (p < n_tail && p < loaded && block_of(early[q] & ID_MASK) != NONE) {
-                packed[q] = early[q];
-            }
-        }
-        // Entries held in registers take their place inside the bucket with the first pass's
-        // atomic (counted in bfill); everything else is counted in bkt and placed behind them
-        // by a second atomic in the second pass.
-        uint32_t place[PREG];
-        for (int pass = 0; pass < 2; ++pass) {
-#pragma unroll
-            for (int q = 0; q < PREG; ++q) {
-                if (packed[q] != NONE) {
-                    const uint32_t b = block_of(packed[q] & ID_MASK);
-                    if (pass == 0) {
-                        place[q] = atomicAdd(&L.bfill[b], 1u);
-                    } else {
-                        L.spec[L.bkt[b] + place[q]] = packed[q];
-                    }
-                }
-            }
-            for (uint32_t p = loaded + tid; p < n_tail; p += NT) {  // what the registers do not hold
-                const uint32_t e = gload(list + (a.pairs_cap - 1u - p));
-                const uint32_t b = block_of(e & ID_MASK);
-                if (b != NONE) {
-                    if (pass == 0) {
-                        atomicAdd(&L.bkt[b], 1u);
-                    } else {
-                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = e;
-                    }
-                }
-            }
-            for (uint32_t i = tid; i < n_bias; i += NT) {
-                const uint32_t b = bias_block(i);
-                if (b != NONE) {
-                    if (pass == 0) {
-                        atomicAdd(&L.bkt[b], 1u);
-                    } else {
-                        L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = L.bias_id[i];
-                    }
-                }
-            }
-            each_barred([&](uint32_t id, uint32_t b) {
-                if (pass == 0) {
-                    atomicAdd(&L.bkt[b], 1u);
-                } else {
-                    L.spec[L.bkt[b] + atomicAdd(&L.bfill[b], 1u)] = id;
-                }
-            });
-            __syncthreads();
-            if (pass == 0) {
-                phase(cfg, 14);
-                if (tid < 64) {  // counts -> exclusive offsets, total in bkt[MAX_BUCKETS]
-                    const uint32_t cnt = L.bkt[tid] + L.bfill[tid];
-                    const uint64_t big =
-                        __ballot(cnt + (L.hseg[tid].y - L.hseg[tid].x) > (uint32_t)NT);
-                    if (tid == 0 && big != 0ull) {
-                        sh.dense_listed = 1u;
-                    }
-                    uint32_t incl = cnt;
-                    for (int o = 1; o < 64; o <<= 1) {
-                        const uint32_t t = __shfl_up(incl, o);
-                        if ((int)tid >= o) {
-                            incl += t;
-                        }
-                    }
-                    L.bkt[tid] = incl - cnt;
-                    if (tid == 63) {
-                        L.bkt[MAX_BUCKETS] = incl;
-                    }
-                }
-                __syncthreads();
-                phase(cfg, 15);
-                if (L.bkt[MAX_BUCKETS] > SPEC_CAP) {
-                    return stream_fail(cfg, 3u);
-                }
-            }
-        }
-    }
     phase(cfg, 1);
 
     // ---- scan
     const uint32_t keff = min(k + k / 8u + 2u, 64u * NWAVE);
     const uint32_t kw = (keff + NWAVE - 1) / NWAVE;
     float lane_max = NEG_INF;
+    float clean_max = NEG_INF;  // this lane's largest chunk maximum among chunks without a listed id
     float T = F32_LOWEST;       // the block's bound, the same in every thread
     float ref_s = 0.0f;         // reference of the double sums
     float row_max = NEG_INF;    // lower bound of the row's largest true value, as of the last refresh
-    float listed_raw_max = NEG_INF, listed_true_max = NEG_INF;  // this thread's listed ids so far
     float skip_b = NEG_INF;     // the block's cut: chunks whose maximum is not above it are not summed
     uint32_t wq = 0;            // this wave's queue fill
     WaveLse wl;
     wl.init();
-    double acc_t = 0.0, acc_r = 0.0, acc_q = 0.0;
+    double acc_t = 0.0, acc_r = 0.0;   // true terms added one by one; raw terms to take off
     constexpr int UP_UNSET = INT_MIN;
     int up = UP_UNSET;          // this thread's double sums are relative to ref_s + up
     uint32_t parity = 0;
     // One term 2^(v*c2 - ref_s - up) of a double sum.  The exponent is formed in double: a
     // row's largest value may lie hundreds of units above the reference (fixed after the
     // first block), where an f32 difference is good to 1e-5 only.  The thread's own
-    // reference ref_s + up starts at its first term and moves up (its three sums scaled down
+    // reference ref_s + up starts at its first term and moves up (its two sums scaled down
     // by the same power of two) when a term lies beyond 2^900 of it, so what a thread drops
     // as too small is small against something it holds - the row's raw maximum, which ref_s
     // comes from, may belong to an id that a mask or a bias takes out.  The threads'
@@ -465,7 +259,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         double d = __builtin_fma((double)v, c2d, -base);
         if (d > 900.0) {
             // The thread's first term, or one beyond 2^900 of its reference: the reference
-            // moves to the term (the three sums, if any, scaled down by the same power of two).
+            // moves to the term (the two sums, if any, scaled down by the same power of two).
             double e = (double)v * c2d - (double)ref_s;
             e = e < 1.0e9 ? (e > -1.0e9 ? e : -1.0e9) : 1.0e9;
             const int now = (int)__builtin_floor(e);
@@ -473,7 +267,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 const int step = now - up;
                 acc_t = __builtin_ldexp(acc_t, -step);
                 acc_r = __builtin_ldexp(acc_r, -step);
-                acc_q = __builtin_ldexp(acc_q, -step);
             }
             up = now;
             base = (double)ref_s + (double)up;
@@ -490,18 +283,17 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t key16 = lane_max > NEG_INF ? (lilym_order_key(lane_max) >> 16) : 0u;
         const uint32_t P = wave_kth_key16(key16, kw);
         const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
-        float wm[3] = {0.0f, 0.0f, 0.0f};
+        float wm[2] = {0.0f, 0.0f};
         if (maxima) {
             wm[0] = wave_max_dpp(lane_max);
-            if (want_lse && listed_row) {
-                wm[1] = wave_max_dpp(listed_raw_max);
-                wm[2] = wave_max_dpp(listed_true_max);
+            if (want_lse && special) {
+                wm[1] = wave_max_dpp(clean_max);
             }
         }
         if (lane == 0) {
             sh.bound[parity][w] = mine;
             if (maxima) {
-                for (int q = 0; q < 3; ++q) {
+                for (int q = 0; q < 2; ++q) {
                     sh.wmax[parity][q][w] = wm[q];
                 }
             }
@@ -513,25 +305,16 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         T = fmaxf(T, lower_by_slack(t));
         if (maxima) {
-            float m[3];
-            for (int q = 0; q < 3; ++q) {
+            float m[2];
+            for (int q = 0; q < 2; ++q) {
                 m[q] = sh.wmax[parity][q][0];
                 for (int i = 1; i < NWAVE; ++i) {
                     m[q] = fmaxf(m[q], sh.wmax[parity][q][i]);
                 }
             }
-            // A lower bound of the row's largest TRUE value: the largest raw value when it
-            // exceeds every listed id's raw value (then it belongs to an id that keeps its
-            // value), and the largest true value of the listed ids in any case.  All three
-            // maxima cover the same blocks.  A block with more listed ids than threads breaks
-            // that (its later rounds lag), so such rows skip nothing.
-            if (!listed_row) {
-                row_max = m[0];
-            } else if (sh.dense_listed != 0u) {
-                row_max = NEG_INF;
-            } else {
-                row_max = m[0] > m[1] ? fmaxf(m[0], m[2]) : m[2];
-            }
+            // A lower bound of the row's largest TRUE value: the largest raw value of the
+            // chunks that hold no listed id (a row where every chunk holds one skips nothing).
+            row_max = special ? m[1] : m[0];
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
                 ref_s = m[0] > NEG_INF ? fminf(fmaxf(m[0] * c2, -1.0e30f), 1.0e30f) : 0.0f;
@@ -540,44 +323,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         parity ^= 1u;
     };
 
-    struct Listed {
-        uint32_t ent;
-        u32x4 chunk;
-    };
-    // A thread's place among block b's listed ids in round `round` (rotated from block to
-    // block so that the same threads do not serve every block's first entries).
-    auto slot_of = [&](uint32_t b, uint32_t round) -> uint32_t {
-        return round * NT + ((tid + NT - ((b * 64u) % NT)) % NT);
-    };
-    // Block b's entries are those of the sorted part between its two bucket starts (ids of
-    // the neighbouring blocks at either end are dropped when the entry is used), then those
-    // of its LDS bucket.  The load is unconditional as well: a thread without an entry reads
-    // some entry of the list (rows without a list read the row's first bytes).
-    const ListEntry* ent_base = pen ? list : reinterpret_cast<const ListEntry*>(g.base);
-    const uint32_t ent_last = pen ? a.pairs_cap - 1u : 0u;
-    auto entry_load = [&](uint32_t b, uint32_t round) -> uint32_t {
-        return gload(ent_base + min(L.hseg[b].x + slot_of(b, round), ent_last));
-    };
-    // `pre`: what entry_load(b, round) returned.  Issues the gather of the entry's chunk; a
-    // thread without an entry reads the slice's last chunk.
-    auto listed_fetch = [&](Listed& r, uint32_t pre, uint32_t b, uint32_t round) {
-        const uint2 seg = L.hseg[b];
-        const uint32_t nh = seg.y - seg.x;
-        const uint32_t lo = L.bkt[b], nl = L.bkt[b + 1] - lo;
-        const uint32_t j = slot_of(b, round);
-        uint32_t ent = NONE;
-        if (j < nh) {
-            if (block_of(pre & ID_MASK) == b) {
-                ent = pre;
-            }
-        } else if (j - nh < nl) {
-            ent = L.spec[min(lo + (j - nh), SPEC_CAP - 1u)];
-        }
-        r.ent = ent;
-        const uint32_t c = min(((ent & ID_MASK) + g.pad) / E, c_last);
-        r.chunk = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
-    };
-    // The id's own logit out of its chunk (one gather per listed id, not two).
     // Element j of a chunk: one compare picks the 8-byte half, one 64-bit shift the element.
     auto elem_of = [&](const u32x4& q, uint32_t j) -> float {
         const bool upper = (j & (uint32_t)(E / 2)) != 0u;
@@ -587,83 +332,131 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         return lilym_bits_f32((uint32_t)(half >> ((j & 1u) * 32u)));
     };
-    auto raw_of = [&](const u32x4& q, uint32_t id) -> float {
-        return elem_of(q, (id + g.pad) % E);
+    // The chunk with the elements of `bits` replaced by -inf.
+    auto without = [&](const u32x4& q, uint32_t bits) -> u32x4 {
+        u32x4 r = q;
+        if (E == 8) {
+            auto fix = [](uint32_t v, uint32_t two) -> uint32_t {
+                const uint32_t m = ((two & 1u) ? 0x0000ffffu : 0u) | ((two & 2u) ? 0xffff0000u : 0u);
+                return (v & ~m) | (0xff80ff80u & m);
+            };
+            r.x = fix(q.x, bits);
+            r.y = fix(q.y, bits >> 2);
+            r.z = fix(q.z, bits >> 4);
+            r.w = fix(q.w, bits >> 6);
+        } else {
+            r.x = (bits & 1u) ? 0xff800000u : q.x;
+            r.y = (bits & 2u) ? 0xff800000u : q.y;
+            r.z = (bits & 4u) ? 0xff800000u : q.z;
+            r.w = (bits & 8u) ? 0xff800000u : q.w;
+        }
+        return r;
     };
-    // Penalties with a repetition factor of at least 1 and non-negative presence and frequency
-    // terms can only lower a value, and a barred id's value is -inf: without a bias list a
-    // listed id's true value never exceeds its raw one.
-    const bool lowering = n_bias == 0u && a.repetition >= 1.0f && a.presence >= 0.0f &&
-                          a.frequency >= 0.0f;
-    // A listed id's raw value, into the thread's maximum of listed raw values (which must
-    // cover every listed id: see row_max).
-    auto listed_raw = [&](const Listed& r) {
-        if (r.ent != NONE) {
-            listed_raw_max = fmaxf(listed_raw_max, raw_of(r.chunk, r.ent & ID_MASK));
+
+    // ---- the bits of a block's chunks
+    // Load u of a block brings the wave 64 consecutive chunks, whose ids' bits fill WPP
+    // consecutive words of a bitmap (one more when the first chunk starts inside a word): lane
+    // u * WPP + q requests word q of piece u, the first four lanes the pieces' extra words.
+    // Words before or after the bitmap are replaced by its first or last word: they belong to
+    // chunks that are not streamed, whose bits nobody looks at.
+    const uint32_t win_sh = (g.cb * (uint32_t)E - g.pad) & 31u;   // a piece's first bit inside its first word
+    struct Bits {
+        uint32_t t, tx;   // listed ids: this lane's word, this lane's extra word
+        uint32_t m, mx;   // allowed ids (masked rows)
+    };
+    const uint32_t* t_words = pen ? a.touched : reinterpret_cast<const uint32_t*>(g.base);
+    const uint32_t* m_words = masked ? a.allow : reinterpret_cast<const uint32_t*>(g.base);
+    auto piece_word0 = [&](uint32_t b, uint32_t u) -> int32_t {
+        const int32_t first = (int32_t)((g.cb + b * BLOCK + u * NT + w * 64u) * (uint32_t)E) - (int32_t)g.pad;
+        return first >> 5;  // arithmetic: ids before the row lie in "word -1"
+    };
+    auto bits_request = [&](Bits& d, uint32_t b) {
+        const uint32_t u = min(lane / WPP, 3u), q = lane % WPP;
+        const int32_t hi = (int32_t)row_words - 1;
+        const uint32_t i0 = (uint32_t)min(max(piece_word0(b, u) + (int32_t)q, 0), hi);
+        const uint32_t i1 = (uint32_t)min(max(piece_word0(b, lane & 3u) + (int32_t)WPP, 0), hi);
+        d.t = gload(t_words + i0);
+        d.tx = gload(t_words + i1);
+        if (MASKS) {
+            d.m = gload(m_words + i0);
+            d.mx = gload(m_words + i1);
         }
     };
-    // A listed id's true value before the temperature (bias in list order, then penalties);
-    // also feeds the thread's maximum of listed true values (a lower bound of the row's largest
-    // true value whichever ids it covers).
-    auto listed_true = [&](const Listed& r, float raw) -> float {
-        const uint32_t id = r.ent & ID_MASK;
-        uint32_t cnt = r.ent >> SPEC_ID_BITS;
-        if (cnt == 4095u) {
-            cnt = gload(a.counts + id);
-            // The value is waited for here, inside the branch: waiting after it would make
-            // every thread drain the loads it has in flight.
-            asm volatile("" : "+v"(cnt));
-        }
-        float t = raw;
-        for (uint32_t j = 0; j < n_bias; ++j) {
-            if (L.bias_id[j] == id) {
-                t += L.bias_delta[j];
+    // The wave passes its words through its own piece of LDS (its own writes and reads only:
+    // LDS serves a wave's operations in order, so no barrier is needed) and every lane takes
+    // the E bits of each of its four chunks.
+    auto bits_take = [&](const Bits& d, uint32_t& tb_all, uint32_t (&mb)[U]) {
+        uint32_t* mine = L.win + w * (2u * WIN_WORDS);
+        const uint32_t u = lane / WPP, q = lane % WPP;
+        if (u < 4u) {
+            mine[u * PIECE + q] = d.t;
+            if (MASKS) {
+                mine[WIN_WORDS + u * PIECE + q] = d.m;
             }
         }
-        if (cnt > 0u) {
-            t = t > 0.0f ? t / a.repetition : t * a.repetition;
-            t -= a.presence + a.frequency * (float)cnt;
+        if (lane < 4u) {
+            mine[lane * PIECE + WPP] = d.tx;
+            if (MASKS) {
+                mine[WIN_WORDS + lane * PIECE + WPP] = d.mx;
+            }
         }
-        if (masked && !bit_of(a.allow, id)) {
-            t = NEG_INF;
+        // (Nothing for the hardware to do; the compiler must not move the reads above the writes
+        // of other lanes.)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t off = win_sh + lane * (uint32_t)E;
+#pragma unroll
+        for (int v = 0; v < U; ++v) {
+            const uint32_t at = (uint32_t)v * PIECE + (off >> 5);
+            const uint64_t two = ((uint64_t)mine[at + 1u] << 32) | mine[at];
+            tb_all |= pen ? ((uint32_t)(two >> (off & 31u)) & EMASK) << (8 * v) : 0u;
+            if (MASKS) {
+                const uint64_t mtwo = ((uint64_t)mine[WIN_WORDS + at + 1u] << 32) | mine[WIN_WORDS + at];
+                mb[v] = masked ? ~(uint32_t)(mtwo >> (off & 31u)) & EMASK : 0u;   // 1 = barred
+            } else {
+                mb[v] = 0u;
+            }
         }
-        listed_true_max = fmaxf(listed_true_max, t);
-        return t;
+        __builtin_amdgcn_wave_barrier();
     };
-    // After the block's bound is known: was the id's chunk queued or summed by its owner (the
-    // owner's tests on the same bits), the id's terms, and the id as a candidate.  When values
-    // can only be lowered, an id whose chunk was neither queued nor summed is below the bound
-    // and below the sum's cut with its true value too: nothing of it is evaluated (most blocks
-    // of most rows hold no other kind, and their waves skip all of this).
-    auto listed_finish = [&](const Listed& r, bool nonneg) {
-        const bool has = r.ent != NONE;
-        const float cm = nonneg ? chunk_max_nonneg<DT>(r.chunk) : chunk_max<DT>(r.chunk);
-        const bool queued = cm >= T;
-        const bool summed = !queued && cm > skip_b;  // the cut is -inf without a row sum
-        if (!has || (lowering && !queued && !(want_lse && summed))) {
-            return;
-        }
-        const uint32_t id = r.ent & ID_MASK;
-        const float raw = raw_of(r.chunk, id);
-        const float t = listed_true(r, raw);
-        if (want_lse) {
-            if (t > skip_b) {  // the same cut as for streamed terms
-                acc_t += term_d(t);
+
+    // Listed ids of a block's chunks that are not queued, on the spot.  `todo`: a byte per chunk
+    // of the block, bit j = element j is a listed id that matters.  One loop for the whole
+    // block: the lanes take their first such element together, so the gathers of its counts
+    // are in flight together and waited for once.
+    //   * Rows without a row sum whose listed ids may rise: the true value is offered as a
+    //     candidate.  (With a row sum such chunks are queued instead.)
+    //   * Rows with a row sum whose listed ids can only be lowered, chunks whose raw terms went
+    //     into the running sum: the raw term is taken off again and the true term (never the
+    //     larger one, so it fits the same reference) added, in the lane's own f32 sum.
+    auto fix_listed = [&](const u32x4 (&cur)[U], uint32_t b, uint32_t todo) {
+        while (todo != 0u) {
+            const uint32_t i = (uint32_t)__builtin_ctz(todo);
+            todo &= todo - 1u;
+            const uint32_t u = i >> 3, j = i & 7u;
+            u32x4 q = cur[0];
+            q = u == 1u ? cur[1] : q;
+            q = u == 2u ? cur[2] : q;
+            q = u == 3u ? cur[3] : q;
+            const float raw = elem_of(q, j);
+            if (!(raw > NEG_INF)) {
+                continue;  // barred as well, or -inf to begin with: no term, no candidate
             }
-            if (summed) {
-                acc_r += term_d(raw);
+            const uint32_t id = g.id_of(g.cb + (b * U + u) * NT + tid, (int)j);
+            if (n_bias != 0u && biased(id)) {
+                continue;  // the pass after the scan speaks for it
             }
-        }
-        if (queued) {
-            const uint32_t at = atomicAdd(&sh.n_drop, 1u);
-            if (at < DROP_CAP) {
-                L.drop[at] = id;
-            }
-        }
-        if (t >= T && t > NEG_INF) {
-            const uint32_t at = atomicAdd(&sh.n_fc, 1u);
-            if (at < FC_CAP) {
-                L.fc[at] = composite_of(t / a.temperature, id);
+            const float t = true_value(id, raw);
+            if (lowering) {
+                const float off = __builtin_amdgcn_exp2f(__builtin_fmaf(raw, c2, -wl.ref));
+                const float on = t > skip_b ? __builtin_amdgcn_exp2f(__builtin_fmaf(t, c2, -wl.ref)) : 0.0f;
+                wl.s += on - off;
+                wl.booked += off;
+            } else if (t >= T && t > NEG_INF) {
+                const uint32_t at = atomicAdd(&sh.n_fc, 1u);
+                if (at < FC_CAP) {
+                    L.fc[at] = composite_of(t / a.temperature, id);
+                }
             }
         }
     };
@@ -672,178 +465,196 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // buffers that swap roles): one block in flight per wave leaves the memory idle whenever
     // a wave's arithmetic outlasts its load.
     const float lse_cut = (log2f((float)g.vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
-    // Memory operations of a wave complete in the order they were issued: a block's listed
-    // gathers are requested BEFORE the next stream block, so using them never waits for it.
-    Listed lst_a, lst_b, lst_c;
-    lst_a.ent = NONE;
-    lst_b.ent = NONE;
-    lst_c.ent = NONE;
-    // The waves of a compute unit's oldest workgroup win the issue slots and its youngest
-    // finishes last, alone.  Rows that carry both listed ids and a row sum (the most
-    // instructions per block) lower their waves' priority as they advance, so a workgroup
-    // that fell behind catches up; lighter rows lose by it and leave the priority alone.
-    const bool paced = listed_row && want_lse;
-    auto work = [&](u32x4 (&cur)[U], Listed& lcur, uint32_t b) {
-        if (paced) {
-            const uint32_t q = b * 4u / nblocks;
-            if (q == 0u) {
-                __builtin_amdgcn_s_setprio(3);
-            } else if (q == 1u) {
-                __builtin_amdgcn_s_setprio(2);
-            } else if (q == 2u) {
-                __builtin_amdgcn_s_setprio(1);
-            } else {
-                __builtin_amdgcn_s_setprio(0);
+    // The scan is compiled twice, for rows whose chunks come with bits and for rows without:
+    // left as a test inside the loop, the bits' loads would be loads that may be skipped, and
+    // every wait behind them would drain the blocks requested ahead.
+    auto scan = [&](auto with_bits) {
+        constexpr bool SP = decltype(with_bits)::value;
+        Bits bits_a = {}, bits_b = {}, bits_c = {};
+        auto work = [&](u32x4 (&cur)[U], const Bits& bcur, uint32_t b) {
+            // tb_all: a byte per chunk of the block, bit j = element j is a listed id.
+            uint32_t tb_all = 0u, mb[U] = {0u, 0u, 0u, 0u};
+            if (SP) {
+                bits_take(bcur, tb_all, mb);
             }
-        }
-        if (!full_block(b)) {
-            const uint32_t ninf = DT == LILY_BF16 ? 0xff80ff80u : 0xff800000u;
+            if (!full_block(b)) {
+                const uint32_t ninf = DT == LILY_BF16 ? 0xff80ff80u : 0xff800000u;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t c = g.cb + (b * U + u) * NT + tid;
+                    if (c < g.main_lo || c >= g.main_hi) {
+                        cur[u] = u32x4{ninf, ninf, ninf, ninf};
+                        tb_all &= ~(0xffu << (8 * u));
+                        mb[u] = 0u;
+                    }
+                }
+            }
+            if (MASKS && masked) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    cur[u] = without(cur[u], mb[u]);
+                }
+            }
+            // The block's own maxima enter the bound before the block is filtered.  Chunks below
+            // the previous bound cannot be queued: their terms are summed right away.
+            const float T_prev = T;
+            // Once the bound is positive only chunks with a positive element can matter to it:
+            // their maximum comes from the cheaper form, which reports +0 for all others (the sum
+            // then takes such a chunk unless the cut is positive too, and the lanes' maxima are
+            // only overstated up to 0, below the bound they could move).
+            const bool nonneg = DT == LILY_BF16 && __builtin_amdgcn_readfirstlane((int)(T_prev > 0.0f)) != 0;
+            float m8[U];
+            float block_max = NEG_INF;
+            if (nonneg) {
+                // No value here is below +0: their bit patterns order like integers, and such a
+                // pattern exceeds that of any negative value the lane's maximum may still hold.
+                int bm = 0;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    m8[u] = chunk_max_nonneg<DT>(cur[u]);
+                    bm = max(bm, (int)lilym_f32_bits(m8[u]));
+                }
+                block_max = lilym_bits_f32((uint32_t)bm);
+                lane_max = lilym_bits_f32((uint32_t)max((int)lilym_f32_bits(lane_max), bm));
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    m8[u] = chunk_max<DT>(cur[u]);
+                    block_max = max2_raw(block_max, m8[u]);
+                }
+                lane_max = max2_raw(lane_max, block_max);
+            }
+            if (SP && LSE && want_lse && __ballot(block_max > row_max) != 0ull) {
+                // Only a chunk above the largest value known so far can raise it (rare after the
+                // first blocks).  (The cheaper maximum is exact only where it is positive.)
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const bool clean = ((tb_all >> (8 * u)) & 0xffu) == 0u && (!nonneg || m8[u] > 0.0f);
+                    clean_max = fmaxf(clean_max, clean ? m8[u] : NEG_INF);
+                }
+            }
+            // Rows with a row sum whose listed ids may rise: a chunk that holds a listed id is
+            // queued whatever its values (the queue's expansion evaluates every element exactly).
+            uint32_t forced = 0u;   // bit u: chunk u is queued for its listed ids
+            if (SP && LSE && want_lse && !lowering) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    forced |= ((tb_all >> (8 * u)) & 0xffu) != 0u ? 1u << u : 0u;
+                }
+            }
+            if (LSE && want_lse) {
+                // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
+                // sum by more than 2^-21 of it, even with every element of the row at that level:
+                // such chunks are left out, by a rule every thread of the block can evaluate.
+                skip_b = row_max - lse_cut;
+                wl.skip_below = skip_b;
+                // Rows with a dominant value skip nearly every block as a whole.
+                if (__ballot(block_max > skip_b) != 0ull) {
+                    wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        wl.template add_prepared<DT>(cur[u], m8[u], c2,
+                                                     !(m8[u] >= T_prev) && ((forced >> u) & 1u) == 0u);
+                    }
+                }
+            }
+            // The bound moves most in the first blocks: refresh it for each of them, then for
+            // every fourth block (each refresh is a ballot search and a barrier).  The row's
+            // maxima behind the sum's cut follow with every other of those.
+            if (b < 4u || (b & 3u) == 0u) {
+                refresh_bound(b == 0, b == 0 || (LSE && want_lse && (b < 4u || (b & 7u) == 0u)));
+                if (LSE && want_lse) {
+                    // The cut follows at once: what is summed from here on (all of block 0, whose
+                    // chunks were held back above for want of a bound) is measured against the
+                    // largest value known now.  Terms between the old cut and the new one that
+                    // were summed already are as negligible as those that were not.
+                    skip_b = row_max - lse_cut;
+                    wl.skip_below = skip_b;
+                }
+            }
+            if (n_bias != 0u && tid == 0) {
+                L.blk_bound[b] = T;
+                L.blk_cut[b] = skip_b;
+                L.blk_flag[b] = nonneg ? 1u : 0u;
+            }
+            const bool any_late = LSE && want_lse && T != T_prev &&
+                                  __ballot(block_max >= T_prev && block_max > skip_b) != 0ull;
+            // When values can only be lowered, a listed id in a chunk that was neither queued nor
+            // summed is below the bound and below the sum's cut with its true value too: nothing
+            // of it is evaluated (most chunks of most rows; rows with a dominant value sum next
+            // to nothing, and their waves skip even the test).
+            uint32_t fix = 0u;   // a byte per chunk: its listed ids that are evaluated on the spot
+            const bool fix_any = SP && (!lowering || (LSE && want_lse && __ballot(block_max > skip_b) != 0ull));
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t c = g.cb + (b * U + u) * NT + tid;
-                if (c < g.main_lo || c >= g.main_hi) {
-                    cur[u] = u32x4{ninf, ninf, ninf, ninf};
+                const bool pass = m8[u] >= T || ((forced >> u) & 1u) != 0u;
+                const uint64_t mask = __ballot(pass);
+                if (mask != 0ull) {
+                    const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+                        (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                    const uint32_t at = wq + rank;
+                    if (pass && at < QSEG) {
+                        L.qraw[w * QSEG + at] = cur[u];
+                        L.qidx[w * QSEG + at] = c;
+                        L.qbits[w * QSEG + at] = (uint8_t)(tb_all >> (8 * u));
+                    }
+                    wq += (uint32_t)__popcll(mask);
+                }
+                if (any_late) {
+                    // At or above the previous bound but below the new one: not queued after all.
+                    const bool late = m8[u] >= T_prev && !pass;
+                    if (__ballot(late) != 0ull) {
+                        wl.prepare(late ? m8[u] : NEG_INF, c2);
+                        wl.template add_prepared<DT>(cur[u], m8[u], c2, late);
+                    }
+                }
+                if (SP && fix_any) {
+                    const uint32_t tb = (tb_all >> (8 * u)) & 0xffu;
+                    const bool matters = !lowering || (LSE && want_lse && m8[u] > skip_b);
+                    fix |= (tb != 0u && !pass && matters) ? tb << (8 * u) : 0u;
                 }
             }
-        }
-        if (listed_row) {
-            listed_raw(lcur);
-        }
-        // The block's own maxima enter the bound before the block is filtered.  Chunks below
-        // the previous bound cannot be queued: their terms are summed right away.
-        const float T_prev = T;
-        // Once the bound is positive only chunks with a positive element can matter to it:
-        // their maximum comes from the cheaper form, which reports +0 for all others (the sum
-        // then takes such a chunk unless the cut is positive too, and the lanes' maxima are
-        // only overstated up to 0, below the bound they could move).
-        const bool nonneg = DT == LILY_BF16 && __builtin_amdgcn_readfirstlane((int)(T_prev > 0.0f)) != 0;
-        float m8[U];
-        float block_max = NEG_INF;
-        if (nonneg) {
-            // No value here is below +0: their bit patterns order like integers, and such a
-            // pattern exceeds that of any negative value the lane's maximum may still hold.
-            int bm = 0;
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                m8[u] = chunk_max_nonneg<DT>(cur[u]);
-                bm = max(bm, (int)lilym_f32_bits(m8[u]));
+            if (SP && fix != 0u) {
+                fix_listed(cur, b, fix);
             }
-            block_max = lilym_bits_f32((uint32_t)bm);
-            lane_max = lilym_bits_f32((uint32_t)max((int)lilym_f32_bits(lane_max), bm));
+        };
+        // A request past the last block asks for the last block again (its lines are in the
+        // cache and nothing uses the result): with the same loads in flight on every path the
+        // wait for a block's data leaves the blocks requested after it in flight, where a request
+        // that may be skipped makes that wait count as if it had been.
+        auto request = [&](u32x4 (&dst)[U], Bits& bdst, uint32_t b) {
+            const uint32_t bb = min(b, nblocks - 1u);
+            if (SP) {
+                bits_request(bdst, bb);
+            }
+            fetch(dst, bb);
+        };
+        if (nblocks == 0) {
+            refresh_bound(true, true);  // the same barriers in every workgroup
         } else {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                m8[u] = chunk_max<DT>(cur[u]);
-                block_max = max2_raw(block_max, m8[u]);
+            if (SP) {
+                bits_request(bits_a, 0);
             }
-            lane_max = max2_raw(lane_max, block_max);
-        }
-        if (LSE && want_lse) {
-            // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
-            // sum by more than 2^-21 of it, even with every element of the row at that level:
-            // such chunks are left out, by a rule every thread of the block can evaluate.
-            skip_b = row_max - lse_cut;
-            wl.skip_below = skip_b;
-            // Rows with a dominant value skip nearly every block as a whole.
-            if (__ballot(block_max > skip_b) != 0ull) {
-                wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    wl.template add_prepared<DT>(cur[u], m8[u], c2, !(m8[u] >= T_prev));
+            request(buf_b, bits_b, 1);
+            for (uint32_t b = 0; b < nblocks; b += 3) {
+                request(buf_c, bits_c, b + 2);
+                work(buf_a, bits_a, b);
+                if (b + 1 < nblocks) {
+                    request(buf_a, bits_a, b + 3);
+                    work(buf_b, bits_b, b + 1);
+                    if (b + 2 < nblocks) {
+                        request(buf_b, bits_b, b + 4);
+                        work(buf_c, bits_c, b + 2);
+                    }
                 }
-            }
-        }
-        // The bound moves most in the first blocks: refresh it for each of them, then for
-        // every fourth block (each refresh is a ballot search and a barrier).  The row's
-        // maxima behind the sum's cut follow with every other of those.
-        if (b < 4u || (b & 3u) == 0u) {
-            refresh_bound(b == 0, b == 0 || (LSE && want_lse && (b < 4u || (b & 7u) == 0u)));
-        }
-        const bool any_late = LSE && want_lse && T != T_prev &&
-                              __ballot(block_max >= T_prev && block_max > skip_b) != 0ull;
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t c = g.cb + (b * U + u) * NT + tid;
-            const bool pass = m8[u] >= T;
-            const uint64_t mask = __ballot(pass);
-            if (mask != 0ull) {
-                const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
-                    (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
-                const uint32_t at = wq + rank;
-                if (pass && at < QSEG) {
-                    L.qraw[w * QSEG + at] = cur[u];
-                    L.qidx[w * QSEG + at] = c;
-                }
-                wq += (uint32_t)__popcll(mask);
-            }
-            if (any_late) {
-                // At or above the previous bound but below the new one: not queued after all.
-                const bool late = m8[u] >= T_prev && !pass;
-                if (__ballot(late) != 0ull) {
-                    wl.prepare(late ? m8[u] : NEG_INF, c2);
-                    wl.template add_prepared<DT>(cur[u], m8[u], c2, late);
-                }
-            }
-        }
-        if (listed_row) {
-            listed_finish(lcur, nonneg);
-            const uint32_t n_b = (L.hseg[b].y - L.hseg[b].x) + (L.bkt[b + 1] - L.bkt[b]);
-            for (uint32_t round = 1; round * NT < n_b; ++round) {
-                // Rare (a block with more listed ids than threads).  Both loads are waited for
-                // right here, inside the loop: left to the first use, their waits would be
-                // placed where every path meets and drain the blocks requested ahead.
-                Listed extra;
-                uint32_t e = entry_load(b, round);
-                asm volatile("" : "+v"(e));
-                listed_fetch(extra, e, b, round);
-                asm volatile("" : "+v"(extra.chunk.x), "+v"(extra.chunk.y), "+v"(extra.chunk.z),
-                             "+v"(extra.chunk.w));
-                listed_raw(extra);
-                listed_finish(extra, nonneg);
             }
         }
     };
-    // A request past the last block asks for the last block again (its lines are in the
-    // cache and nothing uses the result): with the same loads in flight on every path the
-    // wait for a block's data leaves the blocks requested after it in flight, where a request
-    // that may be skipped makes that wait count as if it had been.
-    // A block's entry of the sorted part is requested two requests ahead of its gather, which
-    // therefore never waits for anything younger than the block the next `work` needs anyway:
-    // `pre` is this block's entry, `ahead` receives the one of the block after next.
-    auto request = [&](u32x4 (&dst)[U], Listed& ldst, uint32_t pre, uint32_t& ahead, uint32_t b) {
-        const uint32_t bb = min(b, nblocks - 1u);
-        if (listed_row) {
-            listed_fetch(ldst, pre, bb, 0);
-            ahead = entry_load(min(b + 2u, nblocks - 1u), 0);
-        }
-        fetch(dst, bb);
-    };
-    if (nblocks == 0) {
-        refresh_bound(true, true);  // the same barriers in every workgroup
+    if (special) {
+        scan(std::true_type{});
     } else {
-        uint32_t pre_a = 0, pre_b = 0, pre_c = 0;
-        if (listed_row) {
-            pre_a = entry_load(0, 0);
-            pre_b = entry_load(min(1u, nblocks - 1u), 0);
-            pre_c = entry_load(min(2u, nblocks - 1u), 0);
-            listed_fetch(lst_a, pre_a, 0, 0);
-        }
-        request(buf_b, lst_b, pre_b, pre_a, 1);
-        for (uint32_t b = 0; b < nblocks; b += 3) {
-            request(buf_c, lst_c, pre_c, pre_b, b + 2);
-            work(buf_a, lst_a, b);
-            if (b + 1 < nblocks) {
-                request(buf_a, lst_a, pre_a, pre_c, b + 3);
-                work(buf_b, lst_b, b + 1);
-                if (b + 2 < nblocks) {
-                    request(buf_b, lst_b, pre_b, pre_a, b + 4);
-                    work(buf_c, lst_c, b + 2);
-                }
-            }
-        }
-    }
-    if (paced) {
-        __builtin_amdgcn_s_setprio(0);  // a row of fewer than four blocks never reached it
+        scan(std::false_type{});
     }
     phase(cfg, 2);
 
@@ -854,7 +665,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     __syncthreads();
     const float filt = T;
     {
-        bool overflow = sh.n_drop > DROP_CAP;
+        bool overflow = false;
         for (int i = 0; i < NWAVE; ++i) {
             overflow = overflow || sh.qfill[i] > QSEG;
         }
@@ -862,24 +673,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             return stream_fail(cfg, 4u);
         }
     }
-    // Listed ids inside queued chunks: mark their element in the chunk's queue slot.  A
-    // wave's segment is in ascending chunk order, so the slot is found by bisection.
-    for (uint32_t d = tid; d < sh.n_drop; d += NT) {
-        const uint32_t id = L.drop[d];
-        const uint32_t c = (id + g.pad) / E, j = (id + g.pad) % E;
-        const uint32_t ow = ((c - g.cb) % NT) / 64u;
-        uint32_t lo = ow * QSEG, hi = lo + sh.qfill[ow];
-        while (lo < hi) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (L.qidx[mid] < c) {
-                lo = mid + 1;
-            } else {
-                hi = mid;
-            }
-        }
-        atomicOr(&L.dmask[lo >> 2], (1u << j) << ((lo & 3u) * 8u));
-    }
-    __syncthreads();
     auto offer = [&](float u, uint32_t id) {
         if (u >= filt && u > NEG_INF) {
             const uint32_t at = atomicAdd(&sh.n_fc, 1u);
@@ -888,9 +681,21 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
     };
+    // Block of a streamed id of this slice, NONE for ids outside it or in a partial chunk.
+    auto block_of = [&](uint32_t id) -> uint32_t {
+        if (id >= g.vocab) {
+            return NONE;
+        }
+        const uint32_t c = (id + g.pad) / E;
+        if (c < g.main_lo || c >= g.main_hi) {
+            return NONE;
+        }
+        return (c - g.cb) / BLOCK;
+    };
     {
         // One thread per queued chunk (the waves' segments counted through in order): its
-        // elements that are not listed ids add their term and are offered.
+        // elements add their term and are offered - listed ones with their true value, ids of
+        // the bias list not at all (the pass below speaks for them).
         uint32_t seg_end[NWAVE], total = 0;
 #pragma unroll
         for (int i = 0; i < NWAVE; ++i) {
@@ -909,32 +714,79 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             const uint32_t slot = ww * QSEG + (ch - before);
             const u32x4 q = L.qraw[slot];
             const uint32_t c = L.qidx[slot];
-            const uint32_t dm = (L.dmask[slot >> 2] >> ((slot & 3u) * 8u)) & 0xffu;
+            const uint32_t dm = L.qbits[slot];
             float v[E];
             unpack<DT>(q, v);
             // Few elements of a queued chunk matter (usually the one that got it queued):
             // they are marked first and then taken one at a time, in ascending order, instead
-            // of eight branches that some lane of the wave enters every time.
-            uint32_t todo = 0;
+            // of eight branches that some lane of the wave enters every time.  A listed element
+            // whose value can only be lowered matters under the same conditions as any other.
+            uint32_t todo = 0, finite = 0;
 #pragma unroll
             for (int j = 0; j < E; ++j) {
                 const bool term = want_lse && v[j] > skip_b;  // the cut of the streamed terms
                 const bool cand = v[j] >= filt && v[j] > NEG_INF;
                 todo |= (term || cand) ? 1u << j : 0u;
+                finite |= v[j] > NEG_INF ? 1u << j : 0u;
             }
-            todo &= ~dm;
+            todo = (todo & ~dm) | (dm & (lowering ? todo : finite));
             while (todo != 0u) {
                 const uint32_t j = (uint32_t)__builtin_ctz(todo);
                 todo &= todo - 1u;
-                const float x = elem_of(q, j);
-                if (want_lse && x > skip_b) {
-                    acc_q += term_d(x);
+                float x = elem_of(q, j);
+                const uint32_t id = g.id_of(c, (int)j);
+                if (n_bias != 0u && biased(id)) {
+                    continue;
                 }
-                offer(x, g.id_of(c, (int)j));
+                if ((dm >> j) & 1u) {
+                    x = true_value(id, x);
+                }
+                if (want_lse && x > skip_b) {
+                    acc_t += term_d(x);
+                }
+                offer(x, id);
             }
         }
     }
     phase(cfg, 8);
+    if (n_bias != 0u) {
+        // The bias list's ids were streamed with their raw values and left alone by everything
+        // above.  One thread per id - the first entry that names it - looks the chunk up again
+        // and redoes its owner's tests with the bound, the cut and the kind of maximum its block
+        // was scanned with: a summed chunk's raw term is booked, the true term (bias in list
+        // order, then penalties) added and the true value offered.
+        for (uint32_t i = tid; i < n_bias; i += NT) {
+            const uint32_t id = L.bias_id[i];
+            bool first = true;
+            for (uint32_t j = 0; j < i; ++j) {
+                first = first && L.bias_id[j] != id;
+            }
+            const uint32_t b = block_of(id);
+            if (!first || b == NONE || (masked && !bit_of(a.allow, id))) {
+                continue;  // an edge id, or a barred id (streamed as -inf)
+            }
+            const uint32_t c = (id + g.pad) / E;
+            u32x4 q = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
+            if (masked) {
+                q = without(q, ~bits32_at(a.allow, row_words, (int64_t)g.id_of(c, 0)) & EMASK);
+            }
+            const float cm = L.blk_flag[b] != 0u ? chunk_max_nonneg<DT>(q) : chunk_max<DT>(q);
+            const float cut = L.blk_cut[b];
+            const bool queued = cm >= L.blk_bound[b];
+            const bool summed = !queued && cm > cut;
+            const float raw = elem_of(q, (id + g.pad) % E);
+            const float t = true_value(id, raw);
+            if (want_lse) {
+                if (summed) {
+                    acc_r += term_d(raw);
+                }
+                if (t > cut) {
+                    acc_t += term_d(t);
+                }
+            }
+            offer(t, id);
+        }
+    }
     // Ids of partial 16-byte chunks at the row's ends were not streamed: exact, one by one.
     for (int side = 0; side < 2; ++side) {
         const uint32_t lo = side == 0 ? g.id_lo : g.edge_hi_begin;
@@ -942,7 +794,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         for (uint32_t id = lo + tid; id < hi; id += NT) {
             const float u = pre_temperature_of<DT>(a, id);
             if (want_lse) {
-                acc_q += term_d(u);
+                acc_t += term_d(u);
             }
             offer(u, id);
         }
@@ -962,16 +814,18 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             ref_w = max(ref_w, (int)__builtin_floor(e));
         }
         const int down = up == UP_UNSET ? 0 : up - ref_w;  // <= 0
-        double part[3];
+        double part[4];
         {
             double d = stream_at - (double)ref_w;  // <= 1 where there is a sum
             d = d < -1000.0 ? -1000.0 : d;
-            part[0] = wl.s > 0.0f ? (double)wl.s * pow2_d(d) : 0.0;
+            const double scale = pow2_d(d);
+            part[0] = wl.s > 0.0f ? (double)wl.s * scale : 0.0;
+            part[3] = wl.booked > 0.0f ? (double)wl.booked * scale : 0.0;
         }
         part[1] = __builtin_ldexp(acc_r, down);
-        part[2] = __builtin_ldexp(acc_t + acc_q, down);
+        part[2] = __builtin_ldexp(acc_t, down);
 #pragma unroll
-        for (int i = 0; i < 3; ++i) {
+        for (int i = 0; i < 4; ++i) {
             part[i] = wave_sum_d(part[i]);
             if (lane == 0) {
                 sh.red3[i][w] = part[i];
@@ -986,7 +840,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             ref_all = max(ref_all, (int)sh.red_i[i]);
         }
 #pragma unroll
-        for (int i = 0; i < 3; ++i) {
+        for (int i = 0; i < 4; ++i) {
             part[i] = 0.0;
             for (int ww = 0; ww < NWAVE; ++ww) {
                 const int at = (int)sh.red_i[ww];
@@ -996,10 +850,13 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (ref_all == UP_UNSET) {
             ref_all = 0;  // no term anywhere: the sums are zero
         }
-        const double streamed = part[0], booked = part[1], exact = part[2];
+        // part[0]: the running sums, the listed ids' raw terms of part[3] already taken off (and
+        // their true terms added); part[1]: raw terms still to take off; part[2]: terms added
+        // one by one.
+        const double streamed = part[0], booked = part[1], exact = part[2], taken = part[3];
         const double rest = streamed - booked;
         // Listed ids held nearly all of what was streamed: the difference is too coarse.
-        const bool coarse = booked > 0.0 && !(rest > 0.05 * streamed);
+        const bool coarse = booked + taken > 0.0 && !(rest > 0.05 * (streamed + taken));
         phase(cfg, 10);
         if (coarse) {
             phase(cfg, 11);

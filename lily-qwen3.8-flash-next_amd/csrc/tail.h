@@ -136,43 +136,13 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
 
 // ------------------------------------------------------------------ tail
 
-// Lists an id that has just been counted for the first time: it joins the tail, which grows
-// downwards from the end of the list's memory (the sorted part grows upwards from its start;
-// when the two would meet the id stays unlisted and the lengths tell that the list is unusable).
-__device__ __forceinline__ void list_new_id(ListEntry* pairs, uint32_t* list_hdr, uint32_t* pos,
-                                            uint32_t pairs_cap, uint32_t id, uint32_t count) {
-    const uint32_t t = atomicAdd(&list_hdr[HDR_TAIL], 1u);
-    const uint32_t n_sorted = list_hdr[HDR_SORTED];
-    const bool fits = (uint64_t)n_sorted + t < pairs_cap;
-    const uint32_t at = fits ? pairs_cap - 1u - t : 0xffffffffu;
-    if (fits) {
-        pairs[at] = list_entry(id, count);
-    }
-    pos[id] = at;  // listed ids always have a meaningful pos
-}
-
-// Counts one emission of `id` in a scratch: the dense count, and the id's entry in the list
-// (`touched` marks the listed ids).
-__device__ __forceinline__ void count_token(uint32_t* counts, uint32_t* touched, ListEntry* pairs,
-                                            uint32_t* list_hdr, uint32_t* pos, uint32_t pairs_cap,
-                                            uint32_t id) {
-    const uint32_t before = atomicAdd(&counts[id], 1u);
-    const uint32_t bit = 1u << (id & 31u);
-    const uint32_t bits = atomicOr(&touched[id >> 5], bit);
-    if ((bits & bit) == 0u) {
-        list_new_id(pairs, list_hdr, pos, pairs_cap, id, before + 1u);
-    } else {
-        const uint32_t p = pos[id];
-        if (p < pairs_cap) {
-            pairs[p] = list_entry(id, before + 1u);
-        }
-    }
-}
-
+// Counts one emission of `id` in a scratch: the dense count, and the id's bit in the bitmap of
+// the ids that were ever counted.
 __device__ __forceinline__ void emit(const RowArgs& a, uint32_t id) {
     *a.out_id = id;
     if (a.flags & F_PEN) {
-        count_token(a.counts, a.touched, a.pairs, a.list_hdr, a.pos, a.pairs_cap, id);
+        atomicAdd(&a.counts[id], 1u);
+        atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
     }
 }
 
@@ -189,9 +159,8 @@ __device__ __forceinline__ uint32_t pick_sequential(const float* prefix, uint32_
 // log p(id) = (u*c2 - mc - log2 s) * ln 2, with the id's exponent u*c2 formed exactly as
 // the row sum formed its terms, so the two cancel when the id carries all the mass.
 // Emits `id` and, when asked, its log-probability, with the memory operations of both in one
-// round trip: the count's atomic increment returns the count the penalties used, the bitmap's
-// atomic OR tells whether the id is listed already, and the logit and the list position load
-// beside them.
+// round trip: the count's atomic increment returns the count the penalties used, and the logit
+// loads beside it.
 template <int DT>
 __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
     *a.out_id = id;
@@ -203,12 +172,10 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
         }
         return;
     }
-    uint32_t before = 0, bits = 0, p = 0xffffffffu;
-    const uint32_t bit = 1u << (id & 31u);
+    uint32_t before = 0;
     if (pen) {
         before = atomicAdd(&a.counts[id], 1u);
-        bits = atomicOr(&a.touched[id >> 5], bit);
-        p = gload(a.pos + id);
+        atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
     }
     if (want) {
         const float l = load_logit<DT>(a.logits, id);
@@ -220,13 +187,6 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
             lp = fminf((float)(e * 0.6931471805599453), 0.0f);  // the sum is approximate: clamp
         }
         *a.out_logprob = lp;
-    }
-    if (pen) {
-        if ((bits & bit) == 0u) {
-            list_new_id(a.pairs, a.list_hdr, a.pos, a.pairs_cap, id, before + 1u);
-        } else if (p < a.pairs_cap) {
-            a.pairs[p] = list_entry(id, before + 1u);
-        }
     }
 }
 

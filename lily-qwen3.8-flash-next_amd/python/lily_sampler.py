@@ -414,7 +414,10 @@ class Plan:
 
     def close(self):
         if self._h:
-            _lib.lily_plan_destroy(self._h)
+            # The library object points at its sampler: once that is gone (a garbage collection
+            # that finalised the sampler first) the handle is only dropped.
+            if self._s._h:
+                _lib.lily_plan_destroy(self._h)
             self._h = None
 
     def __del__(self):
@@ -436,7 +439,10 @@ class SamplerScratch:
 
     def close(self):
         if self._h:
-            _lib.lily_scratch_destroy(self._h)
+            # The library object points at its sampler: once that is gone (a garbage collection
+            # that finalised the sampler first) the handle is only dropped.
+            if self._s._h:
+                _lib.lily_scratch_destroy(self._h)
             self._h = None
 
     def __del__(self):
@@ -491,7 +497,10 @@ class DraftDists:
 
     def close(self):
         if self._h:
-            _lib.lily_draft_dists_destroy(self._h)
+            # The library object points at its sampler: once that is gone (a garbage collection
+            # that finalised the sampler first) the handle is only dropped.
+            if self._s._h:
+                _lib.lily_draft_dists_destroy(self._h)
             self._h = None
 
     def __del__(self):
