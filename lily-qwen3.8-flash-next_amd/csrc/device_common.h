@@ -222,10 +222,13 @@ struct Shared {
     double lse_s;    // sum of 2^(x * log2e / T - lse_mc) over the row
     // streaming select
     float bound[2][NWAVE];   // each wave's lower bound of its share of the k-th largest (two parities)
-    float wmax[2][2][NWAVE];  // each wave's largest raw value, and its largest among chunks without a
-                              // listed id
+    float wmax[2][NWAVE];     // each wave's largest raw value
+    uint32_t wfill[2][NWAVE]; // each wave's queue fill at the last refresh
+    uint32_t wnote[2][NWAVE]; // each wave's count for the scan's choice of mode
     uint32_t qfill[NWAVE];   // chunks each wave queued
+    uint32_t nfill[NWAVE];   // chunks each wave noted
     uint32_t n_fc;           // final candidates
+    uint32_t n_hits;   // noted chunks found to hold a listed id
     uint32_t fail;
     double red3[4][NWAVE];
 };

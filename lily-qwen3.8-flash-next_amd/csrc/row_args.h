@@ -103,6 +103,7 @@ constexpr uint32_t SPECIAL_LIST_CAP = 2048;  // ids of penalised / biased tokens
 constexpr uint32_t STREAM_K_MAX = 64;
 constexpr uint32_t STREAM_UNROLL = 4;      // 16-byte chunks per thread per block
 constexpr uint32_t Q_CAP = 768;            // queued chunks (those holding a value at or above the bound)
+constexpr uint32_t S_CAP = 4096;           // noted chunks (summed before their listed ids were looked at)
 constexpr uint32_t FC_CAP = 1024;          // final candidates
 constexpr uint32_t MAX_BLOCKS = 64;        // blocks of one slice
 constexpr uint32_t STREAM_BIAS_CAP = 64;   // bias pairs kept in LDS
@@ -113,15 +114,15 @@ constexpr uint32_t WIN_PIECE_MAX = 64 * 8 / 32 + 1;           // bf16: 64 chunks
 constexpr uint32_t WIN_WORDS = STREAM_UNROLL * WIN_PIECE_MAX; // per wave and bitmap
 constexpr uint32_t OFF_QRAW = 0;
 constexpr uint32_t OFF_QIDX = OFF_QRAW + Q_CAP * 16;
-constexpr uint32_t OFF_QBITS = OFF_QIDX + Q_CAP * 4;          // a byte per queue slot: its listed elements
-constexpr uint32_t OFF_WIN = OFF_QBITS + Q_CAP;               // [4 waves][2 bitmaps][WIN_WORDS]
+constexpr uint32_t OFF_NOTED = OFF_QIDX + Q_CAP * 4;          // [4 waves][S_CAP / 4] x 16 bits
+constexpr uint32_t OFF_WIN = OFF_NOTED + S_CAP * 2;           // [4 waves][2 bitmaps][WIN_WORDS]
 constexpr uint32_t OFF_BLK = OFF_WIN + 4 * 2 * WIN_WORDS * 4; // [MAX_BLOCKS] x (bound, cut, flags)
 constexpr uint32_t OFF_BIAS = OFF_BLK + MAX_BLOCKS * 12;      // ids then deltas
 // The final candidates lie above everything the tail and the merge use (the sorted candidates
 // and the tail's three float arrays: K_CAP * 8 + 3 * K_CAP * 4 bytes from the start).
-constexpr uint32_t OFF_FC = 20480;
+constexpr uint32_t OFF_FC = (OFF_BIAS + STREAM_BIAS_CAP * 8 + 15u) / 16u * 16u;
 constexpr uint32_t STREAM_LDS_BYTES = OFF_FC + FC_CAP * 8;
-static_assert(OFF_BIAS + STREAM_BIAS_CAP * 8 <= OFF_FC, "stream LDS layout");
+static_assert(OFF_FC >= 20480, "stream LDS layout");
 static_assert(OFF_FC % 8 == 0 && OFF_WIN % 4 == 0 && STREAM_LDS_BYTES % 16 == 0, "stream LDS layout");
 
 }  // namespace lily

@@ -103,7 +103,7 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
 
     if ((a.flags & F_FORCED) && !want_lse) {
         if (s == 0 && tid == 0) {
-            emit(a, a.forced);
+            emit(a, a.forced, vocab);
         }
         return;
     }
@@ -124,10 +124,10 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         uint32_t took = 2;
         if (cfg.path == 0u && (a.flags & F_STREAM)) {
             done = select_stream<DT, LSE, KIND != 2>(a, g, a.k, sh, cfg, sorted, found);
-            took = done ? 0u : took;
             if (!done) {
                 __syncthreads();
             }
+            took = done ? 0u : took;
         }
         if (KIND == 1 && !done && cfg.path == 0u && a.allow != nullptr) {
             done = select_sparse<DT, LSE>(a, g, a.k, cand, min(cfg.dyn_slots, MERGE_CAP), sh, sorted);

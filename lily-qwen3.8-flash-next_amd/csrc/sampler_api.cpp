@@ -80,7 +80,8 @@ struct lily_scratch {
     uint32_t vocab = 0;
     uint32_t words = 0;
     uint32_t* counts = nullptr;   // [vocab]; the one allocation, the bitmap follows it
-    uint32_t* touched = nullptr;  // [words + 4] bit per id that was ever counted
+    uint32_t* touched = nullptr;  // [words + 4] bit per id that was ever counted, then the largest
+                                  // count any id has reached
 };
 
 struct lily_draft_dists {
@@ -836,7 +837,8 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
     HIP_TRY(hipSetDevice(dst->s->device));
     HIP_TRY(hipMemcpyAsync(dst->counts, src->counts, (size_t)src->vocab * 4, hipMemcpyDeviceToDevice,
                            dst->s->stream));
-    HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)src->words * 4,
+    // (the bitmap and the largest count behind it)
+    HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)(src->words + 1) * 4,
                            hipMemcpyDeviceToDevice, dst->s->stream));
     return LILY_OK;
 }

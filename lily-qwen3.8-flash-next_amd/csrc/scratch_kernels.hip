@@ -15,14 +15,16 @@ __global__ void k_fill_u32(uint32_t* p, uint32_t n, uint32_t v) {
     }
 }
 
-// counts[id] += 1 per occurrence, and the id's bit in `touched`.
+// counts[id] += 1 per occurrence, the id's bit in `touched`, and the largest count reached (the
+// first spare word behind the bitmap).
 __global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         const uint32_t id = ids[i];
         if (id < sc.vocab) {
-            atomicAdd(&sc.counts[id], 1u);
+            const uint32_t before = atomicAdd(&sc.counts[id], 1u);
             atomicOr(&sc.touched[id >> 5], 1u << (id & 31u));
+            atomicMax(&sc.touched[(sc.vocab + 31u) / 32u], before + 1u);
         }
     }
 }
@@ -60,19 +62,25 @@ __global__ void k_uncount_after(ScratchView sc, const uint32_t* draws, uint32_t 
     }
 }
 
-// After counts were written whole: touched[w] = bits of the non-zero counts in word w.
+// After counts were written whole: touched[w] = bits of the non-zero counts in word w, and the
+// largest count (the word behind the bitmap, cleared before the launch).
 __global__ void k_touch_from_counts(ScratchView sc) {
     const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t words = (sc.vocab + 31u) / 32u;
     if (w < words) {
-        uint32_t bits = 0;
+        uint32_t bits = 0, most = 0;
         for (uint32_t b = 0; b < 32u; ++b) {
             const uint32_t id = w * 32u + b;
-            if (id < sc.vocab && sc.counts[id] != 0u) {
+            const uint32_t c = id < sc.vocab ? sc.counts[id] : 0u;
+            if (c != 0u) {
                 bits |= 1u << b;
+                most = max(most, c);
             }
         }
         sc.touched[w] = bits;
+        if (most != 0u) {
+            atomicMax(&sc.touched[words], most);
+        }
     }
 }
 
@@ -170,6 +178,7 @@ hipError_t launch_uncount_after(hipStream_t stream, const ScratchView& sc, const
 
 hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc) {
     const uint32_t words = (sc.vocab + 31u) / 32u;
+    hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, stream, sc.touched + words, 1u, 0u);
     hipLaunchKernelGGL(k_touch_from_counts, dim3((words + 255) / 256), dim3(256), 0, stream, sc);
     return hipGetLastError();
 }

@@ -22,14 +22,19 @@ namespace lily {
 //     chunk (16 raw bytes + its index) to its wave's queue and leaves it out of the running
 //     sum of exponentials; all other chunks only feed the lane maximum and the sum.
 //   * Listed ids (ids a scratch ever counted: their true value differs from the raw one) are
-//     bits of the scratch's bitmap.  Each wave reads the words that cover its own chunks of a
-//     block (64 bytes per load of 64 bf16 chunks), so a lane knows which of its elements are
-//     listed without anybody gathering anything.  When penalties can only lower a value, a
-//     listed element matters only if its chunk is queued (it is then evaluated exactly when the
-//     queue is expanded, its count gathered from the dense histogram) or summed (its raw term
-//     is booked and its true term added on the spot); otherwise every listed element is
-//     evaluated on the spot.  Barred ids of a masked row are bits of the same kind and are
-//     replaced by -inf as the chunk arrives.
+//     bits of the scratch's bitmap.  Where a row needs them beside its chunks, each wave reads
+//     the words that cover its own chunks of a block (64 bytes per load of 64 bf16 chunks), so
+//     a lane knows which of its elements are listed without anybody gathering anything.  When
+//     penalties can only lower a value, a listed element matters only if its chunk is queued
+//     (it is then evaluated exactly when the queue is expanded, its count gathered from the
+//     dense histogram) or summed (its raw term is booked and its true term added); otherwise
+//     every listed element is evaluated on the spot.  Which rows read bits during the scan and
+//     which look them up afterwards is described where the scan's modes are chosen.  Barred
+//     ids of a masked row are bits of the same kind and are replaced by -inf as the chunk
+//     arrives.
+//   * The sum's cut is measured against a lower bound of the row's largest TRUE value: with
+//     penalties that only lower, the image of the largest raw value under the penalty an id
+//     with the scratch's largest count would get.
 //   * The bias list's ids (at most STREAM_BIAS_CAP) are streamed as they are; after the scan
 //     one thread per id looks its chunk up again, redoes the owner's tests with the bound and
 //     the cut its block was scanned with, books the raw term and offers the true value.
@@ -43,7 +48,7 @@ namespace lily {
 struct StreamLds {
     u32x4* qraw;
     uint32_t* qidx;
-    uint8_t* qbits;     // per queue slot: bit j set = element j is a listed id
+    uint16_t* noted;    // [NWAVE][S_CAP / NWAVE] numbers (within the slice) of summed chunks
     uint32_t* win;      // [NWAVE][2][WIN_WORDS]
     float* blk_bound;   // [MAX_BLOCKS] the bound block b was filtered with
     float* blk_cut;     // [MAX_BLOCKS] the sum's cut of block b
@@ -55,7 +60,7 @@ struct StreamLds {
         char* b = reinterpret_cast<char*>(dyn_lds);
         qraw = reinterpret_cast<u32x4*>(b + OFF_QRAW);
         qidx = reinterpret_cast<uint32_t*>(b + OFF_QIDX);
-        qbits = reinterpret_cast<uint8_t*>(b + OFF_QBITS);
+        noted = reinterpret_cast<uint16_t*>(b + OFF_NOTED);
         win = reinterpret_cast<uint32_t*>(b + OFF_WIN);
         blk_bound = reinterpret_cast<float*>(b + OFF_BLK);
         blk_cut = reinterpret_cast<float*>(b + OFF_BLK + MAX_BLOCKS * 4);
@@ -116,6 +121,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     constexpr int U = STREAM_UNROLL;
     constexpr uint32_t BLOCK = NT * U;
     constexpr uint32_t QSEG = Q_CAP / NWAVE;
+    constexpr uint32_t SSEG = S_CAP / NWAVE;
     constexpr uint32_t NONE = 0xffffffffu;
     constexpr uint32_t EMASK = (1u << E) - 1u;
     constexpr uint32_t WPP = 64u * E / 32u;   // bitmap words that hold the bits of a wave's 64 chunks
@@ -161,6 +167,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     if (tid == 0) {
         sh.n_fc = 0;
         sh.fail = 0;
+        sh.n_hits = 0;
     }
     for (uint32_t i = tid; i < n_bias; i += NT) {
         L.bias_id[i] = gload(&a.bias[i].id);
@@ -187,15 +194,35 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             n_allowed += sh.red_i[i];
         }
         __syncthreads();
-        if (n_allowed <= min(cfg.dyn_slots, MERGE_CAP)) {
+        if (n_allowed <= min(cfg.dyn_slots, MERGE_CAP) && n_allowed <= (g.id_hi - g.id_lo) / 4u) {
             return false;  // not a failure: the sparse select takes the row
         }
     }
     // Penalties with a repetition factor of at least 1 and non-negative presence and frequency
     // terms can only lower a value.  `lowering`: no listed id's true value exceeds its raw one
     // (ids the bias list names are dealt with apart, after the scan, listed or not).
-    const bool special = pen || masked;   // the row's chunks come with bits
     const bool lowering = a.repetition >= 1.0f && a.presence >= 0.0f && a.frequency >= 0.0f;
+    // How a row's chunks are scanned:
+    //   * without bits (mode 0): rows without penalties or masks, and rows whose listed ids can
+    //     only be lowered and that want no row sum - a listed id then matters in queued chunks
+    //     only, and the expansion looks their bits up itself;
+    //   * with bits (mode 1): every block's bits arrive beside its values - masked rows, rows
+    //     whose listed ids may rise, rows with a row sum and listed ids.  A chunk above the sum's
+    //     cut is summed as it arrives and the listed ids among its elements corrected on the spot;
+    //   * noting (mode 2), for rows with a row sum whose listed ids can only be lowered (no
+    //     mask, no bias list): scanned without bits.  A chunk above the cut is summed as it is
+    //     and its number noted in a list (16 bits an entry, a segment per wave); after the scan
+    //     one thread per entry looks the chunk's bits up and, for the few chunks that hold a
+    //     listed id, takes the raw term off and adds the true one.  Rows with a dominant value
+    //     note a few dozen chunks, or a few hundred before that value has been seen.  A flat row
+    //     fills its list within a few blocks: the refresh of the bound that finds a segment
+    //     three quarters full hands the blocks after the current one to mode 1 (chunks that a
+    //     full segment cannot note are corrected on the spot from bits fetched there and then).
+    const bool noting = pen && lowering && want_lse && !masked && n_bias == 0u;
+    const bool special = masked || (pen && (!lowering || want_lse));
+    // The largest count any id of the scratch ever had (kept in the first spare word behind
+    // the bitmap) bounds how far penalties can lower a value.
+    const uint32_t max_count = pen ? *(const LILY_CONST uint32_t*)(a.touched + row_words) : 0u;
     // Whether id is named by the bias list (its true value then comes from the pass after the scan).
     auto biased = [&](uint32_t id) -> bool {
         bool hit = false;
@@ -233,12 +260,16 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     const uint32_t keff = min(k + k / 8u + 2u, 64u * NWAVE);
     const uint32_t kw = (keff + NWAVE - 1) / NWAVE;
     float lane_max = NEG_INF;
-    float clean_max = NEG_INF;  // this lane's largest chunk maximum among chunks without a listed id
     float T = F32_LOWEST;       // the block's bound, the same in every thread
     float ref_s = 0.0f;         // reference of the double sums
     float row_max = NEG_INF;    // lower bound of the row's largest true value, as of the last refresh
     float skip_b = NEG_INF;     // the block's cut: chunks whose maximum is not above it are not summed
     uint32_t wq = 0;            // this wave's queue fill
+    bool give_up = false;       // a wave's queue segment overflowed (the same in every thread)
+    bool stop = false;          // mode 2 ends with block `resume` - 1 (the same in every thread)
+    uint32_t resume = 0;
+    uint32_t sfill = 0;         // this wave's noted chunks
+    uint32_t note_max = 0;      // the fullest segment of noted chunks, as of the last refresh
     WaveLse wl;
     wl.init();
     double acc_t = 0.0, acc_r = 0.0;   // true terms added one by one; raw terms to take off
@@ -283,19 +314,13 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t key16 = lane_max > NEG_INF ? (lilym_order_key(lane_max) >> 16) : 0u;
         const uint32_t P = wave_kth_key16(key16, kw);
         const float mine = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
-        float wm[2] = {0.0f, 0.0f};
-        if (maxima) {
-            wm[0] = wave_max_dpp(lane_max);
-            if (want_lse && special) {
-                wm[1] = wave_max_dpp(clean_max);
-            }
-        }
+        const float wm = maxima ? wave_max_dpp(lane_max) : 0.0f;
         if (lane == 0) {
             sh.bound[parity][w] = mine;
+            sh.wfill[parity][w] = wq;
+            sh.wnote[parity][w] = sfill;
             if (maxima) {
-                for (int q = 0; q < 2; ++q) {
-                    sh.wmax[parity][q][w] = wm[q];
-                }
+                sh.wmax[parity][w] = wm;
             }
         }
         __syncthreads();
@@ -304,20 +329,33 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             t = fminf(t, sh.bound[parity][i]);
         }
         T = fmaxf(T, lower_by_slack(t));
+        // A wave's queue segment is full: the row gives up at once (every thread sees it).
+        note_max = 0;
+        for (int i = 0; i < NWAVE; ++i) {
+            give_up = give_up || sh.wfill[parity][i] > QSEG;
+            note_max = max(note_max, sh.wnote[parity][i]);
+        }
         if (maxima) {
-            float m[2];
-            for (int q = 0; q < 2; ++q) {
-                m[q] = sh.wmax[parity][q][0];
-                for (int i = 1; i < NWAVE; ++i) {
-                    m[q] = fmaxf(m[q], sh.wmax[parity][q][i]);
-                }
+            float m = sh.wmax[parity][0];
+            for (int i = 1; i < NWAVE; ++i) {
+                m = fmaxf(m, sh.wmax[parity][i]);
             }
-            // A lower bound of the row's largest TRUE value: the largest raw value of the
-            // chunks that hold no listed id (a row where every chunk holds one skips nothing).
-            row_max = special ? m[1] : m[0];
+            // A lower bound of the row's largest TRUE value.  The largest raw value may belong
+            // to a listed id: penalties that can only lower take at most what they take from an
+            // id with the scratch's largest count, and that map is monotone, so the image of the
+            // largest raw value bounds the largest true value from below.  (Barred ids are -inf
+            // before any maximum is taken; bias ids are few and only the sum's cut depends on
+            // this bound, so a positive bias on the row's best id merely cuts less.)  Listed
+            // ids that may rise leave the raw maximum as it is.
+            row_max = m;
+            if (pen && lowering && m > NEG_INF) {
+                float t = m > 0.0f ? m / a.repetition : m * a.repetition;
+                t -= a.presence + a.frequency * (float)max_count;
+                row_max = t;
+            }
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
-                ref_s = m[0] > NEG_INF ? fminf(fmaxf(m[0] * c2, -1.0e30f), 1.0e30f) : 0.0f;
+                ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
             }
         }
         parity ^= 1u;
@@ -366,15 +404,18 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     };
     const uint32_t* t_words = pen ? a.touched : reinterpret_cast<const uint32_t*>(g.base);
     const uint32_t* m_words = masked ? a.allow : reinterpret_cast<const uint32_t*>(g.base);
-    auto piece_word0 = [&](uint32_t b, uint32_t u) -> int32_t {
-        const int32_t first = (int32_t)((g.cb + b * BLOCK + u * NT + w * 64u) * (uint32_t)E) - (int32_t)g.pad;
+    auto piece_word0 = [&](uint32_t u) -> int32_t {   // in block 0
+        const int32_t first = (int32_t)((g.cb + u * NT + w * 64u) * (uint32_t)E) - (int32_t)g.pad;
         return first >> 5;  // arithmetic: ids before the row lie in "word -1"
     };
+    // This lane's two words of block 0's window; a block's chunks cover BLOCK * E / 32 words.
+    const int32_t win_w0 = piece_word0(min(lane / WPP, 3u)) + (int32_t)(lane % WPP);
+    const int32_t win_w1 = piece_word0(lane & 3u) + (int32_t)WPP;
+    const int32_t win_hi = (int32_t)row_words - 1;
     auto bits_request = [&](Bits& d, uint32_t b) {
-        const uint32_t u = min(lane / WPP, 3u), q = lane % WPP;
-        const int32_t hi = (int32_t)row_words - 1;
-        const uint32_t i0 = (uint32_t)min(max(piece_word0(b, u) + (int32_t)q, 0), hi);
-        const uint32_t i1 = (uint32_t)min(max(piece_word0(b, lane & 3u) + (int32_t)WPP, 0), hi);
+        const int32_t step = (int32_t)(b * (BLOCK * (uint32_t)E / 32u));
+        const uint32_t i0 = (uint32_t)min(max(win_w0 + step, 0), win_hi);
+        const uint32_t i1 = (uint32_t)min(max(win_w1 + step, 0), win_hi);
         d.t = gload(t_words + i0);
         d.tx = gload(t_words + i1);
         if (MASKS) {
@@ -468,10 +509,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // The scan is compiled twice, for rows whose chunks come with bits and for rows without:
     // left as a test inside the loop, the bits' loads would be loads that may be skipped, and
     // every wait behind them would drain the blocks requested ahead.
-    auto scan = [&](auto with_bits) {
+    auto scan = [&](auto with_bits, auto queueing, uint32_t b_first) {
         constexpr bool SP = decltype(with_bits)::value;
+        constexpr bool QM = LSE && decltype(queueing)::value;   // mode 2
         Bits bits_a = {}, bits_b = {}, bits_c = {};
         auto work = [&](u32x4 (&cur)[U], const Bits& bcur, uint32_t b) {
+            if (give_up || stop) {
+                return;
+            }
             // tb_all: a byte per chunk of the block, bit j = element j is a listed id.
             uint32_t tb_all = 0u, mb[U] = {0u, 0u, 0u, 0u};
             if (SP) {
@@ -524,15 +569,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 }
                 lane_max = max2_raw(lane_max, block_max);
             }
-            if (SP && LSE && want_lse && __ballot(block_max > row_max) != 0ull) {
-                // Only a chunk above the largest value known so far can raise it (rare after the
-                // first blocks).  (The cheaper maximum is exact only where it is positive.)
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const bool clean = ((tb_all >> (8 * u)) & 0xffu) == 0u && (!nonneg || m8[u] > 0.0f);
-                    clean_max = fmaxf(clean_max, clean ? m8[u] : NEG_INF);
-                }
-            }
             // Rows with a row sum whose listed ids may rise: a chunk that holds a listed id is
             // queued whatever its values (the queue's expansion evaluates every element exactly).
             uint32_t forced = 0u;   // bit u: chunk u is queued for its listed ids
@@ -542,6 +578,32 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     forced |= ((tb_all >> (8 * u)) & 0xffu) != 0u ? 1u << u : 0u;
                 }
             }
+            // Mode 2: the lanes whose chunk u was just summed note its number; a lane whose
+            // wave's segment is full has the chunk's bits fetched here instead (`fix`).
+            uint32_t fix = 0u;   // a byte per chunk: its listed ids that are evaluated on the spot
+            auto note_summed = [&](int u, bool summed) {
+                const uint64_t mask = __ballot(summed);
+                if (mask != 0ull) {
+                    const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+                        (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                    const uint32_t at = sfill + rank;
+                    if (summed && at < SSEG) {
+                        L.noted[w * SSEG + at] = (uint16_t)((b * U + (uint32_t)u) * NT + tid);
+                    }
+                    if (sfill + (uint32_t)__popcll(mask) > SSEG) {
+                        uint32_t dm = 0u;
+                        if (summed && at >= SSEG) {
+                            const uint32_t c = g.cb + (b * U + (uint32_t)u) * NT + tid;
+                            dm = bits32_at(a.touched, row_words, (int64_t)g.id_of(c, 0)) & EMASK;
+                            // Waited for inside the branch: waiting behind it would make every
+                            // wave drain the loads it has in flight, not just these.
+                            asm volatile("" : "+v"(dm));
+                        }
+                        fix |= dm << (8 * u);
+                    }
+                    sfill = min(sfill + (uint32_t)__popcll(mask), SSEG);
+                }
+            };
             if (LSE && want_lse) {
                 // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
                 // sum by more than 2^-21 of it, even with every element of the row at that level:
@@ -553,8 +615,11 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
-                        wl.template add_prepared<DT>(cur[u], m8[u], c2,
-                                                     !(m8[u] >= T_prev) && ((forced >> u) & 1u) == 0u);
+                        const bool sum_it = !(m8[u] >= T_prev) && ((forced >> u) & 1u) == 0u;
+                        wl.template add_prepared<DT>(cur[u], m8[u], c2, sum_it);
+                        if (QM) {
+                            note_summed(u, sum_it && m8[u] > skip_b);
+                        }
                     }
                 }
             }
@@ -571,6 +636,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     skip_b = row_max - lse_cut;
                     wl.skip_below = skip_b;
                 }
+                if (QM && note_max >= SSEG * 3u / 4u) {
+                    stop = true;
+                    resume = b + 1u;   // this block is still finished here
+                }
             }
             if (n_bias != 0u && tid == 0) {
                 L.blk_bound[b] = T;
@@ -583,7 +652,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // summed is below the bound and below the sum's cut with its true value too: nothing
             // of it is evaluated (most chunks of most rows; rows with a dominant value sum next
             // to nothing, and their waves skip even the test).
-            uint32_t fix = 0u;   // a byte per chunk: its listed ids that are evaluated on the spot
             const bool fix_any = SP && (!lowering || (LSE && want_lse && __ballot(block_max > skip_b) != 0ull));
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -597,7 +665,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     if (pass && at < QSEG) {
                         L.qraw[w * QSEG + at] = cur[u];
                         L.qidx[w * QSEG + at] = c;
-                        L.qbits[w * QSEG + at] = (uint8_t)(tb_all >> (8 * u));
                     }
                     wq += (uint32_t)__popcll(mask);
                 }
@@ -607,6 +674,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     if (__ballot(late) != 0ull) {
                         wl.prepare(late ? m8[u] : NEG_INF, c2);
                         wl.template add_prepared<DT>(cur[u], m8[u], c2, late);
+                        if (QM) {
+                            note_summed(u, late && m8[u] > skip_b);
+                        }
                     }
                 }
                 if (SP && fix_any) {
@@ -615,7 +685,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     fix |= (tb != 0u && !pass && matters) ? tb << (8 * u) : 0u;
                 }
             }
-            if (SP && fix != 0u) {
+            if ((SP || QM) && fix != 0u) {
                 fix_listed(cur, b, fix);
             }
         };
@@ -632,12 +702,15 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         };
         if (nblocks == 0) {
             refresh_bound(true, true);  // the same barriers in every workgroup
-        } else {
-            if (SP) {
-                bits_request(bits_a, 0);
+        } else if (b_first < nblocks) {
+            if (b_first != 0u) {
+                fetch(buf_a, b_first);   // (block 0 was requested at the very start)
             }
-            request(buf_b, bits_b, 1);
-            for (uint32_t b = 0; b < nblocks; b += 3) {
+            if (SP) {
+                bits_request(bits_a, b_first);
+            }
+            request(buf_b, bits_b, b_first + 1u);
+            for (uint32_t b = b_first; b < nblocks && !give_up && !stop; b += 3) {
                 request(buf_c, bits_c, b + 2);
                 work(buf_a, bits_a, b);
                 if (b + 1 < nblocks) {
@@ -651,21 +724,28 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             }
         }
     };
-    if (special) {
-        scan(std::true_type{});
+    if (noting) {
+        scan(std::false_type{}, std::true_type{}, 0u);
+        if (stop && !give_up) {
+            stop = false;
+            scan(std::true_type{}, std::false_type{}, resume);
+        }
+    } else if (special) {
+        scan(std::true_type{}, std::false_type{}, 0u);
     } else {
-        scan(std::false_type{});
+        scan(std::false_type{}, std::false_type{}, 0u);
     }
     phase(cfg, 2);
 
     // ---- after the scan
     if (lane == 0) {
         sh.qfill[w] = wq;
+        sh.nfill[w] = sfill;
     }
     __syncthreads();
     const float filt = T;
     {
-        bool overflow = false;
+        bool overflow = give_up;
         for (int i = 0; i < NWAVE; ++i) {
             overflow = overflow || sh.qfill[i] > QSEG;
         }
@@ -714,7 +794,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             const uint32_t slot = ww * QSEG + (ch - before);
             const u32x4 q = L.qraw[slot];
             const uint32_t c = L.qidx[slot];
-            const uint32_t dm = L.qbits[slot];
+            // Its listed elements, from the scratch's bitmap (barred ids are -inf already).
+            const uint32_t dm =
+                pen ? bits32_at(a.touched, row_words, (int64_t)g.id_of(c, 0)) & EMASK : 0u;
             float v[E];
             unpack<DT>(q, v);
             // Few elements of a queued chunk matter (usually the one that got it queued):
@@ -746,6 +828,79 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 }
                 offer(x, id);
             }
+        }
+    }
+    if (LSE && noting) {
+        // One thread per noted chunk: all of its elements went into the running sum with their
+        // raw values.  For the few that hold a listed id, that id's raw term is booked and its
+        // true term (above the final cut) added.
+        uint32_t seg_end[NWAVE], total = 0;
+#pragma unroll
+        for (int i = 0; i < NWAVE; ++i) {
+            total += sh.nfill[i];
+            seg_end[i] = total;
+        }
+        // First the chunks' bits, four entries per thread at a time (their loads in flight
+        // together); the chunks that hold a listed id are gathered in the queue's memory, which
+        // the expansion above has left.
+        uint32_t* hits = reinterpret_cast<uint32_t*>(L.qraw);
+        constexpr uint32_t HIT_CAP = Q_CAP * 4u;
+        auto chunk_at = [&](uint32_t e) -> uint32_t {
+            uint32_t ww = 0, before = 0;
+#pragma unroll
+            for (int i = 0; i + 1 < NWAVE; ++i) {
+                if (e >= seg_end[i]) {
+                    ww = (uint32_t)i + 1u;
+                    before = seg_end[i];
+                }
+            }
+            return (uint32_t)L.noted[ww * SSEG + (e - before)];
+        };
+        auto fix_chunk = [&](uint32_t c, uint32_t dm) {
+            const u32x4 q = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
+            while (dm != 0u) {
+                const uint32_t j = (uint32_t)__builtin_ctz(dm);
+                dm &= dm - 1u;
+                const float raw = elem_of(q, j);
+                if (!(raw > NEG_INF)) {
+                    continue;
+                }
+                const float t = true_value(g.id_of(c, (int)j), raw);
+                acc_r += term_d(raw);
+                if (t > skip_b) {
+                    acc_t += term_d(t);
+                }
+            }
+        };
+        __syncthreads();   // (the expansion's reads of the queue are over)
+        for (uint32_t e0 = tid; e0 < total; e0 += 4u * NT) {
+            uint32_t rel[4], dm[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t e = e0 + (uint32_t)i * NT;
+                rel[i] = chunk_at(min(e, total - 1u));
+                dm[i] = bits32_at(a.touched, row_words, (int64_t)g.id_of(g.cb + rel[i], 0)) & EMASK;
+                // (A chunk outside the slice was scanned as -inf throughout, and may have been
+                // "summed" where chunk maxima are the kind that reports +0 for it.)
+                const uint32_t c = g.cb + rel[i];
+                dm[i] = e < total && c >= g.main_lo && c < g.main_hi ? dm[i] : 0u;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (dm[i] != 0u) {
+                    const uint32_t at = atomicAdd(&sh.n_hits, 1u);
+                    if (at < HIT_CAP) {
+                        hits[at] = rel[i] | (dm[i] << 16);
+                    } else {
+                        fix_chunk(g.cb + rel[i], dm[i]);   // (nearly every chunk holds a listed id)
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const uint32_t n_hits = min(sh.n_hits, HIT_CAP);
+        for (uint32_t h = tid; h < n_hits; h += NT) {
+            fix_chunk(g.cb + (hits[h] & 0xffffu), hits[h] >> 16);
         }
     }
     phase(cfg, 8);
@@ -855,8 +1010,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         // one by one.
         const double streamed = part[0], booked = part[1], exact = part[2], taken = part[3];
         const double rest = streamed - booked;
-        // Listed ids held nearly all of what was streamed: the difference is too coarse.
-        const bool coarse = booked + taken > 0.0 && !(rest > 0.05 * (streamed + taken));
+        // The streamed sums are f32: taking the listed ids' raw terms off again leaves an error of
+        // about 1e-6 of what was streamed.  Where that is more than 20 times the row's sum (listed
+        // ids held nearly everything that was streamed, and nothing larger was added exactly) the
+        // difference is too coarse.
+        const bool coarse = booked + taken > 0.0 &&
+                            !((rest > 0.0 ? rest : 0.0) + exact > 0.05 * (streamed + taken));
         phase(cfg, 10);
         if (coarse) {
             phase(cfg, 11);

@@ -136,13 +136,20 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
 
 // ------------------------------------------------------------------ tail
 
-// Counts one emission of `id` in a scratch: the dense count, and the id's bit in the bitmap of
-// the ids that were ever counted.
-__device__ __forceinline__ void emit(const RowArgs& a, uint32_t id) {
+// Counts one emission of `id` in a scratch: the dense count, the id's bit in the bitmap of the
+// ids that were ever counted, and the largest count any id has reached (the first spare word
+// behind the bitmap).  Returns the count before.
+__device__ __forceinline__ uint32_t count_token(const RowArgs& a, uint32_t id, uint32_t vocab) {
+    const uint32_t before = atomicAdd(&a.counts[id], 1u);
+    atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
+    atomicMax(&a.touched[(vocab + 31u) / 32u], before + 1u);
+    return before;
+}
+
+__device__ __forceinline__ void emit(const RowArgs& a, uint32_t id, uint32_t vocab) {
     *a.out_id = id;
-    if (a.flags & F_PEN) {
-        atomicAdd(&a.counts[id], 1u);
-        atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
+    if ((a.flags & F_PEN) && id < vocab) {
+        count_token(a, id, vocab);
     }
 }
 
@@ -174,8 +181,7 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
     }
     uint32_t before = 0;
     if (pen) {
-        before = atomicAdd(&a.counts[id], 1u);
-        atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
+        before = count_token(a, id, vocab);
     }
     if (want) {
         const float l = load_logit<DT>(a.logits, id);
@@ -206,7 +212,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             if (a.out_logprob) {
                 *a.out_logprob = NEG_INF;
             }
-            emit(a, 0);
+            emit(a, 0, vocab);
             if (a.dbg_counts) {
                 a.dbg_counts[0] = 0;
                 a.dbg_counts[1] = 1;  // the reference keeps rank 0 whatever its value
