@@ -21,9 +21,19 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "lily-qwen3.8-flash-next_amd", "python"))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per 1024-row launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised
-# in profiles/k_rows_table_bf16_config5_b1024.md (valid for --rows 1024 only).
-MEASURED_TRAFFIC_BYTES = 333.7e6
+# HBM bytes per 1024-row launch come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# very command, summarised in this file (a line "traffic_bytes_per_launch: N"; 1024 rows only).
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "k_rows_table_bf16_config5_b1024.md")
+
+
+def measured_traffic(rows):
+    """Bytes per launch from the committed counter summary, or None (other sizes, no summary)."""
+    if rows != 1024 or not os.path.exists(TRAFFIC_SUMMARY):
+        return None
+    for line in open(TRAFFIC_SUMMARY):
+        if line.startswith("traffic_bytes_per_launch:"):
+            return float(line.split(":", 1)[1])
+    return None
 
 
 def parse():
@@ -58,6 +68,19 @@ def time_steps(stream, fn, steps, warmup):
     stop.synchronize()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
+
+
+def paths_of(sampler, fn):
+    """Which selects served one more (untimed) run of fn: workgroups by the streaming select, by
+    the sparse / bitmap selects, by the exhaustive select, and the reasons the first gave up."""
+    import torch
+    stats = torch.zeros(4, dtype=torch.int32, device="cuda")
+    sampler.set_path_stats(stats)
+    fn(0)
+    sampler.synchronize()
+    sampler.set_path_stats(None)
+    st = stats.cpu().tolist()
+    return {"streaming": st[0], "sparse_or_bitmap": st[1], "exhaustive": st[2], "gave_up_bits": st[3]}
 
 
 def make_scratches(LS, sampler, history, vocab, device):
@@ -139,7 +162,16 @@ def main():
     achieved = rows * bytes_row / (ms * 1e-3) / 1e9
     ids_host = out_ids.cpu().numpy()
     assert ids_host.min() >= 0 and ids_host.max() < vocab
+    paths5 = paths_of(sampler, lambda i: plan.run(a.warmup + a.steps))
     plan.close()
+    # the reference's call shape at this size: host descriptors packed and uploaded every step
+    ms_call = time_steps(stream, lambda i: sampler.sample_rows(logits, params, [i] * rows, out_ids,
+                                                               scratch=scratches, out_logprobs=out_lp),
+                         max(5, a.steps // 5), 2)
+    # the ceiling of a row-per-workgroup launch of this size: the same rows only read
+    probe_out = torch.zeros(rows, dtype=torch.int32, device=device)
+    ms_read = time_steps(stream, lambda i: sampler.probe_read(logits, probe_out), a.steps, a.warmup)
+    plain_read = rows * vocab * 2 / (ms_read * 1e-3) / 1e9
 
     if a.copy_probe:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=device).normal_()
@@ -159,6 +191,7 @@ def main():
     plan2 = sampler.plan(l2, p2, [0] * 4, o2, scratch=s2)
     ms2 = time_steps(stream, lambda i: plan2.run(i), max(a.steps, 200), max(a.warmup, 20))
     # the reference's call shape: host descriptors every step (lily_sample_rows)
+    paths2 = paths_of(sampler, lambda i: plan2.run(1000))
     ms2_call = time_steps(stream, lambda i: sampler.sample_rows(l2, p2, [i] * 4, o2, scratch=s2),
                           max(a.steps, 200), max(a.warmup, 20))
     bytes2 = 4 * W.algorithmic_bytes_per_row(vocab, 4, history=c2["history"].shape[1])
@@ -213,7 +246,8 @@ def main():
         bytes4 = 64 * W.algorithmic_bytes_per_row(vocab, 2, mask_words=c4["allow"].shape[1], bias_pairs=32,
                                                   logprob=True)
         others["config4_constrained"] = {"us_per_step": us4, "rows": 64,
-                                         "achieved_GBs": bytes4 / (us4 * 1e-6) / 1e9}
+                                         "achieved_GBs": bytes4 / (us4 * 1e-6) / 1e9,
+                                         "paths": paths_of(sampler, lambda i: p4.run(0))}
         p4.close()
 
     line = {
@@ -227,7 +261,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16",
         "data": "synthetic",
         "config": {
             "workload": f"{rows} rows x {vocab} bf16 logits (90% N(0,2^2) + 10% Student-t(3)x4), "
@@ -236,11 +270,14 @@ def main():
             "rows": rows, "vocab": vocab, "logits": "bf16",
         },
         "us_per_step": ms * 1e3,
+        "us_per_step_host_descriptors": ms_call * 1e3,
+        "paths": paths5,
         "decode_b4": {
             "workload": "4 rows x 151936 f32 logits, 8192-id Zipf history, rep 1.05 / pres 0.3 / "
                         "freq 0.2, k 20, p 0.95, min_p 0.05, T 0.6 (BASELINE config 2)",
             "us_per_step": ms2 * 1e3,
             "us_per_step_host_descriptors": ms2_call * 1e3,
+            "paths": paths2,
             "rows_per_s": 4 / (ms2 * 1e-3),
             "achieved_GBs": bytes2 / (ms2 * 1e-3) / 1e9,
             "target_us": 20.0,
@@ -252,7 +289,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES if rows == 1024 else None,
+            "traffic": measured_traffic(rows),
+            "plain_read_GBs": plain_read,
+            "frac_of_plain_read": (rows * vocab * 2 / (ms * 1e-3) / 1e9) / plain_read,
             "kernel": "k_rows_table<bf16, streaming select, log-sum-exp>",
             "bytes_per_row": bytes_row,
         },

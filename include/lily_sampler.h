@@ -121,9 +121,18 @@ int lily_sampler_synchronize(lily_sampler_t* s);
 int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_t capacity_words);
 /* Diagnostics with no counterpart in the reference: while stats_dev (device, u32[4], cleared by
  * the caller) is set, every workgroup of a sampled row adds 1 to [0] when the streaming select
- * (k <= 64, no allow-mask) produced its slice, [1] for the selects of masked rows and of
- * k > 64 (sparse or bitmap), [2] for the exhaustive select.  NULL stops. */
+ * (k <= 64) produced its slice, [1] for the selects of sparsely masked rows and of k > 64
+ * (sparse or bitmap), [2] for the exhaustive select; [3] collects a bit per reason the streaming
+ * select gave a slice up.  NULL stops. */
 int lily_sampler_set_path_stats(lily_sampler_t* s, uint32_t* stats_dev);
+/* Measurement aid with no counterpart in the reference: one launch that only reads `rows` rows of
+ * row_bytes bytes (stride_bytes apart) with the row kernel's shape - a workgroup of 256 threads a
+ * row, 16-byte loads, three blocks requested ahead - and writes each row's largest 32-bit word
+ * (as an unsigned integer, combined with atomicMax) to out_dev[rows].  Its rate is the ceiling a
+ * row-per-workgroup launch of that size can reach on the device.  base_dev 16-byte aligned,
+ * row_bytes and stride_bytes multiples of 16. */
+int lily_probe_read(lily_sampler_t* s, const void* base_dev, uint32_t rows, uint64_t row_bytes,
+                    uint64_t stride_bytes, uint32_t* out_dev);
 /* Workgroups per row the next launch of `rows` rows with candidate count k would use. */
 uint32_t lily_sampler_slices_for(const lily_sampler_t* s, uint32_t rows, uint32_t k, uint32_t vocab,
                                  lily_dtype dtype);

@@ -1023,6 +1023,22 @@ int lily_copy_row_u32(lily_sampler_t* s, const uint32_t* src_dev, uint32_t rows,
     return LILY_OK;
 }
 
+int lily_probe_read(lily_sampler_t* s, const void* base_dev, uint32_t rows, uint64_t row_bytes,
+                    uint64_t stride_bytes, uint32_t* out_dev) {
+    if (s == nullptr || base_dev == nullptr || out_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "probe_read needs base and out");
+    }
+    if (rows == 0 || row_bytes < 16 || row_bytes % 16 != 0 || stride_bytes % 16 != 0 ||
+        stride_bytes < row_bytes || (reinterpret_cast<uintptr_t>(base_dev) & 15u) != 0) {
+        return fail(LILY_ERR_INVALID_ARG,
+                    "probe_read: rows > 0, 16-byte aligned base, row_bytes and stride_bytes multiples "
+                    "of 16 with 16 <= row_bytes <= stride_bytes");
+    }
+    HIP_TRY(hipSetDevice(s->device));
+    HIP_TRY(launch_probe_read(s->stream, base_dev, rows, row_bytes, stride_bytes, out_dev));
+    return LILY_OK;
+}
+
 int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype, uint32_t vocab,
                      uint64_t row_stride, uint32_t m, lily_scratch_t* scratch,
                      const lily_sampling_params* params, uint32_t step0,

@@ -116,6 +116,53 @@ __global__ void k_copy_row_u32(const uint32_t* src, uint32_t* dst, uint32_t word
     dst[i] = src[(size_t)row * words + i];
 }
 
+// The row kernel's access pattern with nothing else: one workgroup of 256 threads per row,
+// 16-byte loads, three blocks of four loads per thread requested ahead, an integer maximum as
+// the only arithmetic.  What this reaches is the ceiling a launch of the same shape can reach.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) k_probe_read(const u32x4* base, uint64_t row_chunks,
+                                                    uint64_t stride_chunks, uint32_t* out) {
+    const u32x4* row = base + (uint64_t)blockIdx.x * stride_chunks;
+    const uint64_t last = row_chunks - 1u;
+    auto fetch = [&](u32x4 (&d)[4], uint64_t b) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint64_t c = b * 1024u + (uint64_t)u * 256u + threadIdx.x;
+            d[u] = row[c < last ? c : last];
+        }
+    };
+    auto fold = [](uint32_t m, const u32x4 (&d)[4]) -> uint32_t {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            m = max(max(m, d[u].x), max(max(d[u].y, d[u].z), d[u].w));
+        }
+        return m;
+    };
+    const uint64_t nblocks = (row_chunks + 1023u) / 1024u;
+    u32x4 a[4], b[4], c[4];
+    uint32_t m = 0;
+    fetch(a, 0);
+    fetch(b, 1 < nblocks ? 1 : nblocks - 1u);
+    for (uint64_t i = 0; i < nblocks; i += 3) {
+        fetch(c, i + 2 < nblocks ? i + 2 : nblocks - 1u);
+        m = fold(m, a);
+        if (i + 1 < nblocks) {
+            fetch(a, i + 3 < nblocks ? i + 3 : nblocks - 1u);
+            m = fold(m, b);
+            if (i + 2 < nblocks) {
+                fetch(b, i + 4 < nblocks ? i + 4 : nblocks - 1u);
+                m = fold(m, c);
+            }
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        m = max(m, (uint32_t)__shfl_xor((int)m, o));
+    }
+    if ((threadIdx.x & 63u) == 0) {
+        atomicMax(out + blockIdx.x, m);
+    }
+}
+
 // ------------------------------------------------------------------ launchers (host)
 
 #define LILY_VARIANT(DT, KIND)                                                                   \
@@ -195,6 +242,13 @@ hipError_t launch_copy_row(hipStream_t stream, const uint32_t* src, uint32_t* ds
                            uint32_t rows, const uint32_t* row_dev) {
     hipLaunchKernelGGL(k_copy_row_u32, dim3((words + 255) / 256), dim3(256), 0, stream, src, dst,
                        words, rows, row_dev);
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_read(hipStream_t stream, const void* base, uint32_t rows, uint64_t row_bytes,
+                             uint64_t stride_bytes, uint32_t* out) {
+    hipLaunchKernelGGL(k_probe_read, dim3(rows), dim3(256), 0, stream,
+                       reinterpret_cast<const u32x4*>(base), row_bytes / 16u, stride_bytes / 16u, out);
     return hipGetLastError();
 }
 

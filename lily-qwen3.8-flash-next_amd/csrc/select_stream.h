@@ -268,6 +268,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     bool give_up = false;       // a wave's queue segment overflowed (the same in every thread)
     bool stop = false;          // mode 2 ends with block `resume` - 1 (the same in every thread)
     uint32_t resume = 0;
+    float own_max = NEG_INF;    // mode 2: what this wave's own lanes bound the row's largest value by
     uint32_t sfill = 0;         // this wave's noted chunks
     uint32_t note_max = 0;      // the fullest segment of noted chunks, as of the last refresh
     WaveLse wl;
@@ -309,6 +310,16 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         return pow2_d(d);
     };
 
+    // What a raw value is worth at least after penalties that can only lower (the penalty of an id
+    // with the scratch's largest count); the value itself for all other rows.
+    auto lowered = [&](float m) -> float {
+        if (pen && lowering && m > NEG_INF) {
+            float t = m > 0.0f ? m / a.repetition : m * a.repetition;
+            t -= a.presence + a.frequency * (float)max_count;
+            return t;
+        }
+        return m;
+    };
     // Brings T up to date with everything the lanes have seen, the current block included.
     auto refresh_bound = [&](bool first, bool maxima) {
         const uint32_t key16 = lane_max > NEG_INF ? (lilym_order_key(lane_max) >> 16) : 0u;
@@ -347,12 +358,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // before any maximum is taken; bias ids are few and only the sum's cut depends on
             // this bound, so a positive bias on the row's best id merely cuts less.)  Listed
             // ids that may rise leave the raw maximum as it is.
-            row_max = m;
-            if (pen && lowering && m > NEG_INF) {
-                float t = m > 0.0f ? m / a.repetition : m * a.repetition;
-                t -= a.presence + a.frequency * (float)max_count;
-                row_max = t;
-            }
+            row_max = lowered(m);
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
                 ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
@@ -608,10 +614,21 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
                 // sum by more than 2^-21 of it, even with every element of the row at that level:
                 // such chunks are left out, by a rule every thread of the block can evaluate.
-                skip_b = row_max - lse_cut;
+                skip_b = fmaxf(row_max, own_max) - lse_cut;
                 wl.skip_below = skip_b;
                 // Rows with a dominant value skip nearly every block as a whole.
-                if (__ballot(block_max > skip_b) != 0ull) {
+                bool some = __ballot(block_max > skip_b) != 0ull;
+                if (QM && some) {
+                    // Between two refreshes of the row's maxima the wave's own lanes may have seen
+                    // more than the row knew then: what they saw bounds the row's largest value
+                    // just as well, and spares a row whose largest value comes late the noting of
+                    // chunk after chunk against a cut that is out of date.
+                    own_max = lowered(wave_max_dpp(lane_max));
+                    skip_b = fmaxf(row_max, own_max) - lse_cut;
+                    wl.skip_below = skip_b;
+                    some = __ballot(block_max > skip_b) != 0ull;
+                }
+                if (some) {
                     wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
@@ -633,7 +650,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     // chunks were held back above for want of a bound) is measured against the
                     // largest value known now.  Terms between the old cut and the new one that
                     // were summed already are as negligible as those that were not.
-                    skip_b = row_max - lse_cut;
+                    skip_b = fmaxf(row_max, own_max) - lse_cut;
                     wl.skip_below = skip_b;
                 }
                 if (QM && note_max >= SSEG * 3u / 4u) {

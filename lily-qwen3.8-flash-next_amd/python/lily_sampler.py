@@ -119,6 +119,7 @@ def _load():
         "lily_sampler_synchronize": [vp],
         "lily_sampler_set_phase_trace": [vp, vp, u64],
         "lily_sampler_set_path_stats": [vp, vp],
+        "lily_probe_read": [vp, vp, C.c_uint32, C.c_uint64, C.c_uint64, vp],
         "lily_scratch_create": [vp, u32, C.POINTER(vp)],
         "lily_scratch_reset_counts": [vp],
         "lily_scratch_uncount": [vp, u32],
@@ -255,6 +256,14 @@ class Sampler:
         self._stats = stats
         _check(_lib.lily_sampler_set_path_stats(
             self._h, _ptr(stats, torch.int32) if stats is not None else None))
+
+    def probe_read(self, rows_tensor, out):
+        """One read-only launch over a 2-D contiguous device tensor, a workgroup per row; out:
+        int32[rows], cleared by the caller.  See lily_probe_read."""
+        assert rows_tensor.dim() == 2 and rows_tensor.is_contiguous()
+        row_bytes = rows_tensor.shape[1] * rows_tensor.element_size()
+        _check(_lib.lily_probe_read(self._h, C.c_void_p(rows_tensor.data_ptr()), rows_tensor.shape[0],
+                                    row_bytes // 16 * 16, row_bytes, _ptr(out, torch.int32)))
 
     def slices_for(self, rows, k, vocab, bf16=False):
         return int(_lib.lily_sampler_slices_for(self._h, rows, k, vocab, 1 if bf16 else 0))
