@@ -838,7 +838,7 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
     HIP_TRY(hipMemcpyAsync(dst->counts, src->counts, (size_t)src->vocab * 4, hipMemcpyDeviceToDevice,
                            dst->s->stream));
     // (the bitmap and the largest count behind it)
-    HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)(src->words + 1) * 4,
+    HIP_TRY(hipMemcpyAsync(dst->touched, src->touched, (size_t)(src->words + 2) * 4,
                            hipMemcpyDeviceToDevice, dst->s->stream));
     return LILY_OK;
 }

@@ -15,8 +15,8 @@ __global__ void k_fill_u32(uint32_t* p, uint32_t n, uint32_t v) {
     }
 }
 
-// counts[id] += 1 per occurrence, the id's bit in `touched`, and the largest count reached (the
-// first spare word behind the bitmap).
+// counts[id] += 1 per occurrence, the id's bit in `touched`, the largest count reached (the first
+// spare word behind the bitmap) and an id that reached it (the second; a hint, see tail.h).
 __global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
@@ -24,7 +24,10 @@ __global__ void k_add_history(ScratchView sc, const uint32_t* ids, uint32_t n) {
         if (id < sc.vocab) {
             const uint32_t before = atomicAdd(&sc.counts[id], 1u);
             atomicOr(&sc.touched[id >> 5], 1u << (id & 31u));
-            atomicMax(&sc.touched[(sc.vocab + 31u) / 32u], before + 1u);
+            const uint32_t words = (sc.vocab + 31u) / 32u;
+            if (atomicMax(&sc.touched[words], before + 1u) <= before + 1u) {
+                sc.touched[words + 1u] = id;
+            }
         }
     }
 }
@@ -68,18 +71,21 @@ __global__ void k_touch_from_counts(ScratchView sc) {
     const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t words = (sc.vocab + 31u) / 32u;
     if (w < words) {
-        uint32_t bits = 0, most = 0;
+        uint32_t bits = 0, most = 0, most_id = 0;
         for (uint32_t b = 0; b < 32u; ++b) {
             const uint32_t id = w * 32u + b;
             const uint32_t c = id < sc.vocab ? sc.counts[id] : 0u;
             if (c != 0u) {
                 bits |= 1u << b;
-                most = max(most, c);
+                if (c > most) {
+                    most = c;
+                    most_id = id;
+                }
             }
         }
         sc.touched[w] = bits;
-        if (most != 0u) {
-            atomicMax(&sc.touched[words], most);
+        if (most != 0u && atomicMax(&sc.touched[words], most) <= most) {
+            sc.touched[words + 1u] = most_id;
         }
     }
 }
@@ -225,7 +231,7 @@ hipError_t launch_uncount_after(hipStream_t stream, const ScratchView& sc, const
 
 hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc) {
     const uint32_t words = (sc.vocab + 31u) / 32u;
-    hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, stream, sc.touched + words, 1u, 0u);
+    hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, stream, sc.touched + words, 2u, 0u);
     hipLaunchKernelGGL(k_touch_from_counts, dim3((words + 255) / 256), dim3(256), 0, stream, sc);
     return hipGetLastError();
 }

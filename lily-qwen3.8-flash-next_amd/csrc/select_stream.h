@@ -254,6 +254,19 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
         return t;
     };
+    // Any id's true value bounds the row's largest from below, wherever in the row it lies (in
+    // another slice, too).  One id is worth the look: the one the scratch counted most often.
+    // Where a sequence keeps coming back to a token its raw value is among the row's largest, and
+    // the sum's cut then stands from the first block on, however late the row's largest values
+    // arrive; and no other id's true value is overstated more by the penalty the cut otherwise
+    // assumes (that of the largest count).
+    float row_floor = NEG_INF;
+    if (want_lse && pen && lowering) {
+        const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + row_words + 1u);
+        if (heavy < g.vocab && max_count != 0u && (!masked || bit_of(a.allow, heavy))) {
+            row_floor = true_value(heavy, load_logit<DT>(a.logits, heavy));
+        }
+    }
     phase(cfg, 1);
 
     // ---- scan
@@ -358,7 +371,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // before any maximum is taken; bias ids are few and only the sum's cut depends on
             // this bound, so a positive bias on the row's best id merely cuts less.)  Listed
             // ids that may rise leave the raw maximum as it is.
-            row_max = lowered(m);
+            row_max = fmaxf(lowered(m), row_floor);
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
                 ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;

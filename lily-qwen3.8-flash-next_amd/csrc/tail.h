@@ -137,12 +137,17 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
 // ------------------------------------------------------------------ tail
 
 // Counts one emission of `id` in a scratch: the dense count, the id's bit in the bitmap of the
-// ids that were ever counted, and the largest count any id has reached (the first spare word
-// behind the bitmap).  Returns the count before.
+// ids that were ever counted, the largest count any id has reached (the first spare word behind
+// the bitmap: never lowered, so an upper bound after un-counting) and an id that reached it (the
+// second spare word).  That id is a hint only - writers race, un-counting leaves it alone - and
+// readers take its count from the histogram.  Returns the count before.
 __device__ __forceinline__ uint32_t count_token(const RowArgs& a, uint32_t id, uint32_t vocab) {
     const uint32_t before = atomicAdd(&a.counts[id], 1u);
     atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
-    atomicMax(&a.touched[(vocab + 31u) / 32u], before + 1u);
+    const uint32_t words = (vocab + 31u) / 32u;
+    if (atomicMax(&a.touched[words], before + 1u) <= before + 1u) {
+        a.touched[words + 1u] = id;
+    }
     return before;
 }
 
