@@ -76,10 +76,22 @@ __device__ __forceinline__ float composite_value(uint64_t c) {
 // penalties; the division by the temperature is the caller's.
 __device__ __forceinline__ float finish_pre_temperature(const RowArgs& a, uint32_t id, float l,
                                                         uint32_t c, bool allowed) {
-    for (uint32_t j = 0; j < a.n_bias; ++j) {
-        const uint32_t bid = gload(&a.bias[j].id);
-        if (bid == id) {
-            l += gload(&a.bias[j].delta);
+    // Eight pairs at a time, loaded whatever they hold (a delta that is loaded only on a match
+    // makes every pair a memory round trip of its own); the additions keep the list's order.
+    for (uint32_t j0 = 0; j0 < a.n_bias; j0 += 8u) {
+        uint32_t bid[8];
+        float delta[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t j = min(j0 + (uint32_t)q, a.n_bias - 1u);
+            bid[q] = gload(&a.bias[j].id);
+            delta[q] = gload(&a.bias[j].delta);
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            if (j0 + (uint32_t)q < a.n_bias && bid[q] == id) {
+                l += delta[q];
+            }
         }
     }
     if (!allowed) {
