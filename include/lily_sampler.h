@@ -113,8 +113,8 @@ int lily_sampler_synchronize(lily_sampler_t* s);
 /* Per-kernel profile transport of the reference (LILY_KERNEL_PROFILE, src/metal.rs:30-33,
  * :140-198) at a finer grain: while trace_dev is set, thread 0 of every workgroup of the row
  * kernels stores the 100 MHz device wall clock at up to 16 phase boundaries into
- * trace_dev[(row * slices + slice) * 16 + phase] (u64; 0 start, 1 listed ids bucketed / bitmap
- * built, 2 scan done, 3 sums merged, 4 slice top-k done, 5 ticket taken, 6 slices merged, 7 row
+ * trace_dev[(row * slices + slice) * 16 + phase] (u64; 0 start, 1 scan about to start, 2 scan
+ * done, 3 sums merged, 4 slice top-k done, 5 ticket taken, 6 slices merged, 7 row
  * done; 8-15 finer marks: 8 queue expanded, 9 edge ids done, 10-11 sum merge, 12 candidates
  * ranked, 13-15 inside phase 1).  capacity_words bounds rows * slices * 16; larger launches run
  * untraced.  NULL stops. */
@@ -180,6 +180,10 @@ int lily_draft_dists_slot(const lily_draft_dists_t* d, uint32_t i, lily_draft_di
  * after its last element are read and discarded (never beyond the aligned blocks the row
  * itself occupies).
  *
+ * NaN logits (the reference states no rule: its kernels compare with <, which a NaN never wins;
+ * its CPU twin sorts with total_cmp) are worth -inf in every draw: never a candidate, no term of
+ * the row sum behind a log-probability.  A row that holds one forms that sum by a slower path.
+ *
  * sample_f32 (sample.rs:373-387): one draw from logits_dev[vocab] into out_dev[0].
  * Greedy without penalties is the exact first-max argmax; otherwise penalties,
  * temperature, top-k, top-p/min-p and the inverse-CDF draw on uniform_for(seed, step).
@@ -219,7 +223,10 @@ int lily_sample_spec_f32_uniforms(lily_sampler_t* s, const float* logits_dev, ui
 int lily_sample_f32_static(void* hip_stream, const float* logits_dev, uint32_t vocab,
                            lily_scratch_t* scratch, const lily_sampling_params* params,
                            uint32_t step, uint32_t* out_dev);
-/* argmax_f32 (src/kernels/elementwise.rs:297-308): first max, lowest index on ties. */
+/* argmax_f32 (src/kernels/elementwise.rs:297-308): first max, lowest index on ties.  The
+ * reference's `partials` tensor (ARGMAX_GROUPS * 8 bytes of caller scratch between its two
+ * dispatches) has no counterpart: the partial maxima of a row spread over several workgroups
+ * live in the sampler's own workspace, and the call is one launch. */
 int lily_argmax_f32(lily_sampler_t* s, const float* x_dev, uint32_t n, uint32_t* out_dev);
 
 /* ---- speculative control --------------------------------------------------------------- */

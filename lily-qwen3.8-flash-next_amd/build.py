@@ -56,7 +56,23 @@ def build(verbose=False, jobs=None):
                 sys.stderr.write(err + "\n")
     objs = [os.path.join(OBJ, obj) for _, obj, _ in units()]
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB])
+    build_harness(hipcc)
     return LIB
+
+
+HARNESS_SRC = os.path.join(os.path.dirname(HERE), "tests", "abi_harness", "harness.cpp")
+HARNESS_BIN = os.path.join(os.path.dirname(HERE), "tests", "abi_harness", "harness.bin")
+
+
+def build_harness(hipcc):
+    """The C++ caller of the library that the tests run: host code only, written against the
+    public header, linked against the library by a path relative to the binary."""
+    if not os.path.exists(HARNESS_SRC):
+        return None
+    _run([hipcc, "-O1", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument",
+          "-I", os.path.join(os.path.dirname(HERE), "include"), HARNESS_SRC, "-o", HARNESS_BIN,
+          "-L", HERE, "-llily_sampler_hip", "-Wl,-rpath,$ORIGIN/../../" + os.path.basename(HERE)])
+    return HARNESS_BIN
 
 
 if __name__ == "__main__":

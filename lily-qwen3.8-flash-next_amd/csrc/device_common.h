@@ -734,13 +734,15 @@ struct WaveLse {
 
 // Workgroup-wide merge of per-thread (reference, sum) pairs: returns through `m`, `sum`
 // (double, valid in every thread).
-__device__ __forceinline__ void wg_merge_lse(Shared& sh, float mc, float s_in, double& m_out, double& sum_out) {
+// Returns whether some thread's sum is a NaN (a NaN logit went into it: such a logit is worth
+// -inf, and the caller forms the row's sum again by the path that looks at every value).
+__device__ __forceinline__ bool wg_merge_lse(Shared& sh, float mc, float s_in, double& m_out, double& sum_out) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     float m = wave_max_f(s_in > 0.0f ? mc : NEG_INF);
     if (lane == 0) {
         sh.red_f[w] = m;
     }
-    __syncthreads();
+    const bool poisoned = __syncthreads_or(s_in != s_in ? 1 : 0) != 0;
     m = sh.red_f[0];
     for (int i = 1; i < NWAVE; ++i) {
         m = fmaxf(m, sh.red_f[i]);
@@ -761,6 +763,7 @@ __device__ __forceinline__ void wg_merge_lse(Shared& sh, float mc, float s_in, d
     __syncthreads();
     m_out = (double)m;
     sum_out = t;
+    return poisoned;
 }
 
 template <int DT>

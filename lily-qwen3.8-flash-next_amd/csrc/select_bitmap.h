@@ -443,20 +443,20 @@ __device__ __forceinline__ bool select_fast(const RowArgs& a, const Geo<DT>& g, 
         if (!lse_done) {
             // Row sum = streamed sum - raw terms of the specials (patch) + their true terms.
             double m_s, s_s, m_t, s_t, m_r = 0.0, s_r = 0.0;
-            wg_merge_lse(sh, wl.ref, wl.s, m_s, s_s);
+            bool bad = wg_merge_lse(sh, wl.ref, wl.s, m_s, s_s);   // a NaN logit among the streamed ones
             wg_merge_lse(sh, lse_true.mc, lse_true.s, m_t, s_t);
             if (patch) {
                 wg_merge_lse(sh, lse_raw.mc, lse_raw.s, m_r, s_r);
             }
             double rest = s_s;
-            bool bad = false;
             if (patch && s_r > 0.0) {
                 rest = s_s - s_r * exp2(m_r - m_s);
-                bad = !(rest > 0.05 * s_s);  // cancellation: the streamed sum is too coarse
+                bad = bad || !(rest > 0.05 * s_s);  // cancellation: the streamed sum is too coarse
             }
             if (bad) {
                 phase(cfg, 12);
-                // Rare: penalised ids held nearly all the raw mass.  Redo the sum exactly.
+                // Rare: penalised ids held nearly all the raw mass, or a logit is a NaN.  Redo
+                // the sum exactly.
                 LseAcc exact;
                 exact.init();
                 exact_terms<DT>(a, g.id_lo, g.id_hi, c2, exact);

@@ -578,8 +578,19 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     m8[u] = chunk_max_nonneg<DT>(cur[u]);
                     bm = max(bm, (int)lilym_f32_bits(m8[u]));
                 }
-                block_max = lilym_bits_f32((uint32_t)bm);
-                lane_max = lilym_bits_f32((uint32_t)max((int)lilym_f32_bits(lane_max), bm));
+                if (__ballot(bm > 0x7f800000) != 0ull) {
+                    // A positive NaN among the block's values (its pattern lies above +inf's):
+                    // the block's maxima are taken again the way that ignores NaNs.
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        m8[u] = chunk_max<DT>(cur[u]);
+                        block_max = max2_raw(block_max, m8[u]);
+                    }
+                    lane_max = max2_raw(lane_max, block_max);
+                } else {
+                    block_max = lilym_bits_f32((uint32_t)bm);
+                    lane_max = lilym_bits_f32((uint32_t)max((int)lilym_f32_bits(lane_max), bm));
+                }
             } else {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -955,7 +966,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             if (masked) {
                 q = without(q, ~bits32_at(a.allow, row_words, (int64_t)g.id_of(c, 0)) & EMASK);
             }
-            const float cm = L.blk_flag[b] != 0u ? chunk_max_nonneg<DT>(q) : chunk_max<DT>(q);
+            float cm = L.blk_flag[b] != 0u ? chunk_max_nonneg<DT>(q) : chunk_max<DT>(q);
+            if (lilym_f32_bits(cm) > 0x7f800000u && !(cm < 0.0f)) {
+                cm = chunk_max<DT>(q);   // a NaN in the chunk: as its owner did
+            }
             const float cut = L.blk_cut[b];
             const bool queued = cm >= L.blk_bound[b];
             const bool summed = !queued && cm > cut;
@@ -1019,7 +1033,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (lane == 0) {
             sh.red_i[w] = (uint32_t)ref_w;
         }
-        __syncthreads();
+        // A NaN logit in a summed chunk leaves its wave's running sum a NaN: such a logit is
+        // worth -inf, and the row's sum is formed again from every value.
+        const bool poisoned = __syncthreads_or(wl.s != wl.s ? 1 : 0) != 0;
         int ref_all = (int)sh.red_i[0];
         for (int i = 1; i < NWAVE; ++i) {
             ref_all = max(ref_all, (int)sh.red_i[i]);
@@ -1044,8 +1060,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         // about 1e-6 of what was streamed.  Where that is more than 20 times the row's sum (listed
         // ids held nearly everything that was streamed, and nothing larger was added exactly) the
         // difference is too coarse.
-        const bool coarse = booked + taken > 0.0 &&
-                            !((rest > 0.0 ? rest : 0.0) + exact > 0.05 * (streamed + taken));
+        const bool coarse = poisoned ||
+                            (booked + taken > 0.0 &&
+                             !((rest > 0.0 ? rest : 0.0) + exact > 0.05 * (streamed + taken)));
         phase(cfg, 10);
         if (coarse) {
             phase(cfg, 11);

@@ -1,0 +1,173 @@
+// A caller of liblily_sampler_hip.so written against include/lily_sampler.h alone (plus the HIP
+// runtime for device memory): what a host other than the Python tests sees.
+//
+//   harness cpu              host helpers only (no GPU): prints "cpu ok"
+//   harness gpu V SEED       two draws through lily_sample_f32, two rows through
+//                            lily_sample_rows and the same rows through a plan; prints
+//                            "ids a b c d e f" - the Python side reproduces the inputs and
+//                            checks the ids against the oracle.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "lily_sampler.h"
+
+#define CHECK(x)                                                                          \
+    do {                                                                                  \
+        int rc_ = (x);                                                                    \
+        if (rc_ != 0) {                                                                   \
+            std::fprintf(stderr, "%s -> %d: %s\n", #x, rc_, lily_last_error());            \
+            return 1;                                                                     \
+        }                                                                                 \
+    } while (0)
+#define HIP(x)                                                                            \
+    do {                                                                                  \
+        hipError_t e_ = (x);                                                              \
+        if (e_ != hipSuccess) {                                                           \
+            std::fprintf(stderr, "%s -> %s\n", #x, hipGetErrorString(e_));                 \
+            return 1;                                                                     \
+        }                                                                                 \
+    } while (0)
+
+// The inputs, reproducible anywhere: a 32-bit multiplicative hash of the index.
+static float logit_of(uint32_t i, uint32_t seed) {
+    uint32_t h = (i + 1u) * 2654435761u + seed * 40503u;
+    h ^= h >> 15;
+    h *= 2246822519u;
+    h ^= h >> 13;
+    return (float)(h >> 8) * (16.0f / 16777216.0f) - 8.0f;   // [-8, 8), a multiple of 2^-20
+}
+
+static int cpu_mode() {
+    lily_sampling_params p;
+    lily_params_greedy(&p);
+    if (!lily_params_is_greedy(&p) || lily_params_uses_penalties(&p) || lily_params_validate(&p) != LILY_OK) {
+        std::fprintf(stderr, "greedy defaults\n");
+        return 1;
+    }
+    p.temperature = 0.7f;
+    p.top_k = 5000;
+    p.repetition_penalty = 1.1f;
+    float t = 0.0f;
+    uint32_t k = 0;
+    lily_params_effective(&p, &t, &k);
+    if (t != 0.7f || k != LILY_SAMPLE_K_CAP || !lily_params_uses_penalties(&p)) {
+        std::fprintf(stderr, "effective: %g %u\n", t, k);
+        return 1;
+    }
+    p.top_p = 0.0f;
+    if (lily_params_validate(&p) != LILY_ERR_PARAMS || std::strlen(lily_last_error()) == 0) {
+        std::fprintf(stderr, "top_p 0 must be rejected with a message\n");
+        return 1;
+    }
+    const float u = lily_uniform_for(1234, 7);
+    if (!(u >= 0.0f && u < 1.0f) || lily_uniform_for(1234, 7) != u || lily_uniform_for(1234, 8) == u) {
+        std::fprintf(stderr, "uniform_for\n");
+        return 1;
+    }
+    if (lily_draft_step(5) == 5 || lily_ctrl_words(2) < LILY_CTRL_STRIDE * 2) {
+        std::fprintf(stderr, "draft_step / ctrl_words\n");
+        return 1;
+    }
+    std::printf("cpu ok uniform %.9g draft_step %u ctrl_words %u\n", u, lily_draft_step(5), lily_ctrl_words(2));
+    return 0;
+}
+
+static int gpu_mode(uint32_t vocab, uint32_t seed) {
+    std::vector<float> x(2 * (size_t)vocab);
+    for (uint32_t r = 0; r < 2; ++r) {
+        for (uint32_t i = 0; i < vocab; ++i) {
+            x[(size_t)r * vocab + i] = logit_of(i, seed + r);
+        }
+    }
+    std::vector<uint32_t> hist(512);
+    for (uint32_t i = 0; i < hist.size(); ++i) {
+        hist[i] = (i * 7919u + seed) % vocab;
+    }
+    float* x_dev = nullptr;
+    uint32_t *hist_dev = nullptr, *out_dev = nullptr;
+    HIP(hipSetDevice(0));
+    HIP(hipMalloc((void**)&x_dev, x.size() * 4));
+    HIP(hipMalloc((void**)&hist_dev, hist.size() * 4));
+    HIP(hipMalloc((void**)&out_dev, 8 * 4));
+    HIP(hipMemcpy(x_dev, x.data(), x.size() * 4, hipMemcpyHostToDevice));
+    HIP(hipMemcpy(hist_dev, hist.data(), hist.size() * 4, hipMemcpyHostToDevice));
+    HIP(hipMemset(out_dev, 0xff, 8 * 4));
+
+    hipStream_t stream;
+    HIP(hipStreamCreate(&stream));
+    lily_sampler_t* s = nullptr;
+    CHECK(lily_sampler_create(0, stream, &s));
+    lily_scratch_t* sc[2] = {nullptr, nullptr};
+    for (int r = 0; r < 2; ++r) {
+        CHECK(lily_scratch_create(s, vocab, &sc[r]));
+        CHECK(lily_scratch_add_history(sc[r], hist_dev, (uint32_t)hist.size()));
+    }
+    lily_sampling_params p;
+    lily_params_greedy(&p);
+    p.temperature = 0.9f;
+    p.top_k = 50;
+    p.top_p = 0.95f;
+    p.repetition_penalty = 1.2f;
+    p.presence_penalty = 0.1f;
+    p.frequency_penalty = 0.05f;
+    p.seed = 77;
+    // two draws of the reference's call shape (row 0, steps 0 and 1)
+    CHECK(lily_sample_f32(s, x_dev, vocab, sc[0], &p, 0, out_dev + 0));
+    CHECK(lily_sample_f32(s, x_dev, vocab, sc[0], &p, 1, out_dev + 1));
+    // both rows in one call (steps 2, 2): row 0 sees the two draws above in its counts
+    lily_sampling_params ps[2] = {p, p};
+    ps[1].seed = 78;
+    const uint32_t steps[2] = {2, 2};
+    lily_rows b;
+    std::memset(&b, 0, sizeof b);
+    b.rows = 2;
+    b.vocab = vocab;
+    b.dtype = LILY_F32;
+    b.logits_dev = x_dev;
+    b.row_stride = vocab;
+    b.params = ps;
+    b.steps = steps;
+    b.scratch = sc;
+    b.out_ids_dev = out_dev + 2;
+    CHECK(lily_sample_rows(s, &b));
+    // and once more through a resident plan (steps 2 + 1)
+    lily_plan_t* plan = nullptr;
+    CHECK(lily_plan_create(s, 2, &plan));
+    b.out_ids_dev = out_dev + 4;
+    CHECK(lily_plan_set(plan, &b));
+    CHECK(lily_plan_run(plan, 1));
+    CHECK(lily_sampler_synchronize(s));
+    uint32_t out[8];
+    HIP(hipMemcpy(out, out_dev, sizeof out, hipMemcpyDeviceToHost));
+    std::printf("ids %u %u %u %u %u %u\n", out[0], out[1], out[2], out[3], out[4], out[5]);
+    // a scratch of another vocabulary is refused before anything is enqueued
+    if (lily_sample_f32(s, x_dev, vocab - 1, sc[0], &p, 9, out_dev + 6) != LILY_ERR_VOCAB) {
+        std::fprintf(stderr, "vocab mismatch must be LILY_ERR_VOCAB\n");
+        return 1;
+    }
+    lily_plan_destroy(plan);
+    lily_scratch_destroy(sc[0]);
+    lily_scratch_destroy(sc[1]);
+    lily_sampler_destroy(s);
+    HIP(hipStreamDestroy(stream));
+    HIP(hipFree(x_dev));
+    HIP(hipFree(hist_dev));
+    HIP(hipFree(out_dev));
+    return 0;
+}
+
+int main(int argc, char** argv) {
+    if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) {
+        return cpu_mode();
+    }
+    if (argc >= 4 && std::strcmp(argv[1], "gpu") == 0) {
+        return gpu_mode((uint32_t)std::atoi(argv[2]), (uint32_t)std::atoi(argv[3]));
+    }
+    std::fprintf(stderr, "usage: harness cpu | harness gpu VOCAB SEED\n");
+    return 2;
+}
