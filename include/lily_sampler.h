@@ -287,6 +287,11 @@ typedef struct lily_rows {
     uint32_t* dbg_counts_dev;            /* [rows][2] = candidates, kept */
 } lily_rows;
 
+/* Host cost and waits: the call packs one 192-byte descriptor per row into one of four pinned
+ * staging buffers and enqueues its upload ahead of the launch.  It blocks only (a) when the
+ * upload of the call four calls back has not finished, (b) the first time `rows` exceeds every
+ * earlier call's (beyond 1024): the row table is reallocated, which drains the stream.  A caller
+ * that must never hit (b) mid-run issues one call at its largest batch size first. */
 int lily_sample_rows(lily_sampler_t* s, const lily_rows* batch);
 
 /* A resident batch: the row table is packed and uploaded once (lily_plan_set, which

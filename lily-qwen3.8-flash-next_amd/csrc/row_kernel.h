@@ -193,11 +193,21 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
                 store_through(&cfg.ws_lse[2 * slot + 1], want_lse ? sh.lse_s : 0.0);
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // The hand-over.  Every thread's partials above are device-scope stores that go through
+        // to memory; the barrier orders them before thread 0's increment of the row's ticket,
+        // which releases them to the device; the workgroup that arrives last acquires what the
+        // others released (a fence behind the increment, paid by that workgroup alone), and the
+        // second barrier passes that on to its other threads, whose reads below are device-scope
+        // loads that bypass the caches of their own XCD.  (The release costs the 4-row step
+        // 0.8 us of its 15: the price of not leaning on how the hardware happens to order a
+        // written-through store and a later atomic.)
         __syncthreads();
         if (tid == 0) {
-            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
+            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELEASE,
                                                       __HIP_MEMORY_SCOPE_AGENT);
+            if (t == S - 1) {
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            }
             sh.last = (t == S - 1) ? 1u : 0u;
         }
         __syncthreads();

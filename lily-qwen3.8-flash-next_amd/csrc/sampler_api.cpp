@@ -45,6 +45,32 @@ int hip_fail(hipError_t e, const char* what) {
         }                                  \
     } while (0)
 
+// Makes `device` the calling thread's current device for the rest of the enclosing scope and
+// puts the caller's own choice back on the way out: a library call must not leave the host
+// thread on another GPU than it came with.
+struct DeviceScope {
+    int before = -1;
+    bool switched = false;
+    hipError_t err = hipSuccess;
+    explicit DeviceScope(int device) {
+        err = hipGetDevice(&before);
+        if (err == hipSuccess && before != device) {
+            err = hipSetDevice(device);
+            switched = err == hipSuccess;
+        }
+    }
+    ~DeviceScope() {
+        if (switched) {
+            DeviceScope device_scope_(before);
+        }
+    }
+    DeviceScope(const DeviceScope&) = delete;
+    DeviceScope& operator=(const DeviceScope&) = delete;
+};
+#define ON_DEVICE(device)                 \
+    DeviceScope device_scope_(device);    \
+    HIP_TRY(device_scope_.err)
+
 constexpr uint32_t WS_ROWS = 4096;      // rows that may span several workgroups
 constexpr uint32_t WS_SLOTS = 1u << 22; // candidate slots of the workspace (rows x slices x k)
 constexpr uint32_t STAGE_SLOTS = 4;
@@ -414,7 +440,7 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
 }
 
 int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n) {
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     const uint32_t kmax = max_k(rows.r, n);
     LaunchCfg cfg;
     const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
@@ -461,12 +487,27 @@ int pack_batch(const lily_rows* b, RowArgs* table) {
     const size_t es = b->dtype == LILY_BF16 ? 2 : 4;
     const uint32_t words = (b->vocab + 31u) / 32u;
     if (b->scratch != nullptr) {
+        // No row under penalties may share its scratch with an earlier row: the rows of a launch
+        // run side by side.  Sorted by scratch, sharers are neighbours.
+        static thread_local std::vector<std::pair<uintptr_t, uint32_t>> owners;
+        owners.clear();
         for (uint32_t r = 0; r < b->rows; ++r) {
-            for (uint32_t q = 0; q < r && b->scratch[r] != nullptr; ++q) {
-                if (b->scratch[q] == b->scratch[r] &&
-                    lily_params_uses_penalties(&b->params[r])) {
-                    return fail(LILY_ERR_INVALID_ARG, "rows %u and %u share a scratch", q, r);
-                }
+            if (b->scratch[r] != nullptr) {
+                owners.emplace_back(reinterpret_cast<uintptr_t>(b->scratch[r]), r);
+            }
+        }
+        std::sort(owners.begin(), owners.end());
+        for (size_t i = 1; i < owners.size(); ++i) {
+            if (owners[i].first != owners[i - 1].first) {
+                continue;
+            }
+            size_t first = i - 1;
+            while (first > 0 && owners[first - 1].first == owners[i].first) {
+                --first;
+            }
+            if (lily_params_uses_penalties(&b->params[owners[i].second])) {
+                return fail(LILY_ERR_INVALID_ARG, "rows %u and %u share a scratch", owners[first].second,
+                            owners[i].second);
             }
         }
     }
@@ -665,7 +706,7 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     if (device < 0 || device >= n) {
         return fail(LILY_ERR_RANGE, "device %d of %d", device, n);
     }
-    HIP_TRY(hipSetDevice(device));
+    ON_DEVICE(device);
     lily_sampler* s = new (std::nothrow) lily_sampler;
     if (s == nullptr) {
         return fail(LILY_ERR_NOMEM, "out of host memory");
@@ -703,7 +744,7 @@ void lily_sampler_destroy(lily_sampler_t* s) {
     if (s == nullptr) {
         return;
     }
-    (void)hipSetDevice(s->device);
+    DeviceScope device_scope_(s->device);
     (void)hipStreamSynchronize(s->stream);
     (void)hipFree(s->ws_cand);
     (void)hipFree(s->ws_lse);
@@ -756,7 +797,7 @@ int lily_scratch_create(lily_sampler_t* s, uint32_t vocab, lily_scratch_t** out)
         return fail(LILY_ERR_INVALID_ARG, "scratch needs a sampler and a vocabulary > 0");
     }
     *out = nullptr;
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     lily_scratch* sc = new (std::nothrow) lily_scratch;
     if (sc == nullptr) {
         return fail(LILY_ERR_NOMEM, "out of host memory");
@@ -781,7 +822,7 @@ void lily_scratch_destroy(lily_scratch_t* sc) {
     if (sc == nullptr) {
         return;
     }
-    (void)hipSetDevice(sc->s->device);
+    DeviceScope device_scope_(sc->s->device);
     (void)hipStreamSynchronize(sc->s->stream);
     (void)hipFree(sc->counts);
     delete sc;
@@ -793,7 +834,7 @@ int lily_scratch_reset_counts(lily_scratch_t* sc) {
     if (sc == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "scratch is null");
     }
-    HIP_TRY(hipSetDevice(sc->s->device));
+    ON_DEVICE(sc->s->device);
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->counts, sc->vocab, 0));
     HIP_TRY(launch_fill_u32(sc->s->stream, sc->touched, sc->words + 4, 0));
     return LILY_OK;
@@ -806,7 +847,7 @@ int lily_scratch_uncount(lily_scratch_t* sc, uint32_t token) {
     if (token >= sc->vocab) {
         return LILY_OK;  // sample.rs:149-151
     }
-    HIP_TRY(hipSetDevice(sc->s->device));
+    ON_DEVICE(sc->s->device);
     HIP_TRY(launch_uncount(sc->s->stream, view_of(sc), token));
     return LILY_OK;
 }
@@ -822,7 +863,7 @@ int lily_scratch_uncount_after(lily_scratch_t* sc, const uint32_t* draws_dev, ui
     if (m == 0 || m > LILY_MAX_VERIFY_ROWS) {
         return fail(LILY_ERR_RANGE, "rollback over %u rows (1..%u)", m, (unsigned)LILY_MAX_VERIFY_ROWS);
     }
-    HIP_TRY(hipSetDevice(sc->s->device));
+    ON_DEVICE(sc->s->device);
     HIP_TRY(launch_uncount_after(sc->s->stream, view_of(sc), draws_dev, m, accepted_dev, accepted_cap));
     return LILY_OK;
 }
@@ -834,7 +875,7 @@ int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src
     if (dst->vocab != src->vocab) {
         return fail(LILY_ERR_VOCAB, "sampler scratches for different vocabularies");
     }
-    HIP_TRY(hipSetDevice(dst->s->device));
+    ON_DEVICE(dst->s->device);
     HIP_TRY(hipMemcpyAsync(dst->counts, src->counts, (size_t)src->vocab * 4, hipMemcpyDeviceToDevice,
                            dst->s->stream));
     // (the bitmap and the largest count behind it)
@@ -847,7 +888,7 @@ int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32
     if (sc == nullptr || (ids_dev == nullptr && n != 0)) {
         return fail(LILY_ERR_INVALID_ARG, "scratch or ids is null");
     }
-    HIP_TRY(hipSetDevice(sc->s->device));
+    ON_DEVICE(sc->s->device);
     HIP_TRY(launch_add_history(sc->s->stream, view_of(sc), ids_dev, n));
     return LILY_OK;
 }
@@ -856,7 +897,7 @@ int lily_scratch_write_counts(lily_scratch_t* sc, const uint32_t* host_counts) {
     if (sc == nullptr || host_counts == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "scratch or counts is null");
     }
-    HIP_TRY(hipSetDevice(sc->s->device));
+    ON_DEVICE(sc->s->device);
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     HIP_TRY(hipMemcpy(sc->counts, host_counts, (size_t)sc->vocab * 4, hipMemcpyHostToDevice));
     HIP_TRY(launch_rebuild_listed(sc->s->stream, view_of(sc)));
@@ -868,7 +909,7 @@ int lily_scratch_read_counts(lily_scratch_t* sc, uint32_t* host_counts) {
     if (sc == nullptr || host_counts == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "scratch or counts is null");
     }
-    HIP_TRY(hipSetDevice(sc->s->device));
+    ON_DEVICE(sc->s->device);
     HIP_TRY(hipStreamSynchronize(sc->s->stream));
     HIP_TRY(hipMemcpy(host_counts, sc->counts, (size_t)sc->vocab * 4, hipMemcpyDeviceToHost));
     return LILY_OK;
@@ -881,7 +922,7 @@ int lily_draft_dists_create(lily_sampler_t* s, uint32_t slots, lily_draft_dists_
         return fail(LILY_ERR_INVALID_ARG, "draft dists need a sampler and slots > 0");
     }
     *out = nullptr;
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     lily_draft_dists* d = new (std::nothrow) lily_draft_dists;
     if (d == nullptr) {
         return fail(LILY_ERR_NOMEM, "out of host memory");
@@ -910,7 +951,7 @@ void lily_draft_dists_destroy(lily_draft_dists_t* d) {
     if (d == nullptr) {
         return;
     }
-    (void)hipSetDevice(d->s->device);
+    DeviceScope device_scope_(d->s->device);
     (void)hipStreamSynchronize(d->s->stream);
     (void)hipFree(d->ids);
     delete d;
@@ -1005,7 +1046,7 @@ int lily_spec_accept(lily_sampler_t* s, const uint32_t* draws_dev, const uint32_
     if (ratio == 0) {
         return fail(LILY_ERR_INVALID_ARG, "indexer block ratio must be nonzero");
     }
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     HIP_TRY(launch_spec_accept(s->stream, draws_dev, ids_dev, ctrl_dev, m, pos0, ratio, chain));
     return LILY_OK;
 }
@@ -1018,7 +1059,7 @@ int lily_copy_row_u32(lily_sampler_t* s, const uint32_t* src_dev, uint32_t rows,
     if (rows == 0 || words == 0) {
         return fail(LILY_ERR_INVALID_ARG, "src must be [rows, words] with both > 0");
     }
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     HIP_TRY(launch_copy_row(s->stream, src_dev, dst_dev, words, rows, row_dev));
     return LILY_OK;
 }
@@ -1034,7 +1075,7 @@ int lily_probe_read(lily_sampler_t* s, const void* base_dev, uint32_t rows, uint
                     "probe_read: rows > 0, 16-byte aligned base, row_bytes and stride_bytes multiples "
                     "of 16 with 16 <= row_bytes <= stride_bytes");
     }
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     HIP_TRY(launch_probe_read(s->stream, base_dev, rows, row_bytes, stride_bytes, out_dev));
     return LILY_OK;
 }
@@ -1138,7 +1179,7 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     if (b == nullptr || b->rows == 0) {
         return fail(LILY_ERR_INVALID_ARG, "empty batch");
     }
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     if (int rc = ensure_table(s, b->rows)) {
         return rc;
     }
@@ -1169,7 +1210,7 @@ int lily_plan_create(lily_sampler_t* s, uint32_t max_rows, lily_plan_t** out) {
         return fail(LILY_ERR_INVALID_ARG, "plan needs a sampler and max_rows > 0");
     }
     *out = nullptr;
-    HIP_TRY(hipSetDevice(s->device));
+    ON_DEVICE(s->device);
     lily_plan* p = new (std::nothrow) lily_plan;
     if (p == nullptr) {
         return fail(LILY_ERR_NOMEM, "out of host memory");
@@ -1190,7 +1231,7 @@ void lily_plan_destroy(lily_plan_t* p) {
     if (p == nullptr) {
         return;
     }
-    (void)hipSetDevice(p->s->device);
+    DeviceScope device_scope_(p->s->device);
     (void)hipStreamSynchronize(p->s->stream);
     (void)hipFree(p->table_dev);
     delete p;
@@ -1208,7 +1249,7 @@ int lily_plan_set(lily_plan_t* p, const lily_rows* b) {
         return rc;
     }
     p->n_parts = plan_parts(p->s, table.data(), b->rows, (int)b->dtype, b->vocab, p->parts);
-    HIP_TRY(hipSetDevice(p->s->device));
+    ON_DEVICE(p->s->device);
     HIP_TRY(hipStreamSynchronize(p->s->stream));
     HIP_TRY(hipMemcpy(p->table_dev, table.data(), (size_t)b->rows * sizeof(RowArgs),
                       hipMemcpyHostToDevice));
@@ -1223,7 +1264,7 @@ int lily_plan_run(lily_plan_t* p, uint32_t step_delta) {
     if (p == nullptr || p->rows == 0) {
         return fail(LILY_ERR_INVALID_ARG, "plan is null or not set");
     }
-    HIP_TRY(hipSetDevice(p->s->device));
+    ON_DEVICE(p->s->device);
     for (uint32_t q = 0; q < p->n_parts; ++q) {
         if (int rc = launch_part(p->s, p->parts[q], p->table_dev, (int)p->dtype, p->vocab, step_delta,
                                  q == 0)) {
