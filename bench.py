@@ -213,7 +213,9 @@ def main():
         m3 = c3["target"].shape[0]
         t3 = torch.from_numpy(c3["target"]).to(device)
         d3 = torch.from_numpy(c3["draft"]).to(device)
-        for name, kw in (("config3_verify_greedy", dict()), ("config3_verify_sampled", c3["params"])):
+        for name, kw in (("config3_verify_greedy", dict()), ("config3_verify_sampled", c3["params"]),
+                         ("config3_verify_penalised", dict(c3["params"], presence_penalty=0.4,
+                                                           repetition_penalty=1.1))):
             lp3 = LS.SamplingParams.greedy(**kw)
             sc3 = LS.SamplerScratch(sampler, vocab)
             dists = LS.DraftDists(sampler, m3)

@@ -241,6 +241,13 @@ struct Shared {
     uint32_t nfill[NWAVE];   // chunks each wave noted
     uint32_t n_fc;           // final candidates
     uint32_t n_hits;   // noted chunks found to hold a listed id
+    // rows that draw in order (one launch): what the rows before drew, the count each of those
+    // ids had right after, the proposals the draws are compared with, and the last draw
+    uint32_t drawn[LILY_MAX_VERIFY_ROWS];
+    uint32_t drawn_count[LILY_MAX_VERIFY_ROWS];
+    uint32_t proposal[LILY_MAX_VERIFY_ROWS];
+    uint32_t chain_n[LILY_MAX_VERIFY_ROWS];   // candidates each row published
+    uint32_t emitted_id;
     uint32_t fail;
     double red3[4][NWAVE];
 };

@@ -54,7 +54,9 @@ struct alignas(16) RowArgs {
     float repetition;
     float uniform;
     float uniform2;
-    uint32_t pad[3];
+    uint32_t k_draw;           // rows of a chained launch: the draw's own candidate count (k is
+                               // then what the select collects); 0 otherwise
+    uint32_t pad[2];
 };
 static_assert(sizeof(RowArgs) == 192, "RowArgs layout");
 
@@ -89,8 +91,28 @@ struct LaunchCfg {
     uint32_t bitmap_layout;    // dynamic LDS holds cand_cap candidates + the bitmap + the id list
     uint32_t dyn_slots;     // 64-bit slots of dynamic LDS in all
     uint32_t* path_stats;   // null, or [4] counters: slices finished by the streaming select, the
-                            // bitmap select, the exhaustive select; [3] unused
+                            // bitmap select, the exhaustive select; [3] a bit per reason the
+                            // streaming select gave a slice up
+    // A chained launch (rows that share one scratch and must draw in order, each seeing the
+    // counts the rows before it left): every row's candidates are collected against the counts
+    // as they stood, published here, and the workgroup that finishes last draws row after row.
+    uint32_t chain_rows;    // 0 = the rows are independent
+    uint64_t* chain_cand;   // [chain_rows][CHAIN_CAP]
+    uint32_t* chain_n;      // [chain_rows] candidates published
+    uint32_t* chain_ticket; // [1] rows that have published, left at 0
+    // spec_accept by the same workgroup once the last row has drawn (null: not asked for)
+    uint32_t* accept_ctrl;
+    const uint32_t* accept_ids;   // [chain_rows] the pass's input ids (ids[j + 1] = proposal j)
+    uint32_t accept_pos0;
+    uint32_t accept_ratio;
+    uint32_t accept_chain;
 };
+
+constexpr uint32_t CHAIN_CAP = LILY_SAMPLE_K_CAP;   // candidates a chained row publishes
+// Where the workgroup that draws the rows keeps what it requested ahead: behind the sorted
+// candidates and the tail's three float arrays, 16 bytes for each of a row's first 64 candidates.
+constexpr uint32_t CHAIN_LDS_OFFSET = LILY_SAMPLE_K_CAP * 8 + 3 * LILY_SAMPLE_K_CAP * 4;
+constexpr uint32_t CHAIN_LDS_BYTES = CHAIN_LDS_OFFSET + LILY_MAX_VERIFY_ROWS * 64 * 16;
 
 constexpr uint32_t PHASE_SLOTS = 16;
 

@@ -85,7 +85,9 @@ __device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowAr
     }
 }
 
-template <int DT, int KIND, bool LSE>
+// CHAIN: the kernel of launches whose rows draw in order (compiled apart from the others: what it
+// adds behind the selects would cost every other launch registers).
+template <int DT, int KIND, bool LSE, bool CHAIN = false>
 __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const LaunchCfg& cfg, Shared& sh) {
     RowArgs a;
     load_row_args(a, src);
@@ -313,6 +315,160 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         }
         return;
     }
+    if (CHAIN && cfg.chain_rows != 0u) {
+        // Rows that draw in order.  This row's candidates - the best t.k under the counts as they
+        // stood when the launch began, t.k being the draw's own count plus one for every row
+        // before it - are published; the workgroup that publishes last takes the rows one after
+        // the other: the ids the earlier rows drew are evaluated again (penalties that can only
+        // lower took them down, so the best k_draw of the row as it stands now are still among
+        // the candidates), and the tail draws from the best k_draw.
+        const uint32_t rows = cfg.chain_rows;
+        for (uint32_t i = tid; i < n; i += NT) {
+            store_through(&cfg.chain_cand[(size_t)row * CHAIN_CAP + i], found[i]);
+        }
+        if (tid == 0) {
+            store_through(&cfg.chain_n[row], n);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const uint32_t arrived = __hip_atomic_fetch_add(cfg.chain_ticket, 1u, __ATOMIC_RELEASE,
+                                                            __HIP_MEMORY_SCOPE_AGENT);
+            if (arrived == rows - 1u) {
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            }
+            sh.last = arrived == rows - 1u ? 1u : 0u;
+        }
+        __syncthreads();
+        if (sh.last == 0u) {
+            return;
+        }
+        if (tid == 0) {
+            store_through(cfg.chain_ticket, 0u);
+        }
+        const LILY_CONST RowArgs* first = src - row;
+        if (cfg.accept_ctrl != nullptr && tid < rows) {
+            sh.proposal[tid] = gload(cfg.accept_ids + tid);
+        }
+        // Every row's first 64 candidates, their raw logits and their counts as they stand before
+        // any of these rows has drawn are requested together (a wave per row, two rounds for
+        // eight rows) and kept in LDS behind the tail's arrays: once the rows draw, nothing waits
+        // for memory but the tail's own reads, and the counts the earlier rows left follow from
+        // what they drew.  Candidates past the 64th are loaded when their row's turn comes.
+        constexpr uint32_t PRE = 64;
+        uint64_t* pre_c = dyn_lds + CHAIN_LDS_OFFSET / 8;                           // [rows][PRE]
+        float* pre_l = reinterpret_cast<float*>(pre_c + LILY_MAX_VERIFY_ROWS * PRE);  // [rows][PRE]
+        uint32_t* pre_cnt = reinterpret_cast<uint32_t*>(pre_l + LILY_MAX_VERIFY_ROWS * PRE);
+        for (uint32_t j0 = 0; j0 < rows; j0 += NWAVE) {
+            const uint32_t j = j0 + (tid >> 6), lane = tid & 63u;
+            if (j < rows) {
+                const uint32_t nj = min(load_through(&cfg.chain_n[j]), CHAIN_CAP);
+                if (lane == 0) {
+                    sh.chain_n[j] = nj;
+                }
+                const uint64_t c = load_through(&cfg.chain_cand[(size_t)j * CHAIN_CAP + lane]);
+                const uint32_t id = min(composite_id(c), vocab - 1u);
+                pre_c[j * PRE + lane] = c;
+                pre_l[j * PRE + lane] = load_logit<DT>((first + j)->logits, id);
+                pre_cnt[j * PRE + lane] = (t.flags & F_PEN) ? load_through(t.counts + id) : 0u;
+            }
+        }
+        __syncthreads();
+        for (uint32_t j = 0; j < rows; ++j) {
+            RowArgs r;
+            {
+                const LILY_CONST RowArgs* from = first + j;
+                asm volatile("" : "+s"(from));
+                load_row_args(r, from);
+            }
+            // What an earlier row drew is evaluated again, with the count it has by now.
+            auto times_drawn = [&](uint32_t id) -> uint32_t {
+                uint32_t times = 0;
+                for (uint32_t q = 0; q < j; ++q) {
+                    times += sh.drawn[q] == id ? 1u : 0u;
+                }
+                return times;
+            };
+            auto with_count = [&](uint32_t id, float l, uint32_t cnt) -> uint64_t {
+                const bool allowed = r.allow == nullptr || bit_of(r.allow, id);
+                return composite_of(finish_pre_temperature(r, id, l, cnt, allowed) / r.temperature, id);
+            };
+            const uint32_t n_now = sh.chain_n[j];
+            if (tid < min(n_now, PRE)) {
+                const uint64_t c = pre_c[j * PRE + tid];
+                const uint32_t id = composite_id(c);
+                const uint32_t times = times_drawn(id);
+                cand[tid] = times == 0u ? c : with_count(id, pre_l[j * PRE + tid], pre_cnt[j * PRE + tid] + times);
+            }
+            if (n_now > PRE) {
+                // Past what was requested ahead: the earlier rows' increments are waited for
+                // (thread 0 issued them) and the counts read as they stand.
+                __threadfence();
+                __syncthreads();
+                for (uint32_t i = tid + PRE; i < n_now; i += NT) {
+                    const uint64_t c = load_through(&cfg.chain_cand[(size_t)j * CHAIN_CAP + i]);
+                    const uint32_t id = composite_id(c);
+                    cand[i] = times_drawn(id) == 0u
+                                  ? c
+                                  : with_count(id, load_logit<DT>(r.logits, id), load_through(r.counts + id));
+                }
+            }
+            __syncthreads();
+            // The few candidates that changed are put back in order: up to a workgroup's worth
+            // each thread counts the candidates that beat its own (composites are distinct).
+            bool ranked = false;
+            if (n_now <= NT) {
+                const uint64_t mine = tid < n_now ? cand[tid] : 0ull;
+                uint32_t ahead = 0;
+                for (uint32_t q = 0; q < n_now; ++q) {
+                    ahead += cand[q] > mine ? 1u : 0u;
+                }
+                __syncthreads();
+                if (tid < n_now) {
+                    cand[ahead] = mine;
+                }
+                __syncthreads();
+                ranked = true;
+            }
+            r.k = r.k_draw;
+            tail<DT, KIND != 2>(r, vocab, r.step + cfg.step_delta, n_now, ranked, cand, sh, cfg);
+            __syncthreads();
+            if (tid == 0) {
+                sh.drawn[j] = sh.emitted_id;
+            }
+            __syncthreads();
+        }
+        // The scratch's largest count (and an id that holds it) follow now, once per draw.  It
+        // must never understate a count: thread 0, which issued every increment, waits for them
+        // before anybody reads a count back.
+        __threadfence();
+        __syncthreads();
+        if (tid < rows && (t.flags & F_PEN) && sh.drawn[tid] < vocab) {
+            const uint32_t id = sh.drawn[tid];
+            const uint32_t words = (vocab + 31u) / 32u;
+            const uint32_t now = load_through(t.counts + id);
+            if (atomicMax(&t.touched[words], now) <= now) {
+                t.touched[words + 1u] = id;
+            }
+        }
+        if (cfg.accept_ctrl != nullptr && tid == 0) {
+            // spec_accept (spec.metal:14-38) on the draws this workgroup just made.
+            uint32_t acc = 0;
+            while (acc + 1 < rows && sh.drawn[acc] == sh.proposal[acc + 1]) {
+                ++acc;
+            }
+            uint32_t* ctrl = cfg.accept_ctrl;
+            ctrl[0] = acc;
+            ctrl[LILY_CTRL_STRIDE] = acc + 1;
+            for (uint32_t i = 0; i < cfg.accept_chain; ++i) {
+                const uint32_t p = cfg.accept_pos0 + acc + 1 + i;
+                ctrl[(2 + 3 * i) * LILY_CTRL_STRIDE] = p;
+                ctrl[(3 + 3 * i) * LILY_CTRL_STRIDE] = p / cfg.accept_ratio;
+                ctrl[(4 + 3 * i) * LILY_CTRL_STRIDE] = ((p + 1) % cfg.accept_ratio == 0) ? 1u : 0u;
+            }
+        }
+        phase(cfg, 7);
+        return;
+    }
     tail<DT, KIND != 2>(t, vocab, step, n, sorted, found, sh, cfg);
     phase(cfg, 7);
 }
@@ -341,6 +497,19 @@ __global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_inline(InlineRow
     row_body<DT, KIND, LSE>(table + blockIdx.y, cfg, sh);
 }
 
+// Rows that draw in order (the verify pass under penalties): see row_body.
+template <int DT, int KIND>
+__global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_chain(InlineRows rows, LaunchCfg cfg) {
+    __shared__ Shared sh;
+    const LILY_CONST RowArgs* table =
+        (const LILY_CONST RowArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+    if (threadIdx.x == 0) {
+        tail_arrays(sh);
+    }
+    __syncthreads();
+    row_body<DT, KIND, false, true>(table + blockIdx.y, cfg, sh);
+}
+
 template <int DT, int KIND, bool LSE>
 __global__ __launch_bounds__(NT, KIND == 1 ? 3 : 4) void k_rows_table(LaunchCfg cfg) {
     __shared__ Shared sh;
@@ -356,6 +525,15 @@ template <int DT, int KIND, bool LSE>
 static hipError_t launch_variant(hipStream_t stream, uint32_t rows, const LaunchCfg& cfg,
                                  const InlineRows* inline_rows, size_t dyn_bytes) {
     const dim3 grid(cfg.slices, rows), block(NT);
+    if (cfg.chain_rows != 0u) {
+        if constexpr (!LSE) {
+            if (inline_rows != nullptr) {
+                hipLaunchKernelGGL((k_rows_chain<DT, KIND>), grid, block, dyn_bytes, stream, *inline_rows, cfg);
+                return hipGetLastError();
+            }
+        }
+        return hipErrorInvalidValue;   // rows that draw in order travel inline and want no row sum
+    }
     if (inline_rows != nullptr) {
         hipLaunchKernelGGL((k_rows_inline<DT, KIND, LSE>), grid, block, dyn_bytes, stream,
                            *inline_rows, cfg);

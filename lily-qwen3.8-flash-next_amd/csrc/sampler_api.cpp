@@ -84,6 +84,9 @@ struct lily_sampler {
     uint64_t* ws_cand = nullptr;
     double* ws_lse = nullptr;
     uint32_t* ws_ticket = nullptr;
+    uint64_t* chain_cand = nullptr;   // [LILY_MAX_VERIFY_ROWS][CHAIN_CAP], then the rows' counts and
+    uint32_t* chain_n = nullptr;      // the ticket of a chained launch
+    uint32_t* chain_ticket = nullptr;
     uint32_t ws_rows = WS_ROWS;    // rows that may span several workgroups
     uint32_t ws_slots = WS_SLOTS;  // candidate slots behind ws_cand
     // Row table of lily_sample_rows batches above INLINE_ROWS.
@@ -439,18 +442,38 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
     return LILY_OK;
 }
 
-int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n) {
+// What spec_accept needs when the launch that draws the rows in order also runs it.
+struct AcceptArgs {
+    uint32_t* ctrl = nullptr;
+    const uint32_t* ids = nullptr;
+    uint32_t pos0 = 0, ratio = 1, chain = 0;
+};
+
+int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& rows, uint32_t n,
+                  bool chained = false, const AcceptArgs& accept = AcceptArgs()) {
     ON_DEVICE(s->device);
     const uint32_t kmax = max_k(rows.r, n);
     LaunchCfg cfg;
     const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
+    if (chained) {
+        cfg.chain_rows = n;
+        cfg.chain_cand = s->chain_cand;
+        cfg.chain_n = s->chain_n;
+        cfg.chain_ticket = s->chain_ticket;
+        cfg.accept_ctrl = accept.ctrl;
+        cfg.accept_ids = accept.ids;
+        cfg.accept_pos0 = accept.pos0;
+        cfg.accept_ratio = accept.ratio;
+        cfg.accept_chain = accept.chain;
+    }
     attach_trace(s, &cfg, n);
     const LaunchShape shp = shape_of(s, rows.r, n, dtype, vocab, slices, kmax);
     cfg.excl_words = shp.excl_words;
     cfg.bitmap_layout = shp.bitmap_layout ? 1u : 0u;
     cfg.cand_cap = shp.cand_cap;
-    HIP_TRY(launch_rows(s->stream, dtype, shp.kind(), shp.lse, n, cfg, &rows, shp.dyn_bytes));
+    const size_t dyn = chained && shp.dyn_bytes < CHAIN_LDS_BYTES ? (size_t)CHAIN_LDS_BYTES : shp.dyn_bytes;
+    HIP_TRY(launch_rows(s->stream, dtype, shp.kind(), shp.lse, n, cfg, &rows, dyn));
     return LILY_OK;
 }
 
@@ -725,6 +748,13 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 16);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
     if (err == hipSuccess) err = hipMemset(s->ws_ticket, 0, WS_ROWS * 4);
+    const size_t chain_bytes = (size_t)LILY_MAX_VERIFY_ROWS * CHAIN_CAP * 8 + (LILY_MAX_VERIFY_ROWS + 1) * 4;
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->chain_cand), chain_bytes);
+    if (err == hipSuccess) err = hipMemset(s->chain_cand, 0, chain_bytes);
+    if (err == hipSuccess) {
+        s->chain_n = reinterpret_cast<uint32_t*>(s->chain_cand + (size_t)LILY_MAX_VERIFY_ROWS * CHAIN_CAP);
+        s->chain_ticket = s->chain_n + LILY_MAX_VERIFY_ROWS;
+    }
     for (uint32_t i = 0; i < STAGE_SLOTS && err == hipSuccess; ++i) {
         err = hipEventCreateWithFlags(&s->stage_done[i], hipEventDisableTiming);
     }
@@ -749,6 +779,7 @@ void lily_sampler_destroy(lily_sampler_t* s) {
     (void)hipFree(s->ws_cand);
     (void)hipFree(s->ws_lse);
     (void)hipFree(s->ws_ticket);
+    (void)hipFree(s->chain_cand);
     (void)hipFree(s->table_dev);
     for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {
         if (s->stage[i]) (void)hipHostFree(s->stage[i]);
@@ -1120,10 +1151,19 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
         }
     }
     const size_t es = dtype == LILY_BF16 ? 2 : 4;
-    // Under penalties row j must see the counts of the rows before it: one launch per row.
-    // Without them the rows are independent and share one launch.
+    // Under penalties row j must see the counts of the rows before it.  Where the penalties can
+    // only lower a value, all rows share one launch whose last workgroup draws them in order
+    // (each row collects m - 1 candidates more than it draws from, see row_body); otherwise one
+    // launch per row.  Without penalties the rows are independent and share one launch.
     static_assert(LILY_MAX_VERIFY_ROWS <= (uint32_t)INLINE_ROWS, "verify rows travel inline");
-    const bool chained = lily_params_uses_penalties(params) != 0;
+    const bool pen = lily_params_uses_penalties(params) != 0;
+    float t_eff;
+    uint32_t k_eff;
+    lily_params_effective(params, &t_eff, &k_eff);
+    const bool in_order = pen && m > 1 && params->repetition_penalty >= 1.0f &&
+                          params->presence_penalty >= 0.0f && params->frequency_penalty >= 0.0f &&
+                          k_eff + m - 1 <= LILY_SAMPLE_K_CAP;
+    const bool chained = pen && !in_order;
     InlineRows rows;
     for (uint32_t j = 0; j < m; ++j) {
         const char* row = static_cast<const char*>(logits_dev) + (size_t)j * row_stride * es;
@@ -1151,9 +1191,30 @@ int lily_spec_verify(lily_sampler_t* s, const void* logits_dev, lily_dtype dtype
             }
         }
     }
+    if (in_order) {
+        for (uint32_t j = 0; j < m; ++j) {
+            RowArgs& r = rows.r[j];
+            r.k_draw = r.k;
+            r.k = r.k + m - 1;
+            if (r.k > STREAM_K_MAX) {
+                r.flags &= ~(uint32_t)F_STREAM;
+            }
+        }
+    }
     if (!chained) {
-        if (int rc = launch_inline(s, dtype, vocab, rows, m)) {
+        AcceptArgs accept;
+        if (in_order && ctrl_dev != nullptr) {
+            accept.ctrl = ctrl_dev;
+            accept.ids = ids_dev;
+            accept.pos0 = pos0;
+            accept.ratio = ratio;
+            accept.chain = chain;
+        }
+        if (int rc = launch_inline(s, dtype, vocab, rows, m, in_order, accept)) {
             return rc;
+        }
+        if (accept.ctrl != nullptr) {
+            return LILY_OK;   // the launch wrote the control block itself
         }
     }
     if (ctrl_dev != nullptr) {

@@ -151,10 +151,27 @@ __device__ __forceinline__ uint32_t count_token(const RowArgs& a, uint32_t id, u
     return before;
 }
 
-__device__ __forceinline__ void emit(const RowArgs& a, uint32_t id, uint32_t vocab) {
+// `sh`: where a launch whose rows draw in order learns what this row drew and the count the id
+// has now (null otherwise: nobody then waits for the increment to come back).
+// The increments alone, nothing waited for: for rows that draw in order within one launch, whose
+// workgroup knows the counts itself and brings the largest count up to date once at the end.
+__device__ __forceinline__ void count_token_blind(const RowArgs& a, uint32_t id) {
+    atomicAdd(&a.counts[id], 1u);
+    atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
+}
+
+// `sh`: where a launch whose rows draw in order learns what this row drew (null otherwise).
+__device__ __forceinline__ void emit(const RowArgs& a, uint32_t id, uint32_t vocab, Shared* sh = nullptr) {
     *a.out_id = id;
     if ((a.flags & F_PEN) && id < vocab) {
-        count_token(a, id, vocab);
+        if (sh != nullptr) {
+            count_token_blind(a, id);
+        } else {
+            count_token(a, id, vocab);
+        }
+    }
+    if (sh != nullptr) {
+        sh->emitted_id = id;
     }
 }
 
@@ -174,7 +191,8 @@ __device__ __forceinline__ uint32_t pick_sequential(const float* prefix, uint32_
 // round trip: the count's atomic increment returns the count the penalties used, and the logit
 // loads beside it.
 template <int DT>
-__device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh, uint32_t id, uint32_t vocab) {
+__device__ __forceinline__ void finish_token(const RowArgs& a, Shared& sh, uint32_t id, uint32_t vocab,
+                                             bool in_order = false) {
     *a.out_id = id;
     const bool pen = (a.flags & F_PEN) != 0;
     const bool want = a.out_logprob != nullptr;
@@ -182,10 +200,19 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, const Shared& sh,
         if (want) {
             *a.out_logprob = NEG_INF;
         }
+        if (in_order) {
+            sh.emitted_id = id;
+        }
         return;
     }
     uint32_t before = 0;
-    if (pen) {
+    if (in_order) {
+        // Rows that draw in order: the next row learns the id; nobody waits for the increments.
+        sh.emitted_id = id;
+        if (pen) {
+            count_token_blind(a, id);
+        }
+    } else if (pen) {
         before = count_token(a, id, vocab);
     }
     if (want) {
@@ -217,7 +244,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             if (a.out_logprob) {
                 *a.out_logprob = NEG_INF;
             }
-            emit(a, 0, vocab);
+            emit(a, 0, vocab, cfg.chain_rows != 0u ? &sh : nullptr);
             if (a.dbg_counts) {
                 a.dbg_counts[0] = 0;
                 a.dbg_counts[1] = 1;  // the reference keeps rank 0 whatever its value
@@ -227,6 +254,13 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             }
         }
         return;
+    }
+    // The speculative draw's proposal and the length of the draft's distribution are asked
+    // for now, so that they have arrived when the candidates are ranked and summed.
+    uint32_t spec_d = 0, spec_qn = 0;
+    if (a.mode == MODE_SPEC) {
+        spec_d = *a.draft;
+        spec_qn = *a.q_n;
     }
     if (!sorted) {
         sort_desc<BIG>(cand, n);
@@ -288,7 +322,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         const uint32_t slot = hits != 0ull ? (uint32_t)__builtin_ctzll(hits) : kept - 1u;
         const uint32_t id = ~(uint32_t)__shfl((int)(uint32_t)c, (int)slot);
         if (lane == 0) {
-            finish_token<DT>(a, sh, id, vocab);
+            finish_token<DT>(a, sh, id, vocab, cfg.chain_rows != 0u);
         }
         return;
     }
@@ -393,14 +427,14 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
         TAIL_MARK(12);
         if (tid == 0) {
             const uint32_t id = composite_id(cand[slot]);
-            finish_token<DT>(a, sh, id, vocab);
+            finish_token<DT>(a, sh, id, vocab, cfg.chain_rows != 0u);
         }
         return;
     }
 
     // Speculative draw (sample.metal:596-658, cpu_spec at tests/unit/kernels/sample.rs:264-283).
-    const uint32_t d = *a.draft;
-    const uint32_t qn = min(*a.q_n, K_CAP);
+    const uint32_t d = spec_d;
+    const uint32_t qn = min(spec_qn, K_CAP);
     for (uint32_t i = tid; i < n_keep; i += NT) {
         if (composite_id(cand[i]) == d) {
             sh.p_d = sh.prob[i] / mass;
@@ -414,17 +448,30 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     __syncthreads();
     if (u1 * sh.q_d < sh.p_d) {
         if (tid == 0) {
-            finish_token<DT>(a, sh, d, vocab);
+            finish_token<DT>(a, sh, d, vocab, cfg.chain_rows != 0u);
         }
         return;
     }
     for (uint32_t i = tid; i < n_keep; i += NT) {
         const uint32_t id = composite_id(cand[i]);
+        // The draft's probability of this id: its entries eight at a time, loaded whatever they
+        // hold (a loop that stops at the match is a memory round trip per entry; ids are
+        // listed once, so going on changes nothing).
         float q_i = 0.0f;
-        for (uint32_t j = 0; j < qn; ++j) {
-            if (a.q_ids[j] == id) {
-                q_i = a.q_probs[j];
-                break;
+        for (uint32_t j0 = 0; j0 < qn; j0 += 8u) {
+            uint32_t qi[8];
+            float qp[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const uint32_t j = min(j0 + (uint32_t)q, qn - 1u);
+                qi[q] = a.q_ids[j];
+                qp[q] = a.q_probs[j];
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                if (j0 + (uint32_t)q < qn && qi[q] == id) {
+                    q_i = qp[q];
+                }
             }
         }
         sh.res[i] = fmaxf(sh.prob[i] / mass - q_i, 0.0f);
@@ -454,7 +501,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             slot = pick_sequential(sh.cum, n_keep, u2 * mass);
         }
         const uint32_t id = composite_id(cand[slot]);
-        finish_token<DT>(a, sh, id, vocab);
+        finish_token<DT>(a, sh, id, vocab, cfg.chain_rows != 0u);
     }
 }
 
