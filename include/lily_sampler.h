@@ -223,6 +223,24 @@ int lily_sample_spec_f32_uniforms(lily_sampler_t* s, const float* logits_dev, ui
 int lily_sample_f32_static(void* hip_stream, const float* logits_dev, uint32_t vocab,
                            lily_scratch_t* scratch, const lily_sampling_params* params,
                            uint32_t step, uint32_t* out_dev);
+/* Draws whose row and step a kernel before them chose - the device-side chaining of
+ * src/qwen4exp/spec.rs:398-528, where the draft pass that follows a verify pass is encoded
+ * before the host knows how many rows were accepted and its dispatches read the control block's
+ * words as arguments (Arg::Gpu / Pos::gpu).  logits_dev is [rows][row_stride]; the draw reads row
+ * min(row_dev[0], rows - 1) at step step_base + step_dev[0].  row_dev / step_dev are device
+ * words written earlier on the stream (typically ctrl + LILY_SLOT_ACCEPTED * LILY_CTRL_STRIDE);
+ * either may be NULL (row 0 / step_base).  Otherwise as lily_sample_f32 / lily_sample_draft_f32.
+ * With lily_spec_verify, lily_scratch_uncount_after and lily_copy_row_u32 this lets
+ * verify -> accept -> rollback -> the next draws be enqueued without a host read between. */
+int lily_sample_f32_at(lily_sampler_t* s, const float* logits_dev, uint32_t vocab, uint64_t row_stride,
+                       uint32_t rows, const uint32_t* row_dev, lily_scratch_t* scratch,
+                       const lily_sampling_params* params, uint32_t step_base,
+                       const uint32_t* step_dev, uint32_t* out_dev);
+int lily_sample_draft_f32_at(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                             uint64_t row_stride, uint32_t rows, const uint32_t* row_dev,
+                             lily_scratch_t* scratch, const lily_sampling_params* params,
+                             uint32_t step_base, const uint32_t* step_dev, uint32_t* out_dev,
+                             const lily_draft_dist* dist);
 /* argmax_f32 (src/kernels/elementwise.rs:297-308): first max, lowest index on ties.  The
  * reference's `partials` tensor (ARGMAX_GROUPS * 8 bytes of caller scratch between its two
  * dispatches) has no counterpart: the partial maxima of a row spread over several workgroups
@@ -287,7 +305,7 @@ typedef struct lily_rows {
     uint32_t* dbg_counts_dev;            /* [rows][2] = candidates, kept */
 } lily_rows;
 
-/* Host cost and waits: the call packs one 192-byte descriptor per row into one of four pinned
+/* Host cost and waits: the call packs one 224-byte descriptor per row into one of four pinned
  * staging buffers and enqueues its upload ahead of the launch.  It blocks only (a) when the
  * upload of the call four calls back has not finished, (b) the first time `rows` exceeds every
  * earlier call's (beyond 1024): the row table is reallocated, which drains the stream.  A caller

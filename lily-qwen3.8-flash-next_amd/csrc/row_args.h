@@ -56,9 +56,17 @@ struct alignas(16) RowArgs {
     float uniform2;
     uint32_t k_draw;           // rows of a chained launch: the draw's own candidate count (k is
                                // then what the select collects); 0 otherwise
-    uint32_t pad[2];
+    uint32_t sel_rows;         // rows behind `logits` that sel_row may pick from
+    uint32_t pad;
+    // A draw whose row and step a kernel before it chose (words of the speculative control
+    // block, typically): the row is logits + min(*sel_row, sel_rows - 1) * sel_stride bytes and
+    // the step is step + *sel_step.  Null pointers: the row and the step as given.
+    const uint32_t* sel_row;
+    const uint32_t* sel_step;
+    uint64_t sel_stride;
+    uint64_t pad2;
 };
-static_assert(sizeof(RowArgs) == 192, "RowArgs layout");
+static_assert(sizeof(RowArgs) == 224, "RowArgs layout");
 
 // A scratch's device state as the small maintenance kernels take it.
 struct ScratchView {

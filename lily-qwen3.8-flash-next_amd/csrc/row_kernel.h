@@ -87,10 +87,22 @@ __device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowAr
 
 // CHAIN: the kernel of launches whose rows draw in order (compiled apart from the others: what it
 // adds behind the selects would cost every other launch registers).
+// The row and the step of a draw that leaves the choice to the device (see RowArgs::sel_row).
+__device__ __forceinline__ void apply_selection(RowArgs& a) {
+    if (a.sel_row != nullptr) {
+        const uint32_t r = min(*(const LILY_CONST uint32_t*)a.sel_row, a.sel_rows - 1u);
+        a.logits = static_cast<const char*>(a.logits) + (size_t)r * a.sel_stride;
+    }
+    if (a.sel_step != nullptr) {
+        a.step += *(const LILY_CONST uint32_t*)a.sel_step;
+    }
+}
+
 template <int DT, int KIND, bool LSE, bool CHAIN = false>
 __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const LaunchCfg& cfg, Shared& sh) {
     RowArgs a;
     load_row_args(a, src);
+    apply_selection(a);
     // KIND: 0 = rows without masks, penalties or bias lists, 1 = rows with any of them (the
     // bitmap select is compiled for them), 2 = streaming rows only (no bitmap select at all).
     constexpr bool EXCL = KIND == 1;
@@ -173,6 +185,7 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         const LILY_CONST RowArgs* again = src;
         asm volatile("" : "+s"(again));
         load_row_args(t, again);
+        apply_selection(t);
     }
     const bool forced = (t.flags & F_FORCED) != 0;
     uint32_t n = (argmax || forced) ? 0u : min(sh.n_cand, cfg.cand_cap);

@@ -172,6 +172,11 @@ struct RowExtras {
     uint32_t* dbg_ids = nullptr;
     float* dbg_probs = nullptr;
     uint32_t* dbg_counts = nullptr;
+    // a row and a step left to the device (lily_sample_f32_at)
+    const uint32_t* sel_row = nullptr;
+    const uint32_t* sel_step = nullptr;
+    uint32_t sel_rows = 0;
+    uint64_t sel_stride = 0;   // bytes
 };
 
 // Validates one row and packs it.  `mode` is the draw the caller asked for.
@@ -244,6 +249,10 @@ int pack_row(RowArgs* out, const void* logits, uint32_t vocab, lily_scratch* scr
         out->flags |= F_FORCED;
         out->forced = x.forced;
     }
+    out->sel_row = x.sel_row;
+    out->sel_step = x.sel_step;
+    out->sel_rows = x.sel_rows;
+    out->sel_stride = x.sel_stride;
     out->out_id = out_id;
     out->out_logprob = x.out_logprob;
     out->dbg_ids = x.dbg_ids;
@@ -1015,6 +1024,48 @@ int lily_sample_draft_f32(lily_sampler_t* s, const float* logits_dev, uint32_t v
                           uint32_t step, uint32_t* out_dev, const lily_draft_dist* dist) {
     return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step, MODE_DRAFT, out_dev, dist,
                    nullptr);
+}
+
+namespace {
+
+int selection(RowExtras* x, uint32_t vocab, uint64_t row_stride, uint32_t rows, const uint32_t* row_dev,
+              const uint32_t* step_dev) {
+    if (rows == 0 || row_stride < vocab) {
+        return fail(LILY_ERR_INVALID_ARG, "logits must be [rows][row_stride] with rows > 0 and "
+                                          "row_stride >= vocab");
+    }
+    x->sel_row = row_dev;
+    x->sel_step = step_dev;
+    x->sel_rows = rows;
+    x->sel_stride = row_stride * 4;
+    return LILY_OK;
+}
+
+}  // namespace
+
+int lily_sample_f32_at(lily_sampler_t* s, const float* logits_dev, uint32_t vocab, uint64_t row_stride,
+                       uint32_t rows, const uint32_t* row_dev, lily_scratch_t* scratch,
+                       const lily_sampling_params* params, uint32_t step_base,
+                       const uint32_t* step_dev, uint32_t* out_dev) {
+    RowExtras x;
+    if (int rc = selection(&x, vocab, row_stride, rows, row_dev, step_dev)) {
+        return rc;
+    }
+    return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step_base, MODE_PLAIN, out_dev,
+                   nullptr, nullptr, x);
+}
+
+int lily_sample_draft_f32_at(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,
+                             uint64_t row_stride, uint32_t rows, const uint32_t* row_dev,
+                             lily_scratch_t* scratch, const lily_sampling_params* params,
+                             uint32_t step_base, const uint32_t* step_dev, uint32_t* out_dev,
+                             const lily_draft_dist* dist) {
+    RowExtras x;
+    if (int rc = selection(&x, vocab, row_stride, rows, row_dev, step_dev)) {
+        return rc;
+    }
+    return one_row(s, logits_dev, LILY_F32, vocab, scratch, params, step_base, MODE_DRAFT, out_dev,
+                   dist, nullptr, x);
 }
 
 int lily_sample_spec_f32(lily_sampler_t* s, const float* logits_dev, uint32_t vocab,

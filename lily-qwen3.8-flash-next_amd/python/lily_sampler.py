@@ -132,6 +132,8 @@ def _load():
         "lily_draft_dists_slot": [vp, u32, C.POINTER(DraftDist)],
         "lily_sample_f32": [vp, vp, u32, vp, P, u32, vp],
         "lily_sample_draft_f32": [vp, vp, u32, vp, P, u32, vp, C.POINTER(DraftDist)],
+        "lily_sample_f32_at": [vp, vp, u32, u64, u32, vp, vp, P, u32, vp, vp],
+        "lily_sample_draft_f32_at": [vp, vp, u32, u64, u32, vp, vp, P, u32, vp, vp, C.POINTER(DraftDist)],
         "lily_sample_spec_f32": [vp, vp, u32, vp, P, u32, C.POINTER(DraftDist), vp, vp],
         "lily_argmax_f32": [vp, vp, u32, vp],
         "lily_sample_f32_static": [vp, vp, u32, vp, P, u32, vp],
@@ -282,6 +284,25 @@ class Sampler:
         _check(_lib.lily_sample_draft_f32(self._h, _ptr(logits, torch.float32), logits.numel(),
                                           scratch._h if scratch else None, C.byref(params), step,
                                           _ptr(out, torch.int32), C.byref(dist)))
+
+    def sample_f32_at(self, logits_rows, row_dev, scratch, params, step_base, step_dev, out):
+        """lily_sample_f32_at: logits_rows [rows, V] f32; row_dev / step_dev: int32 device tensors
+        (or views) holding the row index and the step offset, or None."""
+        rows, vocab = logits_rows.shape
+        _check(_lib.lily_sample_f32_at(
+            self._h, _ptr(logits_rows, torch.float32), vocab, logits_rows.stride(0), rows,
+            _ptr(row_dev, torch.int32) if row_dev is not None else None,
+            scratch._h if scratch else None, C.byref(params), step_base,
+            _ptr(step_dev, torch.int32) if step_dev is not None else None, _ptr(out, torch.int32)))
+
+    def sample_draft_f32_at(self, logits_rows, row_dev, scratch, params, step_base, step_dev, out, dist):
+        rows, vocab = logits_rows.shape
+        _check(_lib.lily_sample_draft_f32_at(
+            self._h, _ptr(logits_rows, torch.float32), vocab, logits_rows.stride(0), rows,
+            _ptr(row_dev, torch.int32) if row_dev is not None else None,
+            scratch._h if scratch else None, C.byref(params), step_base,
+            _ptr(step_dev, torch.int32) if step_dev is not None else None, _ptr(out, torch.int32),
+            C.byref(dist)))
 
     def sample_spec_f32(self, logits, scratch, params, step, dist, draft, out, uniforms=None):
         """uniforms: None (seeded draws) or (u1, u2) for the accept test and the residual draw."""
