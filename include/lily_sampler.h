@@ -159,6 +159,9 @@ int lily_scratch_uncount_after(lily_scratch_t* sc, const uint32_t* draws_dev, ui
                                const uint32_t* accepted_dev, uint32_t accepted_cap);
 /* SamplerScratch::copy_counts_from (sample.rs:168-174): LILY_ERR_VOCAB on a size mismatch. */
 int lily_scratch_copy_counts_from(lily_scratch_t* dst, const lily_scratch_t* src);
+/* move_sampler_counts (src/qwen4exp/batch.rs:138-162, engine slot <-> batch slot): `to` takes
+ * `from`'s counts in stream order; from == to does nothing. */
+int lily_scratch_move_counts(lily_scratch_t* from, lily_scratch_t* to);
 /* No counterpart in the reference (its histogram only ever grows by the kernel's own
  * draws): counts[id] += multiplicity of id in ids_dev[0..n); ids >= vocab are ignored. */
 int lily_scratch_add_history(lily_scratch_t* sc, const uint32_t* ids_dev, uint32_t n);
@@ -173,6 +176,29 @@ int lily_scratch_read_counts(lily_scratch_t* sc, uint32_t* host_counts);
 int lily_draft_dists_create(lily_sampler_t* s, uint32_t slots, lily_draft_dists_t** out);
 void lily_draft_dists_destroy(lily_draft_dists_t* d);
 int lily_draft_dists_slot(const lily_draft_dists_t* d, uint32_t i, lily_draft_dist* out);
+
+/* ---- the decode loop's output slots ------------------------------------------------------ */
+
+/* The ping-pong `next_token` slots of the decode loop and its polled completion
+ * (src/generate.rs:776-891: a step reads slot_in and writes the other slot, the following step is
+ * encoded while this one runs, `wait_polled` + `read_slot`).  `slots` device arrays of `words`
+ * u32 each (one word per row of a batched step) with a pinned host mirror and an event per slot.
+ * A draw is given lily_token_slots_device(t, i) as its out_dev / out_ids_dev; the next step's
+ * kernels read the same address.  lily_token_slots_publish enqueues, behind the work already on
+ * the sampler's stream, the slot's copy to the mirror and an event; lily_token_slots_poll
+ * never blocks: ready = 1 and the slot's words in host_out once that event has passed.
+ * lily_token_slots_wait_polled polls until then (max_polls = 0: without limit; else
+ * LILY_ERR_RANGE after that many polls) - the host thread spins instead of sleeping in the
+ * driver, which is what wakes it within microseconds of the step's end.  A slot must be read
+ * (ready = 1) before it is published again. */
+typedef struct lily_token_slots lily_token_slots_t;
+int lily_token_slots_create(lily_sampler_t* s, uint32_t slots, uint32_t words, lily_token_slots_t** out);
+void lily_token_slots_destroy(lily_token_slots_t* t);
+uint32_t* lily_token_slots_device(const lily_token_slots_t* t, uint32_t slot);
+int lily_token_slots_publish(lily_token_slots_t* t, uint32_t slot);
+int lily_token_slots_poll(lily_token_slots_t* t, uint32_t slot, uint32_t* host_out, int* ready);
+int lily_token_slots_wait_polled(lily_token_slots_t* t, uint32_t slot, uint32_t* host_out,
+                                 uint64_t max_polls);
 
 /* ---- single-row draws (the reference's call signature) --------------------------------- */
 

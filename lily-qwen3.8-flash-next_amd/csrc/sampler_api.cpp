@@ -121,6 +121,15 @@ struct lily_draft_dists {
     uint32_t* counts = nullptr;
 };
 
+struct lily_token_slots {
+    lily_sampler* s = nullptr;
+    uint32_t slots = 0, words = 0;
+    uint32_t* dev = nullptr;    // [slots][words]
+    uint32_t* host = nullptr;   // pinned mirror, [slots][words]
+    hipEvent_t* done = nullptr; // [slots] recorded behind each slot's copy to the mirror
+    bool* published = nullptr;  // [slots] an event has been recorded since the slot was last read
+};
+
 // One launch over consecutive rows of a packed table.
 struct LaunchPart {
     uint32_t first = 0;
@@ -995,6 +1004,123 @@ void lily_draft_dists_destroy(lily_draft_dists_t* d) {
     (void)hipStreamSynchronize(d->s->stream);
     (void)hipFree(d->ids);
     delete d;
+}
+
+// ---- token slots (the decode loop's ping-pong outputs)
+
+int lily_token_slots_create(lily_sampler_t* s, uint32_t slots, uint32_t words, lily_token_slots_t** out) {
+    if (s == nullptr || out == nullptr || slots == 0 || words == 0 || slots > 64 || words > (1u << 20)) {
+        return fail(LILY_ERR_INVALID_ARG, "token slots need a sampler, 1..64 slots and 1..2^20 words");
+    }
+    *out = nullptr;
+    ON_DEVICE(s->device);
+    lily_token_slots* t = new (std::nothrow) lily_token_slots;
+    if (t == nullptr) {
+        return fail(LILY_ERR_NOMEM, "out of host memory");
+    }
+    t->s = s;
+    t->slots = slots;
+    t->words = words;
+    t->done = new (std::nothrow) hipEvent_t[slots]();
+    t->published = new (std::nothrow) bool[slots]();
+    const size_t bytes = (size_t)slots * words * 4;
+    hipError_t e = t->done && t->published ? hipSuccess : hipErrorOutOfMemory;
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&t->dev), bytes);
+    if (e == hipSuccess) e = hipMemsetAsync(t->dev, 0xff, bytes, s->stream);
+    if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void**>(&t->host), bytes, hipHostMallocDefault);
+    for (uint32_t i = 0; e == hipSuccess && i < slots; ++i) {
+        e = hipEventCreateWithFlags(&t->done[i], hipEventDisableTiming);
+    }
+    if (e != hipSuccess) {
+        lily_token_slots_destroy(t);
+        return hip_fail(e, "token slots allocation");
+    }
+    std::memset(t->host, 0xff, bytes);
+    *out = t;
+    return LILY_OK;
+}
+
+void lily_token_slots_destroy(lily_token_slots_t* t) {
+    if (t == nullptr) {
+        return;
+    }
+    DeviceScope device_scope_(t->s->device);
+    (void)hipStreamSynchronize(t->s->stream);
+    for (uint32_t i = 0; t->done != nullptr && i < t->slots; ++i) {
+        if (t->done[i]) (void)hipEventDestroy(t->done[i]);
+    }
+    if (t->dev) (void)hipFree(t->dev);
+    if (t->host) (void)hipHostFree(t->host);
+    delete[] t->done;
+    delete[] t->published;
+    delete t;
+}
+
+uint32_t* lily_token_slots_device(const lily_token_slots_t* t, uint32_t slot) {
+    if (t == nullptr || slot >= t->slots) {
+        (void)fail(LILY_ERR_RANGE, "token slot out of range");
+        return nullptr;
+    }
+    return t->dev + (size_t)slot * t->words;
+}
+
+int lily_token_slots_publish(lily_token_slots_t* t, uint32_t slot) {
+    if (t == nullptr || slot >= t->slots) {
+        return fail(LILY_ERR_RANGE, "token slot out of range");
+    }
+    ON_DEVICE(t->s->device);
+    const size_t off = (size_t)slot * t->words;
+    HIP_TRY(hipMemcpyAsync(t->host + off, t->dev + off, (size_t)t->words * 4, hipMemcpyDeviceToHost,
+                           t->s->stream));
+    HIP_TRY(hipEventRecord(t->done[slot], t->s->stream));
+    t->published[slot] = true;
+    return LILY_OK;
+}
+
+int lily_token_slots_poll(lily_token_slots_t* t, uint32_t slot, uint32_t* host_out, int* ready) {
+    if (t == nullptr || slot >= t->slots || ready == nullptr) {
+        return fail(LILY_ERR_RANGE, "token slot out of range, or ready is null");
+    }
+    *ready = 0;
+    if (!t->published[slot]) {
+        return fail(LILY_ERR_INVALID_ARG, "token slot %u was not published since it was last read", slot);
+    }
+    const hipError_t e = hipEventQuery(t->done[slot]);
+    if (e == hipErrorNotReady) {
+        return LILY_OK;
+    }
+    HIP_TRY(e);
+    if (host_out != nullptr) {
+        std::memcpy(host_out, t->host + (size_t)slot * t->words, (size_t)t->words * 4);
+    }
+    t->published[slot] = false;
+    *ready = 1;
+    return LILY_OK;
+}
+
+int lily_token_slots_wait_polled(lily_token_slots_t* t, uint32_t slot, uint32_t* host_out,
+                                 uint64_t max_polls) {
+    for (uint64_t i = 0; max_polls == 0 || i < max_polls; ++i) {
+        int ready = 0;
+        if (int rc = lily_token_slots_poll(t, slot, host_out, &ready)) {
+            return rc;
+        }
+        if (ready) {
+            return LILY_OK;
+        }
+    }
+    return fail(LILY_ERR_RANGE, "token slot %u not ready after %llu polls", slot,
+                (unsigned long long)max_polls);
+}
+
+int lily_scratch_move_counts(lily_scratch_t* from, lily_scratch_t* to) {
+    if (from == nullptr || to == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "move_counts needs two scratches");
+    }
+    if (from == to) {
+        return LILY_OK;   // batch.rs:147-149
+    }
+    return lily_scratch_copy_counts_from(to, from);
 }
 
 int lily_draft_dists_slot(const lily_draft_dists_t* d, uint32_t i, lily_draft_dist* out) {

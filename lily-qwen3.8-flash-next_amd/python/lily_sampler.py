@@ -132,6 +132,11 @@ def _load():
         "lily_draft_dists_slot": [vp, u32, C.POINTER(DraftDist)],
         "lily_sample_f32": [vp, vp, u32, vp, P, u32, vp],
         "lily_sample_draft_f32": [vp, vp, u32, vp, P, u32, vp, C.POINTER(DraftDist)],
+        "lily_token_slots_create": [vp, u32, u32, C.POINTER(vp)],
+        "lily_token_slots_publish": [vp, u32],
+        "lily_token_slots_poll": [vp, u32, vp, C.POINTER(C.c_int)],
+        "lily_token_slots_wait_polled": [vp, u32, vp, u64],
+        "lily_scratch_move_counts": [vp, vp],
         "lily_sample_f32_at": [vp, vp, u32, u64, u32, vp, vp, P, u32, vp, vp],
         "lily_sample_draft_f32_at": [vp, vp, u32, u64, u32, vp, vp, P, u32, vp, vp, C.POINTER(DraftDist)],
         "lily_sample_spec_f32": [vp, vp, u32, vp, P, u32, C.POINTER(DraftDist), vp, vp],
@@ -153,9 +158,11 @@ def _load():
         getattr(L, name).restype = C.c_int
         getattr(L, name).argtypes = args
     for name in ("lily_sampler_destroy", "lily_scratch_destroy", "lily_draft_dists_destroy",
-                 "lily_plan_destroy"):
+                 "lily_plan_destroy", "lily_token_slots_destroy"):
         getattr(L, name).restype = None
         getattr(L, name).argtypes = [vp]
+    L.lily_token_slots_device.restype = vp
+    L.lily_token_slots_device.argtypes = [vp, u32]
     return L
 
 
@@ -496,6 +503,10 @@ class SamplerScratch:
     def reset_counts(self):
         _check(_lib.lily_scratch_reset_counts(self._h))
 
+    def move_counts_to(self, other):
+        """move_sampler_counts (src/qwen4exp/batch.rs:138-162): `other` takes these counts."""
+        _check(_lib.lily_scratch_move_counts(self._h, other._h))
+
     def copy_counts_from(self, other):
         _check(_lib.lily_scratch_copy_counts_from(self._h, other._h))
 
@@ -513,6 +524,67 @@ class SamplerScratch:
         out = torch.empty(self.vocab(), dtype=torch.int32)
         _check(_lib.lily_scratch_read_counts(self._h, C.c_void_p(out.data_ptr())))
         return out
+
+
+class _DeviceWords:
+    """Device memory owned by the library, as something torch can wrap without copying."""
+
+    def __init__(self, ptr, n):
+        self.__cuda_array_interface__ = {"shape": (n,), "typestr": "<i4", "data": (int(ptr), False),
+                                         "version": 2}
+
+
+def _device_view(ptr, n, device):
+    return torch.as_tensor(_DeviceWords(ptr, n), device=torch.device("cuda", device))
+
+
+class TokenSlots:
+    """The decode loop's ping-pong output slots with polled completion (src/generate.rs:776-891):
+    `slots` device arrays of `words` int32 each, a pinned host mirror, an event per slot."""
+
+    def __init__(self, sampler, slots=2, words=1):
+        self._s = sampler
+        self.slots, self.words = slots, words
+        h = C.c_void_p()
+        _check(_lib.lily_token_slots_create(sampler._h, slots, words, C.byref(h)))
+        self._h = h
+        sampler._children.add(self)
+        self._views = []
+        for i in range(slots):
+            ptr = _lib.lily_token_slots_device(self._h, i)
+            self._views.append(_device_view(ptr, words, sampler.device))
+
+    def device(self, i):
+        """Slot i as an int32 device tensor over the library's memory (valid until close())."""
+        return self._views[i]
+
+    def publish(self, i):
+        _check(_lib.lily_token_slots_publish(self._h, i))
+
+    def poll(self, i):
+        """None while the slot's step is still running, else its words as a list."""
+        out = (C.c_uint32 * self.words)()
+        ready = C.c_int(0)
+        _check(_lib.lily_token_slots_poll(self._h, i, out, C.byref(ready)))
+        return list(out) if ready.value else None
+
+    def wait_polled(self, i, max_polls=0):
+        out = (C.c_uint32 * self.words)()
+        _check(_lib.lily_token_slots_wait_polled(self._h, i, out, max_polls))
+        return list(out)
+
+    def close(self):
+        if self._h:
+            self._views = []
+            if self._s._h:
+                _lib.lily_token_slots_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class DraftDists:
