@@ -88,6 +88,30 @@ int lily_params_uses_penalties(const lily_sampling_params* p);
 int lily_params_validate(const lily_sampling_params* p);
 /* src/kernels/sample.rs:83-94 effective: the temperature and candidate count the kernel uses */
 void lily_params_effective(const lily_sampling_params* p, float* temperature, uint32_t* top_k);
+/* A request's sampling fields over the server's defaults (resolve_sampling,
+ * src/serve/api.rs:798-834; the fields are SamplingFields, :440-456): a field is taken when its
+ * bit of `has` is set, else the default's; top_k < 0 means 0 (off); a request without a seed gets
+ * `fresh_seed` (the reference draws it from the clock and the process id: the caller supplies
+ * its own entropy here, which keeps the function pure).  The result is validated:
+ * LILY_OK or LILY_ERR_PARAMS with the rule's message, `out` written either way. */
+enum {
+    LILY_HAS_TEMPERATURE = 1, LILY_HAS_TOP_P = 2, LILY_HAS_TOP_K = 4, LILY_HAS_MIN_P = 8,
+    LILY_HAS_SEED = 16, LILY_HAS_PRESENCE = 32, LILY_HAS_FREQUENCY = 64, LILY_HAS_REPETITION = 128
+};
+typedef struct lily_sampling_fields {
+    uint32_t has;             /* LILY_HAS_* bits */
+    float temperature;
+    float top_p;
+    float min_p;
+    int64_t top_k;
+    int64_t seed;             /* taken as u64, as the reference's `s as u64` */
+    float presence_penalty;
+    float frequency_penalty;
+    float repetition_penalty;
+    uint32_t reserved;        /* must be 0 */
+} lily_sampling_fields;
+int lily_params_resolve(const lily_sampling_fields* fields, const lily_sampling_params* defaults,
+                        uint64_t fresh_seed, lily_sampling_params* out);
 /* src/kernels/sample.rs:227-234 draft_params */
 void lily_draft_params(const lily_sampling_params* p, lily_sampling_params* out);
 /* src/kernels/sample.rs:220-222 draft_step */

@@ -707,6 +707,28 @@ int lily_params_validate(const lily_sampling_params* p) {
     return LILY_OK;
 }
 
+int lily_params_resolve(const lily_sampling_fields* f, const lily_sampling_params* d,
+                        uint64_t fresh_seed, lily_sampling_params* out) {
+    if (f == nullptr || d == nullptr || out == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "resolve needs fields, defaults and out");
+    }
+    lily_sampling_params p = *d;
+    p.reserved = 0;
+    if (f->has & LILY_HAS_TEMPERATURE) p.temperature = f->temperature;
+    if (f->has & LILY_HAS_TOP_P) p.top_p = f->top_p;
+    if (f->has & LILY_HAS_MIN_P) p.min_p = f->min_p;
+    if (f->has & LILY_HAS_PRESENCE) p.presence_penalty = f->presence_penalty;
+    if (f->has & LILY_HAS_FREQUENCY) p.frequency_penalty = f->frequency_penalty;
+    if (f->has & LILY_HAS_REPETITION) p.repetition_penalty = f->repetition_penalty;
+    if (f->has & LILY_HAS_TOP_K) {
+        // api.rs:803-807: a negative k is "off"; beyond u32 the cap applies anyway.
+        p.top_k = f->top_k < 0 ? 0u : (f->top_k > 0xffffffffll ? 0xffffffffu : (uint32_t)f->top_k);
+    }
+    p.seed = (f->has & LILY_HAS_SEED) ? (uint64_t)f->seed : fresh_seed;
+    *out = p;
+    return lily_params_validate(out);
+}
+
 void lily_params_effective(const lily_sampling_params* p, float* temperature, uint32_t* top_k) {
     if (lily_params_is_greedy(p)) {
         *temperature = 1.0f;

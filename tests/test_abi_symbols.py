@@ -41,3 +41,57 @@ def test_pure_host_helpers_need_no_gpu():
     assert lib.lily_ctrl_words(3) == (2 + 9) * 4
     lib.lily_draft_step.restype = ctypes.c_uint32
     assert lib.lily_draft_step(5) == 5 | 0x40000000
+
+
+class _Params(ctypes.Structure):
+    _fields_ = [("temperature", ctypes.c_float), ("top_k", ctypes.c_uint32), ("top_p", ctypes.c_float),
+                ("min_p", ctypes.c_float), ("presence_penalty", ctypes.c_float),
+                ("frequency_penalty", ctypes.c_float), ("repetition_penalty", ctypes.c_float),
+                ("reserved", ctypes.c_uint32), ("seed", ctypes.c_uint64)]
+
+
+class _Fields(ctypes.Structure):
+    _fields_ = [("has", ctypes.c_uint32), ("temperature", ctypes.c_float), ("top_p", ctypes.c_float),
+                ("min_p", ctypes.c_float), ("top_k", ctypes.c_int64), ("seed", ctypes.c_int64),
+                ("presence_penalty", ctypes.c_float), ("frequency_penalty", ctypes.c_float),
+                ("repetition_penalty", ctypes.c_float), ("reserved", ctypes.c_uint32)]
+
+
+HAS = dict(temperature=1, top_p=2, top_k=4, min_p=8, seed=16, presence_penalty=32,
+           frequency_penalty=64, repetition_penalty=128)
+
+
+def test_request_fields_resolve_over_the_defaults():
+    """resolve_sampling (src/serve/api.rs:798-834): fields over defaults, negative top_k = off,
+    a missing seed replaced by fresh entropy, the result validated."""
+    lib = ctypes.CDLL(LIB)
+    lib.lily_params_resolve.restype = ctypes.c_int
+    lib.lily_params_resolve.argtypes = [ctypes.POINTER(_Fields), ctypes.POINTER(_Params), ctypes.c_uint64,
+                                        ctypes.POINTER(_Params)]
+    lib.lily_last_error.restype = ctypes.c_char_p
+    defaults = _Params(0.6, 20, 0.95, 0.0, 0.0, 0.0, 1.05, 0, 99)
+
+    def resolve(fresh=4242, **given):
+        f = _Fields()
+        for k, v in given.items():
+            f.has |= HAS[k]
+            setattr(f, k, v)
+        out = _Params()
+        rc = lib.lily_params_resolve(ctypes.byref(f), ctypes.byref(defaults), fresh, ctypes.byref(out))
+        return rc, out
+
+    rc, p = resolve()
+    assert rc == 0
+    assert (p.temperature, p.top_k, p.top_p, p.repetition_penalty) == (defaults.temperature, 20,
+                                                                      defaults.top_p, defaults.repetition_penalty)
+    assert p.seed == 4242                      # no seed in the request: the fresh one, not the defaults'
+    rc, p = resolve(temperature=0.0, top_k=-1, seed=-1, presence_penalty=1.5, min_p=0.1)
+    assert rc == 0
+    assert p.temperature == 0.0 and p.top_k == 0 and p.seed == 0xFFFFFFFFFFFFFFFF
+    assert p.presence_penalty == 1.5 and abs(p.min_p - 0.1) < 1e-7 and p.top_p == defaults.top_p
+    rc, p = resolve(top_k=5_000_000_000)
+    assert rc == 0 and p.top_k == 0xFFFFFFFF   # beyond u32: still "more than the cap"
+    for bad in (dict(top_p=0.0), dict(top_p=1.5), dict(min_p=-0.1), dict(temperature=-1.0),
+                dict(repetition_penalty=0.0), dict(frequency_penalty=float("inf"))):
+        rc, p = resolve(**bad)
+        assert rc == -2 and lib.lily_last_error(), bad     # LILY_ERR_PARAMS with the rule's text
