@@ -247,6 +247,8 @@ struct Shared {
     uint32_t drawn_count[LILY_MAX_VERIFY_ROWS];
     uint32_t proposal[LILY_MAX_VERIFY_ROWS];
     uint32_t chain_n[LILY_MAX_VERIFY_ROWS];   // candidates each row published
+    uint32_t proposal_of[LILY_MAX_VERIFY_ROWS];   // each speculative row's proposal ...
+    uint32_t q_n_of[LILY_MAX_VERIFY_ROWS];        // ... and the length of its draft distribution
     uint32_t emitted_id;
     uint32_t fail;
     double red3[4][NWAVE];

@@ -118,9 +118,10 @@ struct LaunchCfg {
 
 constexpr uint32_t CHAIN_CAP = LILY_SAMPLE_K_CAP;   // candidates a chained row publishes
 // Where the workgroup that draws the rows keeps what it requested ahead: behind the sorted
-// candidates and the tail's three float arrays, 16 bytes for each of a row's first 64 candidates.
+// candidates and the tail's three float arrays, 16 bytes for each of a row's first 64 candidates
+// and 8 for each of the first 64 entries of its draft distribution.
 constexpr uint32_t CHAIN_LDS_OFFSET = LILY_SAMPLE_K_CAP * 8 + 3 * LILY_SAMPLE_K_CAP * 4;
-constexpr uint32_t CHAIN_LDS_BYTES = CHAIN_LDS_OFFSET + LILY_MAX_VERIFY_ROWS * 64 * 16;
+constexpr uint32_t CHAIN_LDS_BYTES = CHAIN_LDS_OFFSET + LILY_MAX_VERIFY_ROWS * 64 * 24;
 
 constexpr uint32_t PHASE_SLOTS = 16;
 

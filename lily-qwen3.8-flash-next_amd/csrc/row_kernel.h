@@ -87,6 +87,12 @@ __device__ __forceinline__ void load_row_args(RowArgs& a, const LILY_CONST RowAr
 
 // CHAIN: the kernel of launches whose rows draw in order (compiled apart from the others: what it
 // adds behind the selects would cost every other launch registers).
+// A workgroup barrier that orders LDS accesses only (outstanding global stores and atomics are
+// not waited for).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // The row and the step of a draw that leaves the choice to the device (see RowArgs::sel_row).
 __device__ __forceinline__ void apply_selection(RowArgs& a) {
     if (a.sel_row != nullptr) {
@@ -371,6 +377,11 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         uint64_t* pre_c = dyn_lds + CHAIN_LDS_OFFSET / 8;                           // [rows][PRE]
         float* pre_l = reinterpret_cast<float*>(pre_c + LILY_MAX_VERIFY_ROWS * PRE);  // [rows][PRE]
         uint32_t* pre_cnt = reinterpret_cast<uint32_t*>(pre_l + LILY_MAX_VERIFY_ROWS * PRE);
+        // ... and, for the rows that are speculative draws, the proposal and the first 64 entries
+        // of the draft's distribution (all of it, as a rule): the tail reads them through the
+        // row's pointers, which are turned to these copies.
+        uint32_t* pre_qid = pre_cnt + LILY_MAX_VERIFY_ROWS * PRE;                     // [rows][PRE]
+        float* pre_qp = reinterpret_cast<float*>(pre_qid + LILY_MAX_VERIFY_ROWS * PRE);
         for (uint32_t j0 = 0; j0 < rows; j0 += NWAVE) {
             const uint32_t j = j0 + (tid >> 6), lane = tid & 63u;
             if (j < rows) {
@@ -383,10 +394,22 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
                 pre_c[j * PRE + lane] = c;
                 pre_l[j * PRE + lane] = load_logit<DT>((first + j)->logits, id);
                 pre_cnt[j * PRE + lane] = (t.flags & F_PEN) ? load_through(t.counts + id) : 0u;
+                const LILY_CONST RowArgs* rj = first + j;
+                if (rj->mode == MODE_SPEC) {
+                    pre_qid[j * PRE + lane] = gload(rj->q_ids + lane);
+                    pre_qp[j * PRE + lane] = gload(rj->q_probs + lane);
+                    if (lane == 0) {
+                        sh.proposal_of[j] = gload(rj->draft);
+                        sh.q_n_of[j] = gload(rj->q_n);
+                    }
+                }
             }
         }
         __syncthreads();
         for (uint32_t j = 0; j < rows; ++j) {
+#ifdef LILY_CHAIN_TRACE
+            phase(cfg, 8 + j);
+#endif
             RowArgs r;
             {
                 const LILY_CONST RowArgs* from = first + j;
@@ -430,10 +453,25 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
             // each thread counts the candidates that beat its own (composites are distinct).
             bool ranked = false;
             if (n_now <= NT) {
-                const uint64_t mine = tid < n_now ? cand[tid] : 0ull;
+                // (read eight at a time, the slots up to the next multiple of eight cleared: a
+                // loop of one dependent LDS read after the other costs a microsecond a row)
+                const uint32_t n_up = (n_now + 7u) & ~7u;
+                if (tid >= n_now && tid < n_up) {
+                    cand[tid] = 0ull;
+                }
+                lds_barrier();
+                const uint64_t mine = tid < n_now ? cand[tid] : ~0ull;
                 uint32_t ahead = 0;
-                for (uint32_t q = 0; q < n_now; ++q) {
-                    ahead += cand[q] > mine ? 1u : 0u;
+                for (uint32_t q0 = 0; q0 < n_up; q0 += 8u) {
+                    uint64_t other[8];
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        other[q] = cand[q0 + (uint32_t)q];
+                    }
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        ahead += other[q] > mine ? 1u : 0u;
+                    }
                 }
                 __syncthreads();
                 if (tid < n_now) {
@@ -443,12 +481,21 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
                 ranked = true;
             }
             r.k = r.k_draw;
-            tail<DT, KIND != 2>(r, vocab, r.step + cfg.step_delta, n_now, ranked, cand, sh, cfg);
-            __syncthreads();
+            if (r.mode == MODE_SPEC && sh.q_n_of[j] <= PRE) {
+                r.draft = &sh.proposal_of[j];
+                r.q_n = &sh.q_n_of[j];
+                r.q_ids = pre_qid + j * PRE;
+                r.q_probs = pre_qp + j * PRE;
+            }
+            tail<DT, KIND != 2, true>(r, vocab, r.step + cfg.step_delta, n_now, ranked, cand, sh, cfg);
+            // The workgroup meets over LDS only: a barrier that also waited for thread 0's stores
+            // and increments to be acknowledged by memory would cost every row a round trip
+            // that nothing here depends on.
+            lds_barrier();
             if (tid == 0) {
                 sh.drawn[j] = sh.emitted_id;
             }
-            __syncthreads();
+            lds_barrier();
         }
         // The scratch's largest count (and an id that holds it) follow now, once per draw.  It
         // must never understate a count: thread 0, which issued every increment, waits for them

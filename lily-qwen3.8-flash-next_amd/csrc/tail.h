@@ -229,7 +229,10 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, Shared& sh, uint3
 }
 
 // cand[0..n) holds the row's candidates (at least its top-k); finishes the row.
-template <int DT, bool BIG>
+// SPEC_WAVE: compile the speculative draw of at most 64 candidates as one wave too (the kernel
+// of rows that draw in order, where every row's tail is a step of a chain; elsewhere its scalar
+// registers would be taken from the scan).
+template <int DT, bool BIG, bool SPEC_WAVE = false>
 __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t step, uint32_t n, bool sorted,
                      uint64_t* cand, Shared& sh, const LaunchCfg& cfg) {
 #ifdef LILY_TAIL_TRACE
@@ -268,7 +271,7 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     TAIL_MARK(8);
     const uint32_t k = min(a.k, n);
     const float top = composite_value(cand[0]);
-    if (k <= 64u && a.mode != MODE_SPEC) {
+    if (k <= 64u && (a.mode != MODE_SPEC || (SPEC_WAVE && spec_qn <= 64u))) {
         // One wave, a candidate per lane.  The sums keep the reference's left-to-right f32
         // order: every lane runs the same chain of 64 additions on values read lane by lane
         // (lanes past k hold 0, which changes nothing), so nothing waits on LDS.
@@ -287,12 +290,6 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             }
         }
         const int pbits = (int)lilym_f32_bits(p);
-        float total = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 64; ++i) {
-            total += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, i));
-        }
-        const float limit = a.top_p * total;
         float cum = 0.0f, before = 0.0f, mine = 0.0f;
 #pragma unroll
         for (int i = 0; i < 64; ++i) {
@@ -300,6 +297,8 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             cum += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(pbits, i));
             mine = lane == (uint32_t)i ? cum : mine;
         }
+        // (the chain's last value is the row total: the same additions in the same order)
+        const float limit = a.top_p * cum;
         const bool stop = lane >= 1u && lane < k && !(before < limit && p >= a.min_p);
         const uint64_t stops = __ballot(stop);
         const uint32_t kept = stops != 0ull ? (uint32_t)__builtin_ctzll(stops) : k;
@@ -318,6 +317,61 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
             }
         }
         const float u1 = (a.flags & F_UNIFORM) ? a.uniform : lilym_uniform_for(a.seed, step);
+        if (SPEC_WAVE && a.mode == MODE_SPEC) {
+            // Speculative draw (sample.metal:596-658, cpu_spec at tests/unit/kernels/sample.rs:264-283)
+            // in the same wave: the draft's distribution (at most 64 entries here) sits an entry
+            // per lane, lookups are ballots and lane reads, and the residual's sums run the same
+            // left-to-right chains as above.
+            const uint32_t d = spec_d, qn = spec_qn;
+            const uint32_t my_id = composite_id(c);
+            const uint32_t q_id = lane < qn ? a.q_ids[lane] : 0xffffffffu;
+            const float q_p = lane < qn ? a.q_probs[lane] : 0.0f;
+            const float p_norm = p / mass;
+            const uint64_t at_p = __ballot(lane < kept && my_id == d);
+            const uint64_t at_q = __ballot(lane < qn && q_id == d);
+            const float p_d = at_p != 0ull ? __shfl(p_norm, (int)__builtin_ctzll(at_p)) : 0.0f;
+            const float q_d = at_q != 0ull ? __shfl(q_p, (int)__builtin_ctzll(at_q)) : 0.0f;
+            if (u1 * q_d < p_d) {
+                if (lane == 0) {
+                    finish_token<DT>(a, sh, d, vocab, cfg.chain_rows != 0u);
+                }
+                return;
+            }
+            // The draft's probability of each candidate, then the residual max(0, p - q).
+            int match = -1;   // the lane that holds this candidate's id in the draft's list
+            const int qid_bits = (int)q_id;
+#pragma unroll
+            for (int j = 0; j < 64; ++j) {
+                const uint32_t idj = (uint32_t)__builtin_amdgcn_readlane(qid_bits, j);
+                match = ((uint32_t)j < qn && idj == my_id) ? j : match;
+            }
+            const float q_there = __shfl(q_p, match < 0 ? 0 : match);
+            const float q_mine = match < 0 ? 0.0f : q_there;
+            const float res = lane < kept ? fmaxf(p_norm - q_mine, 0.0f) : 0.0f;
+            const int rbits = (int)lilym_f32_bits(res);
+            const float u2 = (a.flags & F_UNIFORM) ? a.uniform2
+                                                   : lilym_uniform_for(a.seed, lilym_residual_step(step));
+            float r_cum = 0.0f, r_mine = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 64; ++i) {
+                r_cum += lilym_bits_f32((uint32_t)__builtin_amdgcn_readlane(rbits, i));
+                r_mine = lane == (uint32_t)i ? r_cum : r_mine;
+            }
+            const float r_total = r_cum;   // lanes past `kept` added 0
+            uint64_t picks;
+            if (r_total > 0.0f) {
+                picks = __ballot(lane < kept && u2 * r_total < r_mine);
+            } else {
+                // Only rounding gives a rejected proposal a massless residual: draw from p.
+                picks = __ballot(lane < kept && u2 * mass < mine);
+            }
+            const uint32_t slot = picks != 0ull ? (uint32_t)__builtin_ctzll(picks) : kept - 1u;
+            const uint32_t id = ~(uint32_t)__shfl((int)(uint32_t)c, (int)slot);
+            if (lane == 0) {
+                finish_token<DT>(a, sh, id, vocab, cfg.chain_rows != 0u);
+            }
+            return;
+        }
         const uint64_t hits = __ballot(lane < kept && u1 * mass < mine);
         const uint32_t slot = hits != 0ull ? (uint32_t)__builtin_ctzll(hits) : kept - 1u;
         const uint32_t id = ~(uint32_t)__shfl((int)(uint32_t)c, (int)slot);
