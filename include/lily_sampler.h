@@ -355,11 +355,12 @@ typedef struct lily_rows {
     uint32_t* dbg_counts_dev;            /* [rows][2] = candidates, kept */
 } lily_rows;
 
-/* Host cost and waits: the call packs one 224-byte descriptor per row into one of four pinned
- * staging buffers and enqueues its upload ahead of the launch.  It blocks only (a) when the
- * upload of the call four calls back has not finished, (b) the first time `rows` exceeds every
- * earlier call's (beyond 1024): the row table is reallocated, which drains the stream.  A caller
- * that must never hit (b) mid-run issues one call at its largest batch size first. */
+/* Host cost and waits: up to 8 rows travel as kernel arguments.  Beyond that the call packs one
+ * 224-byte descriptor per row into one of four pinned staging buffers, which the launch reads in
+ * place.  It blocks only (a) when the launch of the call four calls back has not finished,
+ * (b) the first time `rows` exceeds every earlier call's (beyond 1024): the staging buffers are
+ * reallocated, which drains the stream.  A caller that must never hit (b) mid-run issues one call
+ * at its largest batch size first. */
 int lily_sample_rows(lily_sampler_t* s, const lily_rows* batch);
 
 /* A resident batch: the row table is packed and uploaded once (lily_plan_set, which

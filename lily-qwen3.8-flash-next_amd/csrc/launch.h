@@ -23,6 +23,7 @@ hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc);
 hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const uint32_t* ids,
                               uint32_t* ctrl, uint32_t m, uint32_t pos0, uint32_t ratio,
                               uint32_t chain);
+hipError_t launch_copy_pieces(hipStream_t stream, const void* src, void* dst, size_t bytes);
 hipError_t launch_probe_read(hipStream_t stream, const void* base, uint32_t rows, uint64_t row_bytes,
                              uint64_t stride_bytes, uint32_t* out);
 hipError_t launch_copy_row(hipStream_t stream, const uint32_t* src, uint32_t* dst, uint32_t words,

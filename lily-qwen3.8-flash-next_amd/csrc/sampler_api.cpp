@@ -537,7 +537,10 @@ int pack_batch(const lily_rows* b, RowArgs* table) {
                 owners.emplace_back(reinterpret_cast<uintptr_t>(b->scratch[r]), r);
             }
         }
-        std::sort(owners.begin(), owners.end());
+        // (scratches made one after the other usually arrive in ascending order already)
+        if (!std::is_sorted(owners.begin(), owners.end())) {
+            std::sort(owners.begin(), owners.end());
+        }
         for (size_t i = 1; i < owners.size(); ++i) {
             if (owners[i].first != owners[i - 1].first) {
                 continue;
@@ -796,7 +799,7 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
         s->chain_ticket = s->chain_n + LILY_MAX_VERIFY_ROWS;
     }
     for (uint32_t i = 0; i < STAGE_SLOTS && err == hipSuccess; ++i) {
-        err = hipEventCreateWithFlags(&s->stage_done[i], hipEventDisableTiming);
+        err = hipEventCreateWithFlags(&s->stage_done[i], hipEventDisableTiming | hipEventReleaseToDevice);
     }
     if (err != hipSuccess) {
         lily_sampler_destroy(s);
@@ -1453,8 +1456,14 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     }
     LaunchPart parts[2];
     const uint32_t n_parts = plan_parts(s, s->stage[slot], b->rows, (int)b->dtype, b->vocab, parts);
-    HIP_TRY(hipMemcpyAsync(s->table_dev, s->stage[slot], (size_t)b->rows * sizeof(RowArgs),
-                           hipMemcpyHostToDevice, s->stream));
+    // A small kernel of the library's own carries the descriptors (224 bytes a row) from the
+    // pinned memory they were packed in to the device, ahead of the row kernels in the same
+    // stream.  (The copy engine's start-up costs about 100 us a call on this system; row kernels
+    // that read the descriptors in place pay a trip across the bus for every field the compiler
+    // chooses to load again, about 55 us on a launch of a thousand rows.)
+    RowArgs* table_mapped = nullptr;
+    HIP_TRY(hipHostGetDevicePointer(reinterpret_cast<void**>(&table_mapped), s->stage[slot], 0));
+    HIP_TRY(launch_copy_pieces(s->stream, table_mapped, s->table_dev, (size_t)b->rows * sizeof(RowArgs)));
     HIP_TRY(hipEventRecord(s->stage_done[slot], s->stream));
     s->stage_used[slot] = true;
     for (uint32_t q = 0; q < n_parts; ++q) {

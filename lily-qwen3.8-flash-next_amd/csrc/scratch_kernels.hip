@@ -122,10 +122,18 @@ __global__ void k_copy_row_u32(const uint32_t* src, uint32_t* dst, uint32_t word
     dst[i] = src[(size_t)row * words + i];
 }
 
+// n 16-byte pieces from src to dst (src may be pinned host memory mapped into the device).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) k_copy_pieces(const u32x4* src, u32x4* dst, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) {
+        dst[i] = src[i];
+    }
+}
+
 // The row kernel's access pattern with nothing else: one workgroup of 256 threads per row,
 // 16-byte loads, three blocks of four loads per thread requested ahead, an integer maximum as
 // the only arithmetic.  What this reaches is the ceiling a launch of the same shape can reach.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(256) k_probe_read(const u32x4* base, uint64_t row_chunks,
                                                     uint64_t stride_chunks, uint32_t* out) {
     const u32x4* row = base + (uint64_t)blockIdx.x * stride_chunks;
@@ -248,6 +256,16 @@ hipError_t launch_copy_row(hipStream_t stream, const uint32_t* src, uint32_t* ds
                            uint32_t rows, const uint32_t* row_dev) {
     hipLaunchKernelGGL(k_copy_row_u32, dim3((words + 255) / 256), dim3(256), 0, stream, src, dst,
                        words, rows, row_dev);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_pieces(hipStream_t stream, const void* src, void* dst, size_t bytes) {
+    const uint32_t n = (uint32_t)(bytes / 16u);
+    if (n == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(k_copy_pieces, dim3((n + 255u) / 256u), dim3(256), 0, stream,
+                       reinterpret_cast<const u32x4*>(src), reinterpret_cast<u32x4*>(dst), n);
     return hipGetLastError();
 }
 

@@ -2,12 +2,17 @@
 // runtime for device memory): what a host other than the Python tests sees.
 //
 //   harness cpu              host helpers only (no GPU): prints "cpu ok"
+//   harness time ROWS V N    N calls of lily_sample_rows over ROWS x V bf16 logits with host
+//                            descriptors every call (params, steps, scratches, penalties, logprobs):
+//                            prints the host time a call takes to return and the time per call
+//                            on the device (HIP events around the N calls)
 //   harness gpu V SEED       two draws through lily_sample_f32, two rows through
 //                            lily_sample_rows and the same rows through a plan; prints
 //                            "ids a b c d e f" - the Python side reproduces the inputs and
 //                            checks the ids against the oracle.
 #include <hip/hip_runtime_api.h>
 
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -161,6 +166,127 @@ static int gpu_mode(uint32_t vocab, uint32_t seed) {
     return 0;
 }
 
+static int time_mode(uint32_t rows, uint32_t vocab, uint32_t n) {
+    HIP(hipSetDevice(0));
+    hipStream_t stream;
+    HIP(hipStreamCreate(&stream));
+    lily_sampler_t* s = nullptr;
+    CHECK(lily_sampler_create(0, stream, &s));
+    // bf16 logits shaped like a language model's: a bulk in [-2, 2) and one id in about a
+    // thousand raised by 12 to 36; every row is a rotation of one such row (distinct rows, cheap
+    // to make)
+    std::vector<uint16_t> one(2 * (size_t)vocab);
+    for (uint32_t i = 0; i < 2 * vocab; ++i) {
+        const uint32_t j = i % vocab;
+        float v = 0.25f * logit_of(j, 3);
+        if ((j * 2654435761u >> 12) % 1021u == 0u) {
+            v += 12.0f + 1.5f * (logit_of(j, 9) + 8.0f);
+        }
+        uint32_t bits;
+        std::memcpy(&bits, &v, 4);
+        one[i] = (uint16_t)(bits >> 16);
+    }
+    uint16_t* x_dev = nullptr;
+    HIP(hipMalloc((void**)&x_dev, (size_t)rows * vocab * 2));
+    for (uint32_t r = 0; r < rows; ++r) {
+        HIP(hipMemcpy(x_dev + (size_t)r * vocab, one.data() + (r * 97u) % vocab, (size_t)vocab * 2,
+                      hipMemcpyHostToDevice));
+    }
+    std::vector<uint32_t> hist(vocab < 4096u ? vocab / 8u + 1u : 512u);
+    for (uint32_t i = 0; i < hist.size(); ++i) {
+        hist[i] = (i * 7919u + 11u) % vocab;
+    }
+    uint32_t *hist_dev = nullptr, *out_dev = nullptr;
+    float* lp_dev = nullptr;
+    HIP(hipMalloc((void**)&hist_dev, hist.size() * 4));
+    HIP(hipMemcpy(hist_dev, hist.data(), hist.size() * 4, hipMemcpyHostToDevice));
+    HIP(hipMalloc((void**)&out_dev, (size_t)rows * 4));
+    HIP(hipMalloc((void**)&lp_dev, (size_t)rows * 4));
+    std::vector<lily_scratch_t*> sc(rows);
+    std::vector<lily_sampling_params> ps(rows);
+    std::vector<uint32_t> steps(rows);
+    for (uint32_t r = 0; r < rows; ++r) {
+        CHECK(lily_scratch_create(s, vocab, &sc[r]));
+        CHECK(lily_scratch_add_history(sc[r], hist_dev, (uint32_t)hist.size()));
+        lily_params_greedy(&ps[r]);
+        ps[r].temperature = 0.8f;
+        ps[r].top_k = 64;
+        ps[r].top_p = 0.9f;
+        ps[r].repetition_penalty = 1.1f;
+        ps[r].presence_penalty = 0.2f;
+        ps[r].frequency_penalty = 0.1f;
+        ps[r].seed = 5000 + r;
+    }
+    lily_rows b;
+    std::memset(&b, 0, sizeof b);
+    b.rows = rows;
+    b.vocab = vocab;
+    b.dtype = LILY_BF16;
+    b.logits_dev = x_dev;
+    b.row_stride = vocab;
+    b.params = ps.data();
+    b.steps = steps.data();
+    b.scratch = sc.data();
+    b.out_ids_dev = out_dev;
+    b.out_logprobs_dev = lp_dev;
+    for (uint32_t w = 0; w < 5; ++w) {
+        CHECK(lily_sample_rows(s, &b));
+    }
+    CHECK(lily_sampler_synchronize(s));
+    hipEvent_t e0, e1;
+    HIP(hipEventCreate(&e0));
+    HIP(hipEventCreate(&e1));
+    double host_us = 0.0;
+    HIP(hipEventRecord(e0, stream));
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t r = 0; r < rows; ++r) {
+            steps[r] = 5 + i;
+        }
+        const auto t0 = std::chrono::steady_clock::now();
+        CHECK(lily_sample_rows(s, &b));
+        host_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+    }
+    HIP(hipEventRecord(e1, stream));
+    HIP(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    HIP(hipEventElapsedTime(&ms, e0, e1));
+    // the same call with the stream drained before each one: what the call itself costs the host
+    double alone_us = 0.0;
+    for (uint32_t i = 0; i < n; ++i) {
+        CHECK(lily_sampler_synchronize(s));
+        const auto t0 = std::chrono::steady_clock::now();
+        CHECK(lily_sample_rows(s, &b));
+        alone_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+    }
+    CHECK(lily_sampler_synchronize(s));
+    // which selects served one more call (workgroups: streaming, sparse or bitmap, exhaustive;
+    // and the reasons the streaming select gave up, as bits)
+    uint32_t* stats_dev = nullptr;
+    uint32_t stats[4] = {0, 0, 0, 0};
+    HIP(hipMalloc((void**)&stats_dev, sizeof stats));
+    HIP(hipMemcpy(stats_dev, stats, sizeof stats, hipMemcpyHostToDevice));
+    CHECK(lily_sampler_set_path_stats(s, stats_dev));
+    CHECK(lily_sample_rows(s, &b));
+    CHECK(lily_sampler_synchronize(s));
+    CHECK(lily_sampler_set_path_stats(s, nullptr));
+    HIP(hipMemcpy(stats, stats_dev, sizeof stats, hipMemcpyDeviceToHost));
+    HIP(hipFree(stats_dev));
+    std::printf("time rows %u vocab %u calls %u host_us_per_call %.1f device_us_per_call %.1f "
+                "host_us_per_call_idle_stream %.1f served_by %u %u %u gave_up_bits %u\n",
+                rows, vocab, n, host_us / n, ms * 1000.0 / n, alone_us / n, stats[0], stats[1], stats[2],
+                stats[3]);
+    for (uint32_t r = 0; r < rows; ++r) {
+        lily_scratch_destroy(sc[r]);
+    }
+    lily_sampler_destroy(s);
+    HIP(hipStreamDestroy(stream));
+    HIP(hipFree(x_dev));
+    HIP(hipFree(hist_dev));
+    HIP(hipFree(out_dev));
+    HIP(hipFree(lp_dev));
+    return 0;
+}
+
 int main(int argc, char** argv) {
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) {
         return cpu_mode();
@@ -168,6 +294,9 @@ int main(int argc, char** argv) {
     if (argc >= 4 && std::strcmp(argv[1], "gpu") == 0) {
         return gpu_mode((uint32_t)std::atoi(argv[2]), (uint32_t)std::atoi(argv[3]));
     }
-    std::fprintf(stderr, "usage: harness cpu | harness gpu VOCAB SEED\n");
+    if (argc >= 5 && std::strcmp(argv[1], "time") == 0) {
+        return time_mode((uint32_t)std::atoi(argv[2]), (uint32_t)std::atoi(argv[3]), (uint32_t)std::atoi(argv[4]));
+    }
+    std::fprintf(stderr, "usage: harness cpu | harness gpu VOCAB SEED | harness time ROWS VOCAB CALLS\n");
     return 2;
 }
