@@ -356,8 +356,8 @@ typedef struct lily_rows {
 } lily_rows;
 
 /* Host cost and waits: up to 8 rows travel as kernel arguments.  Beyond that the call packs one
- * 224-byte descriptor per row into one of four pinned staging buffers, which the launch reads in
- * place.  It blocks only (a) when the launch of the call four calls back has not finished,
+ * 224-byte descriptor per row into one of four pinned staging buffers, which a small kernel of
+ * the library carries to the device ahead of the draws.  It blocks only (a) when the launch of the call four calls back has not finished,
  * (b) the first time `rows` exceeds every earlier call's (beyond 1024): the staging buffers are
  * reallocated, which drains the stream.  A caller that must never hit (b) mid-run issues one call
  * at its largest batch size first. */
@@ -371,6 +371,52 @@ int lily_plan_create(lily_sampler_t* s, uint32_t max_rows, lily_plan_t** out);
 void lily_plan_destroy(lily_plan_t* p);
 int lily_plan_set(lily_plan_t* p, const lily_rows* batch);
 int lily_plan_run(lily_plan_t* p, uint32_t step_delta);
+
+/* ---- The producer of the logits and the draws from its summaries.
+ *
+ * Replaces the language-model head in front of the draws: `project_mat(mixed, lm_head, logits)`
+ * followed by one `sample_f32` per row (src/qwen4exp/batch.rs:573-593) and the single-row
+ * `gemv_quant(lm_head, mixed, logits)` + `sample_f32` (src/qwen4exp/model.rs:2959-2966,
+ * 4157-4169), for a head held in bf16 (the reference's quantised formats are dequantised by
+ * their owner first).  logits[r][v] = sum_i hidden[r][i] * weight[v][i], accumulated in f32 on
+ * the matrix cores and rounded to bf16 (nearest even).  Beside the logits the producer leaves,
+ * for every LILY_LOGIT_TILE_COLS columns of every row, the largest value and the sum of
+ * 2^((x - largest) * log2(e) / T[r]) over the tile - "summaries".  A row without allow-mask,
+ * penalties or bias list that is greedy or draws among at most 64 candidates is then drawn from
+ * the summaries and the few tiles that can hold a candidate (about k tiles of 256 bytes instead
+ * of the row); every other row of the batch is drawn from the logits as lily_sample_rows
+ * draws it.  Ids and log-probabilities are those of lily_sample_rows on the same logits. */
+#define LILY_LOGIT_TILE_COLS 128u
+
+typedef struct lily_lm_head {
+    const void* hidden_dev;   /* bf16 [rows][hidden_stride], d valid elements a row */
+    uint64_t hidden_stride;   /* elements; a multiple of 8; rows start at multiples of 16 bytes */
+    const void* weight_dev;   /* bf16 [vocab][weight_stride]: row v holds the weights of id v */
+    uint64_t weight_stride;   /* elements; a multiple of 8 */
+    uint32_t d;               /* a multiple of 64 */
+    uint32_t reserved;        /* must be 0 */
+    float* tile_max_dev;      /* out [rows][lily_lm_head_tiles(vocab)] */
+    float* tile_sum_dev;      /* out, same shape */
+} lily_lm_head;
+
+/* Summaries a row: ceil(vocab / LILY_LOGIT_TILE_COLS); at most 2048 are supported. */
+uint32_t lily_lm_head_tiles(uint32_t vocab);
+
+/* The producer alone.  temperatures: host [rows], the temperature each row will be drawn at, as
+ * lily_params_effective reports it (1 for a greedy row); NULL or an entry that is not a positive
+ * finite number: the sums of that row are not to be used.
+ * logits_dev: bf16 [rows][row_stride]. */
+int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* head, uint32_t rows, uint32_t vocab,
+                      const float* temperatures, void* logits_dev, uint64_t row_stride);
+
+/* The draws alone: batch->logits_dev (bf16, rows at multiples of 16 bytes) and the summaries must
+ * come from one producer call made with the temperatures of batch->params. */
+int lily_sample_rows_tiled(lily_sampler_t* s, const lily_rows* batch, const float* tile_max_dev,
+                           const float* tile_sum_dev);
+
+/* Both, in the sampler's stream: batch->logits_dev is where the logits are written (it is
+ * written to although the field is const), batch->vocab and batch->rows size the product. */
+int lily_lm_head_sample_rows(lily_sampler_t* s, const lily_lm_head* head, const lily_rows* batch);
 
 #ifdef __cplusplus
 }

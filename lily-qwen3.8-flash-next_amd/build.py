@@ -32,6 +32,8 @@ def units():
            for dt, kind in VARIANTS]
     out.append(("scratch_kernels.hip", "scratch_kernels.o", []))
     out.append(("static_entry.hip", "static_entry.o", []))
+    out.append(("lm_head.hip", "lm_head.o", []))
+    out.append(("rows_tiles.hip", "rows_tiles.o", []))
     out.append(("sampler_api.cpp", "sampler_api.o", []))
     return out
 

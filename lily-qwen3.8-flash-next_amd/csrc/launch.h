@@ -23,6 +23,18 @@ hipError_t launch_rebuild_listed(hipStream_t stream, const ScratchView& sc);
 hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const uint32_t* ids,
                               uint32_t* ctrl, uint32_t m, uint32_t pos0, uint32_t ratio,
                               uint32_t chain);
+// logits[rows, vocab] = hidden[rows, d] x weight[vocab, d]^T (bf16, strides in elements, d a
+// multiple of 64), with the largest value and the sum of 2^((x - largest) * c2_of_row[row]) of
+// every LILY_TILE_COLS columns in tile_max / tile_sum [rows, ceil(vocab / LILY_TILE_COLS)].
+hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
+                               const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
+                               uint32_t vocab, const float* c2_of_row, void* logits,
+                               uint64_t logits_stride, float* tile_max, float* tile_sum);
+// The draw of `rows` rows of cfg.table from the summaries ([.., tiles] each) and the few tiles of
+// the bf16 logits that matter; tile_row[r] = the summaries' row of table row r.
+hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const LaunchCfg& cfg,
+                             const float* tile_max, const float* tile_sum, uint32_t tiles,
+                             const uint32_t* tile_row);
 hipError_t launch_copy_pieces(hipStream_t stream, const void* src, void* dst, size_t bytes);
 hipError_t launch_probe_read(hipStream_t stream, const void* base, uint32_t rows, uint64_t row_bytes,
                              uint64_t stride_bytes, uint32_t* out);

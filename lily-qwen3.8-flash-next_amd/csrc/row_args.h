@@ -8,6 +8,11 @@
 
 namespace lily {
 
+// Columns of the logits that one summary (largest value, sum of exponentials) of the
+// logits' producer covers.
+#define LILY_TILE_COLS 128   // = LILY_LOGIT_TILE_COLS of the public header
+
+
 enum Mode : uint32_t {
     MODE_ARGMAX = 0,  // exact first-max over the raw row (greedy, nothing else asked)
     MODE_PLAIN = 1,   // sample_f32

@@ -1,0 +1,232 @@
+// rows_tiles.hip - the draw of rows whose logits came with the producer's summaries (the largest
+// value and the sum of exponentials of every LILY_TILE_COLS columns): the row is not read,
+// only the summaries and the few tiles that can hold one of its k largest values.
+#include <algorithm>
+
+#include "row_kernel.h"
+
+namespace lily {
+
+constexpr uint32_t TILES_PER_THREAD = 8;                 // wg_kth_largest takes 8 values a thread
+constexpr uint32_t TILES_MAX = NT * TILES_PER_THREAD;    // summaries of a row
+constexpr uint32_t TILE_CAND_CAP = 2048;                 // candidates gathered from the tiles
+
+// One workgroup per row (rows without mask, penalties or bias list, k <= STREAM_K_MAX; bf16).
+//   * The row's largest value is the largest summary; with at least k summaries at or above
+//     x, at least k values are: the k-th largest summary bounds the k-th largest value from
+//     below, and only tiles whose summary reaches it are read (16 lanes a tile, 16 bytes a
+//     lane); their values at or above the bound are the candidates.
+//   * The row's sum of exponentials is the summaries' sums brought to the row's reference.
+//   * More candidates than the buffer holds (ties by the thousand): the exhaustive select
+//     over the whole row takes over.
+// `tile_row[r]` is the row of the summaries that belongs to row r of the table.
+template <bool LSE>
+__global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float* tile_max,
+                                                      const float* tile_sum, uint32_t tiles,
+                                                      const uint32_t* tile_row) {
+    __shared__ Shared sh;
+    __shared__ uint16_t listed[TILES_MAX];
+    __shared__ uint32_t n_listed;
+    const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    if (tid == 0) {
+        tail_arrays(sh);
+        n_listed = 0;
+    }
+    RowArgs a;
+    load_row_args(a, table + blockIdx.y);
+    const uint32_t vocab = cfg.vocab;
+    const uint32_t step = a.step + cfg.step_delta;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    uint64_t* cand = dyn_lds;
+    const bool forced = (a.flags & F_FORCED) != 0;
+    if (forced && !want_lse) {
+        if (tid == 0) {
+            emit(a, a.forced, vocab);
+        }
+        return;
+    }
+    const size_t srow = (size_t)tile_row[blockIdx.y] * tiles;
+    float ms[TILES_PER_THREAD];
+    float best = NEG_INF;
+#pragma unroll
+    for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+        const uint32_t t = tid + j * NT;
+        ms[j] = t < tiles ? tile_max[srow + t] : NEG_INF;
+        best = fmaxf(best, ms[j]);
+    }
+    best = wave_max_f(best);
+    if (lane == 0) {
+        sh.red_f[w] = best;
+    }
+    __syncthreads();
+    float top = sh.red_f[0];
+    for (int i = 1; i < NWAVE; ++i) {
+        top = fmaxf(top, sh.red_f[i]);
+    }
+    __syncthreads();
+    phase(cfg, 1);
+
+    if (a.mode == MODE_ARGMAX && !forced) {
+        // The first of the largest values: the lowest tile that holds it, its lowest column.
+        uint32_t first = 0xffffffffu;
+#pragma unroll
+        for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+            if (ms[j] == top && top > NEG_INF) {
+                first = min(first, tid + j * NT);
+            }
+        }
+        first = wave_min_u32(first);
+        if (lane == 0) {
+            sh.red_i[w] = first;
+        }
+        __syncthreads();
+        first = min(min(sh.red_i[0], sh.red_i[1]), min(sh.red_i[2], sh.red_i[3]));
+        if (w == 0) {
+            uint32_t id = 0xffffffffu;
+            if (first != 0xffffffffu) {
+#pragma unroll
+                for (uint32_t h = 0; h < LILY_TILE_COLS / 64u; ++h) {
+                    const uint32_t col = first * LILY_TILE_COLS + h * 64u + lane;
+                    if (col < vocab && load_logit<LILY_BF16>(a.logits, col) == top) {
+                        id = min(id, col);
+                    }
+                }
+            }
+            id = wave_min_u32(id);
+            if (lane == 0) {
+                *a.out_id = id == 0xffffffffu ? 0u : id;
+            }
+        }
+        return;
+    }
+
+    if (want_lse) {
+        // sum over the tiles of tile_sum * 2^(tile_max * c2 - top * c2)
+        const float mc = top * a.c2;
+        double s = 0.0;
+#pragma unroll
+        for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+            const uint32_t t = tid + j * NT;
+            if (t < tiles && ms[j] > NEG_INF) {
+                s += (double)tile_sum[srow + t] * exp2((double)(ms[j] * a.c2) - (double)mc);
+            }
+        }
+        s = wave_sum_d(s);
+        if (lane == 0) {
+            sh.red_d[w] = s;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            double t = 0.0;
+            for (int i = 0; i < NWAVE; ++i) {
+                t += sh.red_d[i];
+            }
+            sh.lse_mc = (double)mc;
+            sh.lse_s = t;
+        }
+        __syncthreads();
+    }
+    if (forced) {
+        if (tid == 0) {
+            finish_token<LILY_BF16>(a, sh, a.forced, vocab);
+        }
+        return;
+    }
+
+    const uint32_t k = a.k;
+    const float bound = wg_kth_largest(ms, k, sh);   // F32_LOWEST with fewer than k finite summaries
+    phase(cfg, 2);
+    if (tid == 0) {
+        sh.n_cand = 0;
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+        if (ms[j] >= bound && ms[j] > NEG_INF) {
+            listed[atomicAdd(&n_listed, 1u)] = (uint16_t)(tid + j * NT);
+        }
+    }
+    __syncthreads();
+    const uint32_t n_t = n_listed;
+    // 16 lanes a tile, 8 values a lane; four rounds of loads asked for before the first is used
+    constexpr uint32_t LANES = LILY_TILE_COLS / 8u, PER_ROUND = NT / LANES;
+    const uint32_t sub = tid % LANES, slot = tid / LANES;
+    for (uint32_t r0 = 0; r0 < n_t; r0 += 4u * PER_ROUND) {
+        u32x4 q[4];
+        uint32_t col0[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t i = r0 + (uint32_t)u * PER_ROUND + slot;
+            const uint32_t t = listed[min(i, n_t - 1u)];
+            const uint32_t c = t * LILY_TILE_COLS + sub * 8u;
+            col0[u] = (i < n_t && c < vocab) ? c : 0xffffffffu;
+            // A row starts at a multiple of 16 bytes (the host checks), so these pieces do too:
+            // one that holds a valid column lies inside the row's pages, and the others are
+            // replaced by the row's last such piece.
+            q[u] = *reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) +
+                                                   (size_t)min(c, (vocab - 1u) & ~7u) * 2u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (col0[u] == 0xffffffffu) {
+                continue;
+            }
+            float v[8];
+            unpack<LILY_BF16>(q[u], v);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t id = col0[u] + (uint32_t)e;
+                if (id < vocab && v[e] >= bound) {
+                    const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                    if (at < TILE_CAND_CAP) {
+                        cand[at] = composite_of(v[e] / a.temperature, id);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    phase(cfg, 3);
+    uint32_t n = sh.n_cand;
+    __syncthreads();
+    bool sorted = false;
+    uint32_t took = 0;
+    if (n > TILE_CAND_CAP) {
+        took = 2;
+        select_exhaustive<LILY_BF16>(a, 0, vocab, k, want_lse, cand, cfg.cand_cap, sh);
+        n = min(sh.n_cand, cfg.cand_cap);
+    } else {
+        n = select_topk(cand, n, k, sh, sorted);
+    }
+    if (cfg.path_stats != nullptr && tid == 0) {
+        atomicAdd(&cfg.path_stats[took], 1u);
+    }
+    phase(cfg, 6);
+    tail<LILY_BF16, false>(a, vocab, step, n, sorted, cand, sh, cfg);
+    phase(cfg, 7);
+}
+
+hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
+                             const float* tile_max, const float* tile_sum, uint32_t tiles,
+                             const uint32_t* tile_row) {
+    if (tiles == 0 || tiles > TILES_MAX) {
+        return hipErrorInvalidValue;
+    }
+    LaunchCfg cfg = cfg_in;
+    cfg.slices = 1;
+    cfg.cand_cap = TILE_CAND_CAP;
+    const size_t tail_bytes = (size_t)LILY_SAMPLE_K_CAP * 8 + 3 * (size_t)LILY_SAMPLE_K_CAP * 4;
+    const size_t dyn_bytes = std::max(tail_bytes, (size_t)TILE_CAND_CAP * 8);
+    cfg.dyn_slots = (uint32_t)(dyn_bytes / 8);
+    const dim3 grid(1, rows), block(NT);
+    if (lse) {
+        hipLaunchKernelGGL(k_rows_tiles<true>, grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum,
+                           tiles, tile_row);
+    } else {
+        hipLaunchKernelGGL(k_rows_tiles<false>, grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum,
+                           tiles, tile_row);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace lily

@@ -74,6 +74,7 @@ struct DeviceScope {
 constexpr uint32_t WS_ROWS = 4096;      // rows that may span several workgroups
 constexpr uint32_t WS_SLOTS = 1u << 22; // candidate slots of the workspace (rows x slices x k)
 constexpr uint32_t STAGE_SLOTS = 4;
+constexpr size_t STAGE_ROW_BYTES = sizeof(RowArgs) + 16;   // a staged row: descriptor + two words + slack
 constexpr uint32_t TARGET_GROUPS = 512;  // workgroups a small batch is spread over
 
 }  // namespace
@@ -624,9 +625,10 @@ int ensure_table(lily_sampler* s, uint32_t rows) {
         s->stage_used[i] = false;
     }
     s->table_cap = s->stage_cap = 0;
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->table_dev), (size_t)cap * sizeof(RowArgs)));
+    // (behind the descriptors: two words a row for the calls that draw from summaries)
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->table_dev), (size_t)cap * STAGE_ROW_BYTES));
     for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {
-        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&s->stage[i]), (size_t)cap * sizeof(RowArgs),
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&s->stage[i]), (size_t)cap * STAGE_ROW_BYTES,
                               hipHostMallocDefault));
     }
     s->table_cap = s->stage_cap = cap;
@@ -1472,6 +1474,210 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
         }
     }
     return LILY_OK;
+}
+
+// ---- the logits' producer and the draws from its summaries
+
+namespace {
+
+size_t round16(size_t n) { return (n + 15u) & ~(size_t)15u; }
+
+// Takes the next staging buffer (waiting, if need be, for the call that used it four calls back).
+int stage_acquire(lily_sampler* s, uint32_t rows, uint32_t* slot_out) {
+    if (int rc = ensure_table(s, rows)) {
+        return rc;
+    }
+    const uint32_t slot = s->stage_next;
+    s->stage_next = (slot + 1) % STAGE_SLOTS;
+    if (s->stage_used[slot]) {
+        HIP_TRY(hipEventSynchronize(s->stage_done[slot]));
+    }
+    *slot_out = slot;
+    return LILY_OK;
+}
+
+// Carries the first `bytes` of the staging buffer to the device (same offsets in table_dev).
+int stage_commit(lily_sampler* s, uint32_t slot, size_t bytes) {
+    void* mapped = nullptr;
+    HIP_TRY(hipHostGetDevicePointer(&mapped, s->stage[slot], 0));
+    HIP_TRY(launch_copy_pieces(s->stream, mapped, s->table_dev, round16(bytes)));
+    HIP_TRY(hipEventRecord(s->stage_done[slot], s->stream));
+    s->stage_used[slot] = true;
+    return LILY_OK;
+}
+
+float c2_of_temperature(float t) {
+    const float c = (float)(1.4426950408889634 / (double)t);
+    return std::isfinite(c) ? c : 0.0f;
+}
+
+int check_head(const lily_lm_head* h, uint32_t rows, uint32_t vocab, const void* logits_dev,
+               uint64_t row_stride) {
+    if (h == nullptr || h->hidden_dev == nullptr || h->weight_dev == nullptr || h->tile_max_dev == nullptr ||
+        h->tile_sum_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "hidden, weight, tile_max and tile_sum are required");
+    }
+    if (rows == 0 || vocab == 0 || logits_dev == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "rows, vocab and the logits buffer are required");
+    }
+    if (h->d == 0 || h->d % 64u != 0) {
+        return fail(LILY_ERR_INVALID_ARG, "d must be a positive multiple of 64");
+    }
+    if (h->hidden_stride < h->d || h->weight_stride < h->d || h->hidden_stride % 8u != 0 ||
+        h->weight_stride % 8u != 0 || reinterpret_cast<uintptr_t>(h->hidden_dev) % 16u != 0 ||
+        reinterpret_cast<uintptr_t>(h->weight_dev) % 16u != 0) {
+        return fail(LILY_ERR_INVALID_ARG,
+                    "hidden and weight rows must start at multiples of 16 bytes and hold d elements");
+    }
+    if (row_stride < vocab) {
+        return fail(LILY_ERR_INVALID_ARG, "row_stride is shorter than the vocabulary");
+    }
+    return LILY_OK;
+}
+
+// Rows the summaries serve: no mask, no penalties, no bias list, the row given as it is, and a
+// greedy row or a plain draw among at most STREAM_K_MAX candidates.
+bool tiles_serve(const RowArgs& r) {
+    if (r.allow != nullptr || (r.flags & F_PEN) || r.n_bias != 0 || r.sel_row != nullptr) {
+        return false;
+    }
+    return r.mode == MODE_ARGMAX || (r.mode == MODE_PLAIN && r.k <= STREAM_K_MAX);
+}
+
+// The draws of batch `b` with the summaries of its logits at hand; with `h` set, the logits and
+// the summaries are produced first, in the same stream.
+int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, const float* tile_max,
+                    const float* tile_sum) {
+    if (b == nullptr || b->rows == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "empty batch");
+    }
+    if (b->dtype != LILY_BF16) {
+        return fail(LILY_ERR_INVALID_ARG, "summaries describe bf16 logits");
+    }
+    if (tile_max == nullptr || tile_sum == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "tile_max and tile_sum are required");
+    }
+    if (reinterpret_cast<uintptr_t>(b->logits_dev) % 16u != 0 || b->row_stride % 8u != 0) {
+        return fail(LILY_ERR_INVALID_ARG, "rows of logits must start at multiples of 16 bytes");
+    }
+    const uint32_t rows = b->rows, tiles = lily_lm_head_tiles(b->vocab);
+    if (tiles > 2048u) {
+        return fail(LILY_ERR_INVALID_ARG, "vocabulary beyond 2048 summaries a row");
+    }
+    if (h != nullptr) {
+        if (int rc = check_head(h, rows, b->vocab, b->logits_dev, b->row_stride)) {
+            return rc;
+        }
+    }
+    ON_DEVICE(s->device);
+    uint32_t slot = 0;
+    if (int rc = stage_acquire(s, rows, &slot)) {
+        return rc;
+    }
+    static thread_local std::vector<RowArgs> packed;
+    packed.resize(rows);
+    if (int rc = pack_batch(b, packed.data())) {
+        return rc;
+    }
+    // staged: the descriptors (rows the summaries serve first), each such row's row of the
+    // summaries, every row's exponent scale (the producer's)
+    char* stage = reinterpret_cast<char*>(s->stage[slot]);
+    RowArgs* table = reinterpret_cast<RowArgs*>(stage);
+    const size_t idx_off = (size_t)rows * sizeof(RowArgs), c2_off = idx_off + round16((size_t)rows * 4);
+    uint32_t* tile_row = reinterpret_cast<uint32_t*>(stage + idx_off);
+    float* c2 = reinterpret_cast<float*>(stage + c2_off);
+    uint32_t served = 0;
+    bool lse = false;
+    for (uint32_t r = 0; r < rows; ++r) {
+        c2[r] = std::isfinite(packed[r].c2) ? packed[r].c2 : 0.0f;
+        if (tiles_serve(packed[r])) {
+            lse = lse || packed[r].out_logprob != nullptr;
+            tile_row[served] = r;
+            table[served++] = packed[r];
+        }
+    }
+    uint32_t others = served;
+    for (uint32_t r = 0; r < rows; ++r) {
+        if (!tiles_serve(packed[r])) {
+            table[others++] = packed[r];
+        }
+    }
+    LaunchPart parts[2];
+    const uint32_t n_parts =
+        served < rows ? plan_parts(s, table + served, rows - served, (int)b->dtype, b->vocab, parts) : 0u;
+    if (int rc = stage_commit(s, slot, c2_off + (size_t)rows * 4)) {
+        return rc;
+    }
+    const char* dev = reinterpret_cast<const char*>(s->table_dev);
+    if (h != nullptr) {
+        HIP_TRY(launch_lm_head_bf16(s->stream, h->hidden_dev, h->hidden_stride, h->weight_dev,
+                                    h->weight_stride, rows, h->d, b->vocab,
+                                    reinterpret_cast<const float*>(dev + c2_off),
+                                    const_cast<void*>(b->logits_dev), b->row_stride, h->tile_max_dev,
+                                    h->tile_sum_dev));
+    }
+    if (served != 0) {
+        LaunchCfg cfg;
+        fill_cfg(s, &cfg, b->vocab, 1, 1, 0, s->table_dev);
+        attach_trace(s, &cfg, served);
+        HIP_TRY(launch_rows_tiles(s->stream, lse, served, cfg, tile_max, tile_sum, tiles,
+                                  reinterpret_cast<const uint32_t*>(dev + idx_off)));
+    }
+    for (uint32_t q = 0; q < n_parts; ++q) {
+        if (int rc = launch_part(s, parts[q], s->table_dev + served, (int)b->dtype, b->vocab, 0, false)) {
+            return rc;
+        }
+    }
+    return LILY_OK;
+}
+
+}  // namespace
+
+static_assert(LILY_TILE_COLS == LILY_LOGIT_TILE_COLS, "the kernels' tile is the header's");
+
+uint32_t lily_lm_head_tiles(uint32_t vocab) {
+    return (vocab + LILY_LOGIT_TILE_COLS - 1u) / LILY_LOGIT_TILE_COLS;
+}
+
+int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* h, uint32_t rows, uint32_t vocab,
+                      const float* temperatures, void* logits_dev, uint64_t row_stride) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    if (int rc = check_head(h, rows, vocab, logits_dev, row_stride)) {
+        return rc;
+    }
+    ON_DEVICE(s->device);
+    uint32_t slot = 0;
+    if (int rc = stage_acquire(s, rows, &slot)) {
+        return rc;
+    }
+    float* c2 = reinterpret_cast<float*>(s->stage[slot]);
+    for (uint32_t r = 0; r < rows; ++r) {
+        c2[r] = temperatures != nullptr ? c2_of_temperature(temperatures[r]) : 0.0f;
+    }
+    if (int rc = stage_commit(s, slot, (size_t)rows * 4)) {
+        return rc;
+    }
+    HIP_TRY(launch_lm_head_bf16(s->stream, h->hidden_dev, h->hidden_stride, h->weight_dev, h->weight_stride,
+                                rows, h->d, vocab, reinterpret_cast<const float*>(s->table_dev), logits_dev,
+                                row_stride, h->tile_max_dev, h->tile_sum_dev));
+    return LILY_OK;
+}
+
+int lily_sample_rows_tiled(lily_sampler_t* s, const lily_rows* b, const float* tile_max_dev,
+                           const float* tile_sum_dev) {
+    if (s == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler is null");
+    }
+    return rows_with_tiles(s, nullptr, b, tile_max_dev, tile_sum_dev);
+}
+
+int lily_lm_head_sample_rows(lily_sampler_t* s, const lily_lm_head* h, const lily_rows* b) {
+    if (s == nullptr || h == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "sampler and head are required");
+    }
+    return rows_with_tiles(s, h, b, h->tile_max_dev, h->tile_sum_dev);
 }
 
 int lily_plan_create(lily_sampler_t* s, uint32_t max_rows, lily_plan_t** out) {

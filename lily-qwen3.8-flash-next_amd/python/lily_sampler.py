@@ -94,6 +94,16 @@ class _Rows(C.Structure):
     ]
 
 
+class _LmHead(C.Structure):
+    _fields_ = [("hidden_dev", C.c_void_p), ("hidden_stride", C.c_uint64),
+                ("weight_dev", C.c_void_p), ("weight_stride", C.c_uint64),
+                ("d", C.c_uint32), ("reserved", C.c_uint32),
+                ("tile_max_dev", C.c_void_p), ("tile_sum_dev", C.c_void_p)]
+
+
+LOGIT_TILE_COLS = 128
+
+
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
@@ -153,7 +163,12 @@ def _load():
         "lily_plan_set": [vp, C.POINTER(_Rows)],
         "lily_plan_run": [vp, u32],
         "lily_params_validate": [P],
+        "lily_lm_head_bf16": [vp, C.POINTER(_LmHead), u32, u32, C.POINTER(C.c_float), vp, u64],
+        "lily_sample_rows_tiled": [vp, C.POINTER(_Rows), vp, vp],
+        "lily_lm_head_sample_rows": [vp, C.POINTER(_LmHead), C.POINTER(_Rows)],
     }
+    L.lily_lm_head_tiles.restype = C.c_uint32
+    L.lily_lm_head_tiles.argtypes = [C.c_uint32]
     for name, args in sigs.items():
         getattr(L, name).restype = C.c_int
         getattr(L, name).argtypes = args
@@ -432,6 +447,45 @@ class Sampler:
 
     def plan(self, logits, params, steps, out_ids, **kw):
         return Plan(self, logits, params, steps, out_ids, **kw)
+
+    # -- the logits' producer and the draws from its summaries,
+    #    src/qwen4exp/batch.rs:573-593, src/qwen4exp/model.rs:4157-4169
+    @staticmethod
+    def _head(hidden, weight, tile_max, tile_sum):
+        for t, name in ((hidden, "hidden"), (weight, "weight")):
+            if t.dtype != torch.bfloat16 or t.dim() != 2 or t.stride(1) != 1:
+                raise SamplerError(-1, f"{name} must be BF16 [rows, d], rows contiguous")
+        if hidden.shape[1] != weight.shape[1]:
+            raise SamplerError(-1, "hidden and weight differ in d")
+        h = _LmHead()
+        h.hidden_dev, h.hidden_stride = hidden.data_ptr(), hidden.stride(0)
+        h.weight_dev, h.weight_stride = weight.data_ptr(), weight.stride(0)
+        h.d = hidden.shape[1]
+        h.tile_max_dev = _ptr(tile_max, torch.float32)
+        h.tile_sum_dev = _ptr(tile_sum, torch.float32)
+        return h
+
+    def lm_head(self, hidden, weight, temperatures, logits, tile_max, tile_sum):
+        """lily_lm_head_bf16: logits[rows, V] (bf16) = hidden @ weight.T with the summaries."""
+        rows, vocab = logits.shape
+        if logits.dtype != torch.bfloat16 or logits.stride(1) != 1:
+            raise SamplerError(-1, "logits must be BF16 [rows, V], rows contiguous")
+        h = self._head(hidden, weight, tile_max, tile_sum)
+        tarr = None if temperatures is None else (C.c_float * rows)(*[float(t) for t in temperatures])
+        _check(_lib.lily_lm_head_bf16(self._h, C.byref(h), rows, vocab, tarr, logits.data_ptr(),
+                                      logits.stride(0) if rows > 1 else vocab))
+
+    def sample_rows_tiled(self, logits, tile_max, tile_sum, params, steps, out_ids, **kw):
+        r, keep = self._rows(logits, params, steps, out_ids, **kw)
+        _check(_lib.lily_sample_rows_tiled(self._h, C.byref(r), _ptr(tile_max, torch.float32),
+                                           _ptr(tile_sum, torch.float32)))
+        return keep
+
+    def lm_head_sample_rows(self, hidden, weight, logits, tile_max, tile_sum, params, steps, out_ids, **kw):
+        r, keep = self._rows(logits, params, steps, out_ids, **kw)
+        h = self._head(hidden, weight, tile_max, tile_sum)
+        _check(_lib.lily_lm_head_sample_rows(self._h, C.byref(h), C.byref(r)))
+        return keep
 
 
 class Plan:

@@ -1,0 +1,271 @@
+"""The logits' producer (bf16 head on the matrix cores, with summaries) and the draws from its
+summaries (src/qwen4exp/batch.rs:573-593, src/qwen4exp/model.rs:4157-4169).
+
+Bar:
+  * logits: each within one bf16 step of hidden @ weight.T computed in f64 from the same bf16
+    inputs (the f32 accumulation of 512 products and the rounding to bf16 are what may differ);
+  * summaries: tile_max bit-exact against the stored logits, tile_sum within 2e-6 relative of
+    the f64 sum over the stored logits;
+  * draws: ids (and the candidate lists) bit-exact against the oracle ON THE STORED LOGITS,
+    log-probabilities within 1e-5 * max(1, |logprob|) - the same bar as lily_sample_rows, whose
+    results the tiled draws must equal.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import lily_sampler as LS
+import lily_workloads as W
+import oracle as O
+from gpu_util import K_CAP, dev, ls_params, o_params
+
+LOGPROB_RTOL = 1e-5
+TILE = LS.LOGIT_TILE_COLS
+
+
+@pytest.fixture(scope="module")
+def sampler():
+    s = LS.Sampler(0)
+    yield s
+    s.close()
+
+
+def _bf16(x):
+    return torch.from_numpy(W.to_bf16_bits(x).view(np.int16)).to(dev()).view(torch.bfloat16)
+
+
+def _bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _peaked_head(rng, rows, d, vocab, peaks=40, gain=6.0):
+    """Hidden states and a head whose logits look like a language model's: a bulk from random
+    weights and, per row, a few ids whose weight rows point along the row's hidden state."""
+    hidden = rng.normal(0.0, 1.0, (rows, d)).astype(np.float32)
+    weight = rng.normal(0.0, 2.0 / np.sqrt(d), (vocab, d)).astype(np.float32)
+    for r in range(rows):
+        ids = rng.choice(vocab, peaks, replace=False)
+        scale = rng.uniform(0.3, 1.0, peaks).astype(np.float32) * gain / d
+        weight[ids] += scale[:, None] * hidden[r][None, :]
+    return hidden, weight
+
+
+def _produce(sampler, hidden, weight, temps, rows, vocab, stride=None):
+    stride = stride or vocab
+    h, w = _bf16(hidden), _bf16(weight)
+    buf = torch.full((rows, stride), 7.0, dtype=torch.bfloat16, device=dev())
+    logits = buf[:, :vocab]
+    tiles = (vocab + TILE - 1) // TILE
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    sampler.lm_head(h, w, temps, logits, tmax, tsum)
+    sampler.synchronize()
+    return h, w, buf, logits, tmax, tsum
+
+
+def _check_product(h, w, logits, tmax, tsum, temps):
+    rows, vocab = logits.shape
+    got = W.bf16_bits_to_f32(_bits(logits.contiguous()))
+    ref = (h.double() @ w.double().T).cpu().numpy()
+    # one bf16 step at the reference's magnitude (2^-8 relative is half a step), plus the f32
+    # accumulation's error on sums that cancel
+    tol = np.abs(ref) * 2.0 ** -7 + 1e-4
+    assert np.all(np.abs(got - ref) <= tol), float(np.max(np.abs(got - ref) - tol))
+    tiles = tmax.shape[1]
+    pad = tiles * TILE - vocab
+    g = np.pad(got, ((0, 0), (0, pad)), constant_values=-np.inf).reshape(rows, tiles, TILE)
+    assert np.array_equal(tmax.cpu().numpy(), g.max(axis=2))
+    for r in range(rows):
+        t = temps[r] if temps is not None else 0.0
+        if not t > 0.0:
+            continue
+        c2 = np.float32(1.4426950408889634 / t)
+        top = (g[r].max(axis=1).astype(np.float32) * c2).astype(np.float64)
+        want = np.exp2(g[r].astype(np.float64) * np.float64(c2) - top[:, None]).sum(axis=1)
+        assert np.allclose(tsum[r].cpu().numpy(), want, rtol=2e-6, atol=0), r
+
+
+@pytest.mark.parametrize("rows,d,vocab", [(5, 256, 1000), (130, 512, 4096 + 77), (1, 64, 128)])
+def test_producer_against_f64_product(sampler, rows, d, vocab):
+    rng = np.random.default_rng(rows * 1000 + d)
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(20, vocab // 8))
+    temps = [0.0 if r % 5 == 4 else 0.5 + 0.1 * (r % 7) for r in range(rows)]
+    stride = ((vocab + 7) // 8) * 8 + 8
+    h, w, buf, logits, tmax, tsum = _produce(sampler, hidden, weight, temps, rows, vocab, stride)
+    _check_product(h, w, logits, tmax, tsum, temps)
+    # nothing behind a row's last column is written
+    assert torch.all(buf[:, vocab:] == 7.0)
+
+
+def _draw_all(sampler, fn, logits, params_kw, steps, scratch=None, **kw):
+    rows = logits.shape[0]
+    out = torch.full((rows,), -1, dtype=torch.int32, device=dev())
+    lp = torch.full((rows,), 123.0, dtype=torch.float32, device=dev())
+    dbg_ids = torch.full((rows, K_CAP), -1, dtype=torch.int32, device=dev())
+    dbg_counts = torch.zeros((rows, 2), dtype=torch.int32, device=dev())
+    keep = fn(out, lp, dbg_ids, dbg_counts)
+    sampler.synchronize()
+    del keep
+    return (out.cpu().numpy().astype(np.int64), lp.cpu().numpy(), dbg_ids.cpu().numpy(),
+            dbg_counts.cpu().numpy())
+
+
+def _check_draws(stored, ids, lps, cand, counts, params_kw, steps, hist_counts=None, forced=None):
+    for r, kw in enumerate(params_kw):
+        if forced is not None and forced[r] is not None:
+            assert ids[r] == forced[r], r
+            continue
+        p = o_params(**kw)
+        if p.temperature == 0.0:
+            assert ids[r] == O.argmax(stored[r]), r
+            continue
+        c = None if hist_counts is None or hist_counts[r] is None else hist_counts[r].copy()
+        d = O.sample(stored[r], c, p, steps[r], want_logprob=True)
+        n_fin = int(np.sum(d.cand_adj > -np.inf))
+        assert counts[r, 0] == n_fin, (r, counts[r, 0], n_fin)
+        assert np.array_equal(cand[r, :n_fin], d.cand_ids[:n_fin].astype(np.int64)), r
+        assert counts[r, 1] == d.n_kept, r
+        assert ids[r] == d.chosen, (r, ids[r], d.chosen)
+        assert abs(lps[r] - d.logprob) <= LOGPROB_RTOL * max(1.0, abs(d.logprob)), (r, lps[r], d.logprob)
+
+
+def _mixed_params(rows):
+    out = []
+    for r in range(rows):
+        if r % 6 == 5:
+            out.append(dict())   # greedy
+        elif r % 6 == 4:
+            out.append(dict(temperature=0.9, top_k=200, top_p=0.95, seed=900 + r))   # k beyond the summaries' reach
+        else:
+            out.append(dict(temperature=0.6 + 0.1 * (r % 4), top_k=(1, 20, 64, 40)[r % 4],
+                            top_p=(1.0, 0.9, 0.95, 0.8)[r % 4], min_p=0.02 * (r % 3), seed=700 + r))
+    return out
+
+
+@pytest.mark.parametrize("rows,d,vocab", [(24, 256, 151_936), (9, 128, 5000), (3, 64, 333)])
+def test_tiled_draws_equal_the_oracle_on_the_stored_logits(sampler, rows, d, vocab):
+    rng = np.random.default_rng(vocab + rows)
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(60, vocab // 6))
+    params_kw = _mixed_params(rows)
+    params = [ls_params(**kw) for kw in params_kw]
+    temps = [p.effective()[0] for p in params]
+    steps = [3 + r for r in range(rows)]
+    h, w, buf, logits, tmax, tsum = _produce(sampler, hidden, weight, temps, rows, vocab,
+                                             ((vocab + 7) // 8) * 8)
+    stored = _bits(logits.contiguous())
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    sampler.set_path_stats(stats)
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    sampler.set_path_stats(None)
+    _check_draws(stored, ids, lps, cand, counts, params_kw, steps)
+    if vocab > 100_000:   # (with fewer summaries than k every value is a candidate: too many)
+        assert stats.cpu().numpy()[2] == 0, "no row fell back to the exhaustive select"
+    # and the ordinary call on the same logits gives the same
+    ids2, lps2, cand2, counts2 = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows(
+            logits, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    assert np.array_equal(ids, ids2)
+    sampled = [r for r, kw in enumerate(params_kw) if kw]
+    assert np.allclose(lps[sampled], lps2[sampled], rtol=LOGPROB_RTOL, atol=LOGPROB_RTOL)
+
+
+def test_fused_call_with_rows_the_summaries_do_not_serve(sampler):
+    """One call: product, then every row's draw - plain rows from the summaries, rows under
+    penalties, masks, bias lists or a forced token by the selects that read the row."""
+    rows, d, vocab = 40, 256, 20_000
+    rng = np.random.default_rng(77)
+    hidden, weight = _peaked_head(rng, rows, d, vocab)
+    params_kw, hist, forced = [], [], []
+    for r in range(rows):
+        kw = dict(temperature=0.7 + 0.05 * (r % 5), top_k=(20, 64, 50)[r % 3], top_p=0.92, seed=100 + r)
+        if r % 4 == 1:
+            kw.update(repetition_penalty=1.1, presence_penalty=0.3, frequency_penalty=0.1)
+        if r % 10 == 7:
+            kw = dict()
+        params_kw.append(kw)
+        hist.append(rng.integers(0, vocab, 300).astype(np.int32) if r % 4 == 1 else None)
+        forced.append(int(rng.integers(0, vocab)) if r % 8 == 6 else None)
+    params = [ls_params(**kw) for kw in params_kw]
+    steps = [11] * rows
+    scratch, hist_counts = [], []
+    for hh in hist:
+        if hh is None:
+            scratch.append(None)
+            hist_counts.append(None)
+        else:
+            sc = LS.SamplerScratch(sampler, vocab)
+            sc.add_history(torch.from_numpy(hh).to(dev()))
+            scratch.append(sc)
+            hist_counts.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+    h, w = _bf16(hidden), _bf16(weight)
+    logits = torch.zeros(rows, vocab, dtype=torch.bfloat16, device=dev())
+    tiles = (vocab + TILE - 1) // TILE
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.lm_head_sample_rows(
+            h, w, logits, tmax, tsum, params, steps, out, scratch=scratch, forced=forced,
+            out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    temps = [p.effective()[0] for p in params]
+    _check_product(h, w, logits, tmax, tsum, temps)
+    stored = _bits(logits)
+    _check_draws(stored, ids, lps, cand, counts, params_kw, steps, hist_counts=hist_counts, forced=forced)
+    # forced rows with a log-probability: that of the forced id under the row's own settings
+    for r in range(rows):
+        if forced[r] is not None and params_kw[r]:
+            d = O.sample(stored[r], None if hist_counts[r] is None else hist_counts[r].copy(),
+                         o_params(**params_kw[r]), steps[r], want_logprob=True, forced=forced[r])
+            assert abs(lps[r] - d.logprob) <= LOGPROB_RTOL * max(1.0, abs(d.logprob)), r
+
+
+def test_ties_by_the_thousand_take_the_exhaustive_select(sampler):
+    """Constant logits: every value ties at the bound, the candidates overflow the buffer and the
+    select that reads the whole row decides - ids still the oracle's."""
+    rows, vocab = 3, 6000
+    x = np.zeros((rows, vocab), dtype=np.float32)
+    x[1, 4000:] = -1.0
+    x[2, ::2] = 0.5
+    bits = W.to_bf16_bits(x)
+    logits = torch.from_numpy(bits.view(np.int16)).to(dev()).view(torch.bfloat16)
+    tiles = (vocab + TILE - 1) // TILE
+    g = np.pad(x, ((0, 0), (0, tiles * TILE - vocab)), constant_values=-np.inf).reshape(rows, tiles, TILE)
+    params_kw = [dict(temperature=1.0, top_k=50, top_p=1.0, seed=5 + r) for r in range(rows)]
+    c2 = np.float32(1.4426950408889634)
+    tmax_np = g.max(axis=2).astype(np.float32)
+    tsum_np = np.exp2(g.astype(np.float64) * c2 - (tmax_np * c2).astype(np.float64)[:, :, None]).sum(axis=2)
+    tmax = torch.from_numpy(tmax_np).to(dev())
+    tsum = torch.from_numpy(tsum_np.astype(np.float32)).to(dev())
+    params = [ls_params(**kw) for kw in params_kw]
+    steps = [0, 1, 2]
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    sampler.set_path_stats(stats)
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    sampler.set_path_stats(None)
+    _check_draws(bits, ids, lps, cand, counts, params_kw, steps)
+    assert stats.cpu().numpy()[2] >= 1
+
+
+def test_rejections(sampler):
+    rows, d, vocab = 2, 64, 256
+    h = torch.zeros(rows, d, dtype=torch.bfloat16, device=dev())
+    w = torch.zeros(vocab, d, dtype=torch.bfloat16, device=dev())
+    logits = torch.zeros(rows, vocab, dtype=torch.bfloat16, device=dev())
+    tmax = torch.zeros(rows, 2, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, 2, dtype=torch.float32, device=dev())
+    with pytest.raises(LS.SamplerError):
+        sampler.lm_head(h[:, :32], w[:, :32], None, logits, tmax, tsum)     # d not a multiple of 64
+    f32 = torch.zeros(rows, vocab, dtype=torch.float32, device=dev())
+    out = torch.zeros(rows, dtype=torch.int32, device=dev())
+    with pytest.raises(LS.SamplerError):
+        sampler.sample_rows_tiled(f32, tmax, tsum, [ls_params()] * rows, [0, 0], out)   # f32 logits
+    sampler.synchronize()
