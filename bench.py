@@ -252,6 +252,67 @@ def main():
                                          "paths": paths_of(sampler, lambda i: p4.run(0))}
         p4.close()
 
+    # ---- the logits' producer (bf16 head on the matrix cores, d = 4096) and the draws from its
+    # summaries: config 5's draw settings without penalties (rows under penalties read the row)
+    head = None
+    if not a.no_others:
+        head = {}
+        d_model = 4096
+        tiles = (vocab + LS.LOGIT_TILE_COLS - 1) // LS.LOGIT_TILE_COLS
+        gen = torch.Generator(device=device)
+        gen.manual_seed(11)
+        w_f32 = torch.randn(vocab, d_model, device=device, generator=gen) * (2.0 / d_model ** 0.5)
+        for b_rows in (4, rows):
+            hid = torch.randn(b_rows, d_model, device=device, generator=gen)
+            # a bulk N(0, 2^2) and, per row, 40 ids whose weights point along the row's hidden state
+            for r in range(min(b_rows, 128)):
+                ids = torch.randint(0, vocab, (40,), device=device, generator=gen)
+                gain = (torch.rand(40, 1, device=device, generator=gen) * 0.7 + 0.3) * (6.0 / d_model)
+                w_f32[ids] += gain * hid[r][None, :]
+            hb, wb = hid.to(torch.bfloat16), w_f32.to(torch.bfloat16)
+            lg = torch.zeros(b_rows, vocab, dtype=torch.bfloat16, device=device)
+            tmax = torch.zeros(b_rows, tiles, dtype=torch.float32, device=device)
+            tsum = torch.zeros(b_rows, tiles, dtype=torch.float32, device=device)
+            hp = [LS.SamplingParams.greedy(temperature=0.8, top_k=64, top_p=0.9, seed=5000 + r)
+                  for r in range(b_rows)]
+            ho = torch.zeros(b_rows, dtype=torch.int32, device=device)
+            hl = torch.zeros(b_rows, dtype=torch.float32, device=device)
+            torch.cuda.synchronize()
+            n_h = 10 if b_rows > 64 else 30
+            ms_head = time_steps(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum),
+                                 n_h, 2)
+            ms_fused = time_steps(stream, lambda i: sampler.lm_head_sample_rows(
+                hb, wb, lg, tmax, tsum, hp, [i] * b_rows, ho, out_logprobs=hl), n_h, 2)
+
+            def behind_a_head(draw, n=4):
+                """GPU time of a draw call: n of them queued while a head launch still runs, so
+                that the host's packing is off the clock."""
+                sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for i in range(n):
+                    draw(i)
+                e1.record(stream)
+                e1.synchronize()
+                return e0.elapsed_time(e1) / n * 1e3
+
+            us_tiled = behind_a_head(lambda i: sampler.sample_rows_tiled(lg, tmax, tsum, hp, [i] * b_rows, ho,
+                                                                        out_logprobs=hl))
+            us_rows = behind_a_head(lambda i: sampler.sample_rows(lg, hp, [i] * b_rows, ho, out_logprobs=hl))
+            flops = 2.0 * b_rows * d_model * vocab
+            head[f"b{b_rows}"] = {
+                "rows": b_rows, "d": d_model,
+                "head_us": ms_head * 1e3,
+                "head_TFLOPs": flops / (ms_head * 1e-3) / 1e12,
+                "head_frac_of_mfma_peak": flops / (ms_head * 1e-3) / 1e12 / 2500.0,
+                "head_weight_GBs": vocab * d_model * 2 / (ms_head * 1e-3) / 1e9,
+                "head_plus_draws_us": ms_fused * 1e3,
+                "draws_from_summaries_us": us_tiled,
+                "draws_from_rows_us": us_rows,
+            }
+            del hb, wb, lg
+        del w_f32
+
     line = {
         "metric": "rows/s and us/step at B=4 and B=1024 x151,936 vocab; achieved HBM GB/s",
         "value": rows / (ms * 1e-3),
@@ -285,6 +346,7 @@ def main():
             "target_us": 20.0,
         },
         "other_configs": others,
+        "lm_head": head,
         "roofline": {
             "bound": "hbm",
             "achieved": achieved,

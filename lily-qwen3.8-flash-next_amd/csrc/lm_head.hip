@@ -14,34 +14,47 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t w32x4 __attribute__((ext_vector_type(4)));
 
-namespace head {
-constexpr int BM = 128;              // rows of a workgroup's tile
-constexpr int BN = LILY_TILE_COLS;   // columns of a workgroup's tile = the width of a summary
-constexpr int BK = 64;               // depth of one staged piece
-constexpr int ROW_BYTES = BK * 2 + 16;   // a staged row and its padding: rows 8 apart share banks
-constexpr int OPERAND_BYTES = BM * ROW_BYTES;
-constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;     // hidden rows, then weight rows
-constexpr int LDS_BYTES = 2 * STAGE_BYTES;         // two stages
-static_assert(BM == BN, "one loader serves both operands");
-static_assert(LDS_BYTES >= 4 * BM * 4 + BM * 4, "the epilogue's reductions reuse the stages");
-}  // namespace head
+// A workgroup's tile and how its four waves share it.  WAVES_M x (4 / WAVES_M) waves, each
+// MI x NI products of 32 x 32; the tile is WAVES_M * MI * 32 rows by 128 columns (the width of a
+// summary), staged BK columns of d at a time, AHEAD stages of loads in flight (what is in flight
+// has to cover the memory's latency at the rate the tiles consume it).
+template <int WAVES_M_, int MI_, int NI_, int BK_, int AHEAD_, int RESIDENT_>
+struct HeadTile {
+    static constexpr int RESIDENT = RESIDENT_;   // workgroups a compute unit is to hold (bounds the registers)
+    static constexpr int WAVES_M = WAVES_M_, WAVES_N = 4 / WAVES_M_, MI = MI_, NI = NI_, BK = BK_;
+    static constexpr int AHEAD = AHEAD_;   // stages asked from memory ahead of the one being multiplied
+    static constexpr int BM = WAVES_M * MI * 32;
+    static constexpr int BN = WAVES_N * NI * 32;
+    static constexpr int PIECES = BK / 8;                  // 16-byte pieces of a staged row
+    static constexpr int ROW_BYTES = BK * 2 + 16;          // padded: 8 rows cover all banks
+    static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;  // hidden rows, then weight rows
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;      // two stages
+    static constexpr int A_PER = BM * PIECES / 256, B_PER = BN * PIECES / 256;   // pieces a thread brings
+    static_assert(BN == LILY_TILE_COLS, "a workgroup's columns are one summary");
+    static_assert(BM * PIECES % 256 == 0 && BN * PIECES % 256 == 0 && A_PER >= 1, "whole pieces per thread");
+    static_assert(LDS_BYTES >= (WAVES_N + 2) * BM * 4, "the epilogue's reductions reuse the stages");
+};
 
-// One workgroup of 256 threads per 128 x 128 tile of the logits; its four waves take a
-// quarter each (64 x 64: 2 x 2 products of 32 x 32 x 16).  Both operands are contiguous along
-// d, which is how a lane of the matrix instruction wants its 8 values: rows are staged in
-// LDS 64 columns of d at a time (16-byte loads from memory one stage ahead of the
-// arithmetic, 16-byte reads out of LDS, rows padded so that 8 rows cover all banks).
+// One workgroup of 256 threads per tile of the logits.  Both operands are contiguous along d,
+// which is how a lane of the matrix instruction wants its 8 values: rows are staged in LDS BK
+// columns of d at a time (16-byte loads from memory several stages ahead of the arithmetic,
+// 16-byte reads out of LDS).  The shapes: 32 rows for a decode step of a few sequences (the weights are
+// then read once at the speed of memory and the matrix cores idle), 256 rows - each wave 128 x
+// 64, six operand reads out of LDS for eight products - for a batch, whose bound is the matrix
+// cores and, just behind, the bandwidth of LDS.
 //
-// Workgroups are numbered so that the tiles over one block of 128 weight rows - one per 128
+// Workgroups are numbered so that the tiles over one block of 128 weight rows - one per BM
 // rows of the batch - run on the same XCD one after the other: the weight rows, the large
 // operand, are then fetched from memory once and served to the other tiles by that XCD's L2.
-__global__ void __launch_bounds__(256)
+template <class T>
+__global__ void __launch_bounds__(256, T::RESIDENT)
 k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
                const uint16_t* __restrict__ weight, uint64_t weight_stride, uint32_t rows,
                uint32_t d, uint32_t vocab, const float* __restrict__ c2_of_row,
                uint16_t* __restrict__ logits, uint64_t logits_stride, float* __restrict__ tile_max,
                float* __restrict__ tile_sum, uint32_t tiles_per_row, uint32_t m_tiles) {
-    using namespace head;
+    constexpr int BM = T::BM, BN = T::BN, BK = T::BK, MI = T::MI, NI = T::NI, ROW_BYTES = T::ROW_BYTES;
     extern __shared__ __align__(16) char lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
@@ -50,42 +63,56 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         return;
     }
     const uint32_t m0 = m_tile * BM, n0 = n_tile * BN;
-    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    const uint32_t wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
 
-    // The loader: thread t brings pieces t, t + 256, ... of 16 bytes; a staged row has 8.
-    const uint16_t* src_h[4];
-    const uint16_t* src_w[4];
-    uint32_t dst[4];
+    // The loader: thread t brings pieces t, t + 256, ... of 16 bytes of either operand.
+    const uint16_t* src_h[T::A_PER];
+    const uint16_t* src_w[T::B_PER];
+    uint32_t dst_h[T::A_PER], dst_w[T::B_PER];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t piece = tid + 256u * (uint32_t)i, r = piece >> 3, kc = piece & 7u;
-        const uint32_t hr = min(m0 + r, rows - 1u), wr = min(n0 + r, vocab - 1u);
-        src_h[i] = hidden + (uint64_t)hr * hidden_stride + kc * 8u;
-        src_w[i] = weight + (uint64_t)wr * weight_stride + kc * 8u;
-        dst[i] = r * ROW_BYTES + kc * 16u;
+    for (int i = 0; i < T::A_PER; ++i) {
+        const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
+        src_h[i] = hidden + (uint64_t)min(m0 + r, rows - 1u) * hidden_stride + kc * 8u;
+        dst_h[i] = r * ROW_BYTES + kc * 16u;
     }
-    w32x4 next_h[4], next_w[4];
-    auto fetch = [&](uint32_t k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            next_h[i] = *reinterpret_cast<const w32x4*>(src_h[i] + k0);
-            next_w[i] = *reinterpret_cast<const w32x4*>(src_w[i] + k0);
+    for (int i = 0; i < T::B_PER; ++i) {
+        const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
+        src_w[i] = weight + (uint64_t)min(n0 + r, vocab - 1u) * weight_stride + kc * 8u;
+        dst_w[i] = T::A_BYTES + r * ROW_BYTES + kc * 16u;
+    }
+    // ring[j]: the loads of a stage on their way (registers), written to LDS one step before use
+    w32x4 ring_h[T::AHEAD][T::A_PER], ring_w[T::AHEAD][T::B_PER];
+    auto fetch = [&](w32x4 (&h)[T::A_PER], w32x4 (&w)[T::B_PER], uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < T::A_PER; ++i) {
+            h[i] = *reinterpret_cast<const w32x4*>(src_h[i] + k0);
+        }
+#pragma unroll
+        for (int i = 0; i < T::B_PER; ++i) {
+            w[i] = *reinterpret_cast<const w32x4*>(src_w[i] + k0);
         }
     };
-    auto stage = [&](uint32_t buf) {
-        char* base = lds + buf * STAGE_BYTES;
+    // (`real` false: a step past the end of d, run so that every pass of the loop is alike -
+    // the hidden rows are staged as zeros and add nothing)
+    auto stage = [&](const w32x4 (&h)[T::A_PER], const w32x4 (&w)[T::B_PER], uint32_t buf, bool real) {
+        char* base = lds + buf * T::STAGE_BYTES;
+        const uint32_t keep = real ? 0xffffffffu : 0u;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<w32x4*>(base + dst[i]) = next_h[i];
-            *reinterpret_cast<w32x4*>(base + OPERAND_BYTES + dst[i]) = next_w[i];
+        for (int i = 0; i < T::A_PER; ++i) {
+            *reinterpret_cast<w32x4*>(base + dst_h[i]) = h[i] & keep;
+        }
+#pragma unroll
+        for (int i = 0; i < T::B_PER; ++i) {
+            *reinterpret_cast<w32x4*>(base + dst_w[i]) = w[i];
         }
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[MI][NI];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
+        for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 acc[mi][ni][v] = 0.0f;
@@ -94,71 +121,90 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     }
     // A lane's operand values: row lane % 32 of the 32, 8 values of d from (lane / 32) * 8 on.
     const uint32_t frag = (lane & 31u) * ROW_BYTES + (lane >> 5) * 16u;
-    const uint32_t a_at = wm * 64u * ROW_BYTES + frag;
-    const uint32_t b_at = OPERAND_BYTES + wn * 64u * ROW_BYTES + frag;
+    const uint32_t a_at = wm * (MI * 32u) * ROW_BYTES + frag;
+    const uint32_t b_at = T::A_BYTES + wn * (NI * 32u) * ROW_BYTES + frag;
 
-    fetch(0);
-    stage(0);
+    // Every load and every write to LDS below is unconditional (past the end of d the last
+    // stage is asked for again): the compiler then counts the loads in flight and waits for
+    // the oldest only; with a branch around any of them it waits for all.
+    const uint32_t steps = d / BK, padded = (steps + T::AHEAD - 1u) / T::AHEAD * T::AHEAD;
+    const uint32_t k_last = d - BK;
+    fetch(ring_h[0], ring_w[0], 0);
+    stage(ring_h[0], ring_w[0], 0, true);
+#pragma unroll
+    for (int j = 0; j < T::AHEAD; ++j) {
+        fetch(ring_h[j], ring_w[j], min(((uint32_t)j + 1u) * BK, k_last));   // ring[j] <- stage j + 1
+    }
     __syncthreads();
-    const uint32_t steps = d / BK;
-    for (uint32_t s = 0; s < steps; ++s) {
-        const uint32_t buf = s & 1u;
-        if (s + 1u < steps) {
-            fetch((s + 1u) * BK);
-        }
-        const char* base = lds + buf * STAGE_BYTES;
+    for (uint32_t s0 = 0; s0 < padded; s0 += T::AHEAD) {
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-            bf16x8 a[2], b[2];
+        for (int j = 0; j < T::AHEAD; ++j) {
+            const uint32_t s = s0 + (uint32_t)j;
+            const uint32_t buf = s & 1u;
+            // ring[j] holds stage s + 1: into the other LDS stage (nobody reads it: the barrier
+            // that closed step s - 1 saw to that), and the registers ask for stage s + 1 + AHEAD
+            stage(ring_h[j], ring_w[j], buf ^ 1u, s + 1u < steps);
+            fetch(ring_h[j], ring_w[j], min((s + 1u + T::AHEAD) * BK, k_last));
+            const char* base = lds + buf * T::STAGE_BYTES;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + kk * 32);
-                b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + kk * 32);
-            }
+            for (int kk = 0; kk < BK / 16; ++kk) {
+                bf16x8 a[MI], b[NI];
 #pragma unroll
-            for (int mi = 0; mi < 2; ++mi) {
+                for (int i = 0; i < MI; ++i) {
+                    a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + kk * 32);
+                }
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni) {
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+                for (int i = 0; i < NI; ++i) {
+                    b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + kk * 32);
+                }
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        acc[mi][ni] =
+                            __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+                    }
                 }
             }
+            __syncthreads();
         }
-        if (s + 1u < steps) {
-            stage(buf ^ 1u);   // nobody reads that stage: the barrier below closed the step before
-        }
-        __syncthreads();
     }
 
     // ---- epilogue.  Element v of a lane's 16 sits in row 8 * (v / 4) + 4 * (lane / 32) + v % 4
-    // of its 32 x 32 product, column lane % 32.  Values are rounded to bf16 first: the maximum
-    // and the sum describe the logits as they are stored.
-    float* red = reinterpret_cast<float*>(lds);              // [2][BM] by column half
-    float* row_max = red + 2 * BM;                           // [BM]
+    // of its 32 x 32 product, column lane % 32.  Values are rounded to bf16 first, in place: the
+    // maximum and the sum describe the logits as they are stored.
+    float* red = reinterpret_cast<float*>(lds);              // [WAVES_N][BM] by column group
+    float* row_max = red + T::WAVES_N * BM;                  // [BM]
     float* row_c2 = row_max + BM;                            // [BM]
     if (tid < (uint32_t)BM) {
         row_c2[tid] = c2_of_row[min(m0 + tid, rows - 1u)];
     }
     const float NEG = -__builtin_huge_valf();
-    uint32_t bits[2][2][16];
-    float val[2][2][16];
+    bool in_vocab[NI];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int ni = 0; ni < NI; ++ni) {
+        in_vocab[ni] = n0 + wn * (NI * 32u) + (uint32_t)ni * 32u + (lane & 31u) < vocab;
+    }
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const bool in_vocab = n0 + wn * 64u + (uint32_t)ni * 32u + (lane & 31u) < vocab;
+    for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const float f = acc[mi][ni][v];   // (a bit_cast of the element itself reads element 0)
                 const uint32_t u = __builtin_bit_cast(uint32_t, f);
-                // round to nearest even; a NaN stays one (quiet), and counts as -inf below
+                // round to nearest even; a NaN stays one (quiet)
                 const uint32_t r = (u & 0x7fffffffu) > 0x7f800000u ? ((u >> 16) | 0x40u)
                                                                    : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-                bits[mi][ni][v] = r;
-                const float x = __builtin_bit_cast(float, r << 16);
-                val[mi][ni][v] = (in_vocab && x == x) ? x : NEG;
+                acc[mi][ni][v] = __builtin_bit_cast(float, r << 16);
             }
         }
     }
+    // what a stored value counts for: a NaN and a column outside the vocabulary count as -inf
+    auto worth = [&](int mi, int ni, int v) -> float {
+        const float x = acc[mi][ni][v];
+        return (in_vocab[ni] && x == x) ? x : NEG;
+    };
     auto across32 = [&](float x, auto op) -> float {
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) {
@@ -167,14 +213,19 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         return x;
     };
     auto row_of = [&](int mi, int v) -> uint32_t {
-        return wm * 64u + (uint32_t)mi * 32u + 8u * (uint32_t)(v >> 2) + 4u * (lane >> 5) + (uint32_t)(v & 3);
+        return wm * (MI * 32u) + (uint32_t)mi * 32u + 8u * (uint32_t)(v >> 2) + 4u * (lane >> 5) +
+               (uint32_t)(v & 3);
     };
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const float m = across32(fmaxf(val[mi][0][v], val[mi][1][v]),
-                                     [](float p, float q) { return fmaxf(p, q); });
+            float m = NEG;
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                m = fmaxf(m, worth(mi, ni, v));
+            }
+            m = across32(m, [](float p, float q) { return fmaxf(p, q); });
             if ((lane & 31u) == 0u) {
                 red[wn * BM + row_of(mi, v)] = m;
             }
@@ -182,19 +233,24 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     }
     __syncthreads();
     if (tid < (uint32_t)BM) {
-        row_max[tid] = fmaxf(red[tid], red[BM + tid]);
+        float m = red[tid];
+#pragma unroll
+        for (int g = 1; g < T::WAVES_N; ++g) {
+            m = fmaxf(m, red[g * BM + tid]);
+        }
+        row_max[tid] = m;
     }
     __syncthreads();
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t r = row_of(mi, v);
             const float c = row_c2[r], top = row_max[r] * c;
             float e = 0.0f;
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni) {
-                const float x = val[mi][ni][v];
+            for (int ni = 0; ni < NI; ++ni) {
+                const float x = worth(mi, ni, v);
                 e += x > NEG ? __builtin_amdgcn_exp2f(__builtin_fmaf(x, c, -top)) : 0.0f;
             }
             e = across32(e, [](float p, float q) { return p + q; });
@@ -206,48 +262,81 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     __syncthreads();
     if (tid < (uint32_t)BM && m0 + tid < rows) {
         const size_t at = (size_t)(m0 + tid) * tiles_per_row + n_tile;
+        float e = red[tid];
+#pragma unroll
+        for (int g = 1; g < T::WAVES_N; ++g) {
+            e += red[g * BM + tid];
+        }
         tile_max[at] = row_max[tid];
-        tile_sum[at] = row_max[tid] > NEG ? red[tid] + red[BM + tid] : 0.0f;
+        tile_sum[at] = row_max[tid] > NEG ? e : 0.0f;
     }
     // the logits themselves
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const uint32_t col = n0 + wn * 64u + (uint32_t)ni * 32u + (lane & 31u);
+        for (int ni = 0; ni < NI; ++ni) {
+            const uint32_t col = n0 + wn * (NI * 32u) + (uint32_t)ni * 32u + (lane & 31u);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t r = m0 + row_of(mi, v);
                 if (r < rows && col < vocab) {
-                    logits[(uint64_t)r * logits_stride + col] = (uint16_t)bits[mi][ni][v];
+                    const float f = acc[mi][ni][v];
+                    logits[(uint64_t)r * logits_stride + col] = (uint16_t)(__builtin_bit_cast(uint32_t, f) >> 16);
                 }
             }
         }
     }
 }
 
-hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
-                               const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
-                               uint32_t vocab, const float* c2_of_row, void* logits,
-                               uint64_t logits_stride, float* tile_max, float* tile_sum) {
-    using namespace head;
-    static bool sized = false;
-    if (!sized) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_lm_head_bf16),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+template <class T>
+static hipError_t launch_head_shape(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
+                                    const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
+                                    uint32_t vocab, const float* c2_of_row, void* logits,
+                                    uint64_t logits_stride, float* tile_max, float* tile_sum) {
+    static bool sized[64] = {};
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        return e;
+    }
+    if (device < 0 || device >= 64 || !sized[device]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_lm_head_bf16<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
         if (e != hipSuccess) {
             return e;
         }
-        sized = true;
+        if (device >= 0 && device < 64) {
+            sized[device] = true;
+        }
     }
-    const uint32_t tiles_per_row = (vocab + BN - 1u) / BN, m_tiles = (rows + BM - 1u) / BM;
+    const uint32_t tiles_per_row = (vocab + T::BN - 1u) / T::BN, m_tiles = (rows + T::BM - 1u) / T::BM;
     const uint32_t groups = (tiles_per_row + 7u) / 8u;
-    hipLaunchKernelGGL(k_lm_head_bf16, dim3(8u * groups * m_tiles), dim3(256), LDS_BYTES, stream,
+    hipLaunchKernelGGL(k_lm_head_bf16<T>, dim3(8u * groups * m_tiles), dim3(256), T::LDS_BYTES, stream,
                        reinterpret_cast<const uint16_t*>(hidden), hidden_stride,
                        reinterpret_cast<const uint16_t*>(weight), weight_stride, rows, d, vocab,
                        c2_of_row, reinterpret_cast<uint16_t*>(logits), logits_stride, tile_max, tile_sum,
                        tiles_per_row, m_tiles);
     return hipGetLastError();
+}
+
+hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
+                               const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
+                               uint32_t vocab, const float* c2_of_row, void* logits,
+                               uint64_t logits_stride, float* tile_max, float* tile_sum) {
+#define LILY_HEAD_ARGS                                                                              \
+    stream, hidden, hidden_stride, weight, weight_stride, rows, d, vocab, c2_of_row, logits,        \
+        logits_stride, tile_max, tile_sum
+    if (rows <= 32u) {
+        return launch_head_shape<HeadTile<1, 1, 1, 64, 4, 3>>(LILY_HEAD_ARGS);
+    }
+    if (rows <= 64u) {
+        return launch_head_shape<HeadTile<1, 2, 1, 64, 3, 3>>(LILY_HEAD_ARGS);
+    }
+    if (rows <= 128u) {
+        return launch_head_shape<HeadTile<2, 2, 2, 64, 3, 2>>(LILY_HEAD_ARGS);
+    }
+    return launch_head_shape<HeadTile<2, 4, 2, 32, 3, 2>>(LILY_HEAD_ARGS);
+#undef LILY_HEAD_ARGS
 }
 
 }  // namespace lily
