@@ -372,6 +372,37 @@ void lily_plan_destroy(lily_plan_t* p);
 int lily_plan_set(lily_plan_t* p, const lily_rows* batch);
 int lily_plan_run(lily_plan_t* p, uint32_t step_delta);
 
+/* ---- Insertions: what the thinking control decides, as the `forced` input of the next steps.
+ *
+ * The reference's ThinkingControl::decide / decide_stop (src/thinking.rs:485-608) read decoded
+ * text and stay on the host; each answers with an Action - Keep, Before(ids), After(ids),
+ * Replace(ids) - about the token a step has just drawn.  This queue turns those answers into
+ * per-row forced tokens of the steps that follow (lily_rows.forced), and does on the device,
+ * in stream order, what the reference's TODO at thinking.rs:587-592 leaves undone: a replaced
+ * draw leaves the row's penalty counts.
+ *   AFTER   (drawn, ids): drawn stays emitted; the next steps are forced to ids[0..n).
+ *   BEFORE  (drawn, ids): ids are emitted first, then drawn again as a forced token; its count
+ *           from the draw is taken back so that it is counted once.
+ *   REPLACE (drawn, ids): drawn is not emitted: its count is taken back; ids follow.
+ * Host state only; the un-counting is lily_scratch_uncount on the row's scratch (NULL: none). */
+typedef struct lily_insertions lily_insertions_t;
+typedef enum lily_insert_kind {
+    LILY_INSERT_AFTER = 0,
+    LILY_INSERT_BEFORE = 1,
+    LILY_INSERT_REPLACE = 2
+} lily_insert_kind;
+int lily_insertions_create(uint32_t rows, lily_insertions_t** out);
+void lily_insertions_destroy(lily_insertions_t* q);
+int lily_insertions_push(lily_insertions_t* q, uint32_t row, lily_insert_kind kind, uint32_t drawn,
+                         const uint32_t* ids, uint32_t n, lily_scratch_t* scratch);
+/* Fills forced_out[0..rows) for the next lily_sample_rows call (LILY_NO_TOKEN = the row draws)
+ * and removes what it hands out.  Returns the number of rows that are forced. */
+uint32_t lily_insertions_next(lily_insertions_t* q, uint32_t* forced_out);
+/* Tokens still queued for `row` (0 for a row out of range). */
+uint32_t lily_insertions_pending(const lily_insertions_t* q, uint32_t row);
+/* Drops what is queued for `row` (a finished or cancelled request). */
+void lily_insertions_clear(lily_insertions_t* q, uint32_t row);
+
 /* ---- The producer of the logits and the draws from its summaries.
  *
  * Replaces the language-model head in front of the draws: `project_mat(mixed, lm_head, logits)`

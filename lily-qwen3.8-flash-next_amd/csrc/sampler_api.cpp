@@ -1476,6 +1476,95 @@ int lily_sample_rows(lily_sampler_t* s, const lily_rows* b) {
     return LILY_OK;
 }
 
+// ---- insertions (src/thinking.rs:485-608: Action::{Before, After, Replace})
+
+struct lily_insertions {
+    std::vector<std::vector<uint32_t>> pending;   // per row, next token first
+    std::vector<size_t> head;                      // tokens of pending[row] already handed out
+};
+
+int lily_insertions_create(uint32_t rows, lily_insertions_t** out) {
+    if (out == nullptr || rows == 0) {
+        return fail(LILY_ERR_INVALID_ARG, "insertions need rows > 0");
+    }
+    *out = nullptr;
+    lily_insertions* q = new (std::nothrow) lily_insertions;
+    if (q == nullptr) {
+        return fail(LILY_ERR_NOMEM, "out of host memory");
+    }
+    q->pending.resize(rows);
+    q->head.assign(rows, 0);
+    *out = q;
+    return LILY_OK;
+}
+
+void lily_insertions_destroy(lily_insertions_t* q) { delete q; }
+
+int lily_insertions_push(lily_insertions_t* q, uint32_t row, lily_insert_kind kind, uint32_t drawn,
+                         const uint32_t* ids, uint32_t n, lily_scratch_t* scratch) {
+    if (q == nullptr || row >= q->pending.size()) {
+        return fail(LILY_ERR_INVALID_ARG, "row outside the insertions' rows");
+    }
+    if (n != 0 && ids == nullptr) {
+        return fail(LILY_ERR_INVALID_ARG, "ids is null");
+    }
+    if (kind != LILY_INSERT_AFTER && kind != LILY_INSERT_BEFORE && kind != LILY_INSERT_REPLACE) {
+        return fail(LILY_ERR_INVALID_ARG, "unknown kind of insertion");
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        if (ids[i] == LILY_NO_TOKEN) {
+            return fail(LILY_ERR_RANGE, "an inserted id cannot be LILY_NO_TOKEN");
+        }
+    }
+    if (kind != LILY_INSERT_AFTER && scratch != nullptr) {
+        // the draw counted `drawn`; BEFORE emits it again as a forced token (counted there),
+        // REPLACE never emits it
+        if (int rc = lily_scratch_uncount(scratch, drawn)) {
+            return rc;
+        }
+    }
+    std::vector<uint32_t>& p = q->pending[row];
+    if (q->head[row] == p.size()) {
+        p.clear();
+        q->head[row] = 0;
+    }
+    p.insert(p.end(), ids, ids + n);
+    if (kind == LILY_INSERT_BEFORE) {
+        p.push_back(drawn);
+    }
+    return LILY_OK;
+}
+
+uint32_t lily_insertions_next(lily_insertions_t* q, uint32_t* forced_out) {
+    if (q == nullptr || forced_out == nullptr) {
+        return 0;
+    }
+    uint32_t forced = 0;
+    for (size_t r = 0; r < q->pending.size(); ++r) {
+        if (q->head[r] < q->pending[r].size()) {
+            forced_out[r] = q->pending[r][q->head[r]++];
+            ++forced;
+        } else {
+            forced_out[r] = LILY_NO_TOKEN;
+        }
+    }
+    return forced;
+}
+
+uint32_t lily_insertions_pending(const lily_insertions_t* q, uint32_t row) {
+    if (q == nullptr || row >= q->pending.size()) {
+        return 0;
+    }
+    return (uint32_t)(q->pending[row].size() - q->head[row]);
+}
+
+void lily_insertions_clear(lily_insertions_t* q, uint32_t row) {
+    if (q != nullptr && row < q->pending.size()) {
+        q->pending[row].clear();
+        q->head[row] = 0;
+    }
+}
+
 // ---- the logits' producer and the draws from its summaries
 
 namespace {

@@ -167,6 +167,18 @@ def _load():
         "lily_sample_rows_tiled": [vp, C.POINTER(_Rows), vp, vp],
         "lily_lm_head_sample_rows": [vp, C.POINTER(_LmHead), C.POINTER(_Rows)],
     }
+    L.lily_insertions_create.restype = C.c_int
+    L.lily_insertions_create.argtypes = [u32, C.POINTER(vp)]
+    L.lily_insertions_push.restype = C.c_int
+    L.lily_insertions_push.argtypes = [vp, u32, C.c_int, u32, C.POINTER(u32), u32, vp]
+    L.lily_insertions_next.restype = u32
+    L.lily_insertions_next.argtypes = [vp, C.POINTER(u32)]
+    L.lily_insertions_pending.restype = u32
+    L.lily_insertions_pending.argtypes = [vp, u32]
+    L.lily_insertions_clear.restype = None
+    L.lily_insertions_clear.argtypes = [vp, u32]
+    L.lily_insertions_destroy.restype = None
+    L.lily_insertions_destroy.argtypes = [vp]
     L.lily_lm_head_tiles.restype = C.c_uint32
     L.lily_lm_head_tiles.argtypes = [C.c_uint32]
     for name, args in sigs.items():
@@ -633,6 +645,47 @@ class TokenSlots:
             if self._s._h:
                 _lib.lily_token_slots_destroy(self._h)
             self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+INSERT_AFTER, INSERT_BEFORE, INSERT_REPLACE = 0, 1, 2
+
+
+class Insertions:
+    """lily_insertions_*: the thinking control's Action::{After, Before, Replace}
+    (src/thinking.rs:485-608) as the forced tokens of the steps that follow."""
+
+    def __init__(self, rows):
+        self._h = C.c_void_p()
+        self.rows = rows
+        _check(_lib.lily_insertions_create(rows, C.byref(self._h)))
+
+    def push(self, row, kind, drawn, ids, scratch=None):
+        arr = (C.c_uint32 * max(1, len(ids)))(*[int(i) for i in ids])
+        _check(_lib.lily_insertions_push(self._h, row, kind, int(drawn), arr, len(ids),
+                                         scratch._h if scratch is not None else None))
+
+    def next(self):
+        """(forced list for lily_rows: None = the row draws, number of forced rows)."""
+        out = (C.c_uint32 * self.rows)()
+        n = _lib.lily_insertions_next(self._h, out)
+        return [None if v == NO_TOKEN else int(v) for v in out], int(n)
+
+    def pending(self, row):
+        return int(_lib.lily_insertions_pending(self._h, row))
+
+    def clear(self, row):
+        _lib.lily_insertions_clear(self._h, row)
+
+    def close(self):
+        if self._h:
+            _lib.lily_insertions_destroy(self._h)
+            self._h = C.c_void_p()
 
     def __del__(self):
         try:

@@ -130,3 +130,55 @@ def test_a_sequence_moved_into_a_batch_slot_and_back_draws_what_it_draws_alone()
     for x in batch + [engine]:
         x.close()
     s.close()
+
+
+def test_insertions_keep_the_counts_the_oracle_keeps():
+    """The thinking control's answers as forced tokens (src/thinking.rs:485-608), with the
+    replaced draw taken out of the penalty counts (the TODO at thinking.rs:587-592).  Two rows
+    decode under SAMPLED; at step 2 row 0's draw is replaced by three ids, at step 3 row 1 gets
+    two ids in front of its draw.  Every token equals the oracle's on the same counts, and the
+    counts at the end hold exactly the tokens that were emitted."""
+    sampler = LS.Sampler(0)
+    rng = np.random.default_rng(31)
+    rows, steps_n, VOCAB = 2, 9, 30_011
+    x = rng.normal(0.0, 2.0, (steps_n, rows, VOCAB)).astype(np.float32)
+    sc = [LS.SamplerScratch(sampler, VOCAB) for _ in range(rows)]
+    counts = [np.zeros(VOCAB, dtype=np.uint32) for _ in range(rows)]
+    q = LS.Insertions(rows)
+    params = [LS.SamplingParams.greedy(**dict(SAMPLED, seed=7 + r)) for r in range(rows)]
+    oparams = [O.params(**dict(SAMPLED, seed=7 + r)) for r in range(rows)]
+    out = torch.zeros(rows, dtype=torch.int32, device=dev())
+    emitted = [[] for _ in range(rows)]
+    replace_ids, before_ids = [VOCAB - 1, 17, 17], [5, 6]
+    for step in range(steps_n):
+        forced, _ = q.next()
+        logits = torch.from_numpy(x[step]).to(dev())
+        keep = sampler.sample_rows(logits, params, [step] * rows, out, scratch=sc, forced=forced)
+        sampler.synchronize()
+        del keep
+        got = out.cpu().numpy()
+        for r in range(rows):
+            d = O.sample(x[step, r], counts[r], oparams[r], step, forced=forced[r])
+            assert got[r] == d.chosen, (step, r)
+            if forced[r] is not None:
+                assert got[r] == forced[r]
+            emitted[r].append(int(got[r]))
+        if step == 2:     # row 0: the draw was a stop token; the close replaces it
+            q.push(0, LS.INSERT_REPLACE, drawn=int(got[0]), ids=replace_ids, scratch=sc[0])
+            counts[0][got[0]] -= 1
+            emitted[0].pop()
+        if step == 3:     # row 1: a close tag in front of the tool call just drawn
+            q.push(1, LS.INSERT_BEFORE, drawn=int(got[1]), ids=before_ids, scratch=sc[1])
+            counts[1][got[1]] -= 1
+            drawn_again = emitted[1].pop()
+        if step == 6:
+            assert emitted[1][5] == drawn_again   # ... which followed the two inserted ids
+    for r in range(rows):
+        assert np.array_equal(sc[r].read_counts().numpy().view(np.uint32), counts[r]), r
+        assert np.array_equal(np.bincount(emitted[r], minlength=VOCAB).astype(np.uint32), counts[r]), r
+    assert emitted[0][2:5] == replace_ids
+    assert emitted[1][3:5] == before_ids
+    q.close()
+    for s_ in sc:
+        s_.close()
+    sampler.close()
