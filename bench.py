@@ -262,9 +262,15 @@ def main():
         gen = torch.Generator(device=device)
         gen.manual_seed(11)
         w_f32 = torch.randn(vocab, d_model, device=device, generator=gen) * (2.0 / d_model ** 0.5)
+        # one weight row in ten scaled by 2|t(3)|: the logits then are, like config 5's, a bulk
+        # N(0, 2^2) with a heavy-tailed tenth
+        t3 = torch.from_numpy(np.random.default_rng(13).standard_t(3.0, vocab).astype(np.float32)).to(device)
+        heavy = torch.rand(vocab, device=device, generator=gen) < 0.1
+        w_f32 *= torch.where(heavy, 2.0 * t3.abs(), torch.ones_like(t3))[:, None]
+        del t3, heavy
         for b_rows in (4, rows):
             hid = torch.randn(b_rows, d_model, device=device, generator=gen)
-            # a bulk N(0, 2^2) and, per row, 40 ids whose weights point along the row's hidden state
+            # and, per row, 40 ids whose weights point along the row's hidden state
             for r in range(min(b_rows, 128)):
                 ids = torch.randint(0, vocab, (40,), device=device, generator=gen)
                 gain = (torch.rand(40, 1, device=device, generator=gen) * 0.7 + 0.3) * (6.0 / d_model)
@@ -299,6 +305,22 @@ def main():
             us_tiled = behind_a_head(lambda i: sampler.sample_rows_tiled(lg, tmax, tsum, hp, [i] * b_rows, ho,
                                                                         out_logprobs=hl))
             us_rows = behind_a_head(lambda i: sampler.sample_rows(lg, hp, [i] * b_rows, ho, out_logprobs=hl))
+            # config 5's draw settings in full: penalties over a 2 048-id history per row
+            pp = [LS.SamplingParams.greedy(temperature=0.8, top_k=64, top_p=0.9, repetition_penalty=1.1,
+                                           presence_penalty=0.2, frequency_penalty=0.1, seed=5000 + r)
+                  for r in range(b_rows)]
+            hist = np.random.default_rng(12).integers(0, vocab, (b_rows, 2048)).astype(np.int32)
+            hs = make_scratches(LS, sampler, hist, vocab, device)
+            torch.cuda.synchronize()
+            us_tiled_pen = behind_a_head(lambda i: sampler.sample_rows_tiled(
+                lg, tmax, tsum, pp, [i] * b_rows, ho, scratch=hs, out_logprobs=hl))
+            paths_pen = paths_of(sampler, lambda i: sampler.sample_rows_tiled(
+                lg, tmax, tsum, pp, [99] * b_rows, ho, scratch=hs, out_logprobs=hl))
+            us_rows_pen = behind_a_head(lambda i: sampler.sample_rows(lg, pp, [i] * b_rows, ho, scratch=hs,
+                                                                     out_logprobs=hl))
+            sampler.synchronize()
+            for sc_ in hs:
+                sc_.close()
             flops = 2.0 * b_rows * d_model * vocab
             head[f"b{b_rows}"] = {
                 "rows": b_rows, "d": d_model,
@@ -309,6 +331,9 @@ def main():
                 "head_plus_draws_us": ms_fused * 1e3,
                 "draws_from_summaries_us": us_tiled,
                 "draws_from_rows_us": us_rows,
+                "penalised_draws_from_summaries_us": us_tiled_pen,
+                "penalised_draws_from_rows_us": us_rows_pen,
+                "penalised_paths": paths_pen,
             }
             del hb, wb, lg
         del w_f32

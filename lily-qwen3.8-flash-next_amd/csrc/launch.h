@@ -31,10 +31,11 @@ hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t 
                                uint32_t vocab, const float* c2_of_row, void* logits,
                                uint64_t logits_stride, float* tile_max, float* tile_sum);
 // The draw of `rows` rows of cfg.table from the summaries ([.., tiles] each) and the few tiles of
-// the bf16 logits that matter; tile_row[r] = the summaries' row of table row r.
+// the bf16 logits that matter; tile_row[r] = the summaries' row of table row r; served[r] is set
+// for rows under penalties (1 = drawn, 0 = declined: the row is better read whole).
 hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const LaunchCfg& cfg,
                              const float* tile_max, const float* tile_sum, uint32_t tiles,
-                             const uint32_t* tile_row);
+                             const uint32_t* tile_row, uint32_t* served);
 hipError_t launch_copy_pieces(hipStream_t stream, const void* src, void* dst, size_t bytes);
 hipError_t launch_probe_read(hipStream_t stream, const void* base, uint32_t rows, uint64_t row_bytes,
                              uint64_t stride_bytes, uint32_t* out);

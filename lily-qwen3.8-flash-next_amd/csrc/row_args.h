@@ -119,6 +119,9 @@ struct LaunchCfg {
     uint32_t accept_pos0;
     uint32_t accept_ratio;
     uint32_t accept_chain;
+    // null, or [rows]: a row whose word is not 0 has been drawn by an earlier launch of the same
+    // call (from the producer's summaries) and is left alone
+    const uint32_t* served;
 };
 
 constexpr uint32_t CHAIN_CAP = LILY_SAMPLE_K_CAP;   // candidates a chained row publishes

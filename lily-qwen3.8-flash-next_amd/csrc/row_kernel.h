@@ -106,6 +106,9 @@ __device__ __forceinline__ void apply_selection(RowArgs& a) {
 
 template <int DT, int KIND, bool LSE, bool CHAIN = false>
 __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const LaunchCfg& cfg, Shared& sh) {
+    if (cfg.served != nullptr && *(const LILY_CONST uint32_t*)(cfg.served + blockIdx.y) != 0u) {
+        return;
+    }
     RowArgs a;
     load_row_args(a, src);
     apply_selection(a);

@@ -10,22 +10,29 @@ namespace lily {
 constexpr uint32_t TILES_PER_THREAD = 8;                 // wg_kth_largest takes 8 values a thread
 constexpr uint32_t TILES_MAX = NT * TILES_PER_THREAD;    // summaries of a row
 constexpr uint32_t TILE_CAND_CAP = 2048;                 // candidates gathered from the tiles
+constexpr uint32_t TILES_DECLINE = 256;                  // a penalised row that needs more tiles is declined
 
-// One workgroup per row (rows without mask, penalties or bias list, k <= STREAM_K_MAX; bf16).
+// One workgroup per row (rows without mask or bias list, penalties only of the kind that can
+// but lower a value, k <= STREAM_K_MAX; bf16).
 //   * The row's largest value is the largest summary; with at least k summaries at or above
 //     x, at least k values are: the k-th largest summary bounds the k-th largest value from
 //     below, and only tiles whose summary reaches it are read (16 lanes a tile, 16 bytes a
 //     lane); their values at or above the bound are the candidates.
 //   * The row's sum of exponentials is the summaries' sums brought to the row's reference.
+//   * Under penalties the bound is the k-th largest summary as the worst penalty would leave it
+//     (more tiles are read), values of listed ids are evaluated with their counts, and the tiles
+//     that matter to the row's sum are summed element by element instead of by their summaries.
 //   * More candidates than the buffer holds (ties by the thousand): the exhaustive select
 //     over the whole row takes over.
-// `tile_row[r]` is the row of the summaries that belongs to row r of the table.
+// `tile_row[r]` is the row of the summaries that belongs to row r of the table; `served[r]` is
+// written for rows under penalties: 1 = drawn here, 0 = left to the launch that follows.
 template <bool LSE>
 __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float* tile_max,
                                                       const float* tile_sum, uint32_t tiles,
-                                                      const uint32_t* tile_row) {
+                                                      const uint32_t* tile_row, uint32_t* served) {
     __shared__ Shared sh;
     __shared__ uint16_t listed[TILES_MAX];
+    __shared__ float listed_max[TILES_MAX];
     __shared__ uint32_t n_listed;
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
@@ -101,33 +108,61 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         return;
     }
 
+    // Rows under penalties that can only lower a value (the host serves no others here): a
+    // summary describes raw values and bounds true ones from above.  `lowered(x)`: what a raw
+    // value x is worth at least (the penalty of an id with the scratch's largest count).
+    const bool pen = (a.flags & F_PEN) != 0;
+    const uint32_t words = (vocab + 31u) / 32u;
+    const uint32_t max_count = pen ? *(const LILY_CONST uint32_t*)(a.touched + words) : 0u;
+    auto lowered = [&](float m) -> float {
+        if (pen && m > NEG_INF) {
+            float t = m > 0.0f ? m / a.repetition : m * a.repetition;
+            t -= a.presence + a.frequency * (float)max_count;
+            return t;
+        }
+        return m;
+    };
+    auto true_value = [&](uint32_t id, float raw) -> float {
+        uint32_t cnt = gload(a.counts + id);
+        asm volatile("" : "+v"(cnt));   // waited for here, inside the caller's branch
+        float t = raw;
+        if (cnt > 0u) {
+            t = t > 0.0f ? t / a.repetition : t * a.repetition;
+            t -= a.presence + a.frequency * (float)cnt;
+        }
+        return t;
+    };
+    // The sum's cut: tiles whose summary lies below it are summed as their summaries give them
+    // (their listed ids' raw terms stand for the true ones: each is below 2^-(log2 V + 21) of
+    // the row's largest term), tiles at or above it element by element.  It hangs from a lower
+    // bound of the row's largest TRUE value: the lowered largest summary or, better where a
+    // sequence keeps coming back to one token, the true value of the scratch's most-counted id.
+    float cut = -__builtin_huge_valf();
+    if (want_lse && pen) {
+        float floor_v = lowered(top);
+        const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
+        if (heavy < vocab && max_count != 0u) {
+            floor_v = fmaxf(floor_v, true_value(heavy, load_logit<LILY_BF16>(a.logits, heavy)));
+        }
+        cut = floor_v - (log2f((float)vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
+    }
+    LseAcc lse;
+    lse.init();
     if (want_lse) {
-        // sum over the tiles of tile_sum * 2^(tile_max * c2 - top * c2)
-        const float mc = top * a.c2;
-        double s = 0.0;
 #pragma unroll
         for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
             const uint32_t t = tid + j * NT;
-            if (t < tiles && ms[j] > NEG_INF) {
-                s += (double)tile_sum[srow + t] * exp2((double)(ms[j] * a.c2) - (double)mc);
+            if (t < tiles && ms[j] > NEG_INF && (!pen || ms[j] < cut)) {
+                // the tile's sum has the reference tile_max * c2
+                const float safe = lse.rebase(ms[j], a.c2);
+                lse.s += tile_sum[srow + t] * __builtin_amdgcn_exp2f(ms[j] * a.c2 - safe);
             }
         }
-        s = wave_sum_d(s);
-        if (lane == 0) {
-            sh.red_d[w] = s;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            double t = 0.0;
-            for (int i = 0; i < NWAVE; ++i) {
-                t += sh.red_d[i];
-            }
-            sh.lse_mc = (double)mc;
-            sh.lse_s = t;
-        }
-        __syncthreads();
     }
-    if (forced) {
+    if (forced) {   // (not under penalties: the host keeps such rows off this kernel)
+        if (want_lse) {
+            lse_reduce(sh, lse);
+        }
         if (tid == 0) {
             finish_token<LILY_BF16>(a, sh, a.forced, vocab);
         }
@@ -135,36 +170,58 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     }
 
     const uint32_t k = a.k;
-    const float bound = wg_kth_largest(ms, k, sh);   // F32_LOWEST with fewer than k finite summaries
+    // with at least k summaries at or above x, at least k raw values are, and their true values
+    // are at or above lowered(x)
+    const float kth = wg_kth_largest(ms, k, sh);   // F32_LOWEST with fewer than k finite summaries
+    const float bound = lowered(kth);
+    const float reach = (want_lse && pen) ? fminf(bound, cut) : bound;   // tiles read
     phase(cfg, 2);
     if (tid == 0) {
         sh.n_cand = 0;
     }
 #pragma unroll
     for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
-        if (ms[j] >= bound && ms[j] > NEG_INF) {
-            listed[atomicAdd(&n_listed, 1u)] = (uint16_t)(tid + j * NT);
+        if (ms[j] >= reach && ms[j] > NEG_INF) {
+            const uint32_t at = atomicAdd(&n_listed, 1u);
+            listed[at] = (uint16_t)(tid + j * NT);
+            listed_max[at] = ms[j];
         }
     }
     __syncthreads();
     const uint32_t n_t = n_listed;
+    // A row under penalties whose bound or cut reaches a large part of its tiles (a flat row) is
+    // read faster as a whole: it is left to the launch that follows (`served` stays 0).
+    if (pen) {
+        const bool decline = n_t > TILES_DECLINE;
+        if (tid == 0) {
+            served[blockIdx.y] = decline ? 0u : 1u;
+        }
+        if (decline) {
+            return;
+        }
+    }
     // 16 lanes a tile, 8 values a lane; four rounds of loads asked for before the first is used
+    // (under penalties the word of the scratch's bitmap that covers the 8 ids comes with them)
     constexpr uint32_t LANES = LILY_TILE_COLS / 8u, PER_ROUND = NT / LANES;
     const uint32_t sub = tid % LANES, slot = tid / LANES;
+    const uint32_t* bitmap = pen ? a.touched : nullptr;
     for (uint32_t r0 = 0; r0 < n_t; r0 += 4u * PER_ROUND) {
         u32x4 q[4];
-        uint32_t col0[4];
+        uint32_t col0[4], bits[4];
+        bool summed[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const uint32_t i = r0 + (uint32_t)u * PER_ROUND + slot;
-            const uint32_t t = listed[min(i, n_t - 1u)];
+            const uint32_t i = min(r0 + (uint32_t)u * PER_ROUND + slot, n_t - 1u);
+            const uint32_t t = listed[i];
             const uint32_t c = t * LILY_TILE_COLS + sub * 8u;
-            col0[u] = (i < n_t && c < vocab) ? c : 0xffffffffu;
+            col0[u] = (r0 + (uint32_t)u * PER_ROUND + slot < n_t && c < vocab) ? c : 0xffffffffu;
+            summed[u] = want_lse && pen && listed_max[i] >= cut;
             // A row starts at a multiple of 16 bytes (the host checks), so these pieces do too:
             // one that holds a valid column lies inside the row's pages, and the others are
             // replaced by the row's last such piece.
-            q[u] = *reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) +
-                                                   (size_t)min(c, (vocab - 1u) & ~7u) * 2u);
+            const uint32_t cc = min(c, (vocab - 1u) & ~7u);
+            q[u] = *reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) + (size_t)cc * 2u);
+            bits[u] = pen ? (gload(bitmap + (cc >> 5)) >> (cc & 31u)) & 0xffu : 0u;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -176,14 +233,24 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t id = col0[u] + (uint32_t)e;
-                if (id < vocab && v[e] >= bound) {
+                float x = (id < vocab && v[e] == v[e]) ? v[e] : NEG_INF;
+                if (((bits[u] >> e) & 1u) != 0u && x > NEG_INF && (x >= bound || summed[u])) {
+                    x = true_value(id, x);
+                }
+                if (summed[u]) {
+                    lse.add_one(x, a.c2);
+                }
+                if (x >= bound && x > NEG_INF) {
                     const uint32_t at = atomicAdd(&sh.n_cand, 1u);
                     if (at < TILE_CAND_CAP) {
-                        cand[at] = composite_of(v[e] / a.temperature, id);
+                        cand[at] = composite_of(x / a.temperature, id);
                     }
                 }
             }
         }
+    }
+    if (want_lse) {
+        lse_reduce(sh, lse);
     }
     __syncthreads();
     phase(cfg, 3);
@@ -208,7 +275,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
 
 hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
                              const float* tile_max, const float* tile_sum, uint32_t tiles,
-                             const uint32_t* tile_row) {
+                             const uint32_t* tile_row, uint32_t* served) {
     if (tiles == 0 || tiles > TILES_MAX) {
         return hipErrorInvalidValue;
     }
@@ -221,10 +288,10 @@ hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const 
     const dim3 grid(1, rows), block(NT);
     if (lse) {
         hipLaunchKernelGGL(k_rows_tiles<true>, grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum,
-                           tiles, tile_row);
+                           tiles, tile_row, served);
     } else {
         hipLaunchKernelGGL(k_rows_tiles<false>, grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum,
-                           tiles, tile_row);
+                           tiles, tile_row, served);
     }
     return hipGetLastError();
 }

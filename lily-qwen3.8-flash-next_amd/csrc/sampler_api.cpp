@@ -74,7 +74,7 @@ struct DeviceScope {
 constexpr uint32_t WS_ROWS = 4096;      // rows that may span several workgroups
 constexpr uint32_t WS_SLOTS = 1u << 22; // candidate slots of the workspace (rows x slices x k)
 constexpr uint32_t STAGE_SLOTS = 4;
-constexpr size_t STAGE_ROW_BYTES = sizeof(RowArgs) + 16;   // a staged row: descriptor + two words + slack
+constexpr size_t STAGE_ROW_BYTES = sizeof(RowArgs) + 16;   // a staged row: descriptor + three words + slack
 constexpr uint32_t TARGET_GROUPS = 512;  // workgroups a small batch is spread over
 
 }  // namespace
@@ -448,9 +448,10 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
 }
 
 int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_dev, int dtype,
-                uint32_t vocab, uint32_t step_delta, bool traced) {
+                uint32_t vocab, uint32_t step_delta, bool traced, const uint32_t* served = nullptr) {
     LaunchCfg cfg;
     fill_cfg(s, &cfg, vocab, part.slices, part.ws_k, step_delta, table_dev + part.first);
+    cfg.served = served != nullptr ? served + part.first : nullptr;
     if (traced) {
         attach_trace(s, &cfg, part.rows);
     }
@@ -625,7 +626,7 @@ int ensure_table(lily_sampler* s, uint32_t rows) {
         s->stage_used[i] = false;
     }
     s->table_cap = s->stage_cap = 0;
-    // (behind the descriptors: two words a row for the calls that draw from summaries)
+    // (behind the descriptors: three words a row for the calls that draw from summaries)
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->table_dev), (size_t)cap * STAGE_ROW_BYTES));
     for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {
         HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&s->stage[i]), (size_t)cap * STAGE_ROW_BYTES,
@@ -1624,13 +1625,23 @@ int check_head(const lily_lm_head* h, uint32_t rows, uint32_t vocab, const void*
     return LILY_OK;
 }
 
-// Rows the summaries serve: no mask, no penalties, no bias list, the row given as it is, and a
-// greedy row or a plain draw among at most STREAM_K_MAX candidates.
+// Rows the summaries serve: no mask, no bias list, penalties only of the lowering kind, the row
+// given as it is, and a greedy row or a plain draw among at most STREAM_K_MAX candidates.
 bool tiles_serve(const RowArgs& r) {
-    if (r.allow != nullptr || (r.flags & F_PEN) || r.n_bias != 0 || r.sel_row != nullptr) {
+    if (r.allow != nullptr || r.n_bias != 0 || r.sel_row != nullptr) {
         return false;
     }
-    return r.mode == MODE_ARGMAX || (r.mode == MODE_PLAIN && r.k <= STREAM_K_MAX);
+    if (r.mode == MODE_ARGMAX) {
+        return true;   // (a greedy row ignores penalties: sample.rs:382-385)
+    }
+    if (r.flags & F_PEN) {
+        // summaries describe raw values: they bound true ones only where penalties lower
+        const bool lowering = r.repetition >= 1.0f && r.presence >= 0.0f && r.frequency >= 0.0f;
+        if (!lowering || (r.flags & F_FORCED)) {
+            return false;
+        }
+    }
+    return r.mode == MODE_PLAIN && r.k <= STREAM_K_MAX;
 }
 
 // The draws of batch `b` with the summaries of its logits at hand; with `h` set, the logits and
@@ -1668,33 +1679,48 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
     if (int rc = pack_batch(b, packed.data())) {
         return rc;
     }
-    // staged: the descriptors (rows the summaries serve first), each such row's row of the
-    // summaries, every row's exponent scale (the producer's)
+    // staged: the descriptors - rows the summaries serve for certain, then rows under penalties
+    // (served from the summaries unless the kernel declines them: the launch of the remaining
+    // rows covers them too and skips those already drawn), then the others -, each row's row of
+    // the summaries, every row's exponent scale (the producer's), a word per row that says
+    // whether the row has been drawn
     char* stage = reinterpret_cast<char*>(s->stage[slot]);
     RowArgs* table = reinterpret_cast<RowArgs*>(stage);
     const size_t idx_off = (size_t)rows * sizeof(RowArgs), c2_off = idx_off + round16((size_t)rows * 4);
+    const size_t served_off = c2_off + round16((size_t)rows * 4);
     uint32_t* tile_row = reinterpret_cast<uint32_t*>(stage + idx_off);
     float* c2 = reinterpret_cast<float*>(stage + c2_off);
-    uint32_t served = 0;
+    uint32_t* served_flags = reinterpret_cast<uint32_t*>(stage + served_off);
+    uint32_t certain = 0, maybe = 0;
     bool lse = false;
+    uint32_t at = 0;
+    for (int group = 0; group < 3; ++group) {
+        for (uint32_t r = 0; r < rows; ++r) {
+            const RowArgs& row = packed[r];
+            const bool serve = tiles_serve(row);
+            const bool pen = serve && row.mode != MODE_ARGMAX && (row.flags & F_PEN) != 0;
+            const int g = !serve ? 2 : (pen ? 1 : 0);
+            if (g != group) {
+                continue;
+            }
+            if (serve) {
+                lse = lse || row.out_logprob != nullptr;
+                tile_row[at] = r;
+                certain += group == 0 ? 1u : 0u;
+                maybe += group == 1 ? 1u : 0u;
+            }
+            served_flags[at] = 0u;
+            table[at++] = row;
+        }
+    }
     for (uint32_t r = 0; r < rows; ++r) {
         c2[r] = std::isfinite(packed[r].c2) ? packed[r].c2 : 0.0f;
-        if (tiles_serve(packed[r])) {
-            lse = lse || packed[r].out_logprob != nullptr;
-            tile_row[served] = r;
-            table[served++] = packed[r];
-        }
     }
-    uint32_t others = served;
-    for (uint32_t r = 0; r < rows; ++r) {
-        if (!tiles_serve(packed[r])) {
-            table[others++] = packed[r];
-        }
-    }
+    const uint32_t served = certain + maybe;
     LaunchPart parts[2];
     const uint32_t n_parts =
-        served < rows ? plan_parts(s, table + served, rows - served, (int)b->dtype, b->vocab, parts) : 0u;
-    if (int rc = stage_commit(s, slot, c2_off + (size_t)rows * 4)) {
+        certain < rows ? plan_parts(s, table + certain, rows - certain, (int)b->dtype, b->vocab, parts) : 0u;
+    if (int rc = stage_commit(s, slot, served_off + (size_t)rows * 4)) {
         return rc;
     }
     const char* dev = reinterpret_cast<const char*>(s->table_dev);
@@ -1705,15 +1731,17 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
                                     const_cast<void*>(b->logits_dev), b->row_stride, h->tile_max_dev,
                                     h->tile_sum_dev));
     }
+    uint32_t* served_dev = reinterpret_cast<uint32_t*>(const_cast<char*>(dev) + served_off);
     if (served != 0) {
         LaunchCfg cfg;
         fill_cfg(s, &cfg, b->vocab, 1, 1, 0, s->table_dev);
         attach_trace(s, &cfg, served);
         HIP_TRY(launch_rows_tiles(s->stream, lse, served, cfg, tile_max, tile_sum, tiles,
-                                  reinterpret_cast<const uint32_t*>(dev + idx_off)));
+                                  reinterpret_cast<const uint32_t*>(dev + idx_off), served_dev));
     }
     for (uint32_t q = 0; q < n_parts; ++q) {
-        if (int rc = launch_part(s, parts[q], s->table_dev + served, (int)b->dtype, b->vocab, 0, false)) {
+        if (int rc = launch_part(s, parts[q], s->table_dev + certain, (int)b->dtype, b->vocab, 0, false,
+                                 maybe != 0 ? served_dev + certain : nullptr)) {
             return rc;
         }
     }

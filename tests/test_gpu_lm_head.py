@@ -269,3 +269,58 @@ def test_rejections(sampler):
     with pytest.raises(LS.SamplerError):
         sampler.sample_rows_tiled(f32, tmax, tsum, [ls_params()] * rows, [0, 0], out)   # f32 logits
     sampler.synchronize()
+
+
+def test_rows_under_lowering_penalties_are_drawn_from_summaries(sampler):
+    """Rows whose penalties can only lower a value (repetition >= 1, presence and frequency
+    >= 0) are served from the summaries too: a wider set of tiles is read, listed ids are
+    evaluated with their counts, and the tiles that matter to the row's sum are summed element
+    by element.  Three decode steps on the same logits, the counts moving with the draws; rows
+    whose penalties may raise a value go through the selects that read the row."""
+    rows, d, vocab = 12, 256, 151_936
+    rng = np.random.default_rng(404)
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=60, gain=9.0)
+    params_kw = []
+    for r in range(rows):
+        kw = dict(temperature=0.8, top_k=(64, 20, 5)[r % 3], top_p=0.9, seed=5000 + r,
+                  repetition_penalty=1.1, presence_penalty=0.2, frequency_penalty=0.1)
+        if r == 7:
+            kw.update(repetition_penalty=0.9)        # may raise: not served from summaries
+        if r == 9:
+            kw.update(presence_penalty=-0.5)         # may raise
+        params_kw.append(kw)
+    params = [ls_params(**kw) for kw in params_kw]
+    temps = [p.effective()[0] for p in params]
+    h, w, buf, logits, tmax, tsum = _produce(sampler, hidden, weight, temps, rows, vocab)
+    stored = _bits(logits.contiguous())
+    stored_f = W.bf16_bits_to_f32(stored)
+    # histories that hold the rows' best ids (what a model that repeats itself has emitted)
+    scratch, hist_counts = [], []
+    for r in range(rows):
+        best = np.argsort(-stored_f[r])[:30].astype(np.int32)
+        hh = np.concatenate([rng.integers(0, vocab, 2000).astype(np.int32), np.repeat(best[:10], 3), best])
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(hh).to(dev()))
+        scratch.append(sc)
+        hist_counts.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+    for step in range(3):
+        steps = [step] * rows
+        stats = torch.zeros(4, dtype=torch.int32, device=dev())
+        sampler.set_path_stats(stats)
+        ids, lps, cand, counts = _draw_all(
+            sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+                logits, tmax, tsum, params, steps, out, scratch=scratch, out_logprobs=lp, dbg_ids=di,
+                dbg_counts=dc),
+            logits, params_kw, steps)
+        sampler.set_path_stats(None)
+        assert stats.cpu().numpy()[2] == 0, "no row fell back to the exhaustive select"
+        for r, kw in enumerate(params_kw):
+            dd = O.sample(stored[r], hist_counts[r], o_params(**kw), step, want_logprob=True)   # bumps the counts
+            n_fin = int(np.sum(dd.cand_adj > -np.inf))
+            assert counts[r, 0] == n_fin, (step, r)
+            assert np.array_equal(cand[r, :n_fin], dd.cand_ids[:n_fin].astype(np.int64)), (step, r)
+            assert counts[r, 1] == dd.n_kept and ids[r] == dd.chosen, (step, r)
+            assert abs(lps[r] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (step, r, lps[r], dd.logprob)
+    for r in range(rows):
+        assert np.array_equal(scratch[r].read_counts().numpy().view(np.uint32), hist_counts[r]), r
+        scratch[r].close()
