@@ -412,11 +412,14 @@ void lily_insertions_clear(lily_insertions_t* q, uint32_t row);
  * their owner first).  logits[r][v] = sum_i hidden[r][i] * weight[v][i], accumulated in f32 on
  * the matrix cores and rounded to bf16 (nearest even).  Beside the logits the producer leaves,
  * for every LILY_LOGIT_TILE_COLS columns of every row, the largest value and the sum of
- * 2^((x - largest) * log2(e) / T[r]) over the tile - "summaries".  A row without allow-mask,
- * penalties or bias list that is greedy or draws among at most 64 candidates is then drawn from
- * the summaries and the few tiles that can hold a candidate (about k tiles of 256 bytes instead
- * of the row); every other row of the batch is drawn from the logits as lily_sample_rows
- * draws it.  Ids and log-probabilities are those of lily_sample_rows on the same logits. */
+ * 2^((x - largest) * log2(e) / T[r]) over the tile - "summaries".  A row without allow-mask or
+ * bias list that is greedy or draws among at most 64 candidates, under no penalties or under
+ * penalties that can only lower a value (repetition >= 1, presence and frequency >= 0), is then
+ * drawn from the summaries and the few tiles that can hold a candidate (about k tiles of 256
+ * bytes instead of the row; a penalised row whose values lie too close together for that is
+ * recognised on the device and read whole); every other row of the batch is drawn from the
+ * logits as lily_sample_rows draws it.  Ids and log-probabilities are those of lily_sample_rows
+ * on the same logits. */
 #define LILY_LOGIT_TILE_COLS 128u
 
 typedef struct lily_lm_head {
