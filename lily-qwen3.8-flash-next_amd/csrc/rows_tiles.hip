@@ -7,10 +7,12 @@
 
 namespace lily {
 
-constexpr uint32_t TILES_PER_THREAD = 8;                 // wg_kth_largest takes 8 values a thread
+constexpr uint32_t TILES_PER_THREAD = 8;
 constexpr uint32_t TILES_MAX = NT * TILES_PER_THREAD;    // summaries of a row
 constexpr uint32_t TILE_CAND_CAP = 2048;                 // candidates gathered from the tiles
-constexpr uint32_t TILES_DECLINE = 256;                  // a penalised row that needs more tiles is declined
+constexpr uint32_t TILES_DECLINE = 256;                  // a penalised row that needs more tiles is declined,
+constexpr uint32_t SUMMED_DECLINE = 96;                  // or more tiles summed element by element
+constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated element by element
 
 // One workgroup per row (rows without mask or bias list, penalties only of the kind that can
 // but lower a value, k <= STREAM_K_MAX; bf16).
@@ -31,14 +33,16 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
                                                       const float* tile_sum, uint32_t tiles,
                                                       const uint32_t* tile_row, uint32_t* served) {
     __shared__ Shared sh;
-    __shared__ uint16_t listed[TILES_MAX];
-    __shared__ float listed_max[TILES_MAX];
-    __shared__ uint32_t n_listed;
+    __shared__ uint16_t listed[TILES_MAX];   // tiles to read; bit 15: summed element by element
+    __shared__ uint32_t refs[REF_CAP];       // pieces to evaluate: first id; bit 31: summed
+    __shared__ uint32_t n_listed, n_refs, n_summed;
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     if (tid == 0) {
         tail_arrays(sh);
         n_listed = 0;
+        n_refs = 0;
+        n_summed = 0;
     }
     RowArgs a;
     load_row_args(a, table + blockIdx.y);
@@ -53,13 +57,21 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         }
         return;
     }
-    const size_t srow = (size_t)tile_row[blockIdx.y] * tiles;
-    float ms[TILES_PER_THREAD];
+    const size_t srow = (size_t)gload(tile_row + blockIdx.y) * tiles;
+    // the summaries: both arrays asked for at once (clamped, so that no load hangs on a test)
+    float ms[TILES_PER_THREAD], ss[TILES_PER_THREAD];
     float best = NEG_INF;
 #pragma unroll
     for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
-        const uint32_t t = tid + j * NT;
-        ms[j] = t < tiles ? tile_max[srow + t] : NEG_INF;
+        const uint32_t t = min(tid + j * NT, tiles - 1u);
+        ms[j] = gload(tile_max + srow + t);
+        ss[j] = gload(tile_sum + srow + t);
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+        if (tid + j * NT >= tiles) {
+            ms[j] = NEG_INF;
+        }
         best = fmaxf(best, ms[j]);
     }
     best = wave_max_f(best);
@@ -155,7 +167,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             if (t < tiles && ms[j] > NEG_INF && (!pen || ms[j] < cut)) {
                 // the tile's sum has the reference tile_max * c2
                 const float safe = lse.rebase(ms[j], a.c2);
-                lse.s += tile_sum[srow + t] * __builtin_amdgcn_exp2f(ms[j] * a.c2 - safe);
+                lse.s += ss[j] * __builtin_amdgcn_exp2f(ms[j] * a.c2 - safe);
             }
         }
     }
@@ -172,7 +184,32 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     const uint32_t k = a.k;
     // with at least k summaries at or above x, at least k raw values are, and their true values
     // are at or above lowered(x)
-    const float kth = wg_kth_largest(ms, k, sh);   // F32_LOWEST with fewer than k finite summaries
+    // (a lower bound of the k-th largest summary, as the streaming select takes it: each wave's
+    // ceil(k / NWAVE)-th largest of its lanes' best summaries - a 16-step search by ballots on the
+    // top half of the order key -, the minimum over the waves; F32_LOWEST when a wave holds fewer)
+    float lane_best = NEG_INF;
+#pragma unroll
+    for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+        lane_best = fmaxf(lane_best, ms[j]);
+    }
+    float kth;
+    if (tiles >= NT) {
+        const uint32_t kw = (k + NWAVE - 1u) / NWAVE;
+        const uint32_t key16 = lane_best > NEG_INF ? (lilym_order_key(lane_best) >> 16) : 0u;
+        const uint32_t P = wave_kth_key16(key16, kw);
+        if (lane == 0) {
+            sh.red_f[w] = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
+        }
+        __syncthreads();
+        kth = sh.red_f[0];
+        for (int i = 1; i < NWAVE; ++i) {
+            kth = fminf(kth, sh.red_f[i]);
+        }
+        __syncthreads();
+    } else {
+        // a short row leaves whole waves without a summary: the exact k-th largest instead
+        kth = wg_kth_largest(ms, k, sh);
+    }
     const float bound = lowered(kth);
     const float reach = (want_lse && pen) ? fminf(bound, cut) : bound;   // tiles read
     phase(cfg, 2);
@@ -182,17 +219,20 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
 #pragma unroll
     for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
         if (ms[j] >= reach && ms[j] > NEG_INF) {
-            const uint32_t at = atomicAdd(&n_listed, 1u);
-            listed[at] = (uint16_t)(tid + j * NT);
-            listed_max[at] = ms[j];
+            const bool sum_it = want_lse && pen && ms[j] >= cut;
+            listed[atomicAdd(&n_listed, 1u)] = (uint16_t)((tid + j * NT) | (sum_it ? 0x8000u : 0u));
+            if (sum_it) {
+                atomicAdd(&n_summed, 1u);
+            }
         }
     }
     __syncthreads();
     const uint32_t n_t = n_listed;
+    phase(cfg, 8);
     // A row under penalties whose bound or cut reaches a large part of its tiles (a flat row) is
     // read faster as a whole: it is left to the launch that follows (`served` stays 0).
     if (pen) {
-        const bool decline = n_t > TILES_DECLINE;
+        const bool decline = n_t > TILES_DECLINE || n_summed > SUMMED_DECLINE;
         if (tid == 0) {
             served[blockIdx.y] = decline ? 0u : 1u;
         }
@@ -200,54 +240,91 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             return;
         }
     }
-    // 16 lanes a tile, 8 values a lane; four rounds of loads asked for before the first is used
-    // (under penalties the word of the scratch's bitmap that covers the 8 ids comes with them)
+    // First the tiles are read, 16 lanes a tile and 16 bytes a lane, ROUNDS rounds of loads asked
+    // for before the first is used; all a lane does with a piece is compare its largest value
+    // with the bound: a piece that reaches it (or belongs to a summed tile) is put on a list.
+    // (Evaluating such pieces on the spot keeps one or two lanes of a wave busy while the
+    // others wait, eight times per round: that was most of the kernel's time.)
     constexpr uint32_t LANES = LILY_TILE_COLS / 8u, PER_ROUND = NT / LANES;
     const uint32_t sub = tid % LANES, slot = tid / LANES;
-    const uint32_t* bitmap = pen ? a.touched : nullptr;
-    for (uint32_t r0 = 0; r0 < n_t; r0 += 4u * PER_ROUND) {
-        u32x4 q[4];
-        uint32_t col0[4], bits[4];
-        bool summed[4];
+    constexpr int ROUNDS = 8;
+    for (uint32_t r0 = 0; r0 < n_t; r0 += (uint32_t)ROUNDS * PER_ROUND) {
+        u32x4 q[ROUNDS];
+        uint32_t col0[ROUNDS];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < ROUNDS; ++u) {
             const uint32_t i = min(r0 + (uint32_t)u * PER_ROUND + slot, n_t - 1u);
             const uint32_t t = listed[i];
-            const uint32_t c = t * LILY_TILE_COLS + sub * 8u;
-            col0[u] = (r0 + (uint32_t)u * PER_ROUND + slot < n_t && c < vocab) ? c : 0xffffffffu;
-            summed[u] = want_lse && pen && listed_max[i] >= cut;
+            const uint32_t c = (t & 0x7fffu) * LILY_TILE_COLS + sub * 8u;
+            col0[u] = (r0 + (uint32_t)u * PER_ROUND + slot < n_t && c < vocab) ? (c | ((t & 0x8000u) << 16))
+                                                                              : 0xffffffffu;
             // A row starts at a multiple of 16 bytes (the host checks), so these pieces do too:
             // one that holds a valid column lies inside the row's pages, and the others are
             // replaced by the row's last such piece.
             const uint32_t cc = min(c, (vocab - 1u) & ~7u);
-            q[u] = *reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) + (size_t)cc * 2u);
-            bits[u] = pen ? (gload(bitmap + (cc >> 5)) >> (cc & 31u)) & 0xffu : 0u;
+            q[u] = gload(reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) + (size_t)cc * 2u));
+        }
+#pragma unroll
+        for (int u = 0; u < ROUNDS; ++u) {
+            // (true values are raw ones or lower: a piece whose largest raw value stays below the
+            // bound holds no candidate)
+            const bool want = col0[u] != 0xffffffffu &&
+                              ((col0[u] >> 31) != 0u || chunk_max<LILY_BF16>(q[u]) >= bound);
+            const uint64_t votes = __ballot(want);
+            if (votes != 0ull) {
+                uint32_t base = 0;
+                if (lane == 0) {
+                    base = atomicAdd(&n_refs, (uint32_t)__popcll(votes));
+                }
+                base = (uint32_t)__shfl((int)base, 0);
+                const uint32_t at = base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull));
+                if (want && at < REF_CAP) {
+                    refs[at] = col0[u];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // Then the listed pieces, a thread per value, four pieces' loads in flight per thread.
+    const uint32_t n_r = n_refs;   // (beyond the list's capacity: the exhaustive select below)
+    const uint32_t e_of = tid & 7u;
+    for (uint32_t p0 = 0; p0 < min(n_r, REF_CAP); p0 += 4u * (NT / 8u)) {
+        uint32_t ref[4], word[4];
+        float raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t p = p0 + (uint32_t)u * (NT / 8u) + (tid >> 3);
+            ref[u] = p < min(n_r, REF_CAP) ? refs[p] : 0xffffffffu;
+            const uint32_t id = min((ref[u] & 0x7fffffffu) + e_of, vocab - 1u);
+            raw[u] = load_logit<LILY_BF16>(a.logits, id);
+            // (the word of the scratch's bitmap that covers the id; the summaries' first word
+            // when there is no scratch to ask: the load stays unconditional)
+            word[u] = gload((pen ? a.touched : reinterpret_cast<const uint32_t*>(tile_max)) + (pen ? (id >> 5) : 0u));
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            if (col0[u] == 0xffffffffu) {
+            const uint32_t id = (ref[u] & 0x7fffffffu) + e_of;
+            if (ref[u] == 0xffffffffu || id >= vocab) {
                 continue;
             }
-            float v[8];
-            unpack<LILY_BF16>(q[u], v);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t id = col0[u] + (uint32_t)e;
-                float x = (id < vocab && v[e] == v[e]) ? v[e] : NEG_INF;
-                if (((bits[u] >> e) & 1u) != 0u && x > NEG_INF && (x >= bound || summed[u])) {
-                    x = true_value(id, x);
-                }
-                if (summed[u]) {
-                    lse.add_one(x, a.c2);
-                }
-                if (x >= bound && x > NEG_INF) {
-                    const uint32_t at = atomicAdd(&sh.n_cand, 1u);
-                    if (at < TILE_CAND_CAP) {
-                        cand[at] = composite_of(x / a.temperature, id);
-                    }
+            const bool summed = (ref[u] >> 31) != 0u;
+            float x = raw[u] == raw[u] ? raw[u] : NEG_INF;
+            if (pen && ((word[u] >> (id & 31u)) & 1u) != 0u && x > NEG_INF && (x >= bound || summed)) {
+                x = true_value(id, x);
+            }
+            if (summed) {
+                lse.add_one(x, a.c2);
+            }
+            if (x >= bound && x > NEG_INF) {
+                const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                if (at < TILE_CAND_CAP) {
+                    cand[at] = composite_of(x / a.temperature, id);
                 }
             }
         }
+    }
+    if (n_r > REF_CAP && tid == 0) {
+        sh.n_cand = TILE_CAND_CAP + 1u;   // too many pieces: as with too many candidates
     }
     if (want_lse) {
         lse_reduce(sh, lse);
