@@ -44,9 +44,8 @@ struct HeadTile {
 // 64, six operand reads out of LDS for eight products - for a batch, whose bound is the matrix
 // cores and, just behind, the bandwidth of LDS.
 //
-// Workgroups are numbered so that the tiles over one block of 128 weight rows - one per BM
-// rows of the batch - run on the same XCD one after the other: the weight rows, the large
-// operand, are then fetched from memory once and served to the other tiles by that XCD's L2.
+// Workgroups are numbered so that an XCD's L2 holds the hidden rows its workgroups share (see
+// the numbering at the top of the kernel).
 template <class T>
 __global__ void __launch_bounds__(256, T::RESIDENT)
 k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
@@ -57,10 +56,28 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     constexpr int BM = T::BM, BN = T::BN, BK = T::BK, MI = T::MI, NI = T::NI, ROW_BYTES = T::ROW_BYTES;
     extern __shared__ __align__(16) char lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    // Which tile: consecutive workgroups go to consecutive XCDs (eight of them, an L2 each).  An
+    // XCD keeps to one block of BM hidden rows for as long as it can - that block (BM x d x 2
+    // bytes) then stays in its L2 and is shared by all its workgroups, which stream different
+    // blocks of weight rows past it; the XCDs that hold other blocks of hidden rows stream the
+    // same weights at about the same time and find them in the memory-side cache.  With up to 8
+    // blocks of hidden rows the XCDs are divided among the blocks and split the weights' blocks
+    // between them; with more, an XCD takes every eighth block in turn.
     const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-    const uint32_t n_tile = (slot / m_tiles) * 8u + xcd, m_tile = slot % m_tiles;
-    if (n_tile >= tiles_per_row) {
-        return;
+    uint32_t m_tile, n_tile;
+    if (m_tiles <= 8u) {
+        m_tile = xcd % m_tiles;
+        const uint32_t rank = xcd / m_tiles, sharers = (8u - m_tile + m_tiles - 1u) / m_tiles;
+        n_tile = rank + slot * sharers;
+        if (n_tile >= tiles_per_row) {
+            return;
+        }
+    } else {
+        m_tile = xcd + 8u * (slot / tiles_per_row);
+        n_tile = slot % tiles_per_row;
+        if (m_tile >= m_tiles) {
+            return;
+        }
     }
     const uint32_t m0 = m_tile * BM, n0 = n_tile * BN;
     const uint32_t wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
@@ -128,12 +145,21 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     // stage is asked for again): the compiler then counts the loads in flight and waits for
     // the oldest only; with a branch around any of them it waits for all.
     const uint32_t steps = d / BK, padded = (steps + T::AHEAD - 1u) / T::AHEAD * T::AHEAD;
-    const uint32_t k_last = d - BK;
-    fetch(ring_h[0], ring_w[0], 0);
+    // Each tile walks d from a place of its own (and wraps round): rows of either operand lie
+    // d x 2 bytes apart, a power of two for the usual d, so the same 64 or 128 bytes of every
+    // row sit behind the same memory channel; tiles that all start at column 0 and advance in
+    // step would queue up at one channel after the other.
+    const uint32_t rot = (n_tile * 5u + m_tile * 3u) % steps;
+    auto k_of = [&](uint32_t stage_no) -> uint32_t {
+        uint32_t at = min(stage_no, steps - 1u) + rot;
+        at = at >= steps ? at - steps : at;
+        return at * BK;
+    };
+    fetch(ring_h[0], ring_w[0], k_of(0));
     stage(ring_h[0], ring_w[0], 0, true);
 #pragma unroll
     for (int j = 0; j < T::AHEAD; ++j) {
-        fetch(ring_h[j], ring_w[j], min(((uint32_t)j + 1u) * BK, k_last));   // ring[j] <- stage j + 1
+        fetch(ring_h[j], ring_w[j], k_of((uint32_t)j + 1u));   // ring[j] <- stage j + 1
     }
     __syncthreads();
     for (uint32_t s0 = 0; s0 < padded; s0 += T::AHEAD) {
@@ -144,7 +170,7 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
             // ring[j] holds stage s + 1: into the other LDS stage (nobody reads it: the barrier
             // that closed step s - 1 saw to that), and the registers ask for stage s + 1 + AHEAD
             stage(ring_h[j], ring_w[j], buf ^ 1u, s + 1u < steps);
-            fetch(ring_h[j], ring_w[j], min((s + 1u + T::AHEAD) * BK, k_last));
+            fetch(ring_h[j], ring_w[j], k_of(s + 1u + T::AHEAD));
             const char* base = lds + buf * T::STAGE_BYTES;
 #pragma unroll
             for (int kk = 0; kk < BK / 16; ++kk) {
@@ -310,8 +336,10 @@ static hipError_t launch_head_shape(hipStream_t stream, const void* hidden, uint
         }
     }
     const uint32_t tiles_per_row = (vocab + T::BN - 1u) / T::BN, m_tiles = (rows + T::BM - 1u) / T::BM;
-    const uint32_t groups = (tiles_per_row + 7u) / 8u;
-    hipLaunchKernelGGL(k_lm_head_bf16<T>, dim3(8u * groups * m_tiles), dim3(256), T::LDS_BYTES, stream,
+    // slots an XCD needs at most (see the kernel's numbering)
+    const uint32_t slots = m_tiles <= 8u ? (tiles_per_row + (8u / m_tiles) - 1u) / (8u / m_tiles)
+                                         : ((m_tiles + 7u) / 8u) * tiles_per_row;
+    hipLaunchKernelGGL(k_lm_head_bf16<T>, dim3(8u * slots), dim3(256), T::LDS_BYTES, stream,
                        reinterpret_cast<const uint16_t*>(hidden), hidden_stride,
                        reinterpret_cast<const uint16_t*>(weight), weight_stride, rows, d, vocab,
                        c2_of_row, reinterpret_cast<uint16_t*>(logits), logits_stride, tile_max, tile_sum,
