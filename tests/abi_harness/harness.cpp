@@ -78,7 +78,26 @@ static int cpu_mode() {
         std::fprintf(stderr, "draft_step / ctrl_words\n");
         return 1;
     }
-    std::printf("cpu ok uniform %.9g draft_step %u ctrl_words %u\n", u, lily_draft_step(5), lily_ctrl_words(2));
+    // the insertions queue (host state only) and the producer's shapes
+    lily_insertions_t* q = nullptr;
+    const uint32_t ids[2] = {10, 11};
+    uint32_t forced[2] = {0, 0};
+    if (lily_insertions_create(2, &q) != LILY_OK ||
+        lily_insertions_push(q, 1, LILY_INSERT_BEFORE, 9, ids, 2, nullptr) != LILY_OK ||
+        lily_insertions_pending(q, 1) != 3 || lily_insertions_next(q, forced) != 1 ||
+        forced[0] != LILY_NO_TOKEN || forced[1] != 10) {
+        std::fprintf(stderr, "insertions: %s\n", lily_last_error());
+        return 1;
+    }
+    lily_insertions_destroy(q);
+    if (lily_lm_head_tiles(151936) != 1187 || lily_lm_head_tiles(129) != 2) {
+        std::fprintf(stderr, "lm_head_tiles\n");
+        return 1;
+    }
+    // (the sizes a compiler gives the structs: the Python mirror's must be the same)
+    std::printf("cpu ok uniform %.9g draft_step %u ctrl_words %u sizes %zu %zu %zu %zu\n", u, lily_draft_step(5),
+                lily_ctrl_words(2), sizeof(lily_sampling_params), sizeof(lily_rows), sizeof(lily_lm_head),
+                sizeof(lily_draft_dist));
     return 0;
 }
 

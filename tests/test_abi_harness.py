@@ -37,6 +37,13 @@ def test_host_helpers_from_cpp_without_a_gpu():
     assert words[:2] == ["cpu", "ok"], res.stdout
     assert np.float32(float(words[3])) == np.float32(O.uniform_for(1234, 7))
     assert int(words[5]) == (5 | 0x40000000)
+    # the structs as a C++ compiler lays them out against the ctypes mirror's
+    import ctypes
+
+    import lily_sampler as LS
+    sizes = [int(w) for w in words[words.index("sizes") + 1:]]
+    assert sizes == [ctypes.sizeof(LS.SamplingParams), ctypes.sizeof(LS._Rows), ctypes.sizeof(LS._LmHead),
+                     ctypes.sizeof(LS.DraftDist)], sizes
 
 
 def _logits(vocab, seed):
