@@ -26,7 +26,12 @@ struct HeadTile {
     static constexpr int BM = WAVES_M * MI * 32;
     static constexpr int BN = WAVES_N * NI * 32;
     static constexpr int PIECES = BK / 8;                  // 16-byte pieces of a staged row
-    static constexpr int ROW_BYTES = BK * 2 + 16;          // padded: 8 rows cover all banks
+    // A staged row: 128 bytes of d and 16 of padding (8 rows then cover all banks), or 64 bytes
+    // without padding whose four 16-byte pieces change places by the row's number (piece ^
+    // (row / 2) % 4): 8 rows' pieces of one column, and the 8 pieces of two rows, then lie in
+    // 8 different groups of banks.
+    static constexpr bool SWIZZLED = BK == 32;
+    static constexpr int ROW_BYTES = SWIZZLED ? BK * 2 : BK * 2 + 16;
     static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;  // hidden rows, then weight rows
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;      // two stages
@@ -90,13 +95,13 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     for (int i = 0; i < T::A_PER; ++i) {
         const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
         src_h[i] = hidden + (uint64_t)min(m0 + r, rows - 1u) * hidden_stride + kc * 8u;
-        dst_h[i] = r * ROW_BYTES + kc * 16u;
+        dst_h[i] = r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 1) & 3u)) : kc) * 16u;
     }
 #pragma unroll
     for (int i = 0; i < T::B_PER; ++i) {
         const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
         src_w[i] = weight + (uint64_t)min(n0 + r, vocab - 1u) * weight_stride + kc * 8u;
-        dst_w[i] = T::A_BYTES + r * ROW_BYTES + kc * 16u;
+        dst_w[i] = T::A_BYTES + r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 1) & 3u)) : kc) * 16u;
     }
     // ring[j]: the loads of a stage on their way (registers), written to LDS one step before use
     w32x4 ring_h[T::AHEAD][T::A_PER], ring_w[T::AHEAD][T::B_PER];
@@ -137,9 +142,16 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         }
     }
     // A lane's operand values: row lane % 32 of the 32, 8 values of d from (lane / 32) * 8 on.
-    const uint32_t frag = (lane & 31u) * ROW_BYTES + (lane >> 5) * 16u;
-    const uint32_t a_at = wm * (MI * 32u) * ROW_BYTES + frag;
-    const uint32_t b_at = T::A_BYTES + wn * (NI * 32u) * ROW_BYTES + frag;
+    // (piece (lane / 32) + 2 * kk of the row; its place in a swizzled row depends on the row's
+    // number, which is the lane's within every block of 32 rows)
+    uint32_t piece_at[BK / 16];
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+        const uint32_t piece = (lane >> 5) + 2u * (uint32_t)kk;
+        piece_at[kk] = (T::SWIZZLED ? (piece ^ ((lane >> 1) & 3u)) : piece) * 16u;
+    }
+    const uint32_t a_at = (wm * (MI * 32u) + (lane & 31u)) * ROW_BYTES;
+    const uint32_t b_at = T::A_BYTES + (wn * (NI * 32u) + (lane & 31u)) * ROW_BYTES;
 
     // Every load and every write to LDS below is unconditional (past the end of d the last
     // stage is asked for again): the compiler then counts the loads in flight and waits for
@@ -177,11 +189,11 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
                 bf16x8 a[MI], b[NI];
 #pragma unroll
                 for (int i = 0; i < MI; ++i) {
-                    a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + kk * 32);
+                    a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + piece_at[kk]);
                 }
 #pragma unroll
                 for (int i = 0; i < NI; ++i) {
-                    b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + kk * 32);
+                    b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + piece_at[kk]);
                 }
 #pragma unroll
                 for (int mi = 0; mi < MI; ++mi) {
