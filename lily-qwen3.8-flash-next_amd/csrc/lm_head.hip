@@ -14,6 +14,13 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t w32x4 __attribute__((ext_vector_type(4)));
 
+// x as the lane CTRL names holds it (DPP controls: 0x120 + n = rotate right by n within each
+// row of 16 lanes).
+template <int CTRL>
+__device__ __forceinline__ float rotated(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+
 // A workgroup's tile and how its four waves share it.  WAVES_M x (4 / WAVES_M) waves, each
 // MI x NI products of 32 x 32; the tile is WAVES_M * MI * 32 rows by 128 columns (the width of a
 // summary), staged BK columns of d at a time, AHEAD stages of loads in flight (what is in flight
@@ -243,12 +250,16 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         const float x = acc[mi][ni][v];
         return (in_vocab[ni] && x == x) ? x : NEG;
     };
+    // A reduction over the 32 lanes that hold one row's columns: rotations by 8, 4, 2 and 1 within
+    // each row of 16 lanes (DPP operands of the arithmetic itself), then one exchange between the
+    // two rows.  (Five exchanges through the LDS crossbar per value, as __shfl_xor compiles, made
+    // the epilogue as long as the products at 1024 rows.)
     auto across32 = [&](float x, auto op) -> float {
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) {
-            x = op(x, __shfl_xor(x, o));
-        }
-        return x;
+        x = op(x, rotated<0x128>(x));
+        x = op(x, rotated<0x124>(x));
+        x = op(x, rotated<0x122>(x));
+        x = op(x, rotated<0x121>(x));
+        return op(x, __shfl_xor(x, 16));
     };
     auto row_of = [&](int mi, int v) -> uint32_t {
         return wm * (MI * 32u) + (uint32_t)mi * 32u + 8u * (uint32_t)(v >> 2) + 4u * (lane >> 5) +

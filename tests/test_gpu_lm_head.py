@@ -87,12 +87,15 @@ def _check_product(h, w, logits, tmax, tsum, temps):
         assert np.allclose(tsum[r].cpu().numpy(), want, rtol=2e-6, atol=0), r
 
 
-@pytest.mark.parametrize("rows,d,vocab", [(5, 256, 1000), (130, 512, 4096 + 77), (1, 64, 128)])
-def test_producer_against_f64_product(sampler, rows, d, vocab):
+@pytest.mark.parametrize("rows,d,vocab,slack", [(5, 256, 1000, 8), (130, 512, 4096 + 77, 8), (1, 64, 128, 8),
+                                                (300, 128, 2000 + 3, 8), (37, 192, 777, 3)])
+def test_producer_against_f64_product(sampler, rows, d, vocab, slack):
+    """slack 8: rows of the logits start at multiples of 16 bytes (stored 16 bytes a lane);
+    slack 3: they do not (stored value by value)."""
     rng = np.random.default_rng(rows * 1000 + d)
     hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(20, vocab // 8))
     temps = [0.0 if r % 5 == 4 else 0.5 + 0.1 * (r % 7) for r in range(rows)]
-    stride = ((vocab + 7) // 8) * 8 + 8
+    stride = ((vocab + 7) // 8) * 8 + slack
     h, w, buf, logits, tmax, tsum = _produce(sampler, hidden, weight, temps, rows, vocab, stride)
     _check_product(h, w, logits, tmax, tsum, temps)
     # nothing behind a row's last column is written
