@@ -186,10 +186,6 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         for (int j = 0; j < T::AHEAD; ++j) {
             const uint32_t s = s0 + (uint32_t)j;
             const uint32_t buf = s & 1u;
-            // ring[j] holds stage s + 1: into the other LDS stage (nobody reads it: the barrier
-            // that closed step s - 1 saw to that), and the registers ask for stage s + 1 + AHEAD
-            stage(ring_h[j], ring_w[j], buf ^ 1u, s + 1u < steps);
-            fetch(ring_h[j], ring_w[j], k_of(s + 1u + T::AHEAD));
             const char* base = lds + buf * T::STAGE_BYTES;
 #pragma unroll
             for (int kk = 0; kk < BK / 16; ++kk) {
@@ -211,6 +207,12 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
                     }
                 }
             }
+            // ring[j] holds stage s + 1: into the other LDS stage (nobody reads it: the barrier
+            // that closed step s - 1 saw to that), and the registers ask for stage s + 1 + AHEAD.
+            // Behind the products, so that a wave that must wait for its loads waits while the
+            // matrix pipe works.
+            stage(ring_h[j], ring_w[j], buf ^ 1u, s + 1u < steps);
+            fetch(ring_h[j], ring_w[j], k_of(s + 1u + T::AHEAD));
             __syncthreads();
         }
     }
