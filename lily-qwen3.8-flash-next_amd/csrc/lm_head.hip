@@ -25,8 +25,11 @@ __device__ __forceinline__ float rotated(float x) {
 // MI x NI products of 32 x 32; the tile is WAVES_M * MI * 32 rows by 128 columns (the width of a
 // summary), staged BK columns of d at a time, AHEAD stages of loads in flight (what is in flight
 // has to cover the memory's latency at the rate the tiles consume it).
-template <int WAVES_M_, int MI_, int NI_, int BK_, int AHEAD_, int RESIDENT_>
+template <int WAVES_M_, int MI_, int NI_, int BK_, int AHEAD_, int RESIDENT_, bool DIRECT_ = false>
 struct HeadTile {
+    // DIRECT: the loads write LDS themselves (global_load_lds_dwordx4, a wave's 64 pieces side by
+    // side), AHEAD + 1 stages in LDS; otherwise they pass through registers into two stages.
+    static constexpr bool DIRECT = DIRECT_;
     static constexpr int RESIDENT = RESIDENT_;   // workgroups a compute unit is to hold (bounds the registers)
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = 4 / WAVES_M_, MI = MI_, NI = NI_, BK = BK_;
     static constexpr int AHEAD = AHEAD_;   // stages asked from memory ahead of the one being multiplied
@@ -41,10 +44,11 @@ struct HeadTile {
     static constexpr int ROW_BYTES = SWIZZLED ? BK * 2 : BK * 2 + 16;
     static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;  // hidden rows, then weight rows
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;      // two stages
+    static constexpr int LDS_BYTES = (DIRECT ? AHEAD + 1 : 2) * STAGE_BYTES;
     static constexpr int A_PER = BM * PIECES / 256, B_PER = BN * PIECES / 256;   // pieces a thread brings
     static_assert(BN == LILY_TILE_COLS, "a workgroup's columns are one summary");
     static_assert(BM * PIECES % 256 == 0 && BN * PIECES % 256 == 0 && A_PER >= 1, "whole pieces per thread");
+    static_assert(!DIRECT || SWIZZLED, "the direct loads fill 64-byte rows");
     static_assert(LDS_BYTES >= (WAVES_N + 2) * BM * 4, "the epilogue's reductions reuse the stages");
 };
 
@@ -53,8 +57,8 @@ struct HeadTile {
 // columns of d at a time (16-byte loads from memory several stages ahead of the arithmetic,
 // 16-byte reads out of LDS).  The shapes: 32 rows for a decode step of a few sequences (the weights are
 // then read once at the speed of memory and the matrix cores idle), 256 rows - each wave 128 x
-// 64, six operand reads out of LDS for eight products - for a batch, whose bound is the matrix
-// cores and, just behind, the bandwidth of LDS.
+// 64, six operand reads out of LDS for eight products, loads that write LDS themselves - for a
+// batch, whose bound is the matrix cores and, just behind, the bandwidth of LDS.
 //
 // Workgroups are numbered so that an XCD's L2 holds the hidden rows its workgroups share (see
 // the numbering at the top of the kernel).
@@ -160,6 +164,92 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     const uint32_t a_at = (wm * (MI * 32u) + (lane & 31u)) * ROW_BYTES;
     const uint32_t b_at = T::A_BYTES + (wn * (NI * 32u) + (lane & 31u)) * ROW_BYTES;
 
+    if constexpr (T::DIRECT) {
+        // Loads that write LDS themselves.  One instruction of a wave fills 1 KB of LDS, lane
+        // after lane: 16 staged rows of 64 bytes; a lane asks memory for the piece that belongs
+        // in its place (the pieces of a row change places by the row's number, see HeadTile).
+        // Every step: wait until this step's own loads have landed (those of the steps asked for
+        // later may still be on their way), meet the other waves - their loads have landed too,
+        // and nobody reads the stage of the step before any more -, ask for the step AHEAD
+        // steps on into that stage, multiply.  All loads are unconditional (past the end of d
+        // the last step is asked for again, into a stage nobody will read).
+        const uint32_t steps = d / BK;
+        const uint32_t rot = (n_tile * 5u + m_tile * 3u) % steps;
+        auto k_of = [&](uint32_t stage_no) -> uint32_t {
+            uint32_t at = min(stage_no, steps - 1u) + rot;
+            at = at >= steps ? at - steps : at;
+            return at * BK;
+        };
+        constexpr int A_LOADS = T::A_BYTES / 4096, B_LOADS = T::B_BYTES / 4096;   // per wave and stage
+        static_assert(T::A_BYTES % 4096 == 0 && T::B_BYTES % 4096 == 0, "whole 1 KB blocks per wave");
+        const uint16_t* from_h[A_LOADS];
+        const uint16_t* from_w[B_LOADS];
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const uint32_t r = ((uint32_t)i * 4u + wave) * 16u + (lane >> 2);
+            const uint32_t kc = (lane & 3u) ^ ((r >> 1) & 3u);
+            from_h[i] = hidden + (uint64_t)min(m0 + r, rows - 1u) * hidden_stride + kc * 8u;
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            const uint32_t r = ((uint32_t)i * 4u + wave) * 16u + (lane >> 2);
+            const uint32_t kc = (lane & 3u) ^ ((r >> 1) & 3u);
+            from_w[i] = weight + (uint64_t)min(n0 + r, vocab - 1u) * weight_stride + kc * 8u;
+        }
+        typedef __attribute__((address_space(1))) const void* gptr;
+        typedef __attribute__((address_space(3))) void* lptr;
+        auto ask = [&](uint32_t stage_no, uint32_t buf) {
+            const uint32_t k0 = k_of(stage_no);
+            char* base = lds + buf * T::STAGE_BYTES + wave * 1024u;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                __builtin_amdgcn_global_load_lds((gptr)(from_h[i] + k0), (lptr)(base + i * 4096), 16, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                __builtin_amdgcn_global_load_lds((gptr)(from_w[i] + k0), (lptr)(base + T::A_BYTES + i * 4096), 16, 0, 0);
+            }
+        };
+        constexpr int NBUF = T::AHEAD + 1;
+#pragma unroll
+        for (int j = 0; j < T::AHEAD; ++j) {
+            ask((uint32_t)j, (uint32_t)j);
+        }
+        uint32_t buf = 0;
+        for (uint32_t s = 0; s < steps; ++s) {
+            // this step's loads: everything but the (AHEAD - 1) x (A_LOADS + B_LOADS) asked later
+            // (the barrier as an instruction: __syncthreads() carries a fence that would wait for
+            // every load in flight, the ones asked ahead included)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((T::AHEAD - 1) * (A_LOADS + B_LOADS))
+                         : "memory");
+            const uint32_t into = buf == 0u ? (uint32_t)NBUF - 1u : buf - 1u;   // the stage of step s - 1
+            ask(s + T::AHEAD, into);
+            const char* base = lds + buf * T::STAGE_BYTES;
+#pragma unroll
+            for (int kk = 0; kk < BK / 16; ++kk) {
+                bf16x8 a[MI], b[NI];
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + piece_at[kk]);
+                }
+#pragma unroll
+                for (int i = 0; i < NI; ++i) {
+                    b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + piece_at[kk]);
+                }
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        acc[mi][ni] =
+                            __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+                    }
+                }
+            }
+            buf = buf + 1u == (uint32_t)NBUF ? 0u : buf + 1u;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads asked past the end
+        __syncthreads();
+    } else {
     // Every load and every write to LDS below is unconditional (past the end of d the last
     // stage is asked for again): the compiler then counts the loads in flight and waits for
     // the oldest only; with a branch around any of them it waits for all.
@@ -215,6 +305,8 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
             fetch(ring_h[j], ring_w[j], k_of(s + 1u + T::AHEAD));
             __syncthreads();
         }
+    }
+
     }
 
     // ---- epilogue.  Element v of a lane's 16 sits in row 8 * (v / 4) + 4 * (lane / 32) + v % 4
@@ -388,7 +480,7 @@ hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t 
     if (rows <= 128u) {
         return launch_head_shape<HeadTile<2, 2, 2, 64, 3, 2>>(LILY_HEAD_ARGS);
     }
-    return launch_head_shape<HeadTile<2, 4, 2, 32, 3, 2>>(LILY_HEAD_ARGS);
+    return launch_head_shape<HeadTile<2, 4, 2, 32, 2, 2, true>>(LILY_HEAD_ARGS);
 #undef LILY_HEAD_ARGS
 }
 
