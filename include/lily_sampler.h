@@ -147,7 +147,9 @@ int lily_sampler_set_phase_trace(lily_sampler_t* s, uint64_t* trace_dev, uint64_
  * the caller) is set, every workgroup of a sampled row adds 1 to [0] when the streaming select
  * (k <= 64) produced its slice, [1] for the selects of sparsely masked rows and of k > 64
  * (sparse or bitmap), [2] for the exhaustive select; [3] collects a bit per reason the streaming
- * select gave a slice up.  NULL stops. */
+ * select gave a slice up.  A row of k > 64 that the two launches for rows of many candidates
+ * draw (plain rows without mask or bias list, penalties none or lowering) adds 1 to [1], or to
+ * [2], once, whatever the number of its workgroups.  NULL stops. */
 int lily_sampler_set_path_stats(lily_sampler_t* s, uint32_t* stats_dev);
 /* Measurement aid with no counterpart in the reference: one launch that only reads `rows` rows of
  * row_bytes bytes (stride_bytes apart) with the row kernel's shape - a workgroup of 256 threads a

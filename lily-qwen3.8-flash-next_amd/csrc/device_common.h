@@ -315,6 +315,21 @@ __device__ __forceinline__ void lse_reduce(Shared& sh, const LseAcc& l) {
 
 // ------------------------------------------------------------------ radix-select plumbing
 
+// Inclusive sums over the lanes of a wave (all 64 at work), lane 0 first, by six data-parallel
+// moves between neighbours: by 1, 2, 4 and 8 lanes within each row of 16 (a lane without such
+// a neighbour adds 0), then the last lane of row 0 into row 1 and of row 2 into row 3, then
+// lane 31 into rows 2 and 3.
+__device__ __forceinline__ uint32_t wave_scan_u32(uint32_t x) {
+    int v = (int)x;
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1, 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2, 3
+    return (uint32_t)v;
+}
+
 // With sh.hist complete: finds the bin in which the count from bin 255 downwards
 // reaches `need`.  Leaves sh.sel_bin, sh.need (what is still needed inside that
 // bin), sh.bin_count, and sh.all_taken = 1 when fewer than `need` were counted.
@@ -322,27 +337,22 @@ __device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
     if (threadIdx.x < 64) {
         const uint32_t lane = threadIdx.x;
         uint32_t h[4], sum = 0;
+#pragma unroll
         for (int j = 0; j < 4; ++j) {
             h[j] = sh.hist[255u - (4u * lane + j)];
             sum += h[j];
         }
-        uint32_t incl = sum;
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t t = __shfl_up(incl, o);
-            if ((int)lane >= o) {
-                incl += t;
-            }
-        }
+        const uint32_t incl = wave_scan_u32(sum);
         const uint32_t excl = incl - sum;
-        const uint32_t total = __shfl(incl, 63);
+        const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
         if (excl < need && need <= incl) {
             uint32_t seen = excl;
+#pragma unroll
             for (int j = 0; j < 4; ++j) {
-                if (seen + h[j] >= need) {
+                if (seen < need && seen + h[j] >= need) {
                     sh.sel_bin = 255u - (4u * lane + j);
                     sh.need = need - seen;
                     sh.bin_count = h[j];
-                    break;
                 }
                 seen += h[j];
             }
@@ -353,6 +363,33 @@ __device__ __forceinline__ void find_bin(Shared& sh, uint32_t need) {
     }
     __syncthreads();
 }
+
+// One thread's counts of one pass of a radix select.  The digit the thread meets first is
+// counted in a register and added once at the end: the keys of a row of logits share their
+// leading digits, adds by the lanes of a wave to one LDS word are served one after the other,
+// and the workgroup's waves share the one LDS - counted key by key, the leading passes are
+// that queue and little else.
+struct HistRun {
+    uint32_t d0, c0;
+    __device__ __forceinline__ void init() {
+        d0 = 0;
+        c0 = 0;
+    }
+    __device__ __forceinline__ void add(uint32_t* hist, uint32_t digit, bool on) {
+        // (no branch but around the add: selects, not jumps, for the common case)
+        const bool same = on & ((c0 == 0u) | (digit == d0));
+        d0 = same ? digit : d0;
+        c0 += same ? 1u : 0u;
+        if (on & !same) {
+            atomicAdd(&hist[digit], 1u);
+        }
+    }
+    __device__ __forceinline__ void flush(uint32_t* hist) {
+        if (c0 != 0u) {
+            atomicAdd(&hist[d0], c0);
+        }
+    }
+};
 
 // The top-k of cand[0..n) (zeros are invalid) compacted, unsorted, to the front;
 // returns how many there are.
@@ -375,12 +412,13 @@ __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, u
             sh.hist[tid] = 0;
         }
         __syncthreads();
+        HistRun run;
+        run.init();
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            if (mine[j] != 0 && (mine[j] & pmask) == prefix) {
-                atomicAdd(&sh.hist[(uint32_t)(mine[j] >> shift) & 255u], 1u);
-            }
+            run.add(sh.hist, (uint32_t)(mine[j] >> shift) & 255u, mine[j] != 0 && (mine[j] & pmask) == prefix);
         }
+        run.flush(sh.hist);
         __syncthreads();
         find_bin(sh, need);
         if (sh.all_taken != 0u) {
@@ -501,11 +539,12 @@ __device__ __forceinline__ float wg_kth_largest(const float (&ms)[8], uint32_t k
             sh.hist[tid] = 0;
         }
         __syncthreads();
+        HistRun run;
+        run.init();
         for (int j = 0; j < 8; ++j) {
-            if (keys[j] != 0u && (keys[j] & pmask) == prefix) {
-                atomicAdd(&sh.hist[(keys[j] >> shift) & 255u], 1u);
-            }
+            run.add(sh.hist, (keys[j] >> shift) & 255u, keys[j] != 0u && (keys[j] & pmask) == prefix);
         }
+        run.flush(sh.hist);
         __syncthreads();
         find_bin(sh, need);
         if (sh.all_taken != 0u) {

@@ -1,0 +1,456 @@
+// rows_wide.hip - rows that draw among many candidates (k > 64, up to the reference's cap of 1024,
+// which is what a request without top_k gets: src/kernels/sample.rs:17, :326-331), spread over
+// as many workgroups as rows of few candidates are.
+//
+// Two launches.  In the first every workgroup reads its slice of the row once and leaves its 256
+// lanes' largest values (penalised ids at their penalised worth); the workgroup that finishes
+// a row last takes the k-th largest of all the row's lane maxima: k lanes reach it, so k values
+// do - a lower bound of the row's k-th largest value that about k * (1 + a few per cent) values
+// reach.  In the second every workgroup reads its slice again (from the L2 now) and appends
+// the values that reach the bound to the row's list; the one that finishes last reads the
+// list - a thousand and some, whatever the number of slices -, selects, and runs the common
+// tail.  (The select of the other kernels keeps k
+// candidates per slice and can therefore spread a row with k = 1024 over 4 workgroups only.)
+#include <algorithm>
+
+#ifdef LILY_WIDE_TRACE
+#define LILY_TAIL_TRACE
+#endif
+
+#include "row_kernel.h"
+
+namespace lily {
+
+// Diagnostic stamps (LaunchCfg::phase_trace), compiled in with -DLILY_WIDE_TRACE (which also
+// turns on the tail's: slots 8 to 12).  First launch: 0 start, 1 slice read, 2 last slice in,
+// 3 keys loaded, 4 bound stored; second: 5 start, 6 slice read, 7 last slice in, 13 list read,
+// 14 selected.
+#ifdef LILY_WIDE_TRACE
+#define WIDE_MARK(i) phase(cfg, i)
+#else
+#define WIDE_MARK(i)
+#endif
+
+// What the two launches share beyond LaunchCfg.
+struct WideArgs {
+    float* lane_max;      // [rows][slices][NT]
+    float* bound;         // [rows]
+    uint32_t* count;      // [rows] candidates the row's slices have left so far (0 between launches)
+};
+
+template <bool INLINE>
+__device__ __forceinline__ const LILY_CONST RowArgs* wide_table(const LaunchCfg& cfg) {
+    if (INLINE) {
+        // the rows are the kernel's first argument: index the kernel-argument segment itself
+        return (const LILY_CONST RowArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+    }
+    return (const LILY_CONST RowArgs*)cfg.table;
+}
+
+// One pass over the slice's chunks, four loads in flight per thread, every load unconditional
+// (a chunk number past the slice is replaced by the slice's last; `use` says whether it counts).
+template <int DT, class F>
+__device__ __forceinline__ void wide_scan(const Geo<DT>& g, F&& per_chunk) {
+    const uint32_t tid = threadIdx.x;
+    if (g.main_hi <= g.main_lo) {
+        return;
+    }
+    for (uint32_t c0 = g.main_lo; c0 < g.main_hi; c0 += 4u * NT) {
+        u32x4 q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t c = min(c0 + (uint32_t)u * NT + tid, g.main_hi - 1u);
+            q[u] = gload(reinterpret_cast<const u32x4*>(g.base + (size_t)c * 16));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t c = c0 + (uint32_t)u * NT + tid;
+            if (c < g.main_hi) {
+                per_chunk(q[u], c);
+            }
+        }
+    }
+}
+
+// What a raw value is worth under the row's penalties (the arithmetic of finish_pre_temperature).
+__device__ __forceinline__ float wide_worth(const RowArgs& a, float x, uint32_t id) {
+    if (bit_of(a.touched, id)) {
+        uint32_t cnt = gload(a.counts + id);
+        asm volatile("" : "+v"(cnt));   // waited for here, inside the branch
+        if (cnt > 0u) {
+            x = x > 0.0f ? x / a.repetition : x * a.repetition;
+            x -= a.presence + a.frequency * (float)cnt;
+        }
+    }
+    return x;
+}
+
+// Bits id0 .. id0 + E - 1 of the bitmap of penalised ids (all below the vocabulary; the word
+// behind the bitmap's last is the row's largest count, so the second load stays in bounds).
+template <int E>
+__device__ __forceinline__ uint32_t wide_bits(const uint32_t* words, uint32_t id0) {
+    const uint32_t w = id0 >> 5, sh = id0 & 31u;
+    uint32_t b = gload(words + w) >> sh;
+    if (sh + (uint32_t)E > 32u) {
+        b |= gload(words + w + 1u) << (32u - sh);
+    }
+    return b & ((1u << E) - 1u);
+}
+
+// The ids of the partial 16-byte chunks at the slice's ends, one by one.
+template <int DT, class F>
+__device__ __forceinline__ void wide_edges(const RowArgs& a, const Geo<DT>& g, F&& per_id) {
+    for (int side = 0; side < 2; ++side) {
+        const uint32_t lo = side == 0 ? g.id_lo : g.edge_hi_begin;
+        const uint32_t hi = side == 0 ? g.edge_lo_end : g.id_hi;
+        for (uint32_t id = lo + threadIdx.x; id < hi; id += NT) {
+            per_id(load_logit<DT>(a.logits, id), id);
+        }
+    }
+}
+
+// The row's ticket: true in every thread of the workgroup that arrives last.  What the slices
+// hand over is stored through to memory (store_through) and read past the caches
+// (load_through), so the ticket needs no release or acquire at the scope of the device, which
+// would write back, and then invalidate, the whole L2 once per workgroup: the stores have
+// completed when the wait before the barrier ends, the ticket is taken after the barrier, and
+// the reads are issued after the ticket's value has come back.
+__device__ __forceinline__ bool wide_last(const LaunchCfg& cfg, uint32_t row, uint32_t S, Shared& sh) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);   // every counter at 0: this thread's stores have completed
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+        if (t == S - 1u) {
+            store_through(&cfg.ws_ticket[row], 0u);
+        }
+        sh.last = t == S - 1u ? 1u : 0u;
+    }
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    return sh.last != 0u;
+}
+
+// ---- first launch: lane maxima, the slice's sum of exponentials, the row's bound
+
+template <int DT, bool LSE, bool INLINE>
+__global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, LaunchCfg cfg, WideArgs w) {
+    __shared__ Shared sh;
+    constexpr int E = Geo<DT>::E;
+    const uint32_t tid = threadIdx.x, s = blockIdx.x, row = blockIdx.y, S = cfg.slices;
+    if (cfg.served != nullptr && *(const LILY_CONST uint32_t*)(cfg.served + row) != 0u) {
+        return;   // drawn by an earlier launch of the same call
+    }
+    WIDE_MARK(0);
+    RowArgs a;
+    load_row_args(a, wide_table<INLINE>(cfg) + row);
+    apply_selection(a);
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    Geo<DT> g;
+    g.init(a.logits, cfg.vocab, s, S);
+    const bool pen = (a.flags & F_PEN) != 0;
+    float lane_max = NEG_INF;
+    LseAcc lse;
+    lse.init();
+    wide_scan<DT>(g, [&](const u32x4& q, uint32_t c) {
+        float v[E];
+        unpack<DT>(q, v);
+        float m;
+        if (pen) {
+            const uint32_t id0 = g.id_of(c, 0);
+            const uint32_t bits = wide_bits<E>(a.touched, id0);
+            if (bits != 0u) {
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    if ((bits >> j) & 1u) {
+                        v[j] = wide_worth(a, v[j], id0 + (uint32_t)j);
+                    }
+                }
+            }
+            m = NEG_INF;
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                m = fmaxf(m, v[j]);   // (a NaN operand loses)
+            }
+        } else {
+            m = chunk_max<DT>(q);   // (NaN operands lose)
+        }
+        lane_max = fmaxf(lane_max, m);
+        if (want_lse && m > NEG_INF) {
+            const float safe = lse.rebase(m, a.c2);
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                if (v[j] > NEG_INF) {   // (false for a NaN: worth -inf)
+                    lse.term(v[j], a.c2, safe);
+                }
+            }
+        }
+    });
+    wide_edges<DT>(a, g, [&](float x, uint32_t id) {
+        if (pen) {
+            x = wide_worth(a, x, id);
+        }
+        if (x > NEG_INF) {
+            lane_max = fmaxf(lane_max, x);
+            if (want_lse) {
+                lse.add_one(x, a.c2);
+            }
+        }
+    });
+    WIDE_MARK(1);
+    const size_t slot = (size_t)row * S + s;
+    store_through(&w.lane_max[slot * NT + tid], lane_max);
+    if (want_lse) {
+        lse_reduce(sh, lse);
+        if (tid == 0) {
+            store_through(&cfg.ws_lse[2 * slot], sh.lse_mc);
+            store_through(&cfg.ws_lse[2 * slot + 1], sh.lse_s);
+        }
+    }
+    if (!wide_last(cfg, row, S, sh)) {
+        return;
+    }
+    WIDE_MARK(2);
+    // The k-th largest of the row's S x NT lane maxima, by a radix select on the leading 16
+    // bits of their order keys, 8 bits a pass: the bound is that key with the other 16 bits
+    // clear, at most 2^-7 of its magnitude below the k-th largest lane maximum, which lets a
+    // few per cent more values through.  A thread keeps its S keys in registers (the loops are
+    // unrolled over MAX_SLICES in groups of eight, a group past S is skipped by the whole
+    // workgroup): one wave per SIMD is at work here, and a pass that fetched each key from
+    // LDS, or the values from the L2 a few at a time, would wait out that latency over and over.
+    static_assert(MAX_SLICES == 64, "the unrolled loops below cover 64 keys a thread");
+    const uint32_t n = S * NT;
+    float got[MAX_SLICES];
+#pragma unroll
+    for (int j0 = 0; j0 < (int)MAX_SLICES; j0 += 8) {
+        if ((uint32_t)j0 < S) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t i = min((uint32_t)(j0 + u) * NT + tid, n - 1u);
+                got[j0 + u] = load_through(&w.lane_max[(size_t)row * S * NT + i]);
+            }
+        }
+    }
+    uint32_t keys[MAX_SLICES];
+#pragma unroll
+    for (int j = 0; j < (int)MAX_SLICES; ++j) {
+        const bool in = (uint32_t)j < S;   // (a group past S was not loaded: what it holds is not read)
+        keys[j] = in && got[j] > NEG_INF ? lilym_order_key(got[j]) : 0u;
+    }
+    WIDE_MARK(3);
+    uint32_t prefix = 0, pmask = 0, need = a.k;
+    bool enough = true;
+    for (int pass = 0; pass < 2 && enough; ++pass) {
+        const int shift = 24 - 8 * pass;
+        sh.hist[tid] = 0;
+        __syncthreads();
+        HistRun run;
+        run.init();
+#pragma unroll
+        for (int j0 = 0; j0 < (int)MAX_SLICES; j0 += 8) {
+            if ((uint32_t)j0 < S) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const uint32_t key = keys[j0 + u];
+                    run.add(sh.hist, (key >> shift) & 255u, key != 0u && (key & pmask) == prefix);
+                }
+            }
+        }
+        run.flush(sh.hist);
+        __syncthreads();
+        find_bin(sh, need);
+        if (sh.all_taken != 0u) {
+            enough = false;   // fewer than k lanes saw a finite value: every value is a candidate
+        } else {
+            prefix |= sh.sel_bin << shift;
+            pmask |= 255u << shift;
+            need = sh.need;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        store_through(&w.bound[row], enough ? lilym_key_value(prefix) : F32_LOWEST);
+    }
+    WIDE_MARK(4);
+}
+
+// ---- second launch: the values that reach the bound, then merge, select and tail
+
+template <int DT, bool LSE, bool INLINE>
+__global__ __launch_bounds__(NT, 4) void k_wide_draw(InlineRows rows_arg, LaunchCfg cfg, WideArgs w) {
+    __shared__ Shared sh;
+    __shared__ uint32_t n_mine;
+    constexpr int E = Geo<DT>::E;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, s = blockIdx.x, row = blockIdx.y, S = cfg.slices;
+    if (cfg.served != nullptr && *(const LILY_CONST uint32_t*)(cfg.served + row) != 0u) {
+        return;
+    }
+    WIDE_MARK(5);
+    if (tid == 0) {
+        tail_arrays(sh);
+        n_mine = 0;
+    }
+    RowArgs a;
+    load_row_args(a, wide_table<INLINE>(cfg) + row);
+    apply_selection(a);
+    const uint32_t vocab = cfg.vocab;
+    const uint32_t step = a.step + cfg.step_delta;
+    const bool want_lse = LSE && a.out_logprob != nullptr;
+    const bool pen = (a.flags & F_PEN) != 0;   // (of the kind that only lowers: the host sees to it)
+    const float bound = gload(w.bound + row);   // of the values' worth under the penalties
+    Geo<DT> g;
+    g.init(a.logits, vocab, s, S);
+    uint64_t* cand = dyn_lds;
+    const uint32_t cap = MERGE_CAP;   // what the slice's own list holds
+    __syncthreads();
+    auto offer = [&](float x, uint32_t id) {
+        if (!(x >= bound)) {
+            return;
+        }
+        if (pen) {
+            x = wide_worth(a, x, id);   // (never more than the raw value: the host sees to it)
+            if (!(x >= bound)) {
+                return;
+            }
+        }
+        const uint32_t at = atomicAdd(&n_mine, 1u);
+        if (at < cap) {
+            cand[at] = composite_of(x / a.temperature, id);
+        }
+    };
+    wide_scan<DT>(g, [&](const u32x4& q, uint32_t c) {
+        if (chunk_max<DT>(q) >= bound) {
+            float v[E];
+            unpack<DT>(q, v);
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                offer(v[j], g.id_of(c, j));
+            }
+        }
+    });
+    wide_edges<DT>(a, g, [&](float x, uint32_t id) { offer(x, id); });
+    __syncthreads();
+    WIDE_MARK(6);
+    // The slice's candidates go behind those the row's other slices have left (any order: the
+    // select does not care).  A row whose list would pass MERGE_CAP is counted on and not
+    // written: the last workgroup sees the count and takes the exhaustive select.
+    const uint32_t mine = n_mine;
+    if (tid == 0) {
+        n_mine = __hip_atomic_fetch_add(&w.count[row], mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const uint32_t base = n_mine;
+    if (base + mine <= MERGE_CAP) {
+        for (uint32_t i = tid; i < mine; i += NT) {
+            store_through(&cfg.ws_cand[(size_t)row * MERGE_CAP + base + i], cand[i]);
+        }
+    }
+    if (!wide_last(cfg, row, S, sh)) {
+        return;
+    }
+    WIDE_MARK(7);
+    if (tid == 0) {
+        sh.need = load_through(&w.count[row]);
+        store_through(&w.count[row], 0u);
+    }
+    __syncthreads();
+    const uint32_t total = sh.need;
+    uint32_t n;
+    bool sorted = false;
+    if (total > MERGE_CAP) {
+        // more than the buffers hold (values that tie by the thousand, a row in ascending
+        // order): the select that is right for any input, over the whole row
+        __syncthreads();
+        select_exhaustive<DT>(a, 0, vocab, a.k, want_lse, cand, min(cfg.dyn_slots, MERGE_CAP), sh);
+        n = min(sh.n_cand, min(cfg.dyn_slots, MERGE_CAP));
+        if (cfg.path_stats != nullptr && tid == 0) {
+            atomicAdd(&cfg.path_stats[2], 1u);
+        }
+    } else {
+        constexpr int PER = MERGE_CAP / NT;
+        for (int j0 = 0; j0 < PER; j0 += 8) {   // eight loads in flight
+            if ((uint32_t)j0 * NT >= total) {
+                break;
+            }
+            uint64_t got[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t i = min((uint32_t)(j0 + u) * NT + tid, total - 1u);
+                got[u] = load_through(&cfg.ws_cand[(size_t)row * MERGE_CAP + i]);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t i = (uint32_t)(j0 + u) * NT + tid;
+                if (i < total) {
+                    cand[i] = got[u];
+                }
+            }
+        }
+        if (want_lse && tid < 64u) {
+            double mt = -__builtin_huge_val(), st = 0.0;
+            if (lane < S) {
+                mt = load_through(&cfg.ws_lse[2 * ((size_t)row * S + lane)]);
+                st = load_through(&cfg.ws_lse[2 * ((size_t)row * S + lane) + 1]);
+                if (!(st > 0.0)) {
+                    mt = -__builtin_huge_val();
+                }
+            }
+            double m = mt;
+            for (int o = 32; o > 0; o >>= 1) {
+                m = fmax(m, __shfl_xor(m, o));
+            }
+            const double sum = wave_sum_d(st > 0.0 ? st * exp2(mt - m) : 0.0);
+            if (tid == 0) {
+                sh.lse_mc = m;
+                sh.lse_s = sum;
+            }
+        }
+        __syncthreads();
+        WIDE_MARK(13);
+        n = select_topk(cand, total, a.k, sh, sorted);
+        WIDE_MARK(14);
+        if (cfg.path_stats != nullptr && tid == 0) {
+            atomicAdd(&cfg.path_stats[1], 1u);
+        }
+    }
+    tail<DT, true>(a, vocab, step, n, sorted, cand, sh, cfg);
+}
+
+template <int DT, bool LSE, bool INLINE>
+static hipError_t launch_wide_variant(hipStream_t stream, uint32_t rows, const LaunchCfg& cfg,
+                                      const InlineRows* inline_rows, const WideArgs& w) {
+    const dim3 grid(cfg.slices, rows), block(NT);
+    static const InlineRows none = {};
+    const InlineRows& r = inline_rows != nullptr ? *inline_rows : none;
+    const size_t dyn2 = (size_t)cfg.dyn_slots * 8;
+    hipLaunchKernelGGL((k_wide_bound<DT, LSE, INLINE>), grid, block, 0, stream, r, cfg, w);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        return e;
+    }
+    hipLaunchKernelGGL((k_wide_draw<DT, LSE, INLINE>), grid, block, dyn2, stream, r, cfg, w);
+    return hipGetLastError();
+}
+
+hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
+                            const InlineRows* inline_rows, float* lane_max, float* bound, uint32_t* count) {
+    LaunchCfg cfg = cfg_in;
+    // the merging workgroup's candidates, then the tail's arrays behind the first K_CAP of them
+    cfg.dyn_slots = MERGE_CAP;
+    cfg.cand_cap = MERGE_CAP;
+    WideArgs w;
+    w.lane_max = lane_max;
+    w.bound = bound;
+    w.count = count;
+    const bool inl = inline_rows != nullptr;
+#define LILY_WIDE(DT)                                                                               \
+    (lse ? (inl ? launch_wide_variant<DT, true, true>(stream, rows, cfg, inline_rows, w)            \
+                : launch_wide_variant<DT, true, false>(stream, rows, cfg, inline_rows, w))          \
+         : (inl ? launch_wide_variant<DT, false, true>(stream, rows, cfg, inline_rows, w)           \
+                : launch_wide_variant<DT, false, false>(stream, rows, cfg, inline_rows, w)))
+    return dtype == LILY_BF16 ? LILY_WIDE(LILY_BF16) : LILY_WIDE(LILY_F32);
+#undef LILY_WIDE
+}
+
+}  // namespace lily

@@ -76,6 +76,7 @@ constexpr uint32_t WS_SLOTS = 1u << 22; // candidate slots of the workspace (row
 constexpr uint32_t STAGE_SLOTS = 4;
 constexpr size_t STAGE_ROW_BYTES = sizeof(RowArgs) + 16;   // a staged row: descriptor + three words + slack
 constexpr uint32_t TARGET_GROUPS = 512;  // workgroups a small batch is spread over
+constexpr uint32_t WIDE_FLOATS = 1u << 20;   // lane maxima the wide rows' workspace holds
 
 }  // namespace
 
@@ -88,6 +89,10 @@ struct lily_sampler {
     uint64_t* chain_cand = nullptr;   // [LILY_MAX_VERIFY_ROWS][CHAIN_CAP], then the rows' counts and
     uint32_t* chain_n = nullptr;      // the ticket of a chained launch
     uint32_t* chain_ticket = nullptr;
+    // rows that draw among many candidates (rows_wide.hip): null in a view without them
+    float* wide_max = nullptr;     // [WIDE_FLOATS] lane maxima, rows x slices x 256
+    float* wide_bound = nullptr;   // [WS_ROWS]
+    uint32_t* wide_count = nullptr;  // [WS_ROWS] candidates listed so far, 0 between launches
     uint32_t ws_rows = WS_ROWS;    // rows that may span several workgroups
     uint32_t ws_slots = WS_SLOTS;  // candidate slots behind ws_cand
     // Row table of lily_sample_rows batches above INLINE_ROWS.
@@ -100,6 +105,7 @@ struct lily_sampler {
     uint32_t stage_next = 0;
     uint32_t force_path = 0;
     uint32_t force_slices = 0;
+    bool no_wide = false;   // LILY_SAMPLER_WIDE=0: rows of many candidates go the other kernels' way
     uint64_t* phase_trace = nullptr;
     uint64_t phase_words = 0;
     uint32_t* path_stats = nullptr;
@@ -143,6 +149,7 @@ struct LaunchPart {
     uint32_t excl_words = 0;
     bool bitmap_layout = false;
     uint32_t cand_cap = 0;
+    bool wide = false;   // every row draws among many candidates: the two launches of rows_wide.hip
 };
 
 struct lily_plan {
@@ -328,6 +335,53 @@ void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t sl
     cfg->list_cap = SPECIAL_LIST_CAP;
 }
 
+// Whether a launch over `rows` goes the way of rows that draw among many candidates, and over how
+// many workgroups a row then: every row a plain draw (not forced, given as it is or selected on
+// the device) without mask or bias list, penalties none or of the kind that only lowers (the
+// second launch passes over chunks whose raw values stay below the bound), some row with
+// k > STREAM_K_MAX, and at least two workgroups a row.  0 = no.
+uint32_t wide_slices(const lily_sampler* s, const RowArgs* rows, uint32_t n, int dtype, uint32_t vocab) {
+    if (s->wide_max == nullptr || s->no_wide || s->force_path != 0 || n > s->ws_rows) {
+        return 0;
+    }
+    uint32_t kmax = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const RowArgs& r = rows[i];
+        if (r.mode != MODE_PLAIN || (r.flags & F_FORCED) || r.allow != nullptr || r.n_bias != 0) {
+            return 0;
+        }
+        if (r.flags & F_PEN) {
+            const bool lowering = r.repetition >= 1.0f && r.presence >= 0.0f && r.frequency >= 0.0f;
+            if (!lowering) {
+                return 0;
+            }
+        }
+        kmax = r.k > kmax ? r.k : kmax;
+    }
+    if (kmax <= STREAM_K_MAX) {
+        return 0;
+    }
+    // (twice the workgroups of the other kernels: what runs long here is the one workgroup a
+    // row that finishes each launch, and the others have left the CUs by then)
+    uint32_t sl = s->force_slices ? s->force_slices : (2 * TARGET_GROUPS + n - 1) / n;
+    const uint32_t e = dtype == LILY_BF16 ? 8 : 4;
+    const uint32_t nch = (vocab + 2 * (e - 1)) / e + 1;
+    const uint32_t by_block = (nch + 256u * STREAM_UNROLL - 1) / (256u * STREAM_UNROLL);
+    sl = sl > by_block ? by_block : sl;
+    sl = sl > MAX_SLICES ? MAX_SLICES : sl;
+    if ((uint64_t)n * MERGE_CAP > s->ws_slots) {   // a row's list of candidates: MERGE_CAP slots
+        return 0;
+    }
+    const uint64_t by_max = (uint64_t)WIDE_FLOATS / ((uint64_t)n * 256u);
+    sl = sl > by_max ? (uint32_t)by_max : sl;
+    // the bound is the k-th largest of slices x 256 lane maxima: with twice k of them it is the
+    // median of the lanes' maxima, which about 1.4 k values reach on rows of Gaussian logits
+    if (sl < 2 || (uint64_t)sl * 256u < 2ull * kmax) {
+        return 0;
+    }
+    return sl;
+}
+
 // Attaches the phase trace when the launch fits the caller's buffer.
 void attach_trace(const lily_sampler* s, LaunchCfg* cfg, uint32_t rows) {
     if (s->phase_trace != nullptr &&
@@ -436,6 +490,10 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
         const RowArgs* sub = table + part.first;
         part.ws_k = max_k(sub, part.rows);
         part.slices = choose_slices(s, part.rows, part.ws_k, vocab, dtype);
+        if (const uint32_t ws = wide_slices(s, sub, part.rows, dtype, vocab)) {
+            part.wide = true;
+            part.slices = ws;
+        }
         const LaunchShape shp = shape_of(s, sub, part.rows, dtype, vocab, part.slices, part.ws_k);
         part.kind = shp.kind();
         part.lse = shp.lse;
@@ -458,6 +516,11 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
     cfg.excl_words = part.excl_words;
     cfg.bitmap_layout = part.bitmap_layout ? 1u : 0u;
     cfg.cand_cap = part.cand_cap;
+    if (part.wide) {
+        HIP_TRY(launch_rows_wide(s->stream, dtype, part.lse, part.rows, cfg, nullptr, s->wide_max,
+                                 s->wide_bound, s->wide_count));
+        return LILY_OK;
+    }
     HIP_TRY(launch_rows(s->stream, dtype, part.kind, part.lse, part.rows, cfg, nullptr, part.dyn_bytes));
     return LILY_OK;
 }
@@ -474,6 +537,18 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     ON_DEVICE(s->device);
     const uint32_t kmax = max_k(rows.r, n);
     LaunchCfg cfg;
+    if (!chained) {
+        if (const uint32_t ws = wide_slices(s, rows.r, n, dtype, vocab)) {
+            fill_cfg(s, &cfg, vocab, ws, kmax, 0, nullptr);
+            bool lse = false;
+            for (uint32_t i = 0; i < n; ++i) {
+                lse = lse || rows.r[i].out_logprob != nullptr;
+            }
+            HIP_TRY(launch_rows_wide(s->stream, dtype, lse, n, cfg, &rows, s->wide_max, s->wide_bound,
+                                     s->wide_count));
+            return LILY_OK;
+        }
+    }
     const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
     fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
     if (chained) {
@@ -788,12 +863,19 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     if (const char* p = std::getenv("LILY_SAMPLER_SLICES")) {
         s->force_slices = (uint32_t)std::atoi(p);
     }
+    if (const char* p = std::getenv("LILY_SAMPLER_WIDE")) {
+        s->no_wide = std::atoi(p) == 0;
+    }
     const size_t slots = (size_t)WS_ROWS * MAX_SLICES;
     hipError_t err = hipMalloc(reinterpret_cast<void**>(&s->ws_cand),
                                (size_t)WS_SLOTS * sizeof(uint64_t));
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_lse), slots * 16);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
     if (err == hipSuccess) err = hipMemset(s->ws_ticket, 0, WS_ROWS * 4);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->wide_max), (size_t)WIDE_FLOATS * 4);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->wide_bound), (size_t)WS_ROWS * 4);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->wide_count), WS_ROWS * 4);
+    if (err == hipSuccess) err = hipMemset(s->wide_count, 0, WS_ROWS * 4);
     const size_t chain_bytes = (size_t)LILY_MAX_VERIFY_ROWS * CHAIN_CAP * 8 + (LILY_MAX_VERIFY_ROWS + 1) * 4;
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->chain_cand), chain_bytes);
     if (err == hipSuccess) err = hipMemset(s->chain_cand, 0, chain_bytes);
@@ -825,6 +907,9 @@ void lily_sampler_destroy(lily_sampler_t* s) {
     (void)hipFree(s->ws_cand);
     (void)hipFree(s->ws_lse);
     (void)hipFree(s->ws_ticket);
+    (void)hipFree(s->wide_max);
+    (void)hipFree(s->wide_bound);
+    (void)hipFree(s->wide_count);
     (void)hipFree(s->chain_cand);
     (void)hipFree(s->table_dev);
     for (uint32_t i = 0; i < STAGE_SLOTS; ++i) {

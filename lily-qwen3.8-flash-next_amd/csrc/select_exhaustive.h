@@ -26,16 +26,17 @@ __device__ __forceinline__ void select_exhaustive(const RowArgs& a, uint32_t e0,
             sh.hist[tid] = 0;
         }
         __syncthreads();
+        HistRun run;
+        run.init();
         for (uint32_t id = e0 + tid; id < e1; id += NT) {
             const float u = pre_temperature_of<DT>(a, id);
             if (pass == 0 && want_lse) {
                 lse.add_one(u, a.c2);
             }
             const uint64_t c = composite_of(u / a.temperature, id);
-            if (c != 0 && (c & pmask) == prefix) {
-                atomicAdd(&sh.hist[(uint32_t)(c >> shift) & 255u], 1u);
-            }
+            run.add(sh.hist, (uint32_t)(c >> shift) & 255u, c != 0 && (c & pmask) == prefix);
         }
+        run.flush(sh.hist);
         __syncthreads();
         find_bin(sh, need);
         take_all = sh.all_taken != 0u;
