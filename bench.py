@@ -209,6 +209,16 @@ def main():
             p1 = sampler.plan(l1, [LS.SamplingParams.greedy(**kw)], [0], o1)
             others[name] = {"us_per_step": time_steps(stream, lambda i: p1.run(i), n_lat, w_lat) * 1e3}
             p1.close()
+        # the decode step of config 2 without top_k: the reference then keeps 1024 candidates
+        # (src/kernels/sample.rs:326-331), the case of a request that names no top_k
+        lp2 = torch.zeros(4, dtype=torch.float32, device=device)
+        for name, with_lp in (("decode_b4_default_top_k", False), ("decode_b4_default_top_k_logprob", True)):
+            pk = [LS.SamplingParams.greedy(**dict(kw, top_k=0)) for kw in c2["params"]]
+            torch.cuda.synchronize()
+            p1 = sampler.plan(l2, pk, [0] * 4, o2, scratch=s2, out_logprobs=lp2 if with_lp else None)
+            others[name] = {"us_per_step": time_steps(stream, lambda i: p1.run(i), n_lat, w_lat) * 1e3, "rows": 4,
+                            "k": 1024, "paths": paths_of(sampler, lambda i: p1.run(0))}
+            p1.close()
         c3 = W.config3()
         m3 = c3["target"].shape[0]
         t3 = torch.from_numpy(c3["target"]).to(device)
@@ -250,6 +260,12 @@ def main():
         others["config4_constrained"] = {"us_per_step": us4, "rows": 64,
                                          "achieved_GBs": bytes4 / (us4 * 1e-6) / 1e9,
                                          "paths": paths_of(sampler, lambda i: p4.run(0))}
+        p4.close()
+        torch.cuda.synchronize()
+        p4 = sampler.plan(l4, [LS.SamplingParams.greedy(**kw) for kw in c4["params"]], [7] * 64, o4)
+        us4 = time_steps(stream, lambda i: p4.run(i), n_lat, w_lat) * 1e3
+        others["config4_rows_unconstrained"] = {"us_per_step": us4, "rows": 64, "k": 1024,
+                                                "paths": paths_of(sampler, lambda i: p4.run(0))}
         p4.close()
 
     # ---- the logits' producer (bf16 head on the matrix cores, d = 4096) and the draws from its
