@@ -153,7 +153,7 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
             took = done ? 0u : took;
         }
         if (KIND == 1 && !done && cfg.path == 0u && a.allow != nullptr) {
-            done = select_sparse<DT, LSE>(a, g, a.k, cand, min(cfg.dyn_slots, MERGE_CAP), sh, sorted);
+            done = select_sparse<DT, LSE>(a, g, a.k, cand, min(cfg.dyn_slots, MERGE_CAP), sh, sorted, cfg);
             took = done ? 1u : took;
         }
         if (KIND != 2 && !done && cfg.path != 1u && cfg.bitmap_layout != 0u) {

@@ -13,9 +13,17 @@ namespace lily {
 // penalties), adds its term to the row sum and becomes a candidate.  Nothing of the row is
 // streamed: the mask's words and one logit per allowed id are all that is read.  Returns
 // false, with nothing changed, when the slice admits more ids than `cap` candidates.
+//
+// Diagnostic stamps with -DLILY_SPARSE_TRACE (LaunchCfg::phase_trace): 1 ids counted, 2 ids
+// listed, 3 ids evaluated, 13 row sum reduced (the caller stamps 4 behind the select).
+#ifdef LILY_SPARSE_TRACE
+#define SPARSE_MARK(i) phase(cfg, i)
+#else
+#define SPARSE_MARK(i)
+#endif
 template <int DT, bool LSE>
 __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g, uint32_t k, uint64_t* cand,
-                                              uint32_t cap, Shared& sh, bool& sorted) {
+                                              uint32_t cap, Shared& sh, bool& sorted, const LaunchCfg& cfg) {
     static_assert(STREAM_BIAS_CAP <= NT, "one thread stages one bias entry");
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const bool want_lse = LSE && a.out_logprob != nullptr;
@@ -35,18 +43,30 @@ __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g
                               gload(&a.bias[tid].id);
         }
     }
+    // The mask's words are asked for eight at a time (every load issued, a word past the
+    // slice replaced by the slice's last and not counted): a load per turn of the loop is a
+    // trip to the L2 per turn.
+    constexpr int WB = 8;
+    const uint32_t n_words = w_hi - w_lo;
+    auto words_of = [&](uint32_t i0, uint32_t (&wv)[WB]) {
+#pragma unroll
+        for (int u = 0; u < WB; ++u) {
+            const uint32_t i = i0 + (uint32_t)u * NT + tid;
+            const uint32_t got = word(w_lo + min(i, n_words - 1u));
+            wv[u] = i < n_words ? got : 0u;
+        }
+    };
     uint32_t mine = 0;
-    for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
-        mine += (uint32_t)__popc(word(i));
-    }
-    // Exclusive scan of the threads' counts: inside the wave, then over the waves.
-    uint32_t incl = mine;
-    for (int o = 1; o < 64; o <<= 1) {
-        const uint32_t t = __shfl_up(incl, o);
-        if ((int)lane >= o) {
-            incl += t;
+    for (uint32_t i0 = 0; i0 < n_words; i0 += WB * NT) {
+        uint32_t wv[WB];
+        words_of(i0, wv);
+#pragma unroll
+        for (int u = 0; u < WB; ++u) {
+            mine += (uint32_t)__popc(wv[u]);
         }
     }
+    // Exclusive scan of the threads' counts: inside the wave, then over the waves.
+    const uint32_t incl = wave_scan_u32(mine);
     if (lane == 63u) {
         sh.red_i[w] = incl;
     }
@@ -61,46 +81,77 @@ __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g
     if (total > cap) {
         return false;
     }
-    for (uint32_t i = w_lo + tid; i < w_hi; i += NT) {
-        uint32_t bits = word(i);
-        while (bits != 0u) {
-            cand[base++] = (uint64_t)(i * 32u + (uint32_t)__builtin_ctz(bits));
-            bits &= bits - 1u;
+    SPARSE_MARK(1);
+    for (uint32_t i0 = 0; i0 < n_words; i0 += WB * NT) {
+        uint32_t wv[WB];
+        words_of(i0, wv);
+#pragma unroll
+        for (int u = 0; u < WB; ++u) {
+            const uint32_t i = w_lo + i0 + (uint32_t)u * NT + tid;
+            uint32_t bits = wv[u];
+            while (bits != 0u) {
+                cand[base++] = (uint64_t)(i * 32u + (uint32_t)__builtin_ctz(bits));
+                bits &= bits - 1u;
+            }
         }
     }
     __syncthreads();
+    SPARSE_MARK(2);
     LseAcc lse;
     lse.init();
-    for (uint32_t i = tid; i < total; i += NT) {
-        const uint32_t id = (uint32_t)cand[i];
-        float l = load_logit<DT>(a.logits, id);
-        const uint32_t c = pen ? gload(a.counts + id) : 0u;
-        float u;
-        if (bias_lds) {
-            for (uint32_t j = 0; j < n_bias; ++j) {
-                const uint64_t e = cand[cap + j];
-                if ((uint32_t)e == id) {
-                    l += lilym_bits_f32((uint32_t)(e >> 32));
+    // Four ids a thread at a time, their logits and counts asked for together (an id past the
+    // list is replaced by id 0 and dropped).
+    constexpr int EB = 4;
+    for (uint32_t i0 = 0; i0 < total; i0 += EB * NT) {
+        uint32_t ids[EB], cs[EB];
+        float ls[EB];
+#pragma unroll
+        for (int q = 0; q < EB; ++q) {
+            const uint32_t i = i0 + (uint32_t)q * NT + tid;
+            ids[q] = i < total ? (uint32_t)cand[i] : 0u;
+        }
+#pragma unroll
+        for (int q = 0; q < EB; ++q) {
+            ls[q] = load_logit<DT>(a.logits, ids[q]);
+            cs[q] = pen ? gload(a.counts + ids[q]) : 0u;
+        }
+#pragma unroll
+        for (int q = 0; q < EB; ++q) {
+            const uint32_t i = i0 + (uint32_t)q * NT + tid;
+            if (i >= total) {
+                continue;
+            }
+            const uint32_t id = ids[q], c = cs[q];
+            float l = ls[q];
+            float u;
+            if (bias_lds) {
+                for (uint32_t j = 0; j < n_bias; ++j) {
+                    const uint64_t e = cand[cap + j];
+                    if ((uint32_t)e == id) {
+                        l += lilym_bits_f32((uint32_t)(e >> 32));
+                    }
                 }
+                if (c > 0u) {
+                    l = l > 0.0f ? l / a.repetition : l * a.repetition;
+                    l -= a.presence + a.frequency * (float)c;
+                }
+                u = l;
+            } else {
+                u = finish_pre_temperature(a, id, l, c, true);
             }
-            if (c > 0u) {
-                l = l > 0.0f ? l / a.repetition : l * a.repetition;
-                l -= a.presence + a.frequency * (float)c;
+            if (want_lse) {
+                lse.add_one(u, a.c2);
             }
-            u = l;
-        } else {
-            u = finish_pre_temperature(a, id, l, c, true);
+            cand[i] = composite_of(u / a.temperature, id);  // 0 for -inf: dropped by the select
         }
-        if (want_lse) {
-            lse.add_one(u, a.c2);
-        }
-        cand[i] = composite_of(u / a.temperature, id);  // 0 for -inf: dropped by the select
     }
+    SPARSE_MARK(3);
     if (want_lse) {
         lse_reduce(sh, lse);
     } else {
         __syncthreads();
     }
+    SPARSE_MARK(13);
     sorted = false;
     const uint32_t n = select_topk(cand, total, k, sh, sorted);
     if (tid == 0) {
