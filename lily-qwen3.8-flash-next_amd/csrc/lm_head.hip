@@ -38,8 +38,8 @@ struct HeadTile {
     static constexpr int PIECES = BK / 8;                  // 16-byte pieces of a staged row
     // A staged row: 128 bytes of d and 16 of padding (8 rows then cover all banks), or 64 bytes
     // without padding whose four 16-byte pieces change places by the row's number (piece ^
-    // (row / 2) % 4): 8 rows' pieces of one column, and the 8 pieces of two rows, then lie in
-    // 8 different groups of banks.
+    // (row / 4) % 4): rows r, r + 4, r + 8 and r + 12 start in the same bank, so the pieces of
+    // one column that 16 lanes read from 16 rows in a row lie in 16 different groups of banks.
     static constexpr bool SWIZZLED = BK == 32;
     static constexpr int ROW_BYTES = SWIZZLED ? BK * 2 : BK * 2 + 16;
     static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
@@ -106,13 +106,13 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     for (int i = 0; i < T::A_PER; ++i) {
         const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
         src_h[i] = hidden + (uint64_t)min(m0 + r, rows - 1u) * hidden_stride + kc * 8u;
-        dst_h[i] = r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 1) & 3u)) : kc) * 16u;
+        dst_h[i] = r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 2) & 3u)) : kc) * 16u;
     }
 #pragma unroll
     for (int i = 0; i < T::B_PER; ++i) {
         const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
         src_w[i] = weight + (uint64_t)min(n0 + r, vocab - 1u) * weight_stride + kc * 8u;
-        dst_w[i] = T::A_BYTES + r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 1) & 3u)) : kc) * 16u;
+        dst_w[i] = T::A_BYTES + r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 2) & 3u)) : kc) * 16u;
     }
     // ring[j]: the loads of a stage on their way (registers), written to LDS one step before use
     w32x4 ring_h[T::AHEAD][T::A_PER], ring_w[T::AHEAD][T::B_PER];
@@ -159,7 +159,7 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
         const uint32_t piece = (lane >> 5) + 2u * (uint32_t)kk;
-        piece_at[kk] = (T::SWIZZLED ? (piece ^ ((lane >> 1) & 3u)) : piece) * 16u;
+        piece_at[kk] = (T::SWIZZLED ? (piece ^ ((lane >> 2) & 3u)) : piece) * 16u;
     }
     const uint32_t a_at = (wm * (MI * 32u) + (lane & 31u)) * ROW_BYTES;
     const uint32_t b_at = T::A_BYTES + (wn * (NI * 32u) + (lane & 31u)) * ROW_BYTES;
@@ -187,13 +187,13 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) {
             const uint32_t r = ((uint32_t)i * 4u + wave) * 16u + (lane >> 2);
-            const uint32_t kc = (lane & 3u) ^ ((r >> 1) & 3u);
+            const uint32_t kc = (lane & 3u) ^ ((r >> 2) & 3u);
             from_h[i] = hidden + (uint64_t)min(m0 + r, rows - 1u) * hidden_stride + kc * 8u;
         }
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i) {
             const uint32_t r = ((uint32_t)i * 4u + wave) * 16u + (lane >> 2);
-            const uint32_t kc = (lane & 3u) ^ ((r >> 1) & 3u);
+            const uint32_t kc = (lane & 3u) ^ ((r >> 2) & 3u);
             from_w[i] = weight + (uint64_t)min(n0 + r, vocab - 1u) * weight_stride + kc * 8u;
         }
         typedef __attribute__((address_space(1))) const void* gptr;
@@ -210,42 +210,65 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
                 __builtin_amdgcn_global_load_lds((gptr)(from_w[i] + k0), (lptr)(base + T::A_BYTES + i * 4096), 16, 0, 0);
             }
         };
+        // NBUF stages in LDS, all asked for before the first product.  The loop works in half
+        // steps (BK = 32 is two operands of 16 along d): while the products of one half run,
+        // the operands of the next half are on their way from LDS into the other set of
+        // registers.  The barrier sits between the halves: before it a wave has read all it
+        // wants of stage s, behind it stage s + 1 has landed for everybody, stage s's place
+        // is asked for stage s + NBUF, and the second half's products run over the reads of
+        // stage s + 1's first operands.
         constexpr int NBUF = T::AHEAD + 1;
+        static_assert(BK == 32, "two halves a step");
 #pragma unroll
-        for (int j = 0; j < T::AHEAD; ++j) {
+        for (int j = 0; j < NBUF; ++j) {
             ask((uint32_t)j, (uint32_t)j);
         }
-        uint32_t buf = 0;
-        for (uint32_t s = 0; s < steps; ++s) {
-            // this step's loads: everything but the (AHEAD - 1) x (A_LOADS + B_LOADS) asked later
-            // (the barrier as an instruction: __syncthreads() carries a fence that would wait for
-            // every load in flight, the ones asked ahead included)
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((T::AHEAD - 1) * (A_LOADS + B_LOADS))
-                         : "memory");
-            const uint32_t into = buf == 0u ? (uint32_t)NBUF - 1u : buf - 1u;   // the stage of step s - 1
-            ask(s + T::AHEAD, into);
-            const char* base = lds + buf * T::STAGE_BYTES;
+        auto operands = [&](bf16x8 (&a)[MI], bf16x8 (&b)[NI], uint32_t from, int kk) {
+            const char* base = lds + from * T::STAGE_BYTES;
 #pragma unroll
-            for (int kk = 0; kk < BK / 16; ++kk) {
-                bf16x8 a[MI], b[NI];
+            for (int i = 0; i < NI; ++i) {
+                b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + piece_at[kk]);
+            }
 #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + piece_at[kk]);
-                }
+            for (int i = 0; i < MI; ++i) {
+                a[i] = *reinterpret_cast<const bf16x8*>(base + a_at + i * 32 * ROW_BYTES + piece_at[kk]);
+            }
+        };
+        auto products = [&](const bf16x8 (&a)[MI], const bf16x8 (&b)[NI]) {
 #pragma unroll
-                for (int i = 0; i < NI; ++i) {
-                    b[i] = *reinterpret_cast<const bf16x8*>(base + b_at + i * 32 * ROW_BYTES + piece_at[kk]);
-                }
+            for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
-                for (int mi = 0; mi < MI; ++mi) {
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        acc[mi][ni] =
-                            __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
-                    }
+                for (int ni = 0; ni < NI; ++ni) {
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
                 }
             }
-            buf = buf + 1u == (uint32_t)NBUF ? 0u : buf + 1u;
+        };
+        // stage 0 has landed when all but the loads of the NBUF - 1 later stages have
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NBUF - 1) * (A_LOADS + B_LOADS)) : "memory");
+        bf16x8 a0[MI], b0[NI], a1[MI], b1[NI];
+        operands(a0, b0, 0, 0);
+        uint32_t buf = 0;
+        for (uint32_t s = 0; s < steps; ++s) {
+            const uint32_t after = buf + 1u == (uint32_t)NBUF ? 0u : buf + 1u;
+            // This half's operands have had eight products' time to arrive.  Said here, as an
+            // instruction the compiler counts, before the reads of the next half are issued:
+            // left to itself it waits behind them, for all of them.
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+            __builtin_amdgcn_sched_barrier(0);
+            operands(a1, b1, buf, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            products(a0, b0);
+            __builtin_amdgcn_sched_barrier(0);
+            // (the barrier as an instruction: __syncthreads() carries a fence that would wait for
+            // every load in flight, the ones asked ahead included)
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): this wave has read what it wants of stage s
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NBUF - 2) * (A_LOADS + B_LOADS)) : "memory");
+            ask(s + (uint32_t)NBUF, buf);
+            operands(a0, b0, after, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            products(a1, b1);
+            __builtin_amdgcn_sched_barrier(0);
+            buf = after;
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads asked past the end
         __syncthreads();
