@@ -89,9 +89,31 @@ __device__ __forceinline__ bool select_sparse(const RowArgs& a, const Geo<DT>& g
         for (int u = 0; u < WB; ++u) {
             const uint32_t i = w_lo + i0 + (uint32_t)u * NT + tid;
             uint32_t bits = wv[u];
-            while (bits != 0u) {
-                cand[base++] = (uint64_t)(i * 32u + (uint32_t)__builtin_ctz(bits));
-                bits &= bits - 1u;
+            // A mask's bits come in clusters (a grammar's token classes): a lane that listed a
+            // full word bit by bit would keep its wave 32 turns.  Words of more than 8 bits are
+            // listed by the wave together, a bit a lane, the word, its place in the list and
+            // its number read from the lane that holds them; the others bit by bit.
+            const uint32_t n_bits = (uint32_t)__popc(bits), place = base;
+            base += n_bits;
+            const bool dense = n_bits > 8u;
+            uint64_t votes = __ballot(dense);
+            while (votes != 0ull) {
+                const int from = __builtin_ctzll(votes);
+                votes &= votes - 1ull;
+                const uint32_t w_bits = (uint32_t)__builtin_amdgcn_readlane((int)bits, from);
+                const uint32_t w_place = (uint32_t)__builtin_amdgcn_readlane((int)place, from);
+                const uint32_t w_index = (uint32_t)__builtin_amdgcn_readlane((int)i, from);
+                if (lane < 32u && ((w_bits >> lane) & 1u) != 0u) {
+                    cand[w_place + (uint32_t)__popc(w_bits & ((1u << lane) - 1u))] =
+                        (uint64_t)(w_index * 32u + lane);
+                }
+            }
+            if (!dense) {
+                uint32_t at = place;
+                while (bits != 0u) {
+                    cand[at++] = (uint64_t)(i * 32u + (uint32_t)__builtin_ctz(bits));
+                    bits &= bits - 1u;
+                }
             }
         }
     }
