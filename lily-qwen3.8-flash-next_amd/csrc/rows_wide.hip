@@ -33,7 +33,8 @@ namespace lily {
 
 // What the two launches share beyond LaunchCfg.
 struct WideArgs {
-    float* lane_max;      // [rows][slices][NT]
+    float* lane_max;      // [rows][slices][lanes]
+    uint32_t lanes;       // values a slice leaves: NT, or NT / 2 (the larger of each pair of lanes)
     float* bound;         // [rows]
     uint32_t* count;      // [rows] candidates the row's slices have left so far (0 between launches)
 };
@@ -200,7 +201,17 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
     });
     WIDE_MARK(1);
     const size_t slot = (size_t)row * S + s;
-    store_through(&w.lane_max[slot * NT + tid], lane_max);
+    if (w.lanes == NT) {
+        store_through(&w.lane_max[slot * NT + tid], lane_max);
+    } else {
+        // (with slices enough that half the lanes still are four times k, half the keys make
+        // the last workgroup's select half as long)
+        const int other = __builtin_amdgcn_update_dpp(0, (int)lilym_f32_bits(lane_max), 0xb1, 0xf, 0xf, true);   // quad_perm [1, 0, 3, 2]
+        lane_max = fmaxf(lane_max, lilym_bits_f32((uint32_t)other));
+        if ((tid & 1u) == 0u) {
+            store_through(&w.lane_max[slot * (NT / 2) + tid / 2u], lane_max);
+        }
+    }
     if (want_lse) {
         lse_reduce(sh, lse);
         if (tid == 0) {
@@ -212,7 +223,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
         return;
     }
     WIDE_MARK(2);
-    // The k-th largest of the row's S x NT lane maxima, by a radix select on the leading 16
+    // The k-th largest of the row's S x lanes lane maxima, by a radix select on the leading 16
     // bits of their order keys, 8 bits a pass: the bound is that key with the other 16 bits
     // clear, at most 2^-7 of its magnitude below the k-th largest lane maximum, which lets a
     // few per cent more values through.  A thread keeps its S keys in registers (the loops are
@@ -220,22 +231,22 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
     // workgroup): one wave per SIMD is at work here, and a pass that fetched each key from
     // LDS, or the values from the L2 a few at a time, would wait out that latency over and over.
     static_assert(MAX_SLICES == 64, "the unrolled loops below cover 64 keys a thread");
-    const uint32_t n = S * NT;
+    const uint32_t n = S * w.lanes, mine_n = (n + NT - 1u) / NT;   // keys in all, keys a thread
     float got[MAX_SLICES];
 #pragma unroll
     for (int j0 = 0; j0 < (int)MAX_SLICES; j0 += 8) {
-        if ((uint32_t)j0 < S) {
+        if ((uint32_t)j0 < mine_n) {
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const uint32_t i = min((uint32_t)(j0 + u) * NT + tid, n - 1u);
-                got[j0 + u] = load_through(&w.lane_max[(size_t)row * S * NT + i]);
+                got[j0 + u] = load_through(&w.lane_max[(size_t)row * n + i]);
             }
         }
     }
     uint32_t keys[MAX_SLICES];
 #pragma unroll
     for (int j = 0; j < (int)MAX_SLICES; ++j) {
-        const bool in = (uint32_t)j < S;   // (a group past S was not loaded: what it holds is not read)
+        const bool in = (uint32_t)j * NT + tid < n;   // (a group past the last was not loaded: what it holds is not read)
         keys[j] = in && got[j] > NEG_INF ? lilym_order_key(got[j]) : 0u;
     }
     WIDE_MARK(3);
@@ -249,7 +260,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
         run.init();
 #pragma unroll
         for (int j0 = 0; j0 < (int)MAX_SLICES; j0 += 8) {
-            if ((uint32_t)j0 < S) {
+            if ((uint32_t)j0 < mine_n) {
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const uint32_t key = keys[j0 + u];
@@ -441,6 +452,7 @@ hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t ro
     cfg.cand_cap = MERGE_CAP;
     WideArgs w;
     w.lane_max = lane_max;
+    w.lanes = (uint64_t)cfg.slices * (NT / 2) >= 4ull * cfg.ws_k ? NT / 2 : NT;
     w.bound = bound;
     w.count = count;
     const bool inl = inline_rows != nullptr;
