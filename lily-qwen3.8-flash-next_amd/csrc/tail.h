@@ -9,6 +9,20 @@ namespace lily {
 
 // ------------------------------------------------------------------ sort
 
+// The value lane ^ M holds, every lane of the wave at work.  Neighbours at distance 1 and 2
+// are inside a group of four lanes: a data-parallel move of each half; farther ones go through
+// the LDS crossbar, whose latency a sort of dependent exchanges waits out stage by stage.
+template <uint32_t M>
+__device__ __forceinline__ uint64_t from_lane_xor(uint64_t v) {
+    if (M == 1u || M == 2u) {
+        constexpr int PERM = M == 1u ? 0xb1 : 0x4e;   // quad_perm [1, 0, 3, 2] / [2, 3, 0, 1]
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, PERM, 0xf, 0xf, true);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), PERM, 0xf, 0xf, true);
+        return ((uint64_t)hi << 32) | lo;
+    }
+    return shfl_xor_u64(v, (int)M);
+}
+
 // Descending bitonic sort of cand[0..n), n <= 4 * NT, four entries per thread (entry
 // 4 * tid + r in register r; absent entries are 0, the smallest).  Exchanges at distance
 // 1 and 2 stay inside a thread, 4 .. 128 are lane shuffles inside a wave, and only the
@@ -50,12 +64,13 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
                 }
                 __syncthreads();
             } else if (stride >= 4u) {
-                const uint32_t m = stride >> 2;
+                const uint32_t m = stride >> 2;   // (a constant once the loops are unrolled)
                 const bool desc = ((tid * 4u) & size) == 0;
                 const bool take_max = ((lane & m) == 0) == desc;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const uint64_t o = shfl_xor_u64(v[r], (int)m);
+                    const uint64_t o = m == 1u ? from_lane_xor<1>(v[r])
+                                     : m == 2u ? from_lane_xor<2>(v[r]) : shfl_xor_u64(v[r], (int)m);
                     v[r] = ((o > v[r]) == take_max) ? o : v[r];
                 }
             } else if (stride == 2u) {
