@@ -218,23 +218,22 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
             }
         }
         // The hand-over.  Every thread's partials above are device-scope stores that go through
-        // to memory; the barrier orders them before thread 0's increment of the row's ticket,
-        // which releases them to the device; the workgroup that arrives last acquires what the
-        // others released (a fence behind the increment, paid by that workgroup alone), and the
-        // second barrier passes that on to its other threads, whose reads below are device-scope
-        // loads that bypass the caches of their own XCD.  (The release costs the 4-row step
-        // 0.8 us of its 15: the price of not leaning on how the hardware happens to order a
-        // written-through store and a later atomic.)
+        // to memory, and the workgroup that arrives last reads them with device-scope loads that
+        // bypass the caches of its own XCD, so the ticket needs no release or acquire at the
+        // scope of the device (each writes back, or invalidates, the XCD's whole L2: 1 us of the
+        // 4-row step's 15, more with more workgroups): a thread's stores have completed when its
+        // wait ends, the barrier gathers the workgroup's, the ticket is taken behind it, and the
+        // reads are issued after the ticket's value has come back.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);   // every counter at 0: this thread's stores have completed
         __syncthreads();
         if (tid == 0) {
-            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELEASE,
+            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
                                                       __HIP_MEMORY_SCOPE_AGENT);
-            if (t == S - 1) {
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-            }
             sh.last = (t == S - 1) ? 1u : 0u;
         }
         __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         phase(cfg, 5);
         if (sh.last == 0u) {
             return;
@@ -351,16 +350,16 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         if (tid == 0) {
             store_through(&cfg.chain_n[row], n);
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);   // (the hand-over of the slices above, once more)
         __syncthreads();
         if (tid == 0) {
-            const uint32_t arrived = __hip_atomic_fetch_add(cfg.chain_ticket, 1u, __ATOMIC_RELEASE,
+            const uint32_t arrived = __hip_atomic_fetch_add(cfg.chain_ticket, 1u, __ATOMIC_RELAXED,
                                                             __HIP_MEMORY_SCOPE_AGENT);
-            if (arrived == rows - 1u) {
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-            }
             sh.last = arrived == rows - 1u ? 1u : 0u;
         }
         __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (sh.last == 0u) {
             return;
         }
