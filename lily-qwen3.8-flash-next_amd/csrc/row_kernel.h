@@ -500,9 +500,10 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
             lds_barrier();
         }
         // The scratch's largest count (and an id that holds it) follow now, once per draw.  It
-        // must never understate a count: thread 0, which issued every increment, waits for them
-        // before anybody reads a count back.
-        __threadfence();
+        // must never understate a count: thread 0, which issued every increment (device atomics,
+        // done where the reads below look), waits for them before anybody reads a count back.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (tid < rows && (t.flags & F_PEN) && sh.drawn[tid] < vocab) {
             const uint32_t id = sh.drawn[tid];
