@@ -40,7 +40,7 @@ hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const 
 // launches (the row's bound, then the values that reach it, merge, select, tail).
 // lane_max [rows][slices][256], bound [rows], count [rows][slices].
 hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg,
-                            const InlineRows* inline_rows, float* lane_max, float* bound, uint32_t* count);
+                            const InlineRows* inline_rows, float* lane_max, uint32_t* count);
 hipError_t launch_copy_pieces(hipStream_t stream, const void* src, void* dst, size_t bytes);
 hipError_t launch_probe_read(hipStream_t stream, const void* base, uint32_t rows, uint64_t row_bytes,
                              uint64_t stride_bytes, uint32_t* out);

@@ -2,15 +2,15 @@
 // which is what a request without top_k gets: src/kernels/sample.rs:17, :326-331), spread over
 // as many workgroups as rows of few candidates are.
 //
-// Two launches.  In the first every workgroup reads its slice of the row once and leaves its 256
-// lanes' largest values (penalised ids at their penalised worth); the workgroup that finishes
-// a row last takes the k-th largest of all the row's lane maxima: k lanes reach it, so k values
-// do - a lower bound of the row's k-th largest value that about k * (1 + a few per cent) values
-// reach.  In the second every workgroup reads its slice again (from the L2 now) and appends
-// the values that reach the bound to the row's list; the one that finishes last reads the
-// list - a thousand and some, whatever the number of slices -, selects, and runs the common
-// tail.  (The select of the other kernels keeps k
-// candidates per slice and can therefore spread a row with k = 1024 over 4 workgroups only.)
+// Two launches.  In the first every workgroup reads its slice of the row once and leaves its
+// lanes' largest values (penalised ids at their penalised worth).  In the second every
+// workgroup first takes the k-th largest of all the row's lane maxima: k lanes reach it, so k
+// values do - a lower bound of the row's k-th largest value that about k * (1 + a few per cent)
+// values reach -, then reads its slice again (from the L2 now) and appends the values that
+// reach the bound to the row's list; the one that finishes last reads the list - a thousand and
+// some, whatever the number of slices -, selects, and runs the common tail.  (The select of the
+// other kernels keeps k candidates per slice and can therefore spread a row with k = 1024 over
+// 4 workgroups only.)
 #include <algorithm>
 
 #ifdef LILY_WIDE_TRACE
@@ -22,9 +22,8 @@
 namespace lily {
 
 // Diagnostic stamps (LaunchCfg::phase_trace), compiled in with -DLILY_WIDE_TRACE (which also
-// turns on the tail's: slots 8 to 12).  First launch: 0 start, 1 slice read, 2 last slice in,
-// 3 keys loaded, 4 bound stored; second: 5 start, 6 slice read, 7 last slice in, 13 list read,
-// 14 selected.
+// turns on the tail's: slots 8 to 12).  First launch: 0 start, 1 slice read, 2 maxima stored;
+// second: 5 start, 6 slice read, 7 last slice in, 13 list read, 14 selected.
 #ifdef LILY_WIDE_TRACE
 #define WIDE_MARK(i) phase(cfg, i)
 #else
@@ -35,7 +34,6 @@ namespace lily {
 struct WideArgs {
     float* lane_max;      // [rows][slices][lanes]
     uint32_t lanes;       // values a slice leaves: NT, or NT / 2 (the larger of each pair of lanes)
-    float* bound;         // [rows]
     uint32_t* count;      // [rows] candidates the row's slices have left so far (0 between launches)
 };
 
@@ -133,7 +131,7 @@ __device__ __forceinline__ bool wide_last(const LaunchCfg& cfg, uint32_t row, ui
     return sh.last != 0u;
 }
 
-// ---- first launch: lane maxima, the slice's sum of exponentials, the row's bound
+// ---- first launch: lane maxima, the slice's sum of exponentials
 
 template <int DT, bool LSE, bool INLINE>
 __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, LaunchCfg cfg, WideArgs w) {
@@ -205,7 +203,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
         store_through(&w.lane_max[slot * NT + tid], lane_max);
     } else {
         // (with slices enough that half the lanes still are four times k, half the keys make
-        // the last workgroup's select half as long)
+        // the select of the bound half as long)
         const int other = __builtin_amdgcn_update_dpp(0, (int)lilym_f32_bits(lane_max), 0xb1, 0xf, 0xf, true);   // quad_perm [1, 0, 3, 2]
         lane_max = fmaxf(lane_max, lilym_bits_f32((uint32_t)other));
         if ((tid & 1u) == 0u) {
@@ -219,17 +217,21 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
             store_through(&cfg.ws_lse[2 * slot + 1], sh.lse_s);
         }
     }
-    if (!wide_last(cfg, row, S, sh)) {
-        return;
-    }
     WIDE_MARK(2);
-    // The k-th largest of the row's S x lanes lane maxima, by a radix select on the leading 16
-    // bits of their order keys, 8 bits a pass: the bound is that key with the other 16 bits
-    // clear, at most 2^-7 of its magnitude below the k-th largest lane maximum, which lets a
-    // few per cent more values through.  A thread keeps its S keys in registers (the loops are
-    // unrolled over MAX_SLICES in groups of eight, a group past S is skipped by the whole
-    // workgroup): one wave per SIMD is at work here, and a pass that fetched each key from
-    // LDS, or the values from the L2 a few at a time, would wait out that latency over and over.
+}
+
+// The row's bound: the k-th largest of its S x lanes lane maxima, by a radix select on the
+// leading 16 bits of their order keys, 8 bits a pass: that key with the other 16 bits clear, at
+// most 2^-7 of its magnitude below the k-th largest lane maximum, which lets a few per cent more
+// values through.  Every workgroup of the second launch works it out for itself, from what the
+// first launch left (a row's slices all arrive at the same value; a workgroup that did it for
+// all of them would have to be waited for).  A thread keeps its keys in registers (the loops
+// are unrolled over MAX_SLICES in groups of eight, a group past the last is skipped by the whole
+// workgroup): a pass that fetched each key from LDS, or the values from the L2 a few at a time,
+// would wait out that latency over and over.  F32_LOWEST when fewer than k lanes saw a finite
+// value: every value is a candidate then.
+__device__ __forceinline__ float wide_bound_of(const WideArgs& w, uint32_t row, uint32_t S, uint32_t k, Shared& sh) {
+    const uint32_t tid = threadIdx.x;
     static_assert(MAX_SLICES == 64, "the unrolled loops below cover 64 keys a thread");
     const uint32_t n = S * w.lanes, mine_n = (n + NT - 1u) / NT;   // keys in all, keys a thread
     float got[MAX_SLICES];
@@ -249,8 +251,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
         const bool in = (uint32_t)j * NT + tid < n;   // (a group past the last was not loaded: what it holds is not read)
         keys[j] = in && got[j] > NEG_INF ? lilym_order_key(got[j]) : 0u;
     }
-    WIDE_MARK(3);
-    uint32_t prefix = 0, pmask = 0, need = a.k;
+    uint32_t prefix = 0, pmask = 0, need = k;
     bool enough = true;
     for (int pass = 0; pass < 2 && enough; ++pass) {
         const int shift = 24 - 8 * pass;
@@ -280,10 +281,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
         }
         __syncthreads();
     }
-    if (tid == 0) {
-        store_through(&w.bound[row], enough ? lilym_key_value(prefix) : F32_LOWEST);
-    }
-    WIDE_MARK(4);
+    return enough ? lilym_key_value(prefix) : F32_LOWEST;
 }
 
 // ---- second launch: the values that reach the bound, then merge, select and tail
@@ -309,7 +307,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_draw(InlineRows rows_arg, Launch
     const uint32_t step = a.step + cfg.step_delta;
     const bool want_lse = LSE && a.out_logprob != nullptr;
     const bool pen = (a.flags & F_PEN) != 0;   // (of the kind that only lowers: the host sees to it)
-    const float bound = gload(w.bound + row);   // of the values' worth under the penalties
+    const float bound = wide_bound_of(w, row, S, a.k, sh);   // of the values' worth under the penalties
     Geo<DT> g;
     g.init(a.logits, vocab, s, S);
     uint64_t* cand = dyn_lds;
@@ -445,7 +443,7 @@ static hipError_t launch_wide_variant(hipStream_t stream, uint32_t rows, const L
 }
 
 hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
-                            const InlineRows* inline_rows, float* lane_max, float* bound, uint32_t* count) {
+                            const InlineRows* inline_rows, float* lane_max, uint32_t* count) {
     LaunchCfg cfg = cfg_in;
     // the merging workgroup's candidates, then the tail's arrays behind the first K_CAP of them
     cfg.dyn_slots = MERGE_CAP;
@@ -453,7 +451,6 @@ hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t ro
     WideArgs w;
     w.lane_max = lane_max;
     w.lanes = (uint64_t)cfg.slices * (NT / 2) >= 4ull * cfg.ws_k ? NT / 2 : NT;
-    w.bound = bound;
     w.count = count;
     const bool inl = inline_rows != nullptr;
 #define LILY_WIDE(DT)                                                                               \

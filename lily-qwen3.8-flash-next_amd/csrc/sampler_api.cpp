@@ -91,7 +91,6 @@ struct lily_sampler {
     uint32_t* chain_ticket = nullptr;
     // rows that draw among many candidates (rows_wide.hip): null in a view without them
     float* wide_max = nullptr;     // [WIDE_FLOATS] lane maxima, rows x slices x 256
-    float* wide_bound = nullptr;   // [WS_ROWS]
     uint32_t* wide_count = nullptr;  // [WS_ROWS] candidates listed so far, 0 between launches
     uint32_t ws_rows = WS_ROWS;    // rows that may span several workgroups
     uint32_t ws_slots = WS_SLOTS;  // candidate slots behind ws_cand
@@ -518,7 +517,7 @@ int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_de
     cfg.cand_cap = part.cand_cap;
     if (part.wide) {
         HIP_TRY(launch_rows_wide(s->stream, dtype, part.lse, part.rows, cfg, nullptr, s->wide_max,
-                                 s->wide_bound, s->wide_count));
+                                 s->wide_count));
         return LILY_OK;
     }
     HIP_TRY(launch_rows(s->stream, dtype, part.kind, part.lse, part.rows, cfg, nullptr, part.dyn_bytes));
@@ -544,8 +543,7 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
             for (uint32_t i = 0; i < n; ++i) {
                 lse = lse || rows.r[i].out_logprob != nullptr;
             }
-            HIP_TRY(launch_rows_wide(s->stream, dtype, lse, n, cfg, &rows, s->wide_max, s->wide_bound,
-                                     s->wide_count));
+            HIP_TRY(launch_rows_wide(s->stream, dtype, lse, n, cfg, &rows, s->wide_max, s->wide_count));
             return LILY_OK;
         }
     }
@@ -873,7 +871,6 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->ws_ticket), WS_ROWS * 4);
     if (err == hipSuccess) err = hipMemset(s->ws_ticket, 0, WS_ROWS * 4);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->wide_max), (size_t)WIDE_FLOATS * 4);
-    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->wide_bound), (size_t)WS_ROWS * 4);
     if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&s->wide_count), WS_ROWS * 4);
     if (err == hipSuccess) err = hipMemset(s->wide_count, 0, WS_ROWS * 4);
     const size_t chain_bytes = (size_t)LILY_MAX_VERIFY_ROWS * CHAIN_CAP * 8 + (LILY_MAX_VERIFY_ROWS + 1) * 4;
@@ -908,7 +905,6 @@ void lily_sampler_destroy(lily_sampler_t* s) {
     (void)hipFree(s->ws_lse);
     (void)hipFree(s->ws_ticket);
     (void)hipFree(s->wide_max);
-    (void)hipFree(s->wide_bound);
     (void)hipFree(s->wide_count);
     (void)hipFree(s->chain_cand);
     (void)hipFree(s->table_dev);
