@@ -337,6 +337,12 @@ def main():
             sampler.synchronize()
             for sc_ in hs:
                 sc_.close()
+            # for reference only: the library's GEMM (torch.matmul, hipBLASLt) on the same
+            # operands, bf16 in and out, without the summaries the head's epilogue leaves
+            ref_out = torch.empty(b_rows, vocab, dtype=torch.bfloat16, device=device)
+            with torch.cuda.stream(stream):
+                ms_lib = time_steps(stream, lambda i: torch.matmul(hb, wb.t(), out=ref_out), n_h, 3)
+            del ref_out
             flops = 2.0 * b_rows * d_model * vocab
             head[f"b{b_rows}"] = {
                 "rows": b_rows, "d": d_model,
@@ -344,6 +350,7 @@ def main():
                 "head_TFLOPs": flops / (ms_head * 1e-3) / 1e12,
                 "head_frac_of_mfma_peak": flops / (ms_head * 1e-3) / 1e12 / 2500.0,
                 "head_weight_GBs": vocab * d_model * 2 / (ms_head * 1e-3) / 1e9,
+                "library_gemm_us": ms_lib * 1e3,
                 "head_plus_draws_us": ms_fused * 1e3,
                 "draws_from_summaries_us": us_tiled,
                 "draws_from_rows_us": us_rows,
