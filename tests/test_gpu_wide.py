@@ -158,3 +158,66 @@ def test_sixty_four_rows_and_the_way_of_the_other_kernels(sampler):
         d = O.sample(x[i], None, o_params(**kw[i]), 2, want_logprob=True)
         check_row_against_oracle(r, i, d)
         _check_logprob(r.logprobs[i], d.logprob, i)
+
+
+def test_random_launches_of_rows_of_many_candidates(sampler):
+    """Forty seeded launches: 1 to 23 rows, vocabularies that leave partial chunks at the slices'
+    ends, f32 and bf16, k from 65 to 1024, Gaussian, heavy-tailed and peaked rows, rows that are
+    mostly -inf, lowering penalties over histories that hold the rows' best ids, with and
+    without a log-probability, as a call and as a plan."""
+    rng = np.random.default_rng(2024)
+    went = 0
+    for case in range(40):
+        rows = int(rng.integers(1, 24))
+        vocab = int(rng.choice([32_003, 50_021, 100_003, 151_936, 151_937, 151_939, 200_001]))
+        bf16 = bool(rng.integers(0, 2))
+        k = int(rng.choice([0, 65, 100, 300, 777, 1024]))
+        pen, logprob, use_plan = (bool(rng.integers(0, 2)) for _ in range(3))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            x = rng.normal(0, 3, (rows, vocab)).astype(np.float32)
+        elif kind == 1:
+            x = (rng.standard_t(3, (rows, vocab)) * 2).astype(np.float32)
+        else:
+            x = rng.normal(0, 0.5, (rows, vocab)).astype(np.float32)
+            x[:, rng.integers(0, vocab, 50)] += 12.0
+        if rng.integers(0, 4) == 0:
+            x[rng.integers(0, rows), rng.random(vocab) < 0.99] = -np.inf
+        xf = x
+        if bf16:
+            x = W.to_bf16_bits(x)
+            xf = W.bf16_bits_to_f32(x)
+        kw = []
+        for r in range(rows):
+            d = dict(temperature=float(rng.uniform(0.3, 1.5)), top_k=k, top_p=float(rng.choice([0.8, 0.95, 1.0])),
+                     min_p=float(rng.choice([0.0, 0.01])), seed=int(rng.integers(0, 1 << 30)))
+            if pen:
+                d.update(repetition_penalty=float(rng.choice([1.0, 1.1, 1.5])),
+                         presence_penalty=float(rng.choice([0.0, 0.5])),
+                         frequency_penalty=float(rng.choice([0.0, 0.2])))
+            kw.append(d)
+        scratch = counts = None
+        if pen:
+            scratch, counts = [], []
+            for r in range(rows):
+                best = np.argsort(-xf[r])[:int(rng.integers(10, 600))].astype(np.int32)
+                hh = np.concatenate([rng.integers(0, vocab, int(rng.integers(0, 5000))).astype(np.int32),
+                                     np.repeat(best[:20], int(rng.integers(1, 6))), best])
+                sc = LS.SamplerScratch(sampler, vocab)
+                sc.add_history(torch.from_numpy(hh).to(dev()))
+                scratch.append(sc)
+                counts.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+        step = int(rng.integers(0, 100))
+        r, stats = _with_stats(sampler, lambda: run_rows(sampler, x, kw, [step] * rows, scratch=scratch,
+                                                         logprobs=logprob, use_plan=use_plan))
+        went += int(stats[1] + stats[2] == rows)
+        for i in range(rows):
+            d = O.sample(x[i], counts[i] if pen else None, o_params(**kw[i]), step, want_logprob=logprob)
+            check_row_against_oracle(r, i, d)
+            if logprob:
+                _check_logprob(r.logprobs[i], d.logprob, (case, i))
+        if pen:
+            for i in range(rows):
+                assert np.array_equal(scratch[i].read_counts().numpy().view(np.uint32), counts[i]), (case, i)
+                scratch[i].close()
+    assert went >= 30, went   # (a launch of one or two rows has too few slices for some k)
