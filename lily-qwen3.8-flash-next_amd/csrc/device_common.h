@@ -176,6 +176,32 @@ __device__ __forceinline__ double wave_sum_d(double v) {
     }
     return v;
 }
+// The wave's sum in every lane without LDS traffic: inclusive sums inside each row of 16 lanes
+// by DPP row shifts (a lane without such a neighbour adds 0), then the four rows' totals read
+// from lanes 15, 31, 47 and 63.
+__device__ __forceinline__ double wave_sum_d_dpp(double v) {
+#define LILY_ROW_SHR_ADD(n)                                                                      \
+    {                                                                                            \
+        const uint64_t b = __builtin_bit_cast(uint64_t, v);                                      \
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)b, 0x110 + (n), 0xf, 0xf, false);        \
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(b >> 32), 0x110 + (n), 0xf, 0xf, false); \
+        v += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);                              \
+    }
+    LILY_ROW_SHR_ADD(1)
+    LILY_ROW_SHR_ADD(2)
+    LILY_ROW_SHR_ADD(4)
+    LILY_ROW_SHR_ADD(8)
+#undef LILY_ROW_SHR_ADD
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    double t = 0.0;
+#pragma unroll
+    for (int l = 15; l < 64; l += 16) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, l);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), l);
+        t += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+    }
+    return t;
+}
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int o) {
     const uint32_t lo = __shfl_xor((uint32_t)v, o);
     const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), o);
@@ -240,7 +266,7 @@ struct Shared {
     uint32_t qfill[NWAVE];   // chunks each wave queued
     uint32_t nfill[NWAVE];   // chunks each wave noted
     uint32_t n_fc;           // final candidates
-    uint32_t n_hits;   // noted chunks found to hold a listed id
+    uint32_t n_pairs;  // (id, raw value) pairs listed from the queued chunks
     // rows that draw in order (one launch): what the rows before drew, the count each of those
     // ids had right after, the proposals the draws are compared with, and the last draw
     uint32_t drawn[LILY_MAX_VERIFY_ROWS];

@@ -5,6 +5,9 @@
 
 #include "device_common.h"
 
+#ifndef LILY_LOOP
+#define LILY_LOOP 0
+#endif
 namespace lily {
 
 // ------------------------------------------------------------------ streaming select
@@ -160,14 +163,23 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t c0 = g.cb + b * BLOCK;
         return c0 >= g.main_lo && c0 + BLOCK <= g.main_hi;
     };
+    // The first three blocks are asked for before anything else: the row's other preparations
+    // (a list of bias pairs, the scratch's largest count and the value of its most-counted id:
+    // round trips to memory that depend on each other) then run beside them.
     u32x4 buf_a[U], buf_b[U], buf_c[U];
     if (nblocks > 0) {
         fetch(buf_a, 0);
+#if LILY_LOOP == 2
+        fetch(buf_b, min(1u, nblocks - 1u));
+        fetch(buf_c, min(2u, nblocks - 1u));
+#elif LILY_LOOP == 1
+        fetch(buf_b, min(1u, nblocks - 1u));
+#endif
     }
     if (tid == 0) {
         sh.n_fc = 0;
         sh.fail = 0;
-        sh.n_hits = 0;
+        sh.n_pairs = 0;
     }
     for (uint32_t i = tid; i < n_bias; i += NT) {
         L.bias_id[i] = gload(&a.bias[i].id);
@@ -260,11 +272,39 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     // the sum's cut then stands from the first block on, however late the row's largest values
     // arrive; and no other id's true value is overstated more by the penalty the cut otherwise
     // assumes (that of the largest count).
+    // Its logit, count and mask bit are the same for every thread: they come by scalar loads, whose
+    // results are waited for apart from the vector loads - the row's first blocks, requested above,
+    // stay in flight meanwhile (a vector load here would be waited for behind all of them).
     float row_floor = NEG_INF;
     if (want_lse && pen && lowering) {
         const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + row_words + 1u);
-        if (heavy < g.vocab && max_count != 0u && (!masked || bit_of(a.allow, heavy))) {
-            row_floor = true_value(heavy, load_logit<DT>(a.logits, heavy));
+        if (heavy < g.vocab && max_count != 0u) {
+            const uint32_t cnt = *(const LILY_CONST uint32_t*)(a.counts + heavy);
+            float raw;
+            if (DT == LILY_BF16) {
+                const uintptr_t at = reinterpret_cast<uintptr_t>(a.logits) + (uintptr_t)heavy * 2u;
+                const uint32_t word = *(const LILY_CONST uint32_t*)(at & ~(uintptr_t)3u);
+                raw = lilym_bits_f32(((at & 2u) ? word >> 16 : word & 0xffffu) << 16);
+            } else {
+                raw = lilym_bits_f32(*(const LILY_CONST uint32_t*)(static_cast<const uint32_t*>(a.logits) + heavy));
+            }
+            bool allowed = true;
+            if (masked) {
+                allowed = ((*(const LILY_CONST uint32_t*)(a.allow + (heavy >> 5)) >> (heavy & 31u)) & 1u) != 0u;
+            }
+            if (allowed) {
+                float t = raw;
+                for (uint32_t j = 0; j < n_bias; ++j) {
+                    if (L.bias_id[j] == heavy) {
+                        t += L.bias_delta[j];
+                    }
+                }
+                if (cnt > 0u) {
+                    t = t > 0.0f ? t / a.repetition : t * a.repetition;
+                    t -= a.presence + a.frequency * (float)cnt;
+                }
+                row_floor = t;
+            }
         }
     }
     phase(cfg, 1);
@@ -521,6 +561,24 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         }
     };
 
+    // The exact terms of one chunk of the slice, one by one in double: every element whose value
+    // (the true one for the listed ids of `dm`) lies above `cut`.
+    auto chunk_terms = [&](const u32x4& q, uint32_t c, uint32_t dm, float cut, auto&& add_term) {
+#pragma unroll 1
+        for (uint32_t j = 0; j < (uint32_t)E; ++j) {
+            float x = elem_of(q, j);
+            if (!(x > cut)) {
+                continue;   // (penalties that only lower: a listed id below the cut stays below it)
+            }
+            if ((dm >> j) & 1u) {
+                x = true_value(g.id_of(c, (int)j), x);
+            }
+            if (x > cut) {
+                add_term(x);
+            }
+        }
+    };
+
     // Blocks b + 1 and b + 2 are on their way while block b is worked on (three register
     // buffers that swap roles): one block in flight per wave leaves the memory idle whenever
     // a wave's arithmetic outlasts its load.
@@ -533,9 +591,37 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         constexpr bool QM = LSE && decltype(queueing)::value;   // mode 2
         Bits bits_a = {}, bits_b = {}, bits_c = {};
         auto work = [&](u32x4 (&cur)[U], const Bits& bcur, uint32_t b) {
-            if (give_up || stop) {
+            if (give_up || stop || b >= nblocks) {
                 return;
             }
+#if defined(LILY_PRIO_PROGRESS)
+            // A wave that has further to go asks to be issued first: the four workgroups that
+            // share a compute unit then advance together instead of in the order they arrived.
+            {
+                const uint32_t q = (b * 4u) / max(nblocks, 1u);
+                if (q == 0u) {
+                    __builtin_amdgcn_s_setprio(3);
+                } else if (q == 1u) {
+                    __builtin_amdgcn_s_setprio(2);
+                } else if (q == 2u) {
+                    __builtin_amdgcn_s_setprio(1);
+                } else {
+                    __builtin_amdgcn_s_setprio(0);
+                }
+            }
+#elif defined(LILY_PRIO_STATIC)
+            // (experiment) later rows of a compute unit first
+            {
+                const uint32_t q = (blockIdx.y * 4u) / max(gridDim.y, 1u);
+                if (q == 3u) {
+                    __builtin_amdgcn_s_setprio(3);
+                } else if (q == 2u) {
+                    __builtin_amdgcn_s_setprio(2);
+                } else if (q == 1u) {
+                    __builtin_amdgcn_s_setprio(1);
+                }
+            }
+#endif
             // tb_all: a byte per chunk of the block, bit j = element j is a listed id.
             uint32_t tb_all = 0u, mb[U] = {0u, 0u, 0u, 0u};
             if (SP) {
@@ -608,32 +694,55 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     forced |= ((tb_all >> (8 * u)) & 0xffu) != 0u ? 1u << u : 0u;
                 }
             }
-            // Mode 2: the lanes whose chunk u was just summed note its number; a lane whose
-            // wave's segment is full has the chunk's bits fetched here instead (`fix`).
             uint32_t fix = 0u;   // a byte per chunk: its listed ids that are evaluated on the spot
-            auto note_summed = [&](int u, bool summed) {
-                const uint64_t mask = __ballot(summed);
+            // Mode 2: a lane whose chunk lies above the cut without being queued notes the chunk's
+            // number; its terms are formed after the scan, against the row's final cut (most of
+            // what a stale cut lets through is dropped there without a single exponential).  A
+            // lane whose wave's segment is full forms its chunk's terms on the spot instead.
+            auto note_chunk = [&](int u, bool wanted) {
+                const uint64_t mask = __ballot(wanted);
                 if (mask != 0ull) {
                     const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
                         (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
                     const uint32_t at = sfill + rank;
-                    if (summed && at < SSEG) {
+                    if (wanted && at < SSEG) {
                         L.noted[w * SSEG + at] = (uint16_t)((b * U + (uint32_t)u) * NT + tid);
                     }
                     if (sfill + (uint32_t)__popcll(mask) > SSEG) {
-                        uint32_t dm = 0u;
-                        if (summed && at >= SSEG) {
+                        if (wanted && at >= SSEG) {
                             const uint32_t c = g.cb + (b * U + (uint32_t)u) * NT + tid;
-                            dm = bits32_at(a.touched, row_words, (int64_t)g.id_of(c, 0)) & EMASK;
-                            // Waited for inside the branch: waiting behind it would make every
-                            // wave drain the loads it has in flight, not just these.
-                            asm volatile("" : "+v"(dm));
+                            if (c >= g.main_lo && c < g.main_hi) {
+                                // Every element's count, asked for whatever the element is worth
+                                // and waited for here, inside the branch: a fixed number of loads
+                                // and no loop around them, so that the waits of the scan's own
+                                // loads keep counting past this branch.
+                                uint32_t cnt[E];
+#pragma unroll
+                                for (int j = 0; j < E; ++j) {
+                                    cnt[j] = gload(a.counts + g.id_of(c, j));
+                                }
+#pragma unroll
+                                for (int j = 0; j < E; ++j) {
+                                    asm volatile("" : "+v"(cnt[j]));
+                                }
+#pragma unroll
+                                for (int j = 0; j < E; ++j) {
+                                    float x = elem_of(cur[u], (uint32_t)j);
+                                    if (cnt[j] > 0u) {
+                                        x = x > 0.0f ? x / a.repetition : x * a.repetition;
+                                        x -= a.presence + a.frequency * (float)cnt[j];
+                                    }
+                                    if (x > skip_b) {
+                                        acc_t += term_d(x);
+                                    }
+                                }
+                            }
                         }
-                        fix |= dm << (8 * u);
                     }
                     sfill = min(sfill + (uint32_t)__popcll(mask), SSEG);
                 }
             };
+            bool some = false;
             if (LSE && want_lse) {
                 // A term 2^(v*c2) below 2^-21 / vocab of the largest one seen cannot move the row
                 // sum by more than 2^-21 of it, even with every element of the row at that level:
@@ -641,7 +750,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 skip_b = fmaxf(row_max, own_max) - lse_cut;
                 wl.skip_below = skip_b;
                 // Rows with a dominant value skip nearly every block as a whole.
-                bool some = __ballot(block_max > skip_b) != 0ull;
+                some = __ballot(block_max > skip_b) != 0ull;
                 if (QM && some) {
                     // Between two refreshes of the row's maxima the wave's own lanes may have seen
                     // more than the row knew then: what they saw bounds the row's largest value
@@ -652,15 +761,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     wl.skip_below = skip_b;
                     some = __ballot(block_max > skip_b) != 0ull;
                 }
-                if (some) {
+                if (!QM && some) {
                     wl.prepare(block_max < T_prev ? block_max : T_prev, c2);  // nothing above T_prev is added
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
                         const bool sum_it = !(m8[u] >= T_prev) && ((forced >> u) & 1u) == 0u;
                         wl.template add_prepared<DT>(cur[u], m8[u], c2, sum_it);
-                        if (QM) {
-                            note_summed(u, sum_it && m8[u] > skip_b);
-                        }
                     }
                 }
             }
@@ -676,6 +782,9 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     // were summed already are as negligible as those that were not.
                     skip_b = fmaxf(row_max, own_max) - lse_cut;
                     wl.skip_below = skip_b;
+                    if (QM && some) {
+                        some = __ballot(block_max > skip_b) != 0ull;
+                    }
                 }
                 if (QM && note_max >= SSEG * 3u / 4u) {
                     stop = true;
@@ -687,7 +796,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 L.blk_cut[b] = skip_b;
                 L.blk_flag[b] = nonneg ? 1u : 0u;
             }
-            const bool any_late = LSE && want_lse && T != T_prev &&
+            const bool any_late = !QM && LSE && want_lse && T != T_prev &&
                                   __ballot(block_max >= T_prev && block_max > skip_b) != 0ull;
             // When values can only be lowered, a listed id in a chunk that was neither queued nor
             // summed is below the bound and below the sum's cut with its true value too: nothing
@@ -715,10 +824,10 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     if (__ballot(late) != 0ull) {
                         wl.prepare(late ? m8[u] : NEG_INF, c2);
                         wl.template add_prepared<DT>(cur[u], m8[u], c2, late);
-                        if (QM) {
-                            note_summed(u, late && m8[u] > skip_b);
-                        }
                     }
+                }
+                if (QM && some) {
+                    note_chunk(u, !pass && m8[u] > skip_b);
                 }
                 if (SP && fix_any) {
                     const uint32_t tb = (tb_all >> (8 * u)) & 0xffu;
@@ -726,7 +835,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     fix |= (tb != 0u && !pass && matters) ? tb << (8 * u) : 0u;
                 }
             }
-            if ((SP || QM) && fix != 0u) {
+            if (SP && fix != 0u) {
                 fix_listed(cur, b, fix);
             }
         };
@@ -744,13 +853,47 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (nblocks == 0) {
             refresh_bound(true, true);  // the same barriers in every workgroup
         } else if (b_first < nblocks) {
+#if LILY_LOOP == 2
+            if (b_first != 0u) {   // (blocks 0, 1 and 2 were requested at the very start)
+                fetch(buf_a, b_first);
+                fetch(buf_b, min(b_first + 1u, nblocks - 1u));
+                fetch(buf_c, min(b_first + 2u, nblocks - 1u));
+            }
+            if (SP) {
+                bits_request(bits_a, b_first);
+                bits_request(bits_b, min(b_first + 1u, nblocks - 1u));
+                bits_request(bits_c, min(b_first + 2u, nblocks - 1u));
+            }
+            // A block's buffer is asked for the block three further on as soon as the block has
+            // been worked on: two blocks are on their way while one is looked at.  Every trip
+            // issues the same requests (past the row's end they ask for its last block again, and
+            // `work` returns at once): a request that some path skips would make every wait count
+            // as if it had been skipped.
+            for (uint32_t b = b_first; b < nblocks && !give_up && !stop; b += 3u) {
+                work(buf_a, bits_a, b);
+                request(buf_a, bits_a, b + 3u);
+                work(buf_b, bits_b, b + 1u);
+                request(buf_b, bits_b, b + 4u);
+                work(buf_c, bits_c, b + 2u);
+                request(buf_c, bits_c, b + 5u);
+            }
+#else
             if (b_first != 0u) {
                 fetch(buf_a, b_first);   // (block 0 was requested at the very start)
             }
             if (SP) {
                 bits_request(bits_a, b_first);
             }
+#if LILY_LOOP == 1
+            if (b_first != 0u) {
+                fetch(buf_b, min(b_first + 1u, nblocks - 1u));
+            }
+            if (SP) {
+                bits_request(bits_b, min(b_first + 1u, nblocks - 1u));
+            }
+#else
             request(buf_b, bits_b, b_first + 1u);
+#endif
             for (uint32_t b = b_first; b < nblocks && !give_up && !stop; b += 3) {
                 request(buf_c, bits_c, b + 2);
                 work(buf_a, bits_a, b);
@@ -763,6 +906,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     }
                 }
             }
+#endif
         }
     };
     if (noting) {
@@ -779,11 +923,39 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     phase(cfg, 2);
 
     // ---- after the scan
+    const float wave_top = (LSE && noting) ? wave_max_dpp(lane_max) : 0.0f;
     if (lane == 0) {
         sh.qfill[w] = wq;
         sh.nfill[w] = sfill;
+        sh.wmax[parity][w] = wave_top;
     }
     __syncthreads();
+    phase(cfg, 14);
+    // Mode 2 forms its terms after the scan, when the row's largest streamed value is known:
+    // they are relative to that value's exponent (none of them exceeds 1: penalties only lower)
+    // and add up in `acc_p`.
+    double ref_p = 0.0, acc_p = 0.0;
+    bool simple_p = false;   // the same in every thread
+    if (LSE && noting) {
+        // The row's cut as the whole scan leaves it: what follows forms no term below it.
+        float m = sh.wmax[parity][0];
+        for (int i = 1; i < NWAVE; ++i) {
+            m = fmaxf(m, sh.wmax[parity][i]);
+        }
+        const float true_low = fmaxf(lowered(m), row_floor);   // the largest true value is not below this
+        skip_b = fmaxf(skip_b, true_low - lse_cut);
+        // One reference serves when every term above the cut is a double relative to it: the
+        // largest raw value may lie far above what the penalties leave of it, and a temperature
+        // near 0 stretches that distance beyond a double's range (such rows keep the references
+        // that move, term_d).
+        simple_p = m > NEG_INF && (m - true_low) * c2 <= 900.0f;
+        ref_p = simple_p ? (double)m * c2d : 0.0;
+        ref_p = ref_p < 1.0e30 ? (ref_p > -1.0e30 ? ref_p : -1.0e30) : 1.0e30;
+    }
+    auto term_p = [&](float v) -> double {
+        const double d = __builtin_fma((double)v, c2d, -ref_p);
+        return d > -1000.0 ? pow2_d(d < 1000.0 ? d : 1000.0) : 0.0;   // (-inf and NaN: nothing)
+    };
     const float filt = T;
     {
         bool overflow = give_up;
@@ -814,16 +986,13 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         return (c - g.cb) / BLOCK;
     };
     {
-        // One thread per queued chunk (the waves' segments counted through in order): its
-        // elements add their term and are offered - listed ones with their true value, ids of
-        // the bias list not at all (the pass below speaks for them).
         uint32_t seg_end[NWAVE], total = 0;
 #pragma unroll
         for (int i = 0; i < NWAVE; ++i) {
             total += sh.qfill[i];
             seg_end[i] = total;
         }
-        for (uint32_t ch = tid; ch < total; ch += NT) {
+        auto queue_slot = [&](uint32_t ch) -> uint32_t {
             uint32_t ww = 0, before = 0;
 #pragma unroll
             for (int i = 0; i + 1 < NWAVE; ++i) {
@@ -832,7 +1001,172 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     before = seg_end[i];
                 }
             }
-            const uint32_t slot = ww * QSEG + (ch - before);
+            return ww * QSEG + (ch - before);
+        };
+        // Mode 2's noted chunks: their 16 bytes and their bits of the scratch's bitmap are asked
+        // for first, four chunks a thread, and looked at behind the queue's listing below, which
+        // touches LDS only.
+        uint32_t n_seg_end[NWAVE], n_total = 0;
+#pragma unroll
+        for (int i = 0; i < NWAVE; ++i) {
+            n_total += (LSE && noting) ? sh.nfill[i] : 0u;
+            n_seg_end[i] = n_total;
+        }
+        auto noted_at = [&](uint32_t e) -> uint32_t {
+            uint32_t ww = 0, before = 0;
+#pragma unroll
+            for (int i = 0; i + 1 < NWAVE; ++i) {
+                if (e >= n_seg_end[i]) {
+                    ww = (uint32_t)i + 1u;
+                    before = n_seg_end[i];
+                }
+            }
+            return (uint32_t)L.noted[ww * SSEG + (e - before)];
+        };
+        uint32_t n_cc[4] = {0u, 0u, 0u, 0u}, n_dm[4] = {0u, 0u, 0u, 0u};
+        u32x4 n_q[4] = {};
+        bool n_ok[4] = {false, false, false, false};
+        auto noted_request = [&](uint32_t e0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t e = e0 + (uint32_t)i * NT;
+                const uint32_t c = g.cb + noted_at(min(e, n_total - 1u));
+                // (A chunk outside the slice was scanned as -inf throughout, and is noted where
+                // chunk maxima are the kind that reports +0 for it.)
+                n_ok[i] = e < n_total && c >= g.main_lo && c < g.main_hi;
+                n_cc[i] = min(c, c_last);
+                n_q[i] = gload(reinterpret_cast<const u32x4*>(g.base + (n_cc[i] << 4)));
+                n_dm[i] = bits32_at(a.touched, row_words, (int64_t)g.id_of(n_cc[i], 0)) & EMASK;
+            }
+        };
+        // A chunk whose largest value lies above the final cut adds its terms (listed ids with
+        // their true values); the others - all that a cut which was out of date while the row's
+        // largest values had yet to come let through - are dropped.
+        auto noted_consume = [&]() {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (n_ok[i] && chunk_max<DT>(n_q[i]) > skip_b) {
+                    chunk_terms(n_q[i], n_cc[i], n_dm[i], skip_b, [&](float x) {
+                        if (simple_p) {
+                            acc_p += term_p(x);
+                        } else {
+                            acc_t += term_d(x);
+                        }
+                    });
+                }
+            }
+        };
+        if (n_total != 0u) {
+            noted_request(tid);
+        }
+        // Rows under penalties that only lower (the common kind): every element of a queued chunk
+        // that matters by its raw value - at or above the bound, or above the sum's cut - is
+        // listed as an (id, raw value) pair, wave by wave; then one thread per pair gathers the
+        // id's count, so that all of the row's gathers are one round trip to memory.  (A listed
+        // id's true value is not above its raw one: what does not matter raw does not matter.)
+        uint64_t* pairs = L.fc;   // the candidates' place: they arrive once the pairs are in registers
+        const bool pair_path = pen && lowering;
+        if (pair_path) {
+            for (uint32_t ch0 = 0; ch0 < total; ch0 += NT) {
+                const uint32_t ch = ch0 + tid;
+                uint32_t todo = 0, c = 0;
+                u32x4 q = {};
+                if (ch < total) {
+                    const uint32_t slot = queue_slot(ch);
+                    q = L.qraw[slot];
+                    c = L.qidx[slot];
+                    float v[E];
+                    unpack<DT>(q, v);
+#pragma unroll
+                    for (int j = 0; j < E; ++j) {
+                        const bool term = want_lse && v[j] > skip_b;
+                        const bool cand = v[j] >= filt && v[j] > NEG_INF;
+                        todo |= (term || cand) ? 1u << j : 0u;
+                    }
+                }
+                while (__ballot(todo != 0u) != 0ull) {
+                    const bool has = todo != 0u;
+                    const uint32_t j = has ? (uint32_t)__builtin_ctz(todo) : 0u;
+                    todo &= todo - 1u;   // (0 stays 0)
+                    const uint32_t id = g.id_of(c, (int)j);
+                    const bool push = has && !(n_bias != 0u && biased(id));
+                    const uint64_t mask = __ballot(push);
+                    if (mask != 0ull) {
+                        const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+                            (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                        uint32_t first = 0;
+                        if (rank == 0u && push) {
+                            first = atomicAdd(&sh.n_pairs, (uint32_t)__popcll(mask));
+                        }
+                        first = (uint32_t)__builtin_amdgcn_readlane((int)first, __builtin_ctzll(mask));
+                        if (push && first + rank < FC_CAP) {
+                            pairs[first + rank] = ((uint64_t)lilym_f32_bits(elem_of(q, j)) << 32) | id;
+                        }
+                    }
+                }
+            }
+        }
+        if (n_total != 0u) {
+            noted_consume();
+            for (uint32_t e0 = tid + 4u * NT; e0 < n_total + tid; e0 += 4u * NT) {   // (the same trips in every thread)
+                noted_request(e0);
+                noted_consume();
+            }
+        }
+        bool paired = false;
+        if (pair_path) {
+            __syncthreads();
+            paired = sh.n_pairs <= FC_CAP;
+        }
+        if (paired) {
+            const uint32_t n_pairs = sh.n_pairs;
+            uint64_t pr[4];
+            uint32_t cnt[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t at = tid + (uint32_t)i * NT;
+                pr[i] = at < n_pairs ? pairs[at] : 0ull;
+                cnt[i] = gload(a.counts + (uint32_t)pr[i]);   // (id 0 for an empty place)
+            }
+            __syncthreads();   // every pair is in a register: the candidates may take their place
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool valid = tid + (uint32_t)i * NT < n_pairs;
+                const uint32_t id = (uint32_t)pr[i];
+                float x = lilym_bits_f32((uint32_t)(pr[i] >> 32));
+                if (cnt[i] > 0u) {
+                    x = x > 0.0f ? x / a.repetition : x * a.repetition;
+                    x -= a.presence + a.frequency * (float)cnt[i];
+                }
+                if (valid && want_lse && x > skip_b) {
+                    if (simple_p) {
+                        acc_p += term_p(x);
+                    } else {
+                        acc_t += term_d(x);
+                    }
+                }
+                const bool cand = valid && x >= filt && x > NEG_INF;
+                const uint64_t mask = __ballot(cand);
+                if (mask != 0ull) {
+                    const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+                        (uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                    uint32_t first = 0;
+                    if (rank == 0u && cand) {
+                        first = atomicAdd(&sh.n_fc, (uint32_t)__popcll(mask));
+                    }
+                    first = (uint32_t)__builtin_amdgcn_readlane((int)first, __builtin_ctzll(mask));
+                    if (cand && first + rank < FC_CAP) {
+                        L.fc[first + rank] = composite_of(x / a.temperature, id);
+                    }
+                }
+            }
+        }
+        // Every other row (and a row whose pairs outgrew their place): one thread per queued
+        // chunk (the waves' segments counted through in order): its elements add their term and
+        // are offered - listed ones with their true value, ids of the bias list not at all (the
+        // pass below speaks for them).
+        for (uint32_t ch = tid; !paired && ch < total; ch += NT) {
+            const uint32_t slot = queue_slot(ch);
             const u32x4 q = L.qraw[slot];
             const uint32_t c = L.qidx[slot];
             // Its listed elements, from the scratch's bitmap (barred ids are -inf already).
@@ -869,79 +1203,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 }
                 offer(x, id);
             }
-        }
-    }
-    if (LSE && noting) {
-        // One thread per noted chunk: all of its elements went into the running sum with their
-        // raw values.  For the few that hold a listed id, that id's raw term is booked and its
-        // true term (above the final cut) added.
-        uint32_t seg_end[NWAVE], total = 0;
-#pragma unroll
-        for (int i = 0; i < NWAVE; ++i) {
-            total += sh.nfill[i];
-            seg_end[i] = total;
-        }
-        // First the chunks' bits, four entries per thread at a time (their loads in flight
-        // together); the chunks that hold a listed id are gathered in the queue's memory, which
-        // the expansion above has left.
-        uint32_t* hits = reinterpret_cast<uint32_t*>(L.qraw);
-        constexpr uint32_t HIT_CAP = Q_CAP * 4u;
-        auto chunk_at = [&](uint32_t e) -> uint32_t {
-            uint32_t ww = 0, before = 0;
-#pragma unroll
-            for (int i = 0; i + 1 < NWAVE; ++i) {
-                if (e >= seg_end[i]) {
-                    ww = (uint32_t)i + 1u;
-                    before = seg_end[i];
-                }
-            }
-            return (uint32_t)L.noted[ww * SSEG + (e - before)];
-        };
-        auto fix_chunk = [&](uint32_t c, uint32_t dm) {
-            const u32x4 q = gload(reinterpret_cast<const u32x4*>(g.base + (c << 4)));
-            while (dm != 0u) {
-                const uint32_t j = (uint32_t)__builtin_ctz(dm);
-                dm &= dm - 1u;
-                const float raw = elem_of(q, j);
-                if (!(raw > NEG_INF)) {
-                    continue;
-                }
-                const float t = true_value(g.id_of(c, (int)j), raw);
-                acc_r += term_d(raw);
-                if (t > skip_b) {
-                    acc_t += term_d(t);
-                }
-            }
-        };
-        __syncthreads();   // (the expansion's reads of the queue are over)
-        for (uint32_t e0 = tid; e0 < total; e0 += 4u * NT) {
-            uint32_t rel[4], dm[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t e = e0 + (uint32_t)i * NT;
-                rel[i] = chunk_at(min(e, total - 1u));
-                dm[i] = bits32_at(a.touched, row_words, (int64_t)g.id_of(g.cb + rel[i], 0)) & EMASK;
-                // (A chunk outside the slice was scanned as -inf throughout, and may have been
-                // "summed" where chunk maxima are the kind that reports +0 for it.)
-                const uint32_t c = g.cb + rel[i];
-                dm[i] = e < total && c >= g.main_lo && c < g.main_hi ? dm[i] : 0u;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (dm[i] != 0u) {
-                    const uint32_t at = atomicAdd(&sh.n_hits, 1u);
-                    if (at < HIT_CAP) {
-                        hits[at] = rel[i] | (dm[i] << 16);
-                    } else {
-                        fix_chunk(g.cb + rel[i], dm[i]);   // (nearly every chunk holds a listed id)
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        const uint32_t n_hits = min(sh.n_hits, HIT_CAP);
-        for (uint32_t h = tid; h < n_hits; h += NT) {
-            fix_chunk(g.cb + (hits[h] & 0xffffu), hits[h] >> 16);
         }
     }
     phase(cfg, 8);
@@ -1000,84 +1261,123 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
     }
     phase(cfg, 9);
     if (want_lse) {
-        // Each wave brings its sums to one reference of its own: the highest of its threads'
-        // references and of the streamed sums' (wave-uniform) reference.  The waves' partial
-        // sums and references meet in LDS and are brought together after one barrier.
-        int ref_w = up;
-        for (int o = 32; o > 0; o >>= 1) {
-            ref_w = max(ref_w, __shfl_xor(ref_w, o));
-        }
-        const double stream_at = (double)wl.ref - (double)ref_s;  // exact
-        if (__ballot(wl.s > 0.0f) != 0ull) {
-            const double e = stream_at < 1.0e9 ? (stream_at > -1.0e9 ? stream_at : -1.0e9) : 1.0e9;
-            ref_w = max(ref_w, (int)__builtin_floor(e));
-        }
-        const int down = up == UP_UNSET ? 0 : up - ref_w;  // <= 0
-        double part[4];
-        {
-            double d = stream_at - (double)ref_w;  // <= 1 where there is a sum
-            d = d < -1000.0 ? -1000.0 : d;
-            const double scale = pow2_d(d);
-            part[0] = wl.s > 0.0f ? (double)wl.s * scale : 0.0;
-            part[3] = wl.booked > 0.0f ? (double)wl.booked * scale : 0.0;
-        }
-        part[1] = __builtin_ldexp(acc_r, down);
-        part[2] = __builtin_ldexp(acc_t, down);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            part[i] = wave_sum_d(part[i]);
-            if (lane == 0) {
-                sh.red3[i][w] = part[i];
-            }
-        }
+        // Mode 2 as a rule holds nothing but its post-scan terms, all relative to one reference:
+        // the waves' sums meet in LDS behind one barrier.  A thread with a sum of another kind
+        // (terms formed during the scan, edge ids, a scan that went on with bits beside the
+        // chunks) sends the row the long way below.
+        const bool other_sums = up != UP_UNSET || !(wl.s == 0.0f) || !(wl.booked == 0.0f);
+        const double p_wave = wave_sum_d_dpp(acc_p);
         if (lane == 0) {
-            sh.red_i[w] = (uint32_t)ref_w;
+            sh.red_d[w] = p_wave;
         }
-        // A NaN logit in a summed chunk leaves its wave's running sum a NaN: such a logit is
-        // worth -inf, and the row's sum is formed again from every value.
-        const bool poisoned = __syncthreads_or(wl.s != wl.s ? 1 : 0) != 0;
-        int ref_all = (int)sh.red_i[0];
-        for (int i = 1; i < NWAVE; ++i) {
-            ref_all = max(ref_all, (int)sh.red_i[i]);
+        const bool long_way = __syncthreads_or((!simple_p || other_sums) ? 1 : 0) != 0;
+        double p_all = 0.0;
+        for (int i = 0; i < NWAVE; ++i) {
+            p_all += sh.red_d[i];
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            part[i] = 0.0;
-            for (int ww = 0; ww < NWAVE; ++ww) {
-                const int at = (int)sh.red_i[ww];
-                part[i] += at == UP_UNSET ? 0.0 : __builtin_ldexp(sh.red3[i][ww], at - ref_all);
-            }
-        }
-        if (ref_all == UP_UNSET) {
-            ref_all = 0;  // no term anywhere: the sums are zero
-        }
-        // part[0]: the running sums, the listed ids' raw terms of part[3] already taken off (and
-        // their true terms added); part[1]: raw terms still to take off; part[2]: terms added
-        // one by one.
-        const double streamed = part[0], booked = part[1], exact = part[2], taken = part[3];
-        const double rest = streamed - booked;
-        // The streamed sums are f32: taking the listed ids' raw terms off again leaves an error of
-        // about 1e-6 of what was streamed.  Where that is more than 20 times the row's sum (listed
-        // ids held nearly everything that was streamed, and nothing larger was added exactly) the
-        // difference is too coarse.
-        const bool coarse = poisoned ||
-                            (booked + taken > 0.0 &&
-                             !((rest > 0.0 ? rest : 0.0) + exact > 0.05 * (streamed + taken)));
-        phase(cfg, 10);
-        if (coarse) {
-            phase(cfg, 11);
-            LseAcc all;
-            all.init();
-            exact_terms<DT>(a, g.id_lo, g.id_hi, c2, all);
-            double m_e, s_e;
-            wg_merge_lse(sh, all.mc, all.s, m_e, s_e);
+        if (!long_way) {
+            phase(cfg, 10);
             if (tid == 0) {
-                sh.lse_mc = m_e;
-                sh.lse_s = s_e;
+                sh.lse_mc = ref_p;
+                sh.lse_s = p_all;
             }
-        } else if (tid == 0) {
-            sh.lse_mc = (double)ref_s + (double)ref_all;
-            sh.lse_s = (rest > 0.0 ? rest : 0.0) + exact;
+        } else {
+            // Each wave brings its sums to one reference of its own: the highest of its threads'
+            // references and of the streamed sums' (wave-uniform) reference.  The waves' partial
+            // sums and references meet in LDS and are brought together after one barrier.
+            int ref_w = up;
+            for (int o = 32; o > 0; o >>= 1) {
+                ref_w = max(ref_w, __shfl_xor(ref_w, o));
+            }
+            const double stream_at = (double)wl.ref - (double)ref_s;  // exact
+            if (__ballot(wl.s > 0.0f) != 0ull) {
+                const double e = stream_at < 1.0e9 ? (stream_at > -1.0e9 ? stream_at : -1.0e9) : 1.0e9;
+                ref_w = max(ref_w, (int)__builtin_floor(e));
+            }
+            const int down = up == UP_UNSET ? 0 : up - ref_w;  // <= 0
+            double part[4];
+            {
+                double d = stream_at - (double)ref_w;  // <= 1 where there is a sum
+                d = d < -1000.0 ? -1000.0 : d;
+                const double scale = pow2_d(d);
+                part[0] = wl.s > 0.0f ? (double)wl.s * scale : 0.0;
+                part[3] = wl.booked > 0.0f ? (double)wl.booked * scale : 0.0;
+            }
+            part[1] = __builtin_ldexp(acc_r, down);
+            part[2] = __builtin_ldexp(acc_t, down);
+    #pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                part[i] = wave_sum_d(part[i]);
+                if (lane == 0) {
+                    sh.red3[i][w] = part[i];
+                }
+            }
+            if (lane == 0) {
+                sh.red_i[w] = (uint32_t)ref_w;
+            }
+            // A NaN logit in a summed chunk leaves its wave's running sum a NaN: such a logit is
+            // worth -inf, and the row's sum is formed again from every value.
+            const bool poisoned = __syncthreads_or(wl.s != wl.s ? 1 : 0) != 0;
+            int ref_all = (int)sh.red_i[0];
+            for (int i = 1; i < NWAVE; ++i) {
+                ref_all = max(ref_all, (int)sh.red_i[i]);
+            }
+    #pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                part[i] = 0.0;
+                for (int ww = 0; ww < NWAVE; ++ww) {
+                    const int at = (int)sh.red_i[ww];
+                    part[i] += at == UP_UNSET ? 0.0 : __builtin_ldexp(sh.red3[i][ww], at - ref_all);
+                }
+            }
+            if (ref_all == UP_UNSET) {
+                ref_all = 0;  // no term anywhere: the sums are zero
+            }
+            // part[0]: the running sums, the listed ids' raw terms of part[3] already taken off (and
+            // their true terms added); part[1]: raw terms still to take off; part[2]: terms added
+            // one by one.
+            const double streamed = part[0], booked = part[1], exact = part[2], taken = part[3];
+            const double rest = streamed - booked;
+            // The streamed sums are f32: taking the listed ids' raw terms off again leaves an error of
+            // about 1e-6 of what was streamed.  Where that is more than 20 times the row's sum (listed
+            // ids held nearly everything that was streamed, and nothing larger was added exactly) the
+            // difference is too coarse.
+            const bool coarse = poisoned ||
+                                (booked + taken > 0.0 &&
+                                 !((rest > 0.0 ? rest : 0.0) + exact > 0.05 * (streamed + taken)));
+            phase(cfg, 10);
+            if (coarse) {
+                phase(cfg, 11);
+                LseAcc all;
+                all.init();
+                exact_terms<DT>(a, g.id_lo, g.id_hi, c2, all);
+                double m_e, s_e;
+                wg_merge_lse(sh, all.mc, all.s, m_e, s_e);
+                if (tid == 0) {
+                    sh.lse_mc = m_e;
+                    sh.lse_s = s_e;
+                }
+            } else if (tid == 0) {
+                double mc = (double)ref_s + (double)ref_all;
+                double sum = (rest > 0.0 ? rest : 0.0) + exact;
+                if (p_all > 0.0) {
+                    // Mode 2's post-scan terms have a reference of their own: the higher of the
+                    // two serves both (what lies 2^1000 below the other adds nothing).
+                    if (!(sum > 0.0)) {
+                        mc = ref_p;
+                        sum = p_all;
+                    } else {
+                        const double top = mc > ref_p ? mc : ref_p;
+                        const double d0 = mc - top, d1 = ref_p - top;
+                        sum = sum * pow2_d(d0 < -1000.0 ? -1000.0 : d0) +
+                              p_all * pow2_d(d1 < -1000.0 ? -1000.0 : d1);
+                        mc = top;
+                    }
+                }
+                sh.lse_mc = mc;
+                sh.lse_s = sum;
+            }
+    
         }
     }
     __syncthreads();
