@@ -5,9 +5,6 @@
 
 #include "device_common.h"
 
-#ifndef LILY_LOOP
-#define LILY_LOOP 0
-#endif
 namespace lily {
 
 // ------------------------------------------------------------------ streaming select
@@ -163,18 +160,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         const uint32_t c0 = g.cb + b * BLOCK;
         return c0 >= g.main_lo && c0 + BLOCK <= g.main_hi;
     };
-    // The first three blocks are asked for before anything else: the row's other preparations
-    // (a list of bias pairs, the scratch's largest count and the value of its most-counted id:
-    // round trips to memory that depend on each other) then run beside them.
+    // The first block is asked for before anything else.  (Asking for the second and third here
+    // as well - twelve loads a thread in flight across the row's preparations - made the launch of
+    // 1 024 rows 8 us longer per extra block.)
     u32x4 buf_a[U], buf_b[U], buf_c[U];
     if (nblocks > 0) {
         fetch(buf_a, 0);
-#if LILY_LOOP == 2
-        fetch(buf_b, min(1u, nblocks - 1u));
-        fetch(buf_c, min(2u, nblocks - 1u));
-#elif LILY_LOOP == 1
-        fetch(buf_b, min(1u, nblocks - 1u));
-#endif
     }
     if (tid == 0) {
         sh.n_fc = 0;
@@ -594,11 +585,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             if (give_up || stop || b >= nblocks) {
                 return;
             }
-#if defined(LILY_PRIO_PROGRESS)
-            // A wave that has further to go asks to be issued first: the four workgroups that
-            // share a compute unit then advance together instead of in the order they arrived.
+            // A wave that has further to go asks to be issued first, so that the workgroups that
+            // share a compute unit advance together instead of in the order they arrived (the
+            // arbiter otherwise favours the oldest wave, and the rows dispatched last scan alone at
+            // the end).  Four levels: the quarter of the way the wave has come, rows dispatched
+            // earlier counted as two blocks further on per generation.
             {
-                const uint32_t q = (b * 4u) / max(nblocks, 1u);
+                const uint32_t gen = min((blockIdx.y * 4u) / max(gridDim.y, 1u), 3u);
+                const uint32_t q = min(((b + 2u * (3u - gen)) * 4u) / (nblocks + 6u), 3u);
                 if (q == 0u) {
                     __builtin_amdgcn_s_setprio(3);
                 } else if (q == 1u) {
@@ -609,19 +603,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     __builtin_amdgcn_s_setprio(0);
                 }
             }
-#elif defined(LILY_PRIO_STATIC)
-            // (experiment) later rows of a compute unit first
-            {
-                const uint32_t q = (blockIdx.y * 4u) / max(gridDim.y, 1u);
-                if (q == 3u) {
-                    __builtin_amdgcn_s_setprio(3);
-                } else if (q == 2u) {
-                    __builtin_amdgcn_s_setprio(2);
-                } else if (q == 1u) {
-                    __builtin_amdgcn_s_setprio(1);
-                }
-            }
-#endif
             // tb_all: a byte per chunk of the block, bit j = element j is a listed id.
             uint32_t tb_all = 0u, mb[U] = {0u, 0u, 0u, 0u};
             if (SP) {
@@ -853,47 +834,13 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         if (nblocks == 0) {
             refresh_bound(true, true);  // the same barriers in every workgroup
         } else if (b_first < nblocks) {
-#if LILY_LOOP == 2
-            if (b_first != 0u) {   // (blocks 0, 1 and 2 were requested at the very start)
-                fetch(buf_a, b_first);
-                fetch(buf_b, min(b_first + 1u, nblocks - 1u));
-                fetch(buf_c, min(b_first + 2u, nblocks - 1u));
-            }
-            if (SP) {
-                bits_request(bits_a, b_first);
-                bits_request(bits_b, min(b_first + 1u, nblocks - 1u));
-                bits_request(bits_c, min(b_first + 2u, nblocks - 1u));
-            }
-            // A block's buffer is asked for the block three further on as soon as the block has
-            // been worked on: two blocks are on their way while one is looked at.  Every trip
-            // issues the same requests (past the row's end they ask for its last block again, and
-            // `work` returns at once): a request that some path skips would make every wait count
-            // as if it had been skipped.
-            for (uint32_t b = b_first; b < nblocks && !give_up && !stop; b += 3u) {
-                work(buf_a, bits_a, b);
-                request(buf_a, bits_a, b + 3u);
-                work(buf_b, bits_b, b + 1u);
-                request(buf_b, bits_b, b + 4u);
-                work(buf_c, bits_c, b + 2u);
-                request(buf_c, bits_c, b + 5u);
-            }
-#else
             if (b_first != 0u) {
                 fetch(buf_a, b_first);   // (block 0 was requested at the very start)
             }
             if (SP) {
                 bits_request(bits_a, b_first);
             }
-#if LILY_LOOP == 1
-            if (b_first != 0u) {
-                fetch(buf_b, min(b_first + 1u, nblocks - 1u));
-            }
-            if (SP) {
-                bits_request(bits_b, min(b_first + 1u, nblocks - 1u));
-            }
-#else
             request(buf_b, bits_b, b_first + 1u);
-#endif
             for (uint32_t b = b_first; b < nblocks && !give_up && !stop; b += 3) {
                 request(buf_c, bits_c, b + 2);
                 work(buf_a, bits_a, b);
@@ -906,7 +853,6 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                     }
                 }
             }
-#endif
         }
     };
     if (noting) {

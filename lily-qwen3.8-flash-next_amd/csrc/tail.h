@@ -157,10 +157,15 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
 // second spare word).  That id is a hint only - writers race, un-counting leaves it alone - and
 // readers take its count from the histogram.  Returns the count before.
 __device__ __forceinline__ uint32_t count_token(const RowArgs& a, uint32_t id, uint32_t vocab) {
+    // The largest count so far is read beside the increment (one round trip for both): a launch
+    // has one writer per scratch, so what the maximum becomes follows from the two, and nothing
+    // waits for the maximum's own update.
+    const uint32_t words = (vocab + 31u) / 32u;
+    const uint32_t top = gload(&a.touched[words]);
     const uint32_t before = atomicAdd(&a.counts[id], 1u);
     atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
-    const uint32_t words = (vocab + 31u) / 32u;
-    if (atomicMax(&a.touched[words], before + 1u) <= before + 1u) {
+    if (top <= before + 1u) {
+        atomicMax(&a.touched[words], before + 1u);
         a.touched[words + 1u] = id;
     }
     return before;
@@ -220,7 +225,12 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, Shared& sh, uint3
         }
         return;
     }
-    uint32_t before = 0;
+    // The id's logit is asked for before the increments (it comes back with the count), and
+    // the logarithm of the row's sum is formed while they are on their way.
+    const float l = want ? load_logit<DT>(a.logits, id) : 0.0f;
+    const bool allowed = !want || a.allow == nullptr || bit_of(a.allow, id);
+    uint32_t before = 0, top = 0;
+    const uint32_t words = (vocab + 31u) / 32u;
     if (in_order) {
         // Rows that draw in order: the next row learns the id; nobody waits for the increments.
         sh.emitted_id = id;
@@ -228,15 +238,22 @@ __device__ __forceinline__ void finish_token(const RowArgs& a, Shared& sh, uint3
             count_token_blind(a, id);
         }
     } else if (pen) {
-        before = count_token(a, id, vocab);
+        // (count_token(), taken apart so that nothing between here and the logarithm below
+        // waits for memory)
+        top = gload(&a.touched[words]);
+        before = atomicAdd(&a.counts[id], 1u);
+        atomicOr(&a.touched[id >> 5], 1u << (id & 31u));
+    }
+    const double base = want ? sh.lse_mc + log2(sh.lse_s) : 0.0;
+    if (pen && !in_order && top <= before + 1u) {
+        atomicMax(&a.touched[words], before + 1u);
+        a.touched[words + 1u] = id;
     }
     if (want) {
-        const float l = load_logit<DT>(a.logits, id);
-        const bool allowed = a.allow == nullptr || bit_of(a.allow, id);
         const float u = finish_pre_temperature(a, id, l, before, allowed);
         float lp = NEG_INF;
         if (u > NEG_INF) {
-            const double e = (double)u * (double)a.c2 - sh.lse_mc - log2(sh.lse_s);
+            const double e = (double)u * (double)a.c2 - base;
             lp = fminf((float)(e * 0.6931471805599453), 0.0f);  // the sum is approximate: clamp
         }
         *a.out_logprob = lp;
