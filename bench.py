@@ -6,7 +6,11 @@
 One "step" is one pass of the sampler over one batch of synthetic logits already
 resident in HBM: the throughput configuration of BASELINE.json (1 024 rows x 151 936
 bf16 logits, top-k 64, top-p 0.9, T 0.8, penalties over a 2 048-id history per row,
-output = token ids + chosen-token log-probabilities).  The 4-row decode-step
+output = token ids + chosen-token log-probabilities).  Every timed step reads other
+logits than the step before it (LOGITS_SETS resident batches taken in turn: a decode
+step never sees the same logits twice, and a sampler that is handed the same rows again
+and again finds the token it drew most often to be the row's dominant one, which it is
+not in general); the figure with one batch replayed is reported beside it.  The 4-row decode-step
 configuration (f32, 8 192-id history, k 20) is timed in the same run and reported in
 the same JSON line under "decode_b4".  The CPU oracle is timed on a bounded sample
 of the same rows on the host's cores as a reported baseline.
@@ -21,6 +25,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "lily-qwen3.8-flash-next_amd", "python"))
 
 HBM_PEAK_GBS = 8000.0
+LOGITS_SETS = 8   # resident batches of logits the timed steps take in turn
 # HBM bytes per 1024-row launch come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # very command, summarised in this file (a line "traffic_bytes_per_launch: N"; 1024 rows only).
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "k_rows_table_bf16_config5_b1024.md")
@@ -70,6 +75,47 @@ def time_steps(stream, fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def median_ms(stream, fn, reps, warmup):
+    """Median milliseconds of single calls of fn, each between its own pair of events."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    stream.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for i, (e0, e1) in enumerate(pairs):
+        e0.record(stream)
+        fn(warmup + i)
+        e1.record(stream)
+    pairs[-1][1].synchronize()
+    times = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return times[len(times) // 2]
+
+
+def cpp_caller(rows, vocab, calls):
+    """lily_sample_rows with host descriptors on every call, from the C++ program that the tests
+    build against the public header (a child process): host time a call takes to return,
+    device time per call, host time with an idle stream."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "abi_harness", "harness.bin")
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe, "time", str(rows), str(vocab), str(calls)], capture_output=True,
+                             text=True, timeout=240)
+    except (OSError, subprocess.TimeoutExpired):
+        return None
+    for line in res.stdout.splitlines():
+        w = line.split()
+        if w[:1] == ["time"]:
+            kv = dict(zip(w[1::2], w[2::2]))
+            return {"rows": rows, "calls": calls,
+                    "host_us_per_call": float(kv["host_us_per_call"]),
+                    "device_us_per_call": float(kv["device_us_per_call"]),
+                    "host_us_per_call_idle_stream": float(kv["host_us_per_call_idle_stream"]),
+                    "logits": "a language-model-shaped row rotated per row (the program's own), replayed"}
+    return None
+
+
 def paths_of(sampler, fn):
     """Which selects served one more (untimed) run of fn: workgroups by the streaming select, by
     the sparse / bitmap selects, by the exhaustive select, and the reasons the first gave up."""
@@ -99,8 +145,8 @@ def cpu_baseline(c, rows_total, seconds):
     import numpy as np
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle as O
-    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
-    cores = max(1, min(cores, 16))
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = max(1, min(avail, 16))   # the GPU box's CPU share is 16 whatever it shows
     x, hist = c["logits"], c["history"]
     vocab = x.shape[1]
     ext, _ = O.make_ext(sort_mode=O.SORT_FULL, want_logprob=True)
@@ -121,7 +167,8 @@ def cpu_baseline(c, rows_total, seconds):
         total_rows += n
         total_dt += dt
     n, dt = total_rows, total_dt
-    return {"value": n / dt, "unit": "rows/s", "cores": cores, "kind": "port",
+    return {"value": n / dt, "unit": "rows/s", "cores": cores, "nproc": os.cpu_count(),
+            "cores_available_to_this_process": avail, "kind": "port",
             "sample": f"{n} row draws (rows 0..{min(chunk, rows_total) - 1} of the {rows_total}, repeated), full-vocabulary index sort per row "
                       f"(as tests/unit/kernels/sample.rs:31-34), id + f64 log-probability, "
                       f"{dt:.1f} s wall"}
@@ -155,15 +202,25 @@ def main():
     scratches = make_scratches(LS, sampler, c5["history"], vocab, device)
     out_ids = torch.zeros(rows, dtype=torch.int32, device=device)
     out_lp = torch.zeros(rows, dtype=torch.float32, device=device)
+    # The other batches: the same rows handed to other requests and turned along the vocabulary
+    # (row r of batch j is row r - 131 j of the first, its ids moved on by 32 792 j), so that a
+    # request's scratch meets other logits at every step.
+    sets = [logits] + [torch.roll(logits, shifts=(131 * j, 32_792 * j), dims=(0, 1)).contiguous()
+                       for j in range(1, LOGITS_SETS)]
     torch.cuda.synchronize()
-    plan = sampler.plan(logits, params, [0] * rows, out_ids, scratch=scratches, out_logprobs=out_lp)
-    ms = time_steps(stream, lambda i: plan.run(i), a.steps, a.warmup)
+    plans = [sampler.plan(x, params, [0] * rows, out_ids, scratch=scratches, out_logprobs=out_lp)
+             for x in sets]
+    ms = time_steps(stream, lambda i: plans[i % LOGITS_SETS].run(i), a.steps, a.warmup)
     bytes_row = W.algorithmic_bytes_per_row(vocab, 2, history=history, logprob=True)
     achieved = rows * bytes_row / (ms * 1e-3) / 1e9
     ids_host = out_ids.cpu().numpy()
     assert ids_host.min() >= 0 and ids_host.max() < vocab
-    paths5 = paths_of(sampler, lambda i: plan.run(a.warmup + a.steps))
-    plan.close()
+    paths5 = paths_of(sampler, lambda i: plans[1].run(a.warmup + a.steps))
+    # for comparison: one batch replayed (what the figure of earlier builds was measured on)
+    ms_replay = time_steps(stream, lambda i: plans[0].run(2 * (a.warmup + a.steps) + i), a.steps, a.warmup)
+    for p_ in plans:
+        p_.close()
+    del sets[1:]
     # the reference's call shape at this size: host descriptors packed and uploaded every step
     ms_call = time_steps(stream, lambda i: sampler.sample_rows(logits, params, [i] * rows, out_ids,
                                                                scratch=scratches, out_logprobs=out_lp),
@@ -300,11 +357,23 @@ def main():
             ho = torch.zeros(b_rows, dtype=torch.int32, device=device)
             hl = torch.zeros(b_rows, dtype=torch.float32, device=device)
             torch.cuda.synchronize()
-            n_h = 10 if b_rows > 64 else 30
-            ms_head = time_steps(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum),
-                                 n_h, 2)
-            ms_fused = time_steps(stream, lambda i: sampler.lm_head_sample_rows(
-                hb, wb, lg, tmax, tsum, hp, [i] * b_rows, ho, out_logprobs=hl), n_h, 2)
+            n_h = 30
+            ms_head = median_ms(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum),
+                                n_h, 3)
+            ms_fused = median_ms(stream, lambda i: sampler.lm_head_sample_rows(
+                hb, wb, lg, tmax, tsum, hp, [i] * b_rows, ho, out_logprobs=hl), n_h, 3)
+            # what was timed is checked: the drawn ids lie in the vocabulary, and a seeded handful
+            # of the stored logits equal the f64 product of the same bf16 operands to one bf16 step
+            sampler.synchronize()
+            ids_h = ho.cpu().numpy()
+            assert ids_h.min() >= 0 and ids_h.max() < vocab, (ids_h.min(), ids_h.max())
+            pick = np.random.default_rng(17 + b_rows)
+            rr = torch.from_numpy(pick.integers(0, b_rows, 64)).to(device)
+            cc = torch.from_numpy(pick.integers(0, vocab, 64)).to(device)
+            want = (hb[rr].double() * wb[cc].double()).sum(dim=1)
+            have = lg[rr, cc].double()
+            assert bool(torch.all((have - want).abs() <= want.abs() * 2.0 ** -7 + 1e-3)), \
+                float((have - want).abs().max())
 
             def behind_a_head(draw, n=4):
                 """GPU time of a draw call: n of them queued while a head launch still runs, so
@@ -341,7 +410,7 @@ def main():
             # operands, bf16 in and out, without the summaries the head's epilogue leaves
             ref_out = torch.empty(b_rows, vocab, dtype=torch.bfloat16, device=device)
             with torch.cuda.stream(stream):
-                ms_lib = time_steps(stream, lambda i: torch.matmul(hb, wb.t(), out=ref_out), n_h, 3)
+                ms_lib = median_ms(stream, lambda i: torch.matmul(hb, wb.t(), out=ref_out), n_h, 3)
             del ref_out
             flops = 2.0 * b_rows * d_model * vocab
             head[f"b{b_rows}"] = {
@@ -351,6 +420,7 @@ def main():
                 "head_frac_of_mfma_peak": flops / (ms_head * 1e-3) / 1e12 / 2500.0,
                 "head_weight_GBs": vocab * d_model * 2 / (ms_head * 1e-3) / 1e9,
                 "library_gemm_us": ms_lib * 1e3,
+                "timing": f"median of {n_h} single launches",
                 "head_plus_draws_us": ms_fused * 1e3,
                 "draws_from_summaries_us": us_tiled,
                 "draws_from_rows_us": us_rows,
@@ -360,6 +430,12 @@ def main():
             }
             del hb, wb, lg
         del w_f32
+
+    # lily_sample_rows as a C++ caller sees it (the Python mirror packs 1 024 descriptors in
+    # Python on every call, which is what "us_per_step_host_descriptors" times)
+    sampler.synchronize()
+    torch.cuda.synchronize()
+    cpp = cpp_caller(rows, vocab, 100)
 
     line = {
         "metric": "rows/s and us/step at B=4 and B=1024 x151,936 vocab; achieved HBM GB/s",
@@ -381,7 +457,11 @@ def main():
             "rows": rows, "vocab": vocab, "logits": "bf16",
         },
         "us_per_step": ms * 1e3,
+        "logits_per_step": f"{LOGITS_SETS} resident batches taken in turn (row and vocabulary rotations of one "
+                           "generated batch): no step reads the logits of the step before it",
+        "us_per_step_replayed_logits": ms_replay * 1e3,
         "us_per_step_host_descriptors": ms_call * 1e3,
+        "host_descriptors_from_cpp": cpp,
         "paths": paths5,
         "decode_b4": {
             "workload": "4 rows x 151936 f32 logits, 8192-id Zipf history, rep 1.05 / pres 0.3 / "
