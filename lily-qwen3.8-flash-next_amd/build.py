@@ -1,6 +1,12 @@
 """Builds liblily_sampler_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
 
-    python lily-qwen3.8-flash-next_amd/build.py
+    python lily-qwen3.8-flash-next_amd/build.py [--strict-handover]
+
+--strict-handover builds liblily_sampler_hip_strict.so instead: the same library without the
+relaxed form of the hand-over between the workgroups of a row (-DLILY_STRICT_HANDOVER, see
+last_to_arrive() in csrc/device_common.h; the default build picks the form by the launch's size,
+and LILY_SAMPLER_HANDOVER=strict picks the strict one at run time).  LILY_SAMPLER_LIBRARY=<path>
+makes the Python mirror load it.
 
 The row kernel is compiled once per (logits type, kernel kind) pair from rows_variant.hip, in
 parallel; the objects are linked with the small kernels and the C-ABI layer.
@@ -47,20 +53,27 @@ def _run(cmd):
     return err
 
 
-def build(verbose=False, jobs=None):
+LIB_STRICT = os.path.join(HERE, "liblily_sampler_hip_strict.so")
+
+
+def build(verbose=False, jobs=None, strict_handover=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    os.makedirs(OBJ, exist_ok=True)
+    obj_dir = OBJ + ("_strict" if strict_handover else "")
+    lib = LIB_STRICT if strict_handover else LIB
+    flags = FLAGS + (["-DLILY_STRICT_HANDOVER"] if strict_handover else [])
+    os.makedirs(obj_dir, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
-    cmds = [[hipcc] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ, obj)]
+    cmds = [[hipcc] + flags + extra + ["-c", os.path.join(CSRC, src), "-o", os.path.join(obj_dir, obj)]
             for src, obj, extra in units()]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         for err in pool.map(_run, cmds):
             if verbose and err.strip():
                 sys.stderr.write(err + "\n")
-    objs = [os.path.join(OBJ, obj) for _, obj, _ in units()]
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB])
-    build_harness(hipcc)
-    return LIB
+    objs = [os.path.join(obj_dir, obj) for _, obj, _ in units()]
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", lib])
+    if not strict_handover:
+        build_harness(hipcc)
+    return lib
 
 
 HARNESS_SRC = os.path.join(os.path.dirname(HERE), "tests", "abi_harness", "harness.cpp")
@@ -79,4 +92,4 @@ def build_harness(hipcc):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, strict_handover="--strict-handover" in sys.argv[1:]))

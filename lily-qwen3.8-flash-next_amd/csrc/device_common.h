@@ -49,6 +49,64 @@ __device__ __forceinline__ T load_through(const T* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+template <class T>
+__device__ __forceinline__ void handed_store(const Handed<T>& h, size_t i, T v) {
+    store_through(h.p + i, v);
+}
+template <class T>
+__device__ __forceinline__ T handed_load(const Handed<T>& h, size_t i) {
+    return load_through(h.p + i);
+}
+
+// The hand-over between the workgroups of a row (or the rows of a chained launch): every
+// workgroup calls this after its handed_store()s; true, in every thread, in the workgroup that
+// arrives last, which then reads with handed_load().  The counter is left at 0 for the next launch.
+//
+// Strict form (`relaxed` false): the ticket is a device-scope release, and an acquire fence of the
+// same scope stands behind it - the hand-over the HIP memory model defines.
+//
+// Relaxed form: the ticket is a relaxed device atomic behind a wait for the thread's stores and a
+// workgroup barrier, and nothing is invalidated behind it.  That leans on the hardware, not on the
+// memory model: handed_store() writes through to memory (sc1) and has completed when
+// s_waitcnt vmcnt(0) returns, handed_load() reads past the L2 of its XCD, so neither a write-back
+// nor an invalidation of that L2 - what the release and the acquire cost, once per workgroup -
+// adds anything.  A plain store to handed memory would break it silently, which is why Handed<T>
+// admits none.  The host asks for this form only for launches of hundreds of workgroups
+// (LaunchCfg::relaxed_handover; LILY_SAMPLER_HANDOVER=strict|relaxed overrides the choice), and
+// -DLILY_STRICT_HANDOVER leaves it out of the build.
+__device__ __forceinline__ bool last_to_arrive(uint32_t* ticket, uint32_t expected, uint32_t& last_lds,
+                                               bool relaxed) {
+#ifdef LILY_STRICT_HANDOVER
+    relaxed = false;
+#endif
+    if (relaxed) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);   // every counter at 0: this thread's stores have completed
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_lds = t == expected - 1u ? 1u : 0u;
+        }
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    } else {
+        __syncthreads();   // (the other threads' stores happen before thread 0's release)
+        if (threadIdx.x == 0) {
+            const uint32_t t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            last_lds = t == expected - 1u ? 1u : 0u;
+        }
+        __syncthreads();
+        if (last_lds != 0u) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        }
+    }
+    const bool last = last_lds != 0u;
+    if (last && threadIdx.x == 0) {
+        store_through(ticket, 0u);
+    }
+    return last;
+}
+
 template <int DT>
 __device__ __forceinline__ float load_logit(const void* p, uint32_t i) {
     if (DT == LILY_BF16) {

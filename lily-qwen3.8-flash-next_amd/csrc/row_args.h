@@ -85,6 +85,15 @@ struct InlineRows {
     RowArgs r[INLINE_ROWS];
 };
 
+// Device memory that one workgroup writes and another reads after taking a ticket.  The type has
+// no indexing and no dereference: kernels reach it through handed_store() / handed_load()
+// (device_common.h) only, which go through to memory and read past the caches - the hand-over
+// depends on every access being of that kind.
+template <class T>
+struct Handed {
+    T* p;
+};
+
 // Launch-wide settings and the workspace of rows that span several workgroups.
 struct LaunchCfg {
     const RowArgs* table;   // device row table, or null when rows travel inline
@@ -92,8 +101,8 @@ struct LaunchCfg {
     uint32_t slices;        // workgroups per row
     uint32_t step_delta;    // added to every row's step
     uint32_t ws_k;          // candidate slots per (row, slice) in ws_cand
-    uint64_t* ws_cand;      // [rows][slices][ws_k] (value key << 32 | ~id)
-    double* ws_lse;         // [rows][slices][2] log2-domain reference, sum of 2^(x - reference)
+    Handed<uint64_t> ws_cand;   // [rows][slices][ws_k] (value key << 32 | ~id)
+    Handed<double> ws_lse;  // [rows][slices][2] log2-domain reference, sum of 2^(x - reference)
     uint32_t* ws_ticket;    // [rows] arrival counter, left at 0
     uint32_t path;          // 0 = automatic, 1 = exhaustive select only, 2 = two-pass select only,
                             // 3 = no streaming select
@@ -110,8 +119,8 @@ struct LaunchCfg {
     // counts the rows before it left): every row's candidates are collected against the counts
     // as they stood, published here, and the workgroup that finishes last draws row after row.
     uint32_t chain_rows;    // 0 = the rows are independent
-    uint64_t* chain_cand;   // [chain_rows][CHAIN_CAP]
-    uint32_t* chain_n;      // [chain_rows] candidates published
+    Handed<uint64_t> chain_cand;   // [chain_rows][CHAIN_CAP]
+    Handed<uint32_t> chain_n;      // [chain_rows] candidates published
     uint32_t* chain_ticket; // [1] rows that have published, left at 0
     // spec_accept by the same workgroup once the last row has drawn (null: not asked for)
     uint32_t* accept_ctrl;
@@ -122,6 +131,9 @@ struct LaunchCfg {
     // null, or [rows]: a row whose word is not 0 has been drawn by an earlier launch of the same
     // call (from the producer's summaries) and is left alone
     const uint32_t* served;
+    // 1 = the slices' hand-over in its relaxed form (last_to_arrive() in device_common.h)
+    uint32_t relaxed_handover;
+    uint32_t pad_cfg;
 };
 
 constexpr uint32_t CHAIN_CAP = LILY_SAMPLE_K_CAP;   // candidates a chained row publishes

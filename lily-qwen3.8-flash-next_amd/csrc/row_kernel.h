@@ -205,47 +205,30 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         // for its stores, the workgroup meets, and one thread takes the row's ticket.
         if (argmax) {
             if (tid == 0) {
-                store_through(&cfg.ws_cand[slot * cfg.ws_k], best);
+                handed_store(cfg.ws_cand, slot * cfg.ws_k, best);
             }
         } else {
             // Every slot is written (0 = no candidate), so the merge needs no counts.
             for (uint32_t i = tid; !forced && i < cfg.ws_k; i += NT) {
-                store_through(&cfg.ws_cand[slot * cfg.ws_k + i], i < n ? found[i] : (uint64_t)0);
+                handed_store(cfg.ws_cand, slot * cfg.ws_k + i, i < n ? found[i] : (uint64_t)0);
             }
             if (tid == 0) {
-                store_through(&cfg.ws_lse[2 * slot], want_lse ? sh.lse_mc : 0.0);
-                store_through(&cfg.ws_lse[2 * slot + 1], want_lse ? sh.lse_s : 0.0);
+                handed_store(cfg.ws_lse, 2 * slot, want_lse ? sh.lse_mc : 0.0);
+                handed_store(cfg.ws_lse, 2 * slot + 1, want_lse ? sh.lse_s : 0.0);
             }
         }
-        // The hand-over.  Every thread's partials above are device-scope stores that go through
-        // to memory, and the workgroup that arrives last reads them with device-scope loads that
-        // bypass the caches of its own XCD, so the ticket needs no release or acquire at the
-        // scope of the device (each writes back, or invalidates, the XCD's whole L2: 1 us of the
-        // 4-row step's 15, more with more workgroups): a thread's stores have completed when its
-        // wait ends, the barrier gathers the workgroup's, the ticket is taken behind it, and the
-        // reads are issued after the ticket's value has come back.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);   // every counter at 0: this thread's stores have completed
-        __syncthreads();
-        if (tid == 0) {
-            const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_AGENT);
-            sh.last = (t == S - 1) ? 1u : 0u;
-        }
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        // The hand-over (last_to_arrive(): a release on the ticket and an acquire behind it, or
+        // the relaxed form described there).
+        const bool last = last_to_arrive(&cfg.ws_ticket[row], S, sh.last, cfg.relaxed_handover != 0u);
         phase(cfg, 5);
-        if (sh.last == 0u) {
+        if (!last) {
             return;
-        }
-        if (tid == 0) {
-            store_through(&cfg.ws_ticket[row], 0u);
         }
         const size_t base = (size_t)row * S;
         if (argmax) {
             best = 0;
             for (uint32_t t = tid; t < S; t += NT) {
-                const uint64_t c = load_through(&cfg.ws_cand[(base + t) * cfg.ws_k]);
+                const uint64_t c = handed_load(cfg.ws_cand, (base + t) * cfg.ws_k);
                 best = c > best ? c : best;
             }
             best = wave_max_u64(best);
@@ -266,13 +249,13 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
 #pragma unroll
             for (int q = 0; q < PER; ++q) {
                 const uint32_t j = tid + (uint32_t)q * NT;
-                mine[q] = (!forced && j < slots) ? load_through(&cfg.ws_cand[base * cfg.ws_k + j]) : 0ull;
+                mine[q] = (!forced && j < slots) ? handed_load(cfg.ws_cand, base * cfg.ws_k + j) : 0ull;
             }
             if (want_lse && tid < 64) {
                 double mt = -__builtin_huge_val(), st = 0.0;
                 if (tid < S) {
-                    mt = load_through(&cfg.ws_lse[2 * (base + tid)]);
-                    st = load_through(&cfg.ws_lse[2 * (base + tid) + 1]);
+                    mt = handed_load(cfg.ws_lse, 2 * (base + tid));
+                    st = handed_load(cfg.ws_lse, 2 * (base + tid) + 1);
                     if (!(st > 0.0)) {
                         mt = -__builtin_huge_val();
                     }
@@ -345,26 +328,13 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         // the candidates), and the tail draws from the best k_draw.
         const uint32_t rows = cfg.chain_rows;
         for (uint32_t i = tid; i < n; i += NT) {
-            store_through(&cfg.chain_cand[(size_t)row * CHAIN_CAP + i], found[i]);
+            handed_store(cfg.chain_cand, (size_t)row * CHAIN_CAP + i, found[i]);
         }
         if (tid == 0) {
-            store_through(&cfg.chain_n[row], n);
+            handed_store(cfg.chain_n, row, n);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);   // (the hand-over of the slices above, once more)
-        __syncthreads();
-        if (tid == 0) {
-            const uint32_t arrived = __hip_atomic_fetch_add(cfg.chain_ticket, 1u, __ATOMIC_RELAXED,
-                                                            __HIP_MEMORY_SCOPE_AGENT);
-            sh.last = arrived == rows - 1u ? 1u : 0u;
-        }
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (sh.last == 0u) {
+        if (!last_to_arrive(cfg.chain_ticket, rows, sh.last, cfg.relaxed_handover != 0u)) {
             return;
-        }
-        if (tid == 0) {
-            store_through(cfg.chain_ticket, 0u);
         }
         const LILY_CONST RowArgs* first = src - row;
         if (cfg.accept_ctrl != nullptr && tid < rows) {
@@ -387,11 +357,11 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         for (uint32_t j0 = 0; j0 < rows; j0 += NWAVE) {
             const uint32_t j = j0 + (tid >> 6), lane = tid & 63u;
             if (j < rows) {
-                const uint32_t nj = min(load_through(&cfg.chain_n[j]), CHAIN_CAP);
+                const uint32_t nj = min(handed_load(cfg.chain_n, j), CHAIN_CAP);
                 if (lane == 0) {
                     sh.chain_n[j] = nj;
                 }
-                const uint64_t c = load_through(&cfg.chain_cand[(size_t)j * CHAIN_CAP + lane]);
+                const uint64_t c = handed_load(cfg.chain_cand, (size_t)j * CHAIN_CAP + lane);
                 const uint32_t id = min(composite_id(c), vocab - 1u);
                 pre_c[j * PRE + lane] = c;
                 pre_l[j * PRE + lane] = load_logit<DT>((first + j)->logits, id);
@@ -443,7 +413,7 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
                 __threadfence();
                 __syncthreads();
                 for (uint32_t i = tid + PRE; i < n_now; i += NT) {
-                    const uint64_t c = load_through(&cfg.chain_cand[(size_t)j * CHAIN_CAP + i]);
+                    const uint64_t c = handed_load(cfg.chain_cand, (size_t)j * CHAIN_CAP + i);
                     const uint32_t id = composite_id(c);
                     cand[i] = times_drawn(id) == 0u
                                   ? c

@@ -32,7 +32,7 @@ namespace lily {
 
 // What the two launches share beyond LaunchCfg.
 struct WideArgs {
-    float* lane_max;      // [rows][slices][lanes]
+    Handed<float> lane_max;   // [rows][slices][lanes]
     uint32_t lanes;       // values a slice leaves: NT, or NT / 2 (the larger of each pair of lanes)
     uint32_t* count;      // [rows] candidates the row's slices have left so far (0 between launches)
 };
@@ -108,27 +108,9 @@ __device__ __forceinline__ void wide_edges(const RowArgs& a, const Geo<DT>& g, F
     }
 }
 
-// The row's ticket: true in every thread of the workgroup that arrives last.  What the slices
-// hand over is stored through to memory (store_through) and read past the caches
-// (load_through), so the ticket needs no release or acquire at the scope of the device, which
-// would write back, and then invalidate, the whole L2 once per workgroup: the stores have
-// completed when the wait before the barrier ends, the ticket is taken after the barrier, and
-// the reads are issued after the ticket's value has come back.
+// The row's ticket: true in every thread of the workgroup that arrives last (last_to_arrive()).
 __device__ __forceinline__ bool wide_last(const LaunchCfg& cfg, uint32_t row, uint32_t S, Shared& sh) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);   // every counter at 0: this thread's stores have completed
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const uint32_t t = __hip_atomic_fetch_add(&cfg.ws_ticket[row], 1u, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT);
-        if (t == S - 1u) {
-            store_through(&cfg.ws_ticket[row], 0u);
-        }
-        sh.last = t == S - 1u ? 1u : 0u;
-    }
-    __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    return sh.last != 0u;
+    return last_to_arrive(&cfg.ws_ticket[row], S, sh.last, cfg.relaxed_handover != 0u);
 }
 
 // ---- first launch: lane maxima, the slice's sum of exponentials
@@ -200,21 +182,21 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
     WIDE_MARK(1);
     const size_t slot = (size_t)row * S + s;
     if (w.lanes == NT) {
-        store_through(&w.lane_max[slot * NT + tid], lane_max);
+        handed_store(w.lane_max, slot * NT + tid, lane_max);
     } else {
         // (with slices enough that half the lanes still are four times k, half the keys make
         // the select of the bound half as long)
         const int other = __builtin_amdgcn_update_dpp(0, (int)lilym_f32_bits(lane_max), 0xb1, 0xf, 0xf, true);   // quad_perm [1, 0, 3, 2]
         lane_max = fmaxf(lane_max, lilym_bits_f32((uint32_t)other));
         if ((tid & 1u) == 0u) {
-            store_through(&w.lane_max[slot * (NT / 2) + tid / 2u], lane_max);
+            handed_store(w.lane_max, slot * (NT / 2) + tid / 2u, lane_max);
         }
     }
     if (want_lse) {
         lse_reduce(sh, lse);
         if (tid == 0) {
-            store_through(&cfg.ws_lse[2 * slot], sh.lse_mc);
-            store_through(&cfg.ws_lse[2 * slot + 1], sh.lse_s);
+            handed_store(cfg.ws_lse, 2 * slot, sh.lse_mc);
+            handed_store(cfg.ws_lse, 2 * slot + 1, sh.lse_s);
         }
     }
     WIDE_MARK(2);
@@ -241,7 +223,7 @@ __device__ __forceinline__ float wide_bound_of(const WideArgs& w, uint32_t row, 
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const uint32_t i = min((uint32_t)(j0 + u) * NT + tid, n - 1u);
-                got[j0 + u] = load_through(&w.lane_max[(size_t)row * n + i]);
+                got[j0 + u] = handed_load(w.lane_max, (size_t)row * n + i);
             }
         }
     }
@@ -352,7 +334,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_draw(InlineRows rows_arg, Launch
     const uint32_t base = n_mine;
     if (base + mine <= MERGE_CAP) {
         for (uint32_t i = tid; i < mine; i += NT) {
-            store_through(&cfg.ws_cand[(size_t)row * MERGE_CAP + base + i], cand[i]);
+            handed_store(cfg.ws_cand, (size_t)row * MERGE_CAP + base + i, cand[i]);
         }
     }
     if (!wide_last(cfg, row, S, sh)) {
@@ -386,7 +368,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_draw(InlineRows rows_arg, Launch
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const uint32_t i = min((uint32_t)(j0 + u) * NT + tid, total - 1u);
-                got[u] = load_through(&cfg.ws_cand[(size_t)row * MERGE_CAP + i]);
+                got[u] = handed_load(cfg.ws_cand, (size_t)row * MERGE_CAP + i);
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
@@ -399,8 +381,8 @@ __global__ __launch_bounds__(NT, 4) void k_wide_draw(InlineRows rows_arg, Launch
         if (want_lse && tid < 64u) {
             double mt = -__builtin_huge_val(), st = 0.0;
             if (lane < S) {
-                mt = load_through(&cfg.ws_lse[2 * ((size_t)row * S + lane)]);
-                st = load_through(&cfg.ws_lse[2 * ((size_t)row * S + lane) + 1]);
+                mt = handed_load(cfg.ws_lse, 2 * ((size_t)row * S + lane));
+                st = handed_load(cfg.ws_lse, 2 * ((size_t)row * S + lane) + 1);
                 if (!(st > 0.0)) {
                     mt = -__builtin_huge_val();
                 }
@@ -449,7 +431,7 @@ hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t ro
     cfg.dyn_slots = MERGE_CAP;
     cfg.cand_cap = MERGE_CAP;
     WideArgs w;
-    w.lane_max = lane_max;
+    w.lane_max = Handed<float>{lane_max};
     w.lanes = (uint64_t)cfg.slices * (NT / 2) >= 4ull * cfg.ws_k ? NT / 2 : NT;
     w.count = count;
     const bool inl = inline_rows != nullptr;

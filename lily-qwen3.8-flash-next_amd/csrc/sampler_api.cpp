@@ -105,6 +105,7 @@ struct lily_sampler {
     uint32_t force_path = 0;
     uint32_t force_slices = 0;
     bool no_wide = false;   // LILY_SAMPLER_WIDE=0: rows of many candidates go the other kernels' way
+    uint32_t handover = 0;  // LILY_SAMPLER_HANDOVER: 0 = by the launch's size, 1 = strict, 2 = relaxed
     uint64_t* phase_trace = nullptr;
     uint64_t phase_words = 0;
     uint32_t* path_stats = nullptr;
@@ -317,16 +318,23 @@ uint32_t choose_slices(const lily_sampler* s, uint32_t rows, uint32_t kmax, uint
     return sl < 1 ? 1 : sl;
 }
 
-void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t vocab, uint32_t slices,
+// Launches of more than this many workgroups hand their slices over in the relaxed form (see
+// last_to_arrive() in device_common.h): there the release / acquire pair costs most (14 us of the
+// 72 that 64 rows of 1 024 candidates take over 2 x 1 024 workgroups; 1.2 us of a 4-row step).
+constexpr uint32_t RELAXED_MIN_GROUPS = 256;
+
+void fill_cfg(const lily_sampler* s, LaunchCfg* cfg, uint32_t rows, uint32_t vocab, uint32_t slices,
               uint32_t kmax, uint32_t step_delta, const RowArgs* table) {
     std::memset(cfg, 0, sizeof *cfg);
+    cfg->relaxed_handover = s->handover == 2u || (s->handover == 0u && (uint64_t)rows * slices > RELAXED_MIN_GROUPS)
+                                ? 1u : 0u;
     cfg->table = table;
     cfg->vocab = vocab;
     cfg->slices = slices;
     cfg->step_delta = step_delta;
     cfg->ws_k = kmax ? kmax : 1;
-    cfg->ws_cand = s->ws_cand;
-    cfg->ws_lse = s->ws_lse;
+    cfg->ws_cand = Handed<uint64_t>{s->ws_cand};
+    cfg->ws_lse = Handed<double>{s->ws_lse};
     cfg->ws_ticket = s->ws_ticket;
     cfg->path = s->force_path;
     cfg->cand_cap = CAND_CAP;
@@ -507,7 +515,7 @@ uint32_t plan_parts(const lily_sampler* s, RowArgs* table, uint32_t rows, int dt
 int launch_part(lily_sampler* s, const LaunchPart& part, const RowArgs* table_dev, int dtype,
                 uint32_t vocab, uint32_t step_delta, bool traced, const uint32_t* served = nullptr) {
     LaunchCfg cfg;
-    fill_cfg(s, &cfg, vocab, part.slices, part.ws_k, step_delta, table_dev + part.first);
+    fill_cfg(s, &cfg, part.rows, vocab, part.slices, part.ws_k, step_delta, table_dev + part.first);
     cfg.served = served != nullptr ? served + part.first : nullptr;
     if (traced) {
         attach_trace(s, &cfg, part.rows);
@@ -538,7 +546,7 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     LaunchCfg cfg;
     if (!chained) {
         if (const uint32_t ws = wide_slices(s, rows.r, n, dtype, vocab)) {
-            fill_cfg(s, &cfg, vocab, ws, kmax, 0, nullptr);
+            fill_cfg(s, &cfg, n, vocab, ws, kmax, 0, nullptr);
             bool lse = false;
             for (uint32_t i = 0; i < n; ++i) {
                 lse = lse || rows.r[i].out_logprob != nullptr;
@@ -548,11 +556,11 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
         }
     }
     const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
-    fill_cfg(s, &cfg, vocab, slices, kmax, 0, nullptr);
+    fill_cfg(s, &cfg, n, vocab, slices, kmax, 0, nullptr);
     if (chained) {
         cfg.chain_rows = n;
-        cfg.chain_cand = s->chain_cand;
-        cfg.chain_n = s->chain_n;
+        cfg.chain_cand = Handed<uint64_t>{s->chain_cand};
+        cfg.chain_n = Handed<uint32_t>{s->chain_n};
         cfg.chain_ticket = s->chain_ticket;
         cfg.accept_ctrl = accept.ctrl;
         cfg.accept_ids = accept.ids;
@@ -863,6 +871,9 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     }
     if (const char* p = std::getenv("LILY_SAMPLER_WIDE")) {
         s->no_wide = std::atoi(p) == 0;
+    }
+    if (const char* p = std::getenv("LILY_SAMPLER_HANDOVER")) {
+        s->handover = std::strcmp(p, "strict") == 0 ? 1u : std::strcmp(p, "relaxed") == 0 ? 2u : 0u;
     }
     const size_t slots = (size_t)WS_ROWS * MAX_SLICES;
     hipError_t err = hipMalloc(reinterpret_cast<void**>(&s->ws_cand),
@@ -1815,7 +1826,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
     uint32_t* served_dev = reinterpret_cast<uint32_t*>(const_cast<char*>(dev) + served_off);
     if (served != 0) {
         LaunchCfg cfg;
-        fill_cfg(s, &cfg, b->vocab, 1, 1, 0, s->table_dev);
+        fill_cfg(s, &cfg, served, b->vocab, 1, 1, 0, s->table_dev);
         attach_trace(s, &cfg, served);
         HIP_TRY(launch_rows_tiles(s->stream, lse, served, cfg, tile_max, tile_sum, tiles,
                                   reinterpret_cast<const uint32_t*>(dev + idx_off), served_dev));

@@ -14,7 +14,9 @@ import weakref
 import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(HERE), "liblily_sampler_hip.so")
+# LILY_SAMPLER_LIBRARY names another build of the library (build.py --strict-handover leaves
+# liblily_sampler_hip_strict.so beside the default one).
+LIB_PATH = os.environ.get("LILY_SAMPLER_LIBRARY") or os.path.join(os.path.dirname(HERE), "liblily_sampler_hip.so")
 
 SAMPLE_K_CAP = 1024
 CTRL_STRIDE = 4
