@@ -4,8 +4,9 @@ summaries (src/qwen4exp/batch.rs:573-593, src/qwen4exp/model.rs:4157-4169).
 Bar:
   * logits: each within one bf16 step of hidden @ weight.T computed in f64 from the same bf16
     inputs (the f32 accumulation of 512 products and the rounding to bf16 are what may differ);
-  * summaries: tile_max bit-exact against the stored logits, tile_sum within 2e-6 relative of
-    the f64 sum over the stored logits;
+  * summaries: tile_max bit-exact against the stored logits, tile_sum within 4e-6 relative of
+    the f64 sum over the stored logits (128 terms whose exponents are formed in f32: 1e-6 each at
+    the magnitudes of these logits);
   * draws: ids (and the candidate lists) bit-exact against the oracle ON THE STORED LOGITS,
     log-probabilities within 1e-5 * max(1, |logprob|) - the same bar as lily_sample_rows, whose
     results the tiled draws must equal.
@@ -84,14 +85,18 @@ def _check_product(h, w, logits, tmax, tsum, temps):
         c2 = np.float32(1.4426950408889634 / t)
         top = (g[r].max(axis=1).astype(np.float32) * c2).astype(np.float64)
         want = np.exp2(g[r].astype(np.float64) * np.float64(c2) - top[:, None]).sum(axis=1)
-        assert np.allclose(tsum[r].cpu().numpy(), want, rtol=2e-6, atol=0), r
+        assert np.allclose(tsum[r].cpu().numpy(), want, rtol=4e-6, atol=0), r
 
 
 @pytest.mark.parametrize("rows,d,vocab,slack", [(5, 256, 1000, 8), (130, 512, 4096 + 77, 8), (1, 64, 128, 8),
-                                                (300, 128, 2000 + 3, 8), (37, 192, 777, 3)])
+                                                (300, 128, 2000 + 3, 8), (37, 192, 777, 3),
+                                                (65, 256, 1500, 8), (96, 320, 2048 + 5, 3), (128, 128, 3000, 8),
+                                                (2049 + 130, 64, 300, 8)])
 def test_producer_against_f64_product(sampler, rows, d, vocab, slack):
-    """slack 8: rows of the logits start at multiples of 16 bytes (stored 16 bytes a lane);
-    slack 3: they do not (stored value by value)."""
+    """Every tile shape of the launcher: up to 32 rows, up to 64, 65 to 128 (three cases), more
+    (256-row tiles), and more than 2 048 rows (more blocks of hidden rows than XCDs: the other
+    branch of the tile numbering).  slack 8: rows of the logits start at multiples of 16 bytes;
+    slack 3: they start at any even address (every value is stored by a 2-byte store)."""
     rng = np.random.default_rng(rows * 1000 + d)
     hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(20, vocab // 8))
     temps = [0.0 if r % 5 == 4 else 0.5 + 0.1 * (r % 7) for r in range(rows)]
@@ -327,3 +332,54 @@ def test_rows_under_lowering_penalties_are_drawn_from_summaries(sampler):
     for r in range(rows):
         assert np.array_equal(scratch[r].read_counts().numpy().view(np.uint32), hist_counts[r]), r
         scratch[r].close()
+
+
+def test_the_benchmarked_shape(sampler):
+    """1 024 rows x 151 936 ids over d = 4 096, the shape bench.py times: a seeded subset of tiles
+    against the f64 product of the same bf16 operands (logits within one bf16 step, tile_max
+    exact on the stored logits, tile_sum within 4e-6), and the draws of 24 rows - through the one
+    call that runs the head and draws every row - against the oracle on the stored logits."""
+    rows, d, vocab = 1024, 4096, 151_936
+    gen = torch.Generator(device=dev())
+    gen.manual_seed(2024)
+    w_f32 = torch.randn(vocab, d, device=dev(), generator=gen) * (2.0 / d ** 0.5)
+    hid = torch.randn(rows, d, device=dev(), generator=gen)
+    for r in range(24):   # peaks, so that the checked rows have candidates worth drawing
+        ids = torch.randint(0, vocab, (40,), device=dev(), generator=gen)
+        gain = (torch.rand(40, 1, device=dev(), generator=gen) * 0.7 + 0.3) * (6.0 / d)
+        w_f32[ids] += gain * hid[r][None, :]
+    hb, wb = hid.to(torch.bfloat16), w_f32.to(torch.bfloat16)
+    del w_f32, hid
+    tiles = (vocab + TILE - 1) // TILE
+    logits = torch.zeros(rows, vocab, dtype=torch.bfloat16, device=dev())
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    params_kw = [dict(temperature=0.8, top_k=64, top_p=0.9, seed=5000 + r) for r in range(rows)]
+    params = [ls_params(**kw) for kw in params_kw]
+    steps = [4] * rows
+    out = torch.full((rows,), -1, dtype=torch.int32, device=dev())
+    lp = torch.zeros(rows, dtype=torch.float32, device=dev())
+    sampler.lm_head_sample_rows(hb, wb, logits, tmax, tsum, params, steps, out, out_logprobs=lp)
+    sampler.synchronize()
+    # ---- a seeded subset of tiles: the first, the last (ragged: 151 936 = 1 187 x 128) and 30 others
+    rng = np.random.default_rng(99)
+    pick = np.unique(np.concatenate([[0, tiles - 1], rng.integers(0, tiles, 30)]))
+    c2 = np.float32(1.4426950408889634 / 0.8)
+    for t in pick:
+        lo, hi = int(t) * TILE, min((int(t) + 1) * TILE, vocab)
+        ref = (hb.double() @ wb[lo:hi].double().T).cpu().numpy()
+        got = W.bf16_bits_to_f32(_bits(logits[:, lo:hi].contiguous()))
+        tol = np.abs(ref) * 2.0 ** -7 + 1e-4
+        assert np.all(np.abs(got - ref) <= tol), (int(t), float(np.max(np.abs(got - ref) - tol)))
+        assert np.array_equal(tmax[:, int(t)].cpu().numpy(), got.max(axis=1)), int(t)
+        top = (got.max(axis=1).astype(np.float32) * c2).astype(np.float64)
+        want = np.exp2(got.astype(np.float64) * np.float64(c2) - top[:, None]).sum(axis=1)
+        assert np.allclose(tsum[:, int(t)].cpu().numpy(), want, rtol=4e-6, atol=0), int(t)
+    # ---- the draws of 24 rows against the oracle on what was stored
+    ids, lps = out.cpu().numpy().astype(np.int64), lp.cpu().numpy()
+    assert ids.min() >= 0 and ids.max() < vocab
+    stored = _bits(logits[:24].contiguous())
+    for r in range(24):
+        dd = O.sample(stored[r], None, o_params(**params_kw[r]), steps[r], want_logprob=True)
+        assert ids[r] == dd.chosen, (r, ids[r], dd.chosen)
+        assert abs(lps[r] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (r, lps[r], dd.logprob)
