@@ -121,3 +121,56 @@ def test_given_uniforms_and_rising_penalties():
             assert got == want, (kw, u is not None, got, want)
             assert ok
     s.close()
+
+
+@pytest.mark.parametrize("outside", [False, True], ids=["q(d) = 2 p(d)", "proposal outside p's kept set"])
+def test_massless_residual_in_the_one_launch_form(outside):
+    """A rejected proposal whose residual max(0, p - q) has no mass: the kernel draws plainly from
+    p on the second uniform (sample.metal:649-651).  Draft heads never export such a distribution,
+    so it is written by hand: q equal to p on p's kept set except at the proposal (twice p there,
+    rejected by u1 = 0.75), or q equal to p with a proposal that p does not keep at all (always
+    rejected).  The rows are penalised, so both draw inside one launch, the speculative row in the
+    wave that runs every row's tail; the next row sees the count the fallback's draw left."""
+    s = LS.Sampler(0)
+    rng = np.random.default_rng(77)
+    vocab, m = 30_011, 2
+    target = rng.normal(0, 2, (m, vocab)).astype(np.float32)
+    kw = dict(temperature=1.0, top_k=12, top_p=1.0, seed=21, repetition_penalty=1.3,
+              presence_penalty=0.4, frequency_penalty=0.2)
+    lp, op = ls_params(**kw), o_params(**kw)
+    hist = rng.integers(0, vocab, 200)
+    t_target = torch.from_numpy(target).to(dev())
+    for which, u2 in ((0, 0.0), (4, 0.31), (11, 0.77), (2, 0.99999994)):
+        scratch = LS.SamplerScratch(s, vocab)
+        scratch.add_history(torch.from_numpy(hist.astype(np.int32)).to(dev()))
+        counts = np.bincount(hist, minlength=vocab).astype(np.uint32)
+        trunk = O.sample(target[0], counts.copy(), op, 3)
+        p_ids, p_pr = trunk.kept_ids, trunk.kept_q
+        dists = LS.DraftDists(s, m)
+        if outside:
+            d = int(np.setdiff1d(np.arange(64), p_ids)[0])
+            q_ids = np.concatenate([p_ids, [d]]).astype(np.uint32)
+            q_pr = np.concatenate([p_pr, [np.float32(0.5)]]).astype(np.float32)
+        else:
+            d = int(p_ids[which])
+            q_ids, q_pr = p_ids.copy(), p_pr.copy()
+            q_pr[which] = np.float32(2.0) * p_pr[which]
+        dists.write(0, q_ids, q_pr)
+        ids = torch.tensor([7, d], dtype=torch.int32, device=dev())
+        verify = torch.full((m,), -1, dtype=torch.int32, device=dev())
+        ctrl = torch.zeros(LS.ctrl_words(1), dtype=torch.int32, device=dev())
+        us = np.array([[0.75, u2], [0.5, 0.0]], dtype=np.float32)
+        s.spec_verify(t_target, scratch, lp, 3, dists, ids, verify, ctrl, pos0=9, ratio=4, chain=1,
+                      uniforms=us)
+        s.synchronize()
+        got = verify.cpu().numpy()
+        tok, acc, zero, gap = O.spec(p_ids, p_pr, q_ids, q_pr, d, op.seed, 3, u1=0.75, u2=u2)
+        assert zero and not acc
+        plain = O.sample(target[0], counts, op, 3, uniform=u2)      # bumps counts[plain.chosen]
+        assert got[0] == plain.chosen, (outside, which, u2, got[0], plain.chosen)
+        nxt = O.sample(target[1], counts, op, 4, uniform=0.5)
+        assert got[1] == nxt.chosen, (outside, which, u2, got[1], nxt.chosen)
+        assert np.array_equal(scratch.read_counts().numpy().view(np.uint32), counts)
+        scratch.close()
+        dists.close()
+    s.close()
