@@ -270,7 +270,10 @@ int lily_sample_spec_f32_uniforms(lily_sampler_t* s, const float* logits_dev, ui
  * until the process ends.  The call allocates and frees nothing and does not synchronise.
  * Same results as lily_sample_f32.  Limits: one row of at most LILY_STATIC_MAX_VOCAB logits
  * (LILY_ERR_RANGE beyond); every call on a GPU shares that GPU's array, so two calls that may
- * overlap on one GPU (different streams, or graphs replayed concurrently) race - order them. */
+ * overlap on one GPU (different streams, or graphs replayed concurrently) race - order them.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress, which may load
+ * the library's code object): make one call outside any stream capture on each device before
+ * capturing calls into a graph. */
 #define LILY_STATIC_MAX_VOCAB 1048576u
 int lily_sample_f32_static(void* hip_stream, const float* logits_dev, uint32_t vocab,
                            lily_scratch_t* scratch, const lily_sampling_params* params,
@@ -341,8 +344,10 @@ typedef struct lily_rows {
     uint64_t row_stride;                 /* elements between rows */
     const lily_sampling_params* params;  /* host [rows] */
     const uint32_t* steps;               /* host [rows] */
-    lily_scratch_t* const* scratch;      /* host [rows] or NULL; entries may be NULL; no
-                                            scratch may appear twice in one call */
+    lily_scratch_t* const* scratch;      /* host [rows] or NULL; entries may be NULL.  A row
+                                            touches its scratch only when its params use
+                                            penalties: a scratch may stand in several rows of one
+                                            call as long as at most one of them does */
     const uint32_t* allow_dev;           /* packed bits, bit id&31 of word id>>5, or NULL */
     uint64_t allow_stride;               /* words between rows; 0 = one mask for all rows */
     const lily_bias* bias_dev;           /* concatenated per-row lists or NULL */

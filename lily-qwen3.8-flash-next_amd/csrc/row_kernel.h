@@ -365,8 +365,8 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
                 const uint32_t id = min(composite_id(c), vocab - 1u);
                 pre_c[j * PRE + lane] = c;
                 pre_l[j * PRE + lane] = load_logit<DT>((first + j)->logits, id);
-                pre_cnt[j * PRE + lane] = (t.flags & F_PEN) ? load_through(t.counts + id) : 0u;
                 const LILY_CONST RowArgs* rj = first + j;
+                pre_cnt[j * PRE + lane] = (rj->flags & F_PEN) ? load_through(rj->counts + id) : 0u;
                 if (rj->mode == MODE_SPEC) {
                     pre_qid[j * PRE + lane] = gload(rj->q_ids + lane);
                     pre_qp[j * PRE + lane] = gload(rj->q_probs + lane);
@@ -475,12 +475,15 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        if (tid < rows && (t.flags & F_PEN) && sh.drawn[tid] < vocab) {
+        if (tid < rows && ((first + tid)->flags & F_PEN) && sh.drawn[tid] < vocab) {
+            // (row tid's own scratch: the launcher hands every row of such a launch the same one,
+            // but nothing here depends on that)
+            const LILY_CONST RowArgs* mine = first + tid;
             const uint32_t id = sh.drawn[tid];
             const uint32_t words = (vocab + 31u) / 32u;
-            const uint32_t now = load_through(t.counts + id);
-            if (atomicMax(&t.touched[words], now) <= now) {
-                t.touched[words + 1u] = id;
+            const uint32_t now = load_through(mine->counts + id);
+            if (atomicMax(&mine->touched[words], now) <= now) {
+                mine->touched[words + 1u] = id;
             }
         }
         if (cfg.accept_ctrl != nullptr && tid == 0) {

@@ -558,6 +558,15 @@ int launch_inline(lily_sampler* s, int dtype, uint32_t vocab, const InlineRows& 
     const uint32_t slices = choose_slices(s, n, kmax, vocab, dtype);
     fill_cfg(s, &cfg, n, vocab, slices, kmax, 0, nullptr);
     if (chained) {
+        // Rows that draw in order count what the rows before them drew into one histogram: the
+        // kernel's bookkeeping (an id drawn j times so far has its count raised by j) holds for
+        // rows of one scratch under one kind of penalty only.
+        for (uint32_t i = 1; i < n; ++i) {
+            if (rows.r[i].counts != rows.r[0].counts || rows.r[i].touched != rows.r[0].touched ||
+                ((rows.r[i].flags ^ rows.r[0].flags) & F_PEN) != 0u) {
+                return fail(LILY_ERR_INVALID_ARG, "rows that draw in order share one scratch (row %u differs)", i);
+            }
+        }
         cfg.chain_rows = n;
         cfg.chain_cand = Handed<uint64_t>{s->chain_cand};
         cfg.chain_n = Handed<uint32_t>{s->chain_n};
@@ -624,18 +633,24 @@ int pack_batch(const lily_rows* b, RowArgs* table) {
         if (!std::is_sorted(owners.begin(), owners.end())) {
             std::sort(owners.begin(), owners.end());
         }
-        for (size_t i = 1; i < owners.size(); ++i) {
-            if (owners[i].first != owners[i - 1].first) {
-                continue;
+        // Rows without penalties never touch their scratch: among the rows that name one scratch
+        // at most one may use penalties (two would count into one histogram at once).
+        for (size_t lo = 0; lo < owners.size();) {
+            size_t hi = lo + 1;
+            while (hi < owners.size() && owners[hi].first == owners[lo].first) {
+                ++hi;
             }
-            size_t first = i - 1;
-            while (first > 0 && owners[first - 1].first == owners[i].first) {
-                --first;
+            uint32_t first_pen = 0, n_pen = 0;
+            for (size_t i = lo; i < hi && hi - lo > 1; ++i) {
+                if (lily_params_uses_penalties(&b->params[owners[i].second])) {
+                    if (n_pen++ != 0) {
+                        return fail(LILY_ERR_INVALID_ARG, "rows %u and %u use penalties and share a scratch",
+                                    first_pen, owners[i].second);
+                    }
+                    first_pen = owners[i].second;
+                }
             }
-            if (lily_params_uses_penalties(&b->params[owners[i].second])) {
-                return fail(LILY_ERR_INVALID_ARG, "rows %u and %u share a scratch", owners[first].second,
-                            owners[i].second);
-            }
+            lo = hi;
         }
     }
     for (uint32_t r = 0; r < b->rows; ++r) {

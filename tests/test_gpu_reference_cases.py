@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 import lily_sampler as LS
 import oracle as O
-from gpu_util import both_params, dev, ls_params, run_rows, check_row_against_oracle
+from gpu_util import both_params, dev, ls_params, o_params, run_rows, check_row_against_oracle
 
 
 @pytest.fixture(scope="module")
@@ -402,3 +402,37 @@ def test_error_behaviour(sampler):
     with pytest.raises(LS.SamplerError):  # penalties need a scratch
         sampler.sample_f32(x, None, ls_params(presence_penalty=0.5), 0, out)
     wrong.close()
+
+
+def test_rows_that_share_a_scratch(sampler):
+    """A row touches its scratch only under penalties: a scratch may stand in several rows of one
+    call as long as at most one of them uses penalties - in either order; two penalised rows on
+    one scratch would count into one histogram at once and are refused."""
+    rng = np.random.default_rng(61)
+    v = 4096
+    x = rng.normal(0, 2, (3, v)).astype(np.float32)
+    hist = rng.integers(0, v, 100).astype(np.int32)
+    hist[:5] = np.argsort(-x[1])[:5]
+    plain = dict(temperature=0.8, top_k=10, top_p=0.9, seed=4)
+    pen = dict(plain, repetition_penalty=1.3, presence_penalty=0.5, frequency_penalty=0.2)
+    t = torch.from_numpy(x).to(dev())
+    out = torch.zeros(3, dtype=torch.int32, device=dev())
+    for kws in ([plain, pen, plain], [pen, plain, plain], [plain, plain, pen]):
+        sc = LS.SamplerScratch(sampler, v)
+        sc.add_history(torch.from_numpy(hist).to(dev()))
+        counts = np.bincount(hist, minlength=v).astype(np.uint32)
+        sampler.sample_rows(t, [ls_params(**kw) for kw in kws], [2, 2, 2], out, scratch=[sc, sc, sc])
+        sampler.synchronize()
+        got = out.cpu().numpy()
+        for r, kw in enumerate(kws):
+            d = O.sample(x[r], counts if kw is pen else None, o_params(**kw), 2)   # bumps counts under penalties
+            assert got[r] == d.chosen, (r, got[r], d.chosen)
+        assert np.array_equal(sc.read_counts().numpy().view(np.uint32), counts)
+        sc.close()
+    sc = LS.SamplerScratch(sampler, v)
+    with pytest.raises(LS.SamplerError) as e:
+        sampler.sample_rows(t, [ls_params(**pen), ls_params(**plain), ls_params(**pen)], [0, 0, 0], out,
+                            scratch=[sc, sc, sc])
+    assert e.value.code == -1 and "share a scratch" in str(e.value)
+    sampler.synchronize()
+    sc.close()

@@ -111,3 +111,38 @@ def test_static_entry_rejects_what_it_cannot_hold():
     assert e.value.code == -2
     with pytest.raises(LS.SamplerError):           # penalties need a scratch
         LS.sample_f32_static(stream, x, None, ls_params(presence_penalty=0.5), 0, out)
+
+
+def test_static_entry_captured_into_a_graph():
+    """Two static draws recorded into one HIP graph and replayed.  The first call on a device
+    looks the static array's address up (a module load that a capture does not admit), so one
+    call outside the capture comes first - as the header asks.  Every replay, with eager work
+    and synchronisations between them, gives the oracle's tokens."""
+    rng = np.random.default_rng(47)
+    big = rng.normal(0, 3, 151_936).astype(np.float32)
+    small = rng.normal(0, 3, 40_000).astype(np.float32)
+    kw = dict(temperature=0.7, top_k=20, top_p=0.95, seed=23)
+    p = ls_params(**kw)
+    tb, ts = torch.from_numpy(big).to(dev()), torch.from_numpy(small).to(dev())
+    outs = torch.full((2,), -1, dtype=torch.int32, device=dev())
+    warm = torch.full((1,), -1, dtype=torch.int32, device=dev())
+    side = torch.cuda.Stream(device=dev())
+    torch.cuda.synchronize()
+    LS.sample_f32_static(side, ts, None, p, 0, warm)          # the warm call, not captured
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        cur = torch.cuda.current_stream(0)
+        LS.sample_f32_static(cur, tb, None, p, 6, outs[0:1])
+        LS.sample_f32_static(cur, ts, None, p, 6, outs[1:2])
+    want = [O.sample(big, None, o_params(**kw), 6).chosen, O.sample(small, None, o_params(**kw), 6).chosen]
+    for replay in range(4):
+        outs.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert outs.cpu().tolist() == want, (replay, outs.cpu().tolist(), want)
+        # eager work on the same array between the replays
+        LS.sample_f32_static(side, tb, None, p, 100 + replay, warm)
+        side.synchronize()
+        assert int(warm.item()) == O.sample(big, None, o_params(**kw), 100 + replay).chosen
