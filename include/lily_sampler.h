@@ -451,7 +451,10 @@ int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* head, uint32_t rows
                       const float* temperatures, void* logits_dev, uint64_t row_stride);
 
 /* The draws alone: batch->logits_dev (bf16, rows at multiples of 16 bytes) and the summaries must
- * come from one producer call made with the temperatures of batch->params. */
+ * come from one producer call made with the temperatures of batch->params.  Where the summaries
+ * are those of this sampler's last producer call, a row that asks for a log-probability at
+ * another temperature than its sums were formed at is drawn from its logits instead (right
+ * token, right log-probability); summaries of any other origin are taken on trust. */
 int lily_sample_rows_tiled(lily_sampler_t* s, const lily_rows* batch, const float* tile_max_dev,
                            const float* tile_sum_dev);
 

@@ -106,6 +106,10 @@ struct lily_sampler {
     uint32_t force_slices = 0;
     bool no_wide = false;   // LILY_SAMPLER_WIDE=0: rows of many candidates go the other kernels' way
     uint32_t handover = 0;  // LILY_SAMPLER_HANDOVER: 0 = by the launch's size, 1 = strict, 2 = relaxed
+    // What the last lily_lm_head_bf16 call of this sampler left: where, and with which exponent
+    // scale per row (tile_sum is only good for a log-probability at that scale).
+    const float* head_sum = nullptr;
+    std::vector<float> head_c2;
     uint64_t* phase_trace = nullptr;
     uint64_t phase_words = 0;
     uint32_t* path_stats = nullptr;
@@ -1801,10 +1805,20 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
     uint32_t certain = 0, maybe = 0;
     bool lse = false;
     uint32_t at = 0;
+    // Summaries this sampler's lily_lm_head_bf16 produced at another temperature than the row's
+    // (or at none) would give the row a wrong log-probability with the right token: such a row
+    // is drawn from its logits instead.  (Summaries of any other origin are taken on trust.)
+    auto sum_at_other_scale = [&](uint32_t r) -> bool {
+        if (h != nullptr || tile_sum != s->head_sum || packed[r].out_logprob == nullptr) {
+            return false;
+        }
+        const float mine = std::isfinite(packed[r].c2) ? packed[r].c2 : 0.0f;
+        return r >= s->head_c2.size() || s->head_c2[r] != mine;
+    };
     for (int group = 0; group < 3; ++group) {
         for (uint32_t r = 0; r < rows; ++r) {
             const RowArgs& row = packed[r];
-            const bool serve = tiles_serve(row);
+            const bool serve = tiles_serve(row) && !sum_at_other_scale(r);
             const bool pen = serve && row.mode != MODE_ARGMAX && (row.flags & F_PEN) != 0;
             const int g = !serve ? 2 : (pen ? 1 : 0);
             if (g != group) {
@@ -1822,6 +1836,10 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
     }
     for (uint32_t r = 0; r < rows; ++r) {
         c2[r] = std::isfinite(packed[r].c2) ? packed[r].c2 : 0.0f;
+    }
+    if (h != nullptr) {
+        s->head_sum = h->tile_sum_dev;
+        s->head_c2.assign(c2, c2 + rows);
     }
     const uint32_t served = certain + maybe;
     LaunchPart parts[2];
@@ -1877,8 +1895,11 @@ int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* h, uint32_t rows, u
         return rc;
     }
     float* c2 = reinterpret_cast<float*>(s->stage[slot]);
+    s->head_sum = h->tile_sum_dev;
+    s->head_c2.resize(rows);
     for (uint32_t r = 0; r < rows; ++r) {
         c2[r] = temperatures != nullptr ? c2_of_temperature(temperatures[r]) : 0.0f;
+        s->head_c2[r] = c2[r];
     }
     if (int rc = stage_commit(s, slot, (size_t)rows * 4)) {
         return rc;

@@ -383,3 +383,29 @@ def test_the_benchmarked_shape(sampler):
         dd = O.sample(stored[r], None, o_params(**params_kw[r]), steps[r], want_logprob=True)
         assert ids[r] == dd.chosen, (r, ids[r], dd.chosen)
         assert abs(lps[r] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (r, lps[r], dd.logprob)
+
+
+def test_sums_formed_at_another_temperature_are_not_used(sampler):
+    """The producer ran with other temperatures than the rows are drawn at (or with none): the
+    sums of the summaries would give a wrong log-probability beside the right token, so rows that
+    ask for one are drawn from their logits - ids and log-probabilities are the oracle's, and the
+    path statistics show the selects that read the row."""
+    rows, d, vocab = 6, 128, 20_000
+    rng = np.random.default_rng(515)
+    hidden, weight = _peaked_head(rng, rows, d, vocab)
+    params_kw = [dict(temperature=0.7, top_k=20, top_p=0.9, seed=60 + r) for r in range(rows)]
+    params = [ls_params(**kw) for kw in params_kw]
+    steps = [2] * rows
+    for temps in ([1.3] * rows, None, [0.7, 0.7, 0.7, 1.3, 0.7, 0.7]):
+        h, w, buf, logits, tmax, tsum = _produce(sampler, hidden, weight, temps, rows, vocab)
+        stored = _bits(logits.contiguous())
+        stats = torch.zeros(4, dtype=torch.int32, device=dev())
+        sampler.set_path_stats(stats)
+        ids, lps, cand, counts = _draw_all(
+            sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+                logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+            logits, params_kw, steps)
+        sampler.set_path_stats(None)
+        _check_draws(stored, ids, lps, cand, counts, params_kw, steps)
+        wrong = rows if temps is None else sum(1 for t in temps if t != 0.7)
+        assert stats.cpu().numpy()[0] >= wrong, (temps, stats.cpu().tolist())
