@@ -415,9 +415,13 @@ void lily_insertions_clear(lily_insertions_t* q, uint32_t row);
  * Replaces the language-model head in front of the draws: `project_mat(mixed, lm_head, logits)`
  * followed by one `sample_f32` per row (src/qwen4exp/batch.rs:573-593) and the single-row
  * `gemv_quant(lm_head, mixed, logits)` + `sample_f32` (src/qwen4exp/model.rs:2959-2966,
- * 4157-4169), for a head held in bf16 (the reference's quantised formats are dequantised by
- * their owner first).  logits[r][v] = sum_i hidden[r][i] * weight[v][i], accumulated in f32 on
- * the matrix cores and rounded to bf16 (nearest even).  Beside the logits the producer leaves,
+ * 4157-4169).  The head is held in bf16 or in one of the reference's affine formats (4- or 8-bit
+ * codes with a bf16 scale and bias per group of a row: QuantWeights, src/weights.rs:27-36; its
+ * lm_head is 4 bits in groups of 64, or 8 under `--q8 head`), whose weights are what
+ * dequant_q4_bf16 / dequant_q8_bf16 make of them (q * scale + bias in f32, rounded to bf16:
+ * src/kernels/metal/quant.metal:179-233).  logits[r][v] = sum_i hidden[r][i] * weight[v][i],
+ * accumulated in f32 on the matrix cores and stored as f32 (what the reference's sampler reads,
+ * src/kernels/sample.rs:263) or rounded to bf16 (nearest even).  Beside the logits the producer leaves,
  * for every LILY_LOGIT_TILE_COLS columns of every row, the largest value and the sum of
  * 2^((x - largest) * log2(e) / T[r]) over the tile - "summaries".  A row without allow-mask or
  * bias list that is greedy or draws among at most 64 candidates, under no penalties or under
@@ -432,12 +436,18 @@ void lily_insertions_clear(lily_insertions_t* q, uint32_t row);
 typedef struct lily_lm_head {
     const void* hidden_dev;   /* bf16 [rows][hidden_stride], d valid elements a row */
     uint64_t hidden_stride;   /* elements; a multiple of 8; rows start at multiples of 16 bytes */
-    const void* weight_dev;   /* bf16 [vocab][weight_stride]: row v holds the weights of id v */
-    uint64_t weight_stride;   /* elements; a multiple of 8 */
+    const void* weight_dev;   /* weight_bits 0: bf16 [vocab][weight_stride], row v the weights of id v;
+                                 4 or 8: the codes, u32 [vocab][weight_stride] (d * bits / 32 words
+                                 hold a row, the lowest code of a word first) */
+    uint64_t weight_stride;   /* bf16 elements (a multiple of 8) or words of codes (a multiple of 4) */
     uint32_t d;               /* a multiple of 64 */
-    uint32_t reserved;        /* must be 0 */
+    uint32_t weight_bits;     /* 0 = bf16 weights; 4 or 8 = affine codes (f32 logits only) */
     float* tile_max_dev;      /* out [rows][lily_lm_head_tiles(vocab)] */
     float* tile_sum_dev;      /* out, same shape */
+    const void* scales_dev;   /* weight_bits 4 / 8: bf16 [vocab][d / group_size]; else unused */
+    const void* biases_dev;   /* same shape */
+    uint32_t group_size;      /* weight_bits 4 / 8: a power of two from 32 on that divides d */
+    uint32_t logits_f32;      /* 0 = the logits are bf16 [rows][row_stride], 1 = f32 */
 } lily_lm_head;
 
 /* Summaries a row: ceil(vocab / LILY_LOGIT_TILE_COLS); at most 2048 are supported. */
@@ -446,11 +456,11 @@ uint32_t lily_lm_head_tiles(uint32_t vocab);
 /* The producer alone.  temperatures: host [rows], the temperature each row will be drawn at, as
  * lily_params_effective reports it (1 for a greedy row); NULL or an entry that is not a positive
  * finite number: the sums of that row are not to be used.
- * logits_dev: bf16 [rows][row_stride]. */
+ * logits_dev: bf16 or f32 (head->logits_f32) [rows][row_stride]. */
 int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* head, uint32_t rows, uint32_t vocab,
                       const float* temperatures, void* logits_dev, uint64_t row_stride);
 
-/* The draws alone: batch->logits_dev (bf16, rows at multiples of 16 bytes) and the summaries must
+/* The draws alone: batch->logits_dev (bf16 or f32, rows at multiples of 16 bytes) and the summaries must
  * come from one producer call made with the temperatures of batch->params.  Where the summaries
  * are those of this sampler's last producer call, a row that asks for a log-probability at
  * another temperature than its sums were formed at is drawn from its logits instead (right

@@ -26,14 +26,24 @@ hipError_t launch_spec_accept(hipStream_t stream, const uint32_t* draws, const u
 // logits[rows, vocab] = hidden[rows, d] x weight[vocab, d]^T (bf16, strides in elements, d a
 // multiple of 64), with the largest value and the sum of 2^((x - largest) * c2_of_row[row]) of
 // every LILY_TILE_COLS columns in tile_max / tile_sum [rows, ceil(vocab / LILY_TILE_COLS)].
+// out_f32: the logits are f32 [rows, logits_stride] instead of bf16.  wq.bits 4 / 8: `weight` points
+// at the reference's affine codes (u32 words, weight_stride words a row), wq.scales / wq.biases at
+// bf16 [vocab, d >> wq.group_shift]; f32 logits only.
+struct HeadWeights {
+    uint32_t bits = 0;          // 0 = bf16 weights
+    const void* scales = nullptr;
+    const void* biases = nullptr;
+    uint32_t group_shift = 6;   // log2 of the group size
+};
 hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
                                const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
                                uint32_t vocab, const float* c2_of_row, void* logits,
-                               uint64_t logits_stride, float* tile_max, float* tile_sum);
+                               uint64_t logits_stride, float* tile_max, float* tile_sum, bool out_f32,
+                               const HeadWeights& wq);
 // The draw of `rows` rows of cfg.table from the summaries ([.., tiles] each) and the few tiles of
-// the bf16 logits that matter; tile_row[r] = the summaries' row of table row r; served[r] is set
+// the logits (bf16 or f32) that matter; tile_row[r] = the summaries' row of table row r; served[r] is set
 // for rows under penalties (1 = drawn, 0 = declined: the row is better read whole).
-hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const LaunchCfg& cfg,
+hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg,
                              const float* tile_max, const float* tile_sum, uint32_t tiles,
                              const uint32_t* tile_row, uint32_t* served);
 // Rows that draw among many candidates (k > 64), spread over cfg.slices workgroups a row: two

@@ -62,13 +62,29 @@ struct HeadTile {
 //
 // Workgroups are numbered so that an XCD's L2 holds the hidden rows its workgroups share (see
 // the numbering at the top of the kernel).
-template <class T>
+//
+// OUT_F32: the logits are stored as the f32 sums they are (the reference's sampler reads F32
+// logits, src/kernels/sample.rs:263), the summaries describe those; otherwise rounded to bf16.
+// WBITS 4 / 8: the weights are the reference's affine codes (QuantWeights, src/weights.rs:27-36:
+// u32 words of eight 4-bit or four 8-bit codes, low code first, a bf16 scale and bias per group
+// of a row), turned into bf16 as dequant_q4_bf16 / dequant_q8_bf16 turn them (w = q * scale +
+// bias in f32, rounded to bf16: src/kernels/metal/quant.metal:179-233) on their way into LDS;
+// `weight` then points at the codes, weight_stride counts words, and a row has
+// (d >> group_shift) groups.  (Tiles whose loads pass through registers only.)
+struct HeadQuant {
+    const uint16_t* scales;   // bf16 [vocab][d >> group_shift]
+    const uint16_t* biases;
+    uint32_t group_shift;
+};
+
+template <class T, bool OUT_F32, int WBITS>
 __global__ void __launch_bounds__(256, T::RESIDENT)
 k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
                const uint16_t* __restrict__ weight, uint64_t weight_stride, uint32_t rows,
                uint32_t d, uint32_t vocab, const float* __restrict__ c2_of_row,
-               uint16_t* __restrict__ logits, uint64_t logits_stride, float* __restrict__ tile_max,
-               float* __restrict__ tile_sum, uint32_t tiles_per_row, uint32_t m_tiles) {
+               void* __restrict__ logits_out, uint64_t logits_stride, float* __restrict__ tile_max,
+               float* __restrict__ tile_sum, uint32_t tiles_per_row, uint32_t m_tiles, HeadQuant quant) {
+    static_assert(WBITS == 0 || !T::DIRECT, "codes pass through registers");
     constexpr int BM = T::BM, BN = T::BN, BK = T::BK, MI = T::MI, NI = T::NI, ROW_BYTES = T::ROW_BYTES;
     extern __shared__ __align__(16) char lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -108,10 +124,23 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         src_h[i] = hidden + (uint64_t)min(m0 + r, rows - 1u) * hidden_stride + kc * 8u;
         dst_h[i] = r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 2) & 3u)) : kc) * 16u;
     }
+    // (codes: the row's words, the piece's eight codes at word (k0 + kc * 8) * WBITS / 32; the
+    // row's scales and biases, the piece's group at (k0 + kc * 8) >> group_shift)
+    const uint16_t* src_s[T::B_PER];
+    const uint16_t* src_b[T::B_PER];
+    uint32_t k_in[T::B_PER];
 #pragma unroll
     for (int i = 0; i < T::B_PER; ++i) {
         const uint32_t piece = tid + 256u * (uint32_t)i, r = piece / T::PIECES, kc = piece % T::PIECES;
-        src_w[i] = weight + (uint64_t)min(n0 + r, vocab - 1u) * weight_stride + kc * 8u;
+        const uint64_t row = min(n0 + r, vocab - 1u);
+        if constexpr (WBITS == 0) {
+            src_w[i] = weight + row * weight_stride + kc * 8u;
+        } else {
+            src_w[i] = weight + (row * weight_stride + kc * (8u * WBITS / 32u)) * 2u;   // (counted in 16-bit units)
+            src_s[i] = quant.scales + row * (uint64_t)(d >> quant.group_shift);
+            src_b[i] = quant.biases + row * (uint64_t)(d >> quant.group_shift);
+            k_in[i] = kc * 8u;
+        }
         dst_w[i] = T::A_BYTES + r * ROW_BYTES + (T::SWIZZLED ? (kc ^ ((r >> 2) & 3u)) : kc) * 16u;
     }
     // ring[j]: the loads of a stage on their way (registers), written to LDS one step before use
@@ -123,8 +152,32 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         }
 #pragma unroll
         for (int i = 0; i < T::B_PER; ++i) {
-            w[i] = *reinterpret_cast<const w32x4*>(src_w[i] + k0);
+            if constexpr (WBITS == 0) {
+                w[i] = *reinterpret_cast<const w32x4*>(src_w[i] + k0);
+            } else {
+                // the piece's codes (8 or 4 bytes), its group's scale and bias
+                const uint32_t* codes = reinterpret_cast<const uint32_t*>(src_w[i]) + k0 * WBITS / 32u;
+                const uint32_t g = (k0 + k_in[i]) >> quant.group_shift;
+                w[i].x = codes[0];
+                w[i].y = WBITS == 8 ? codes[1] : 0u;
+                w[i].z = (uint32_t)src_s[i][g] | ((uint32_t)src_b[i][g] << 16);
+                w[i].w = 0u;
+            }
         }
+    };
+    // eight codes and their group's (scale, bias) as eight bf16 weights: q * scale + bias in f32
+    // (a product and a sum, each rounded), rounded to bf16 (nearest even)
+    auto dequantised = [&](const w32x4& c) -> w32x4 {
+        const float sc = __builtin_bit_cast(float, c.z << 16), bi = __builtin_bit_cast(float, c.z & 0xffff0000u);
+        uint32_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t q = WBITS == 8 ? (((j < 4 ? c.x : c.y) >> (8 * (j & 3))) & 0xffu) : ((c.x >> (4 * j)) & 0xfu);
+            const float f = (float)q * sc + bi;
+            const uint32_t u = __builtin_bit_cast(uint32_t, f);
+            h[j] = (u & 0x7fffffffu) > 0x7f800000u ? ((u >> 16) | 0x40u) : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+        }
+        return w32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
     };
     // (`real` false: a step past the end of d, run so that every pass of the loop is alike -
     // the hidden rows are staged as zeros and add nothing)
@@ -137,7 +190,11 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
         }
 #pragma unroll
         for (int i = 0; i < T::B_PER; ++i) {
-            *reinterpret_cast<w32x4*>(base + dst_w[i]) = w[i];
+            if constexpr (WBITS == 0) {
+                *reinterpret_cast<w32x4*>(base + dst_w[i]) = w[i];
+            } else {
+                *reinterpret_cast<w32x4*>(base + dst_w[i]) = dequantised(w[i]);
+            }
         }
     };
 
@@ -347,18 +404,20 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
     for (int ni = 0; ni < NI; ++ni) {
         in_vocab[ni] = n0 + wn * (NI * 32u) + (uint32_t)ni * 32u + (lane & 31u) < vocab;
     }
+    if constexpr (!OUT_F32) {
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
+        for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni) {
+            for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float f = acc[mi][ni][v];   // (a bit_cast of the element itself reads element 0)
-                const uint32_t u = __builtin_bit_cast(uint32_t, f);
-                // round to nearest even; a NaN stays one (quiet)
-                const uint32_t r = (u & 0x7fffffffu) > 0x7f800000u ? ((u >> 16) | 0x40u)
-                                                                   : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-                acc[mi][ni][v] = __builtin_bit_cast(float, r << 16);
+                for (int v = 0; v < 16; ++v) {
+                    const float f = acc[mi][ni][v];   // (a bit_cast of the element itself reads element 0)
+                    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+                    // round to nearest even; a NaN stays one (quiet)
+                    const uint32_t r = (u & 0x7fffffffu) > 0x7f800000u ? ((u >> 16) | 0x40u)
+                                                                       : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+                    acc[mi][ni][v] = __builtin_bit_cast(float, r << 16);
+                }
             }
         }
     }
@@ -447,18 +506,24 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
                 const uint32_t r = m0 + row_of(mi, v);
                 if (r < rows && col < vocab) {
                     const float f = acc[mi][ni][v];
-                    logits[(uint64_t)r * logits_stride + col] = (uint16_t)(__builtin_bit_cast(uint32_t, f) >> 16);
+                    if constexpr (OUT_F32) {
+                        static_cast<float*>(logits_out)[(uint64_t)r * logits_stride + col] = f;
+                    } else {
+                        static_cast<uint16_t*>(logits_out)[(uint64_t)r * logits_stride + col] =
+                            (uint16_t)(__builtin_bit_cast(uint32_t, f) >> 16);
+                    }
                 }
             }
         }
     }
 }
 
-template <class T>
+template <class T, bool OUT_F32, int WBITS>
 static hipError_t launch_head_shape(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
                                     const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
                                     uint32_t vocab, const float* c2_of_row, void* logits,
-                                    uint64_t logits_stride, float* tile_max, float* tile_sum) {
+                                    uint64_t logits_stride, float* tile_max, float* tile_sum,
+                                    const HeadQuant& quant) {
     static bool sized[64] = {};
     int device = 0;
     hipError_t e = hipGetDevice(&device);
@@ -466,7 +531,7 @@ static hipError_t launch_head_shape(hipStream_t stream, const void* hidden, uint
         return e;
     }
     if (device < 0 || device >= 64 || !sized[device]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_lm_head_bf16<T>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_lm_head_bf16<T, OUT_F32, WBITS>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
         if (e != hipSuccess) {
             return e;
@@ -479,31 +544,60 @@ static hipError_t launch_head_shape(hipStream_t stream, const void* hidden, uint
     // slots an XCD needs at most (see the kernel's numbering)
     const uint32_t slots = m_tiles <= 8u ? (tiles_per_row + (8u / m_tiles) - 1u) / (8u / m_tiles)
                                          : ((m_tiles + 7u) / 8u) * tiles_per_row;
-    hipLaunchKernelGGL(k_lm_head_bf16<T>, dim3(8u * slots), dim3(256), T::LDS_BYTES, stream,
+    hipLaunchKernelGGL((k_lm_head_bf16<T, OUT_F32, WBITS>), dim3(8u * slots), dim3(256), T::LDS_BYTES, stream,
                        reinterpret_cast<const uint16_t*>(hidden), hidden_stride,
                        reinterpret_cast<const uint16_t*>(weight), weight_stride, rows, d, vocab,
-                       c2_of_row, reinterpret_cast<uint16_t*>(logits), logits_stride, tile_max, tile_sum,
-                       tiles_per_row, m_tiles);
+                       c2_of_row, logits, logits_stride, tile_max, tile_sum, tiles_per_row, m_tiles, quant);
     return hipGetLastError();
 }
 
 hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
                                const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
                                uint32_t vocab, const float* c2_of_row, void* logits,
-                               uint64_t logits_stride, float* tile_max, float* tile_sum) {
+                               uint64_t logits_stride, float* tile_max, float* tile_sum, bool out_f32,
+                               const HeadWeights& wq) {
+    HeadQuant quant;
+    quant.scales = static_cast<const uint16_t*>(wq.scales);
+    quant.biases = static_cast<const uint16_t*>(wq.biases);
+    quant.group_shift = wq.group_shift;
 #define LILY_HEAD_ARGS                                                                              \
     stream, hidden, hidden_stride, weight, weight_stride, rows, d, vocab, c2_of_row, logits,        \
-        logits_stride, tile_max, tile_sum
+        logits_stride, tile_max, tile_sum, quant
+    typedef HeadTile<1, 1, 1, 64, 4, 3> Tile32;
+    typedef HeadTile<1, 2, 1, 64, 3, 3> Tile64;
+    typedef HeadTile<2, 2, 2, 64, 3, 2> Tile128;
+    typedef HeadTile<2, 4, 2, 32, 2, 2, true> Tile256;
+    if (wq.bits != 0u) {
+        // codes: f32 logits only (what the reference's quantised head produces), and the tiles
+        // whose loads pass through registers, whatever the number of rows
+        if (!out_f32 || (wq.bits != 4u && wq.bits != 8u)) {
+            return hipErrorInvalidValue;
+        }
+#define LILY_HEAD_Q(TILE)                                                                           \
+    (wq.bits == 8u ? launch_head_shape<TILE, true, 8>(LILY_HEAD_ARGS)                               \
+                   : launch_head_shape<TILE, true, 4>(LILY_HEAD_ARGS))
+        if (rows <= 32u) {
+            return LILY_HEAD_Q(Tile32);
+        }
+        if (rows <= 64u) {
+            return LILY_HEAD_Q(Tile64);
+        }
+        return LILY_HEAD_Q(Tile128);
+#undef LILY_HEAD_Q
+    }
+#define LILY_HEAD_B(TILE)                                                                           \
+    (out_f32 ? launch_head_shape<TILE, true, 0>(LILY_HEAD_ARGS) : launch_head_shape<TILE, false, 0>(LILY_HEAD_ARGS))
     if (rows <= 32u) {
-        return launch_head_shape<HeadTile<1, 1, 1, 64, 4, 3>>(LILY_HEAD_ARGS);
+        return LILY_HEAD_B(Tile32);
     }
     if (rows <= 64u) {
-        return launch_head_shape<HeadTile<1, 2, 1, 64, 3, 3>>(LILY_HEAD_ARGS);
+        return LILY_HEAD_B(Tile64);
     }
     if (rows <= 128u) {
-        return launch_head_shape<HeadTile<2, 2, 2, 64, 3, 2>>(LILY_HEAD_ARGS);
+        return LILY_HEAD_B(Tile128);
     }
-    return launch_head_shape<HeadTile<2, 4, 2, 32, 2, 2, true>>(LILY_HEAD_ARGS);
+    return LILY_HEAD_B(Tile256);
+#undef LILY_HEAD_B
 #undef LILY_HEAD_ARGS
 }
 

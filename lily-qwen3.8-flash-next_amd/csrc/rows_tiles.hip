@@ -15,11 +15,11 @@ constexpr uint32_t SUMMED_DECLINE = 96;                  // or more tiles summed
 constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated element by element
 
 // One workgroup per row (rows without mask or bias list, penalties only of the kind that can
-// but lower a value, k <= STREAM_K_MAX; bf16).
+// but lower a value, k <= STREAM_K_MAX; bf16 or f32 logits, rows at multiples of 16 bytes).
 //   * The row's largest value is the largest summary; with at least k summaries at or above
 //     x, at least k values are: the k-th largest summary bounds the k-th largest value from
-//     below, and only tiles whose summary reaches it are read (16 lanes a tile, 16 bytes a
-//     lane); their values at or above the bound are the candidates.
+//     below, and only tiles whose summary reaches it are read (16 bytes a lane: 16 lanes a tile
+//     of bf16 logits, 32 of f32); their values at or above the bound are the candidates.
 //   * The row's sum of exponentials is the summaries' sums brought to the row's reference.
 //   * Under penalties the bound is the k-th largest summary as the worst penalty would leave it
 //     (more tiles are read), values of listed ids are evaluated with their counts, and the tiles
@@ -28,7 +28,7 @@ constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated ele
 //     over the whole row takes over.
 // `tile_row[r]` is the row of the summaries that belongs to row r of the table; `served[r]` is
 // written for rows under penalties: 1 = drawn here, 0 = left to the launch that follows.
-template <bool LSE>
+template <int DT, bool LSE>
 __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float* tile_max,
                                                       const float* tile_sum, uint32_t tiles,
                                                       const uint32_t* tile_row, uint32_t* served) {
@@ -36,6 +36,8 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     __shared__ uint16_t listed[TILES_MAX];   // tiles to read; bit 15: summed element by element
     __shared__ uint32_t refs[REF_CAP];       // pieces to evaluate: first id; bit 31: summed
     __shared__ uint32_t n_listed, n_refs, n_summed;
+    constexpr uint32_t E = (uint32_t)Geo<DT>::E;          // values in a piece of 16 bytes
+    constexpr uint32_t ELEM = DT == LILY_BF16 ? 2u : 4u;  // bytes a value
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     if (tid == 0) {
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
 #pragma unroll
                 for (uint32_t h = 0; h < LILY_TILE_COLS / 64u; ++h) {
                     const uint32_t col = first * LILY_TILE_COLS + h * 64u + lane;
-                    if (col < vocab && load_logit<LILY_BF16>(a.logits, col) == top) {
+                    if (col < vocab && load_logit<DT>(a.logits, col) == top) {
                         id = min(id, col);
                     }
                 }
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         float floor_v = lowered(top);
         const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
         if (heavy < vocab && max_count != 0u) {
-            floor_v = fmaxf(floor_v, true_value(heavy, load_logit<LILY_BF16>(a.logits, heavy)));
+            floor_v = fmaxf(floor_v, true_value(heavy, load_logit<DT>(a.logits, heavy)));
         }
         cut = floor_v - (log2f((float)vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
     }
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             lse_reduce(sh, lse);
         }
         if (tid == 0) {
-            finish_token<LILY_BF16>(a, sh, a.forced, vocab);
+            finish_token<DT>(a, sh, a.forced, vocab);
         }
         return;
     }
@@ -245,7 +247,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     // with the bound: a piece that reaches it (or belongs to a summed tile) is put on a list.
     // (Evaluating such pieces on the spot keeps one or two lanes of a wave busy while the
     // others wait, eight times per round: that was most of the kernel's time.)
-    constexpr uint32_t LANES = LILY_TILE_COLS / 8u, PER_ROUND = NT / LANES;
+    constexpr uint32_t LANES = LILY_TILE_COLS / E, PER_ROUND = NT / LANES;
     const uint32_t sub = tid % LANES, slot = tid / LANES;
     constexpr int ROUNDS = 8;
     for (uint32_t r0 = 0; r0 < n_t; r0 += (uint32_t)ROUNDS * PER_ROUND) {
@@ -255,21 +257,21 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         for (int u = 0; u < ROUNDS; ++u) {
             const uint32_t i = min(r0 + (uint32_t)u * PER_ROUND + slot, n_t - 1u);
             const uint32_t t = listed[i];
-            const uint32_t c = (t & 0x7fffu) * LILY_TILE_COLS + sub * 8u;
+            const uint32_t c = (t & 0x7fffu) * LILY_TILE_COLS + sub * E;
             col0[u] = (r0 + (uint32_t)u * PER_ROUND + slot < n_t && c < vocab) ? (c | ((t & 0x8000u) << 16))
                                                                               : 0xffffffffu;
             // A row starts at a multiple of 16 bytes (the host checks), so these pieces do too:
             // one that holds a valid column lies inside the row's pages, and the others are
             // replaced by the row's last such piece.
-            const uint32_t cc = min(c, (vocab - 1u) & ~7u);
-            q[u] = gload(reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) + (size_t)cc * 2u));
+            const uint32_t cc = min(c, (vocab - 1u) & ~(E - 1u));
+            q[u] = gload(reinterpret_cast<const u32x4*>(static_cast<const char*>(a.logits) + (size_t)cc * ELEM));
         }
 #pragma unroll
         for (int u = 0; u < ROUNDS; ++u) {
             // (true values are raw ones or lower: a piece whose largest raw value stays below the
             // bound holds no candidate)
             const bool want = col0[u] != 0xffffffffu &&
-                              ((col0[u] >> 31) != 0u || chunk_max<LILY_BF16>(q[u]) >= bound);
+                              ((col0[u] >> 31) != 0u || chunk_max<DT>(q[u]) >= bound);
             const uint64_t votes = __ballot(want);
             if (votes != 0ull) {
                 uint32_t base = 0;
@@ -287,16 +289,16 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     __syncthreads();
     // Then the listed pieces, a thread per value, four pieces' loads in flight per thread.
     const uint32_t n_r = n_refs;   // (beyond the list's capacity: the exhaustive select below)
-    const uint32_t e_of = tid & 7u;
-    for (uint32_t p0 = 0; p0 < min(n_r, REF_CAP); p0 += 4u * (NT / 8u)) {
+    const uint32_t e_of = tid % E;
+    for (uint32_t p0 = 0; p0 < min(n_r, REF_CAP); p0 += 4u * (NT / E)) {
         uint32_t ref[4], word[4];
         float raw[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const uint32_t p = p0 + (uint32_t)u * (NT / 8u) + (tid >> 3);
+            const uint32_t p = p0 + (uint32_t)u * (NT / E) + tid / E;
             ref[u] = p < min(n_r, REF_CAP) ? refs[p] : 0xffffffffu;
             const uint32_t id = min((ref[u] & 0x7fffffffu) + e_of, vocab - 1u);
-            raw[u] = load_logit<LILY_BF16>(a.logits, id);
+            raw[u] = load_logit<DT>(a.logits, id);
             // (the word of the scratch's bitmap that covers the id; the summaries' first word
             // when there is no scratch to ask: the load stays unconditional)
             word[u] = gload((pen ? a.touched : reinterpret_cast<const uint32_t*>(tile_max)) + (pen ? (id >> 5) : 0u));
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     uint32_t took = 0;
     if (n > TILE_CAND_CAP) {
         took = 2;
-        select_exhaustive<LILY_BF16>(a, 0, vocab, k, want_lse, cand, cfg.cand_cap, sh);
+        select_exhaustive<DT>(a, 0, vocab, k, want_lse, cand, cfg.cand_cap, sh);
         n = min(sh.n_cand, cfg.cand_cap);
     } else {
         n = select_topk(cand, n, k, sh, sorted);
@@ -346,11 +348,11 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         atomicAdd(&cfg.path_stats[took], 1u);
     }
     phase(cfg, 6);
-    tail<LILY_BF16, false>(a, vocab, step, n, sorted, cand, sh, cfg);
+    tail<DT, false>(a, vocab, step, n, sorted, cand, sh, cfg);
     phase(cfg, 7);
 }
 
-hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
+hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
                              const float* tile_max, const float* tile_sum, uint32_t tiles,
                              const uint32_t* tile_row, uint32_t* served) {
     if (tiles == 0 || tiles > TILES_MAX) {
@@ -363,13 +365,21 @@ hipError_t launch_rows_tiles(hipStream_t stream, bool lse, uint32_t rows, const 
     const size_t dyn_bytes = std::max(tail_bytes, (size_t)TILE_CAND_CAP * 8);
     cfg.dyn_slots = (uint32_t)(dyn_bytes / 8);
     const dim3 grid(1, rows), block(NT);
-    if (lse) {
-        hipLaunchKernelGGL(k_rows_tiles<true>, grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum,
-                           tiles, tile_row, served);
+#define LILY_TILES(DT, LSE)                                                                       \
+    hipLaunchKernelGGL((k_rows_tiles<DT, LSE>), grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum, \
+                       tiles, tile_row, served)
+    if (dtype == LILY_BF16) {
+        if (lse) {
+            LILY_TILES(LILY_BF16, true);
+        } else {
+            LILY_TILES(LILY_BF16, false);
+        }
+    } else if (lse) {
+        LILY_TILES(LILY_F32, true);
     } else {
-        hipLaunchKernelGGL(k_rows_tiles<false>, grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum,
-                           tiles, tile_row, served);
+        LILY_TILES(LILY_F32, false);
     }
+#undef LILY_TILES
     return hipGetLastError();
 }
 

@@ -1724,16 +1724,58 @@ int check_head(const lily_lm_head* h, uint32_t rows, uint32_t vocab, const void*
     if (h->d == 0 || h->d % 64u != 0) {
         return fail(LILY_ERR_INVALID_ARG, "d must be a positive multiple of 64");
     }
-    if (h->hidden_stride < h->d || h->weight_stride < h->d || h->hidden_stride % 8u != 0 ||
-        h->weight_stride % 8u != 0 || reinterpret_cast<uintptr_t>(h->hidden_dev) % 16u != 0 ||
+    if (h->hidden_stride < h->d || h->hidden_stride % 8u != 0 ||
+        reinterpret_cast<uintptr_t>(h->hidden_dev) % 16u != 0 ||
         reinterpret_cast<uintptr_t>(h->weight_dev) % 16u != 0) {
         return fail(LILY_ERR_INVALID_ARG,
                     "hidden and weight rows must start at multiples of 16 bytes and hold d elements");
+    }
+    if (h->weight_bits == 0u) {
+        if (h->weight_stride < h->d || h->weight_stride % 8u != 0) {
+            return fail(LILY_ERR_INVALID_ARG,
+                        "hidden and weight rows must start at multiples of 16 bytes and hold d elements");
+        }
+    } else {
+        if (h->weight_bits != 4u && h->weight_bits != 8u) {
+            return fail(LILY_ERR_INVALID_ARG, "weight_bits is 0 (bf16), 4 or 8");
+        }
+        const uint64_t words = (uint64_t)h->d * h->weight_bits / 32u;
+        if (h->weight_stride < words || h->weight_stride % 4u != 0) {
+            return fail(LILY_ERR_INVALID_ARG, "rows of codes hold d * bits / 32 words and start at multiples of 16 bytes");
+        }
+        const uint32_t gs = h->group_size;
+        if (gs < 32u || (gs & (gs - 1u)) != 0u || h->d % gs != 0u) {
+            return fail(LILY_ERR_INVALID_ARG, "group_size is a power of two from 32 on that divides d");
+        }
+        if (h->scales_dev == nullptr || h->biases_dev == nullptr) {
+            return fail(LILY_ERR_INVALID_ARG, "codes come with scales and biases");
+        }
+        if (h->logits_f32 == 0u) {
+            return fail(LILY_ERR_INVALID_ARG, "a head of codes produces f32 logits (logits_f32 = 1)");
+        }
+    }
+    if (h->logits_f32 > 1u) {
+        return fail(LILY_ERR_INVALID_ARG, "logits_f32 is 0 or 1");
     }
     if (row_stride < vocab) {
         return fail(LILY_ERR_INVALID_ARG, "row_stride is shorter than the vocabulary");
     }
     return LILY_OK;
+}
+
+struct HeadWeightsOf : HeadWeights {
+    explicit HeadWeightsOf(const lily_lm_head* h);
+};
+HeadWeightsOf::HeadWeightsOf(const lily_lm_head* h) {
+    HeadWeights& w = *this;
+    w.bits = h->weight_bits;
+    w.scales = h->scales_dev;
+    w.biases = h->biases_dev;
+    uint32_t shift = 0;
+    while (h->weight_bits != 0u && (1u << shift) < h->group_size) {
+        ++shift;
+    }
+    w.group_shift = shift;
 }
 
 // Rows the summaries serve: no mask, no bias list, penalties only of the lowering kind, the row
@@ -1762,13 +1804,17 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
     if (b == nullptr || b->rows == 0) {
         return fail(LILY_ERR_INVALID_ARG, "empty batch");
     }
-    if (b->dtype != LILY_BF16) {
-        return fail(LILY_ERR_INVALID_ARG, "summaries describe bf16 logits");
+    if (b->dtype != LILY_BF16 && b->dtype != LILY_F32) {
+        return fail(LILY_ERR_INVALID_ARG, "logits are bf16 or f32");
+    }
+    if (h != nullptr && (h->logits_f32 != 0u) != (b->dtype == LILY_F32)) {
+        return fail(LILY_ERR_INVALID_ARG, "the head's logits_f32 and the batch's dtype disagree");
     }
     if (tile_max == nullptr || tile_sum == nullptr) {
         return fail(LILY_ERR_INVALID_ARG, "tile_max and tile_sum are required");
     }
-    if (reinterpret_cast<uintptr_t>(b->logits_dev) % 16u != 0 || b->row_stride % 8u != 0) {
+    if (reinterpret_cast<uintptr_t>(b->logits_dev) % 16u != 0 ||
+        b->row_stride % (b->dtype == LILY_BF16 ? 8u : 4u) != 0) {
         return fail(LILY_ERR_INVALID_ARG, "rows of logits must start at multiples of 16 bytes");
     }
     const uint32_t rows = b->rows, tiles = lily_lm_head_tiles(b->vocab);
@@ -1854,14 +1900,14 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
                                     h->weight_stride, rows, h->d, b->vocab,
                                     reinterpret_cast<const float*>(dev + c2_off),
                                     const_cast<void*>(b->logits_dev), b->row_stride, h->tile_max_dev,
-                                    h->tile_sum_dev));
+                                    h->tile_sum_dev, h->logits_f32 != 0u, HeadWeightsOf(h)));
     }
     uint32_t* served_dev = reinterpret_cast<uint32_t*>(const_cast<char*>(dev) + served_off);
     if (served != 0) {
         LaunchCfg cfg;
         fill_cfg(s, &cfg, served, b->vocab, 1, 1, 0, s->table_dev);
         attach_trace(s, &cfg, served);
-        HIP_TRY(launch_rows_tiles(s->stream, lse, served, cfg, tile_max, tile_sum, tiles,
+        HIP_TRY(launch_rows_tiles(s->stream, (int)b->dtype, lse, served, cfg, tile_max, tile_sum, tiles,
                                   reinterpret_cast<const uint32_t*>(dev + idx_off), served_dev));
     }
     for (uint32_t q = 0; q < n_parts; ++q) {
@@ -1906,7 +1952,8 @@ int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* h, uint32_t rows, u
     }
     HIP_TRY(launch_lm_head_bf16(s->stream, h->hidden_dev, h->hidden_stride, h->weight_dev, h->weight_stride,
                                 rows, h->d, vocab, reinterpret_cast<const float*>(s->table_dev), logits_dev,
-                                row_stride, h->tile_max_dev, h->tile_sum_dev));
+                                row_stride, h->tile_max_dev, h->tile_sum_dev, h->logits_f32 != 0u,
+                                HeadWeightsOf(h)));
     return LILY_OK;
 }
 

@@ -99,8 +99,23 @@ class _Rows(C.Structure):
 class _LmHead(C.Structure):
     _fields_ = [("hidden_dev", C.c_void_p), ("hidden_stride", C.c_uint64),
                 ("weight_dev", C.c_void_p), ("weight_stride", C.c_uint64),
-                ("d", C.c_uint32), ("reserved", C.c_uint32),
-                ("tile_max_dev", C.c_void_p), ("tile_sum_dev", C.c_void_p)]
+                ("d", C.c_uint32), ("weight_bits", C.c_uint32),
+                ("tile_max_dev", C.c_void_p), ("tile_sum_dev", C.c_void_p),
+                ("scales_dev", C.c_void_p), ("biases_dev", C.c_void_p),
+                ("group_size", C.c_uint32), ("logits_f32", C.c_uint32)]
+
+
+class QuantWeights:
+    """The reference's affine weights (src/weights.rs:27-36): codes int32 [out, in * bits / 32]
+    (u32 words, the lowest code first), scales and biases bf16 [out, in / group_size]."""
+
+    def __init__(self, codes, scales, biases, group_size, bits):
+        self.codes, self.scales, self.biases = codes, scales, biases
+        self.group_size, self.bits = int(group_size), int(bits)
+
+    @property
+    def in_features(self):
+        return self.codes.shape[1] * (32 // self.bits)
 
 
 LOGIT_TILE_COLS = 128
@@ -465,26 +480,40 @@ class Sampler:
     # -- the logits' producer and the draws from its summaries,
     #    src/qwen4exp/batch.rs:573-593, src/qwen4exp/model.rs:4157-4169
     @staticmethod
-    def _head(hidden, weight, tile_max, tile_sum):
-        for t, name in ((hidden, "hidden"), (weight, "weight")):
-            if t.dtype != torch.bfloat16 or t.dim() != 2 or t.stride(1) != 1:
-                raise SamplerError(-1, f"{name} must be BF16 [rows, d], rows contiguous")
-        if hidden.shape[1] != weight.shape[1]:
-            raise SamplerError(-1, "hidden and weight differ in d")
+    def _head(hidden, weight, tile_max, tile_sum, logits):
+        """weight: a bf16 tensor [V, d] or a QuantWeights; logits: bf16 or f32 [rows, V]."""
+        if hidden.dtype != torch.bfloat16 or hidden.dim() != 2 or hidden.stride(1) != 1:
+            raise SamplerError(-1, "hidden must be BF16 [rows, d], rows contiguous")
+        if logits.dtype not in (torch.bfloat16, torch.float32) or logits.stride(1) != 1:
+            raise SamplerError(-1, "logits must be BF16 or F32 [rows, V], rows contiguous")
         h = _LmHead()
         h.hidden_dev, h.hidden_stride = hidden.data_ptr(), hidden.stride(0)
-        h.weight_dev, h.weight_stride = weight.data_ptr(), weight.stride(0)
         h.d = hidden.shape[1]
+        if isinstance(weight, QuantWeights):
+            if weight.codes.dtype != torch.int32 or weight.codes.stride(1) != 1 or weight.in_features != h.d:
+                raise SamplerError(-1, "codes must be int32 [V, d * bits / 32], rows contiguous")
+            for t in (weight.scales, weight.biases):
+                if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.shape != (weight.codes.shape[0], h.d // weight.group_size):
+                    raise SamplerError(-1, "scales and biases must be BF16 [V, d / group_size], contiguous")
+            h.weight_dev, h.weight_stride = weight.codes.data_ptr(), weight.codes.stride(0)
+            h.weight_bits, h.group_size = weight.bits, weight.group_size
+            h.scales_dev, h.biases_dev = weight.scales.data_ptr(), weight.biases.data_ptr()
+        else:
+            if weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.stride(1) != 1:
+                raise SamplerError(-1, "weight must be BF16 [V, d], rows contiguous")
+            if hidden.shape[1] != weight.shape[1]:
+                raise SamplerError(-1, "hidden and weight differ in d")
+            h.weight_dev, h.weight_stride = weight.data_ptr(), weight.stride(0)
+        h.logits_f32 = 1 if logits.dtype == torch.float32 else 0
         h.tile_max_dev = _ptr(tile_max, torch.float32)
         h.tile_sum_dev = _ptr(tile_sum, torch.float32)
         return h
 
     def lm_head(self, hidden, weight, temperatures, logits, tile_max, tile_sum):
-        """lily_lm_head_bf16: logits[rows, V] (bf16) = hidden @ weight.T with the summaries."""
+        """lily_lm_head_bf16: logits[rows, V] (bf16 or f32) = hidden @ weight.T with the summaries;
+        weight a bf16 tensor or a QuantWeights."""
         rows, vocab = logits.shape
-        if logits.dtype != torch.bfloat16 or logits.stride(1) != 1:
-            raise SamplerError(-1, "logits must be BF16 [rows, V], rows contiguous")
-        h = self._head(hidden, weight, tile_max, tile_sum)
+        h = self._head(hidden, weight, tile_max, tile_sum, logits)
         tarr = None if temperatures is None else (C.c_float * rows)(*[float(t) for t in temperatures])
         _check(_lib.lily_lm_head_bf16(self._h, C.byref(h), rows, vocab, tarr, logits.data_ptr(),
                                       logits.stride(0) if rows > 1 else vocab))
@@ -497,7 +526,7 @@ class Sampler:
 
     def lm_head_sample_rows(self, hidden, weight, logits, tile_max, tile_sum, params, steps, out_ids, **kw):
         r, keep = self._rows(logits, params, steps, out_ids, **kw)
-        h = self._head(hidden, weight, tile_max, tile_sum)
+        h = self._head(hidden, weight, tile_max, tile_sum, logits)
         _check(_lib.lily_lm_head_sample_rows(self._h, C.byref(h), C.byref(r)))
         return keep
 

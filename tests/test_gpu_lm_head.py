@@ -275,7 +275,7 @@ def test_rejections(sampler):
     f32 = torch.zeros(rows, vocab, dtype=torch.float32, device=dev())
     out = torch.zeros(rows, dtype=torch.int32, device=dev())
     with pytest.raises(LS.SamplerError):
-        sampler.sample_rows_tiled(f32, tmax, tsum, [ls_params()] * rows, [0, 0], out)   # f32 logits
+        sampler.sample_rows_tiled(f32[:, 1:], tmax, tsum, [ls_params()] * rows, [0, 0], out)   # rows off 16-byte boundaries
     sampler.synchronize()
 
 
@@ -409,3 +409,128 @@ def test_sums_formed_at_another_temperature_are_not_used(sampler):
         _check_draws(stored, ids, lps, cand, counts, params_kw, steps)
         wrong = rows if temps is None else sum(1 for t in temps if t != 0.7)
         assert stats.cpu().numpy()[0] >= wrong, (temps, stats.cpu().tolist())
+
+
+def _f32_bound(h, w):
+    """What the f32 accumulation of d products may differ from the f64 product by."""
+    return (h.double().abs() @ w.double().abs().T).cpu().numpy() * 2.0 ** -21 + 1e-6
+
+
+def _check_f32_product(h, w, logits, tmax, tsum, temps):
+    rows, vocab = logits.shape
+    got = logits.cpu().numpy()
+    ref = (h.double() @ w.double().T).cpu().numpy()
+    tol = _f32_bound(h, w)
+    assert np.all(np.abs(got - ref) <= tol), float(np.max(np.abs(got - ref) - tol))
+    tiles = tmax.shape[1]
+    g = np.pad(got, ((0, 0), (0, tiles * TILE - vocab)), constant_values=-np.inf).reshape(rows, tiles, TILE)
+    assert np.array_equal(tmax.cpu().numpy(), g.max(axis=2))
+    for r in range(rows):
+        t = temps[r] if temps is not None else 0.0
+        if not t > 0.0:
+            continue
+        c2 = np.float32(1.4426950408889634 / t)
+        top = (g[r].max(axis=1).astype(np.float32) * c2).astype(np.float64)
+        want = np.exp2(g[r].astype(np.float64) * np.float64(c2) - top[:, None]).sum(axis=1)
+        assert np.allclose(tsum[r].cpu().numpy(), want, rtol=4e-6, atol=0), r
+
+
+@pytest.mark.parametrize("rows,d,vocab", [(4, 256, 20_000), (70, 128, 3000 + 4), (150, 192, 2000)])
+def test_f32_logits_and_draws_from_their_summaries(sampler, rows, d, vocab):
+    """The producer with f32 logits (what the reference's sampler reads, src/kernels/sample.rs:263):
+    the stored values are the f32 sums, the summaries describe them, and the draws from the
+    summaries are the oracle's on the stored f32 logits."""
+    rng = np.random.default_rng(rows + d)
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(40, vocab // 8))
+    params_kw = _mixed_params(rows)
+    params = [ls_params(**kw) for kw in params_kw]
+    temps = [p.effective()[0] for p in params]
+    steps = [2 + r for r in range(rows)]
+    h, w = _bf16(hidden), _bf16(weight)
+    stride = ((vocab + 3) // 4) * 4 + 4
+    buf = torch.full((rows, stride), 7.0, dtype=torch.float32, device=dev())
+    logits = buf[:, :vocab]
+    tiles = (vocab + TILE - 1) // TILE
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    sampler.lm_head(h, w, temps, logits, tmax, tsum)
+    sampler.synchronize()
+    _check_f32_product(h, w, logits, tmax, tsum, temps)
+    assert torch.all(buf[:, vocab:] == 7.0)
+    stored = logits.contiguous().cpu().numpy()
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    _check_draws(stored, ids, lps, cand, counts, params_kw, steps)
+    # and the one call for both
+    logits.zero_()
+    ids2, lps2, cand2, counts2 = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.lm_head_sample_rows(
+            h, w, logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    assert np.array_equal(logits.contiguous().cpu().numpy(), stored)
+    assert np.array_equal(ids, ids2)
+
+
+def _quantised(rng, vocab, d, bits, group):
+    """Random affine weights in the reference's layout and what dequant_q4/q8_bf16 makes of them
+    (src/kernels/metal/quant.metal:179-233): q * scale + bias in f32, rounded to bf16."""
+    q = rng.integers(0, 1 << bits, (vocab, d)).astype(np.uint32)
+    scales = W.to_bf16_bits(rng.uniform(0.5, 1.5, (vocab, d // group)).astype(np.float32) * (2.0 / (1 << bits)) / np.sqrt(d))
+    biases = W.to_bf16_bits(-W.bf16_bits_to_f32(scales) * np.float32((1 << bits) / 2) +
+                            rng.normal(0, 0.02 / np.sqrt(d), (vocab, d // group)).astype(np.float32))
+    per = 32 // bits
+    words = np.zeros((vocab, d // per), dtype=np.uint32)
+    for j in range(per):
+        words |= q[:, j::per] << np.uint32(bits * j)
+    s = np.repeat(W.bf16_bits_to_f32(scales), group, axis=1)
+    b = np.repeat(W.bf16_bits_to_f32(biases), group, axis=1)
+    prod = (q.astype(np.float32) * s).astype(np.float32)
+    dense = W.to_bf16_bits((prod + b).astype(np.float32))
+    t = lambda a, dt: torch.from_numpy(a.view(np.int16) if dt is torch.bfloat16 else a.view(np.int32)).to(dev())
+    qw = LS.QuantWeights(t(words, torch.int32), t(scales, torch.bfloat16).view(torch.bfloat16),
+                         t(biases, torch.bfloat16).view(torch.bfloat16), group, bits)
+    return qw, torch.from_numpy(dense.view(np.int16)).to(dev()).view(torch.bfloat16)
+
+
+@pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 32), (8, 128)])
+@pytest.mark.parametrize("rows", [3, 40, 100, 300])
+def test_heads_of_affine_codes(sampler, bits, group, rows):
+    """The reference's quantised head formats (QuantWeights, src/weights.rs:27-36; lm_head is 4 bits
+    in groups of 64, 8 under --q8 head): logits against the f64 product of the hidden rows with
+    the weights as dequant_q4/q8_bf16 give them, for every tile shape the codes pass through;
+    greedy rows drawn by the same call pick the oracle's token on the stored logits."""
+    d, vocab = 256, 2000 + 8 * bits
+    rng = np.random.default_rng(1000 * bits + group + rows)
+    hidden = rng.normal(0, 1, (rows, d)).astype(np.float32)
+    qw, dense = _quantised(rng, vocab, d, bits, group)
+    h = _bf16(hidden)
+    params_kw = [dict(temperature=0.8, top_k=20, top_p=0.9, seed=r) if r % 2 else dict() for r in range(rows)]
+    params = [ls_params(**kw) for kw in params_kw]
+    temps = [p.effective()[0] for p in params]
+    logits = torch.zeros(rows, vocab, dtype=torch.float32, device=dev())
+    tiles = (vocab + TILE - 1) // TILE
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    steps = [1] * rows
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.lm_head_sample_rows(
+            h, qw, logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    _check_f32_product(h, dense, logits, tmax, tsum, temps)
+    _check_draws(logits.cpu().numpy(), ids, lps, cand, counts, params_kw, steps)
+
+
+def test_codes_ask_for_f32_logits(sampler):
+    rng = np.random.default_rng(5)
+    qw, _ = _quantised(rng, 256, 64, 8, 64)
+    h = torch.zeros(2, 64, dtype=torch.bfloat16, device=dev())
+    tmax = torch.zeros(2, 2, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(2, 2, dtype=torch.float32, device=dev())
+    with pytest.raises(LS.SamplerError):
+        sampler.lm_head(h, qw, None, torch.zeros(2, 256, dtype=torch.bfloat16, device=dev()), tmax, tsum)
+    bad = LS.QuantWeights(qw.codes, qw.scales, qw.biases, 48, 8)
+    with pytest.raises(LS.SamplerError):
+        sampler.lm_head(h, bad, None, torch.zeros(2, 256, dtype=torch.float32, device=dev()), tmax, tsum)
+    sampler.synchronize()
