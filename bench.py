@@ -91,6 +91,27 @@ def median_ms(stream, fn, reps, warmup):
     return times[len(times) // 2]
 
 
+def queued_ms(stream, fn, reps, warmup, rounds=3):
+    """Milliseconds per call of fn over `reps` calls queued back to back between one pair of
+    events (the host's work for a call hides behind the device's work for the one before), the
+    best of `rounds`."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    best = None
+    for _ in range(rounds):
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(reps):
+            fn(i)
+        e1.record(stream)
+        e1.synchronize()
+        t = e0.elapsed_time(e1) / reps
+        best = t if best is None else min(best, t)
+    return best
+
+
 def cpp_caller(rows, vocab, calls):
     """lily_sample_rows with host descriptors on every call, from the C++ program that the tests
     build against the public header (a child process): host time a call takes to return,
@@ -358,7 +379,7 @@ def main():
             hl = torch.zeros(b_rows, dtype=torch.float32, device=device)
             torch.cuda.synchronize()
             n_h = 30
-            ms_head = median_ms(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum),
+            ms_head = queued_ms(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum),
                                 n_h, 3)
             ms_fused = median_ms(stream, lambda i: sampler.lm_head_sample_rows(
                 hb, wb, lg, tmax, tsum, hp, [i] * b_rows, ho, out_logprobs=hl), n_h, 3)
@@ -406,11 +427,32 @@ def main():
             sampler.synchronize()
             for sc_ in hs:
                 sc_.close()
+            # the same head held in the reference's affine formats (random codes, scales of the
+            # weights' size; lm_head is 4 bits in groups of 64, 8 under --q8 head), f32 logits
+            quant = {}
+            lg32 = torch.zeros(b_rows, vocab, dtype=torch.float32, device=device)
+            for bits in (8, 4):
+                per = 32 // bits
+                q = torch.randint(0, 1 << bits, (vocab, d_model // per, per), device=device, generator=gen,
+                                  dtype=torch.int64)
+                words = (q << (bits * torch.arange(per, device=device, dtype=torch.int64))).sum(dim=2)
+                words = torch.where(words >= 2 ** 31, words - 2 ** 32, words).to(torch.int32).contiguous()
+                del q
+                sc = (torch.rand(vocab, d_model // 64, device=device, generator=gen) + 0.5) * (4.0 / (1 << bits) / d_model ** 0.5)
+                bi = -sc * (1 << bits) / 2
+                qw = LS.QuantWeights(words, sc.to(torch.bfloat16), bi.to(torch.bfloat16), 64, bits)
+                ms_q = queued_ms(stream, lambda i: sampler.lm_head(hb, qw, [0.8] * b_rows, lg32, tmax, tsum), n_h, 3)
+                code_bytes = vocab * d_model * bits / 8 + 2 * vocab * (d_model // 64) * 2
+                quant[f"q{bits}_g64"] = {"head_us": ms_q * 1e3, "weight_GBs": code_bytes / (ms_q * 1e-3) / 1e9,
+                                         "TFLOPs": 2.0 * b_rows * d_model * vocab / (ms_q * 1e-3) / 1e12}
+                del words, qw
+            ms_f32 = queued_ms(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg32, tmax, tsum), n_h, 3)
+            del lg32
             # for reference only: the library's GEMM (torch.matmul, hipBLASLt) on the same
             # operands, bf16 in and out, without the summaries the head's epilogue leaves
             ref_out = torch.empty(b_rows, vocab, dtype=torch.bfloat16, device=device)
             with torch.cuda.stream(stream):
-                ms_lib = median_ms(stream, lambda i: torch.matmul(hb, wb.t(), out=ref_out), n_h, 3)
+                ms_lib = queued_ms(stream, lambda i: torch.matmul(hb, wb.t(), out=ref_out), n_h, 3)
             del ref_out
             flops = 2.0 * b_rows * d_model * vocab
             head[f"b{b_rows}"] = {
@@ -420,7 +462,10 @@ def main():
                 "head_frac_of_mfma_peak": flops / (ms_head * 1e-3) / 1e12 / 2500.0,
                 "head_weight_GBs": vocab * d_model * 2 / (ms_head * 1e-3) / 1e9,
                 "library_gemm_us": ms_lib * 1e3,
-                "timing": f"median of {n_h} single launches",
+                "timing": f"the producers alone: per launch over {n_h} queued back to back, best of 3; "
+                          f"head_plus_draws_us: median of {n_h} single calls",
+                "head_f32_logits_us": ms_f32 * 1e3,
+                "quantised_heads_f32_logits": quant,
                 "head_plus_draws_us": ms_fused * 1e3,
                 "draws_from_summaries_us": us_tiled,
                 "draws_from_rows_us": us_rows,

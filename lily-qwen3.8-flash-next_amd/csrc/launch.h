@@ -40,6 +40,15 @@ hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t 
                                uint32_t vocab, const float* c2_of_row, void* logits,
                                uint64_t logits_stride, float* tile_max, float* tile_sum, bool out_f32,
                                const HeadWeights& wq);
+// The same over codes for up to 16 rows in the reference's form for few rows (the codes are not
+// turned into weights: scale * sum(q * x) + bias * sum(x) per group, f32 logits); `serves` says
+// whether a shape can take it (groups of 64 or more, operands within 4 GB).
+bool lm_head_codes_serves(uint32_t rows, uint32_t d, uint32_t vocab, uint64_t hidden_stride, uint64_t weight_stride,
+                          const HeadWeights& wq);
+hipError_t launch_lm_head_codes(hipStream_t stream, const void* hidden, uint64_t hidden_stride, const void* weight,
+                                uint64_t weight_stride, uint32_t rows, uint32_t d, uint32_t vocab,
+                                const float* c2_of_row, void* logits, uint64_t logits_stride, float* tile_max,
+                                float* tile_sum, const HeadWeights& wq);
 // The draw of `rows` rows of cfg.table from the summaries ([.., tiles] each) and the few tiles of
 // the logits (bf16 or f32) that matter; tile_row[r] = the summaries' row of table row r; served[r] is set
 // for rows under penalties (1 = drawn, 0 = declined: the row is better read whole).

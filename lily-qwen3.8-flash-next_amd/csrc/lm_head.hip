@@ -68,7 +68,8 @@ struct HeadTile {
 // WBITS 4 / 8: the weights are the reference's affine codes (QuantWeights, src/weights.rs:27-36:
 // u32 words of eight 4-bit or four 8-bit codes, low code first, a bf16 scale and bias per group
 // of a row), turned into bf16 as dequant_q4_bf16 / dequant_q8_bf16 turn them (w = q * scale +
-// bias in f32, rounded to bf16: src/kernels/metal/quant.metal:179-233) on their way into LDS;
+// bias in f32 - here one fused operation -, rounded to bf16: src/kernels/metal/quant.metal:179-233)
+// on their way into LDS;
 // `weight` then points at the codes, weight_stride counts words, and a row has
 // (d >> group_shift) groups.  (Tiles whose loads pass through registers only.)
 struct HeadQuant {
@@ -165,19 +166,26 @@ k_lm_head_bf16(const uint16_t* __restrict__ hidden, uint64_t hidden_stride,
             }
         }
     };
-    // eight codes and their group's (scale, bias) as eight bf16 weights: q * scale + bias in f32
-    // (a product and a sum, each rounded), rounded to bf16 (nearest even)
+    // eight codes and their group's (scale, bias) as eight bf16 weights: q * scale + bias as one
+    // fused f32 operation (the exact value rounded once), then to bf16 (nearest even) two at a
+    // time by the hardware's conversion
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
     auto dequantised = [&](const w32x4& c) -> w32x4 {
         const float sc = __builtin_bit_cast(float, c.z << 16), bi = __builtin_bit_cast(float, c.z & 0xffff0000u);
-        uint32_t h[8];
+        uint32_t out[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t q = WBITS == 8 ? (((j < 4 ? c.x : c.y) >> (8 * (j & 3))) & 0xffu) : ((c.x >> (4 * j)) & 0xfu);
-            const float f = (float)q * sc + bi;
-            const uint32_t u = __builtin_bit_cast(uint32_t, f);
-            h[j] = (u & 0x7fffffffu) > 0x7f800000u ? ((u >> 16) | 0x40u) : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+        for (int p = 0; p < 4; ++p) {
+            f32x2 f;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int j = 2 * p + e;
+                const uint32_t q = WBITS == 8 ? (((j < 4 ? c.x : c.y) >> (8 * (j & 3))) & 0xffu) : ((c.x >> (4 * j)) & 0xfu);
+                f[e] = __builtin_fmaf((float)q, sc, bi);
+            }
+            out[p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
         }
-        return w32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+        return w32x4{out[0], out[1], out[2], out[3]};
     };
     // (`real` false: a step past the end of d, run so that every pass of the loop is alike -
     // the hidden rows are staged as zeros and add nothing)
@@ -572,6 +580,10 @@ hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t 
         // whose loads pass through registers, whatever the number of rows
         if (!out_f32 || (wq.bits != 4u && wq.bits != 8u)) {
             return hipErrorInvalidValue;
+        }
+        if (lm_head_codes_serves(rows, d, vocab, hidden_stride, weight_stride, wq)) {
+            return launch_lm_head_codes(stream, hidden, hidden_stride, weight, weight_stride, rows, d, vocab,
+                                        c2_of_row, logits, logits_stride, tile_max, tile_sum, wq);
         }
 #define LILY_HEAD_Q(TILE)                                                                           \
     (wq.bits == 8u ? launch_head_shape<TILE, true, 8>(LILY_HEAD_ARGS)                               \

@@ -412,15 +412,16 @@ def test_sums_formed_at_another_temperature_are_not_used(sampler):
 
 
 def _f32_bound(h, w):
-    """What the f32 accumulation of d products may differ from the f64 product by."""
+    """What the f32 accumulation of d products may differ from the f64 product by (w: the
+    magnitudes that are summed)."""
     return (h.double().abs() @ w.double().abs().T).cpu().numpy() * 2.0 ** -21 + 1e-6
 
 
-def _check_f32_product(h, w, logits, tmax, tsum, temps):
+def _check_f32_product(h, w, logits, tmax, tsum, temps, summed=None):
     rows, vocab = logits.shape
     got = logits.cpu().numpy()
     ref = (h.double() @ w.double().T).cpu().numpy()
-    tol = _f32_bound(h, w)
+    tol = _f32_bound(h, w if summed is None else summed)
     assert np.all(np.abs(got - ref) <= tol), float(np.max(np.abs(got - ref) - tol))
     tiles = tmax.shape[1]
     g = np.pad(got, ((0, 0), (0, tiles * TILE - vocab)), constant_values=-np.inf).reshape(rows, tiles, TILE)
@@ -474,8 +475,11 @@ def test_f32_logits_and_draws_from_their_summaries(sampler, rows, d, vocab):
 
 
 def _quantised(rng, vocab, d, bits, group):
-    """Random affine weights in the reference's layout and what dequant_q4/q8_bf16 makes of them
-    (src/kernels/metal/quant.metal:179-233): q * scale + bias in f32, rounded to bf16."""
+    """Random affine weights in the reference's layout; what dequant_q4/q8_bf16 makes of them
+    (src/kernels/metal/quant.metal:179-233: q * scale + bias in f32 (fused), rounded to bf16), the
+    weights themselves (f64: what gemv_q4/q8_bf16_f32out multiply by, quant.metal:8-60 and
+    130-176) and the magnitudes the few-row form sums in f32 (4-bit codes enter as 128 + q and the
+    128 leaves with the bias)."""
     q = rng.integers(0, 1 << bits, (vocab, d)).astype(np.uint32)
     scales = W.to_bf16_bits(rng.uniform(0.5, 1.5, (vocab, d // group)).astype(np.float32) * (2.0 / (1 << bits)) / np.sqrt(d))
     biases = W.to_bf16_bits(-W.bf16_bits_to_f32(scales) * np.float32((1 << bits) / 2) +
@@ -486,25 +490,34 @@ def _quantised(rng, vocab, d, bits, group):
         words |= q[:, j::per] << np.uint32(bits * j)
     s = np.repeat(W.bf16_bits_to_f32(scales), group, axis=1)
     b = np.repeat(W.bf16_bits_to_f32(biases), group, axis=1)
-    prod = (q.astype(np.float32) * s).astype(np.float32)
-    dense = W.to_bf16_bits((prod + b).astype(np.float32))
+    # (one fused operation: the exact q * s + b rounded once to f32 - exact in f64, whose 53 bits
+    # hold an 8-bit code times an 8-bit scale plus a bias of like magnitude)
+    exact = q.astype(np.float64) * s.astype(np.float64) + b.astype(np.float64)
+    dense = W.to_bf16_bits(exact.astype(np.float32))
+    off = 128.0 if bits == 4 else 0.0
+    summed = (q + off) * s.astype(np.float64) + np.abs(b.astype(np.float64) - off * s)
     t = lambda a, dt: torch.from_numpy(a.view(np.int16) if dt is torch.bfloat16 else a.view(np.int32)).to(dev())
     qw = LS.QuantWeights(t(words, torch.int32), t(scales, torch.bfloat16).view(torch.bfloat16),
                          t(biases, torch.bfloat16).view(torch.bfloat16), group, bits)
-    return qw, torch.from_numpy(dense.view(np.int16)).to(dev()).view(torch.bfloat16)
+    return (qw, torch.from_numpy(dense.view(np.int16)).to(dev()).view(torch.bfloat16),
+            torch.from_numpy(exact).to(dev()), torch.from_numpy(summed).to(dev()))
 
 
 @pytest.mark.parametrize("bits,group", [(4, 64), (8, 64), (4, 32), (8, 128)])
-@pytest.mark.parametrize("rows", [3, 40, 100, 300])
+@pytest.mark.parametrize("rows", [1, 3, 16, 17, 40, 100, 300])
 def test_heads_of_affine_codes(sampler, bits, group, rows):
     """The reference's quantised head formats (QuantWeights, src/weights.rs:27-36; lm_head is 4 bits
-    in groups of 64, 8 under --q8 head): logits against the f64 product of the hidden rows with
-    the weights as dequant_q4/q8_bf16 give them, for every tile shape the codes pass through;
-    greedy rows drawn by the same call pick the oracle's token on the stored logits."""
-    d, vocab = 256, 2000 + 8 * bits
+    in groups of 64, 8 under --q8 head).  Up to 16 rows of groups of 64 or more take the
+    reference's form for few rows - the codes are not turned into weights - and are held against
+    the f64 product with the affine weights themselves; the others against the f64 product with
+    the weights as dequant_q4/q8_bf16 give them, for every tile shape the codes pass through.
+    Greedy rows drawn by the same call pick the oracle's token on the stored logits.  (d = 1280:
+    five or ten stages of the few-row form, which walks them three at a time.)"""
+    d, vocab = 1280, 2000 + 8 * bits
     rng = np.random.default_rng(1000 * bits + group + rows)
     hidden = rng.normal(0, 1, (rows, d)).astype(np.float32)
-    qw, dense = _quantised(rng, vocab, d, bits, group)
+    qw, dense, exact, summed = _quantised(rng, vocab, d, bits, group)
+    few = rows <= 16 and group >= 64 and (d // group) % 2 == 0 and d % (1024 // bits) == 0
     h = _bf16(hidden)
     params_kw = [dict(temperature=0.8, top_k=20, top_p=0.9, seed=r) if r % 2 else dict() for r in range(rows)]
     params = [ls_params(**kw) for kw in params_kw]
@@ -518,13 +531,16 @@ def test_heads_of_affine_codes(sampler, bits, group, rows):
         sampler, lambda out, lp, di, dc: sampler.lm_head_sample_rows(
             h, qw, logits, tmax, tsum, params, steps, out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
         logits, params_kw, steps)
-    _check_f32_product(h, dense, logits, tmax, tsum, temps)
+    if few:
+        _check_f32_product(h, exact, logits, tmax, tsum, temps, summed=summed)
+    else:
+        _check_f32_product(h, dense, logits, tmax, tsum, temps)
     _check_draws(logits.cpu().numpy(), ids, lps, cand, counts, params_kw, steps)
 
 
 def test_codes_ask_for_f32_logits(sampler):
     rng = np.random.default_rng(5)
-    qw, _ = _quantised(rng, 256, 64, 8, 64)
+    qw, _, _, _ = _quantised(rng, 256, 64, 8, 64)
     h = torch.zeros(2, 64, dtype=torch.bfloat16, device=dev())
     tmax = torch.zeros(2, 2, dtype=torch.float32, device=dev())
     tsum = torch.zeros(2, 2, dtype=torch.float32, device=dev())
