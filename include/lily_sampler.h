@@ -417,9 +417,15 @@ void lily_insertions_clear(lily_insertions_t* q, uint32_t row);
  * `gemv_quant(lm_head, mixed, logits)` + `sample_f32` (src/qwen4exp/model.rs:2959-2966,
  * 4157-4169).  The head is held in bf16 or in one of the reference's affine formats (4- or 8-bit
  * codes with a bf16 scale and bias per group of a row: QuantWeights, src/weights.rs:27-36; its
- * lm_head is 4 bits in groups of 64, or 8 under `--q8 head`), whose weights are what
- * dequant_q4_bf16 / dequant_q8_bf16 make of them (q * scale + bias in f32, rounded to bf16:
- * src/kernels/metal/quant.metal:179-233).  logits[r][v] = sum_i hidden[r][i] * weight[v][i],
+ * lm_head is 4 bits in groups of 64, or 8 under `--q8 head`).  Codes follow the reference's two
+ * forms.  Up to 16 rows - a decode or verify step - take its form for few rows (gemv_q4_bf16 /
+ * gemv_q8_bf16 and their _f32out kinds, src/kernels/metal/quant.metal:8-60 and 130-176): the
+ * codes are not turned into weights, a group's part of a logit is scale * sum(q * x) + bias *
+ * sum(x) with f32 sums, the weight is exactly q * scale + bias.  (Groups of 64 or more, an even
+ * number of them a row, d a multiple of 256 (4 bits) or 128 (8 bits).)  Every other shape takes
+ * its form for batches: the weights are what dequant_q4_bf16 / dequant_q8_bf16 make of the
+ * codes (q * scale + bias in f32, rounded to bf16: src/kernels/metal/quant.metal:179-233), on
+ * their way into the product.  logits[r][v] = sum_i hidden[r][i] * weight[v][i],
  * accumulated in f32 on the matrix cores and stored as f32 (what the reference's sampler reads,
  * src/kernels/sample.rs:263) or rounded to bf16 (nearest even).  Beside the logits the producer leaves,
  * for every LILY_LOGIT_TILE_COLS columns of every row, the largest value and the sum of
