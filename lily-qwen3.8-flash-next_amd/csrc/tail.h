@@ -424,26 +424,57 @@ __device__ __forceinline__ void tail(const RowArgs& a, uint32_t vocab, uint32_t 
     }
     __syncthreads();
     TAIL_MARK(9);
-    // The reference's left-to-right f32 sums: one wave runs the chain of additions, 64
-    // candidates at a time with a candidate per lane, and keeps every prefix.  Each step adds
-    // the lane's value to the running sum of the lane below (a shift by one lane across the
-    // whole wave; lane 0 has no lane below and keeps what it has): after step j the lanes up
-    // to j hold their final prefix, which further steps only reproduce.  The row total is
-    // the last prefix, and the sum the reference holds before rank r is the prefix of rank
-    // r - 1: the cut by top-p and min-p and the inverse-CDF pick then are searches every
-    // thread takes part in.
+    // The reference's left-to-right f32 sums, by one wave, 64 candidates at a time with a
+    // candidate per lane; every prefix is kept.  The row total is the last prefix, and the sum
+    // the reference holds before rank r is the prefix of rank r - 1: the cut by top-p and min-p
+    // and the inverse-CDF pick then are searches every thread takes part in.
+    //
+    // While the running sum S stays inside one binade it is an integer m in units of its last
+    // place u, and adding p <= S rounds to m + floor(p / u) + (frac(p / u) > 1/2): integer
+    // additions, which a wave sums in six data-parallel moves, exactly.  (p / u, its integer
+    // part and its fraction are exact in f32: u is a power of two and p has no more bits than
+    // S.)  A block of 64 in which some fraction is exactly 1/2 (the rounding then depends on
+    // m's parity) or the sum leaves its binade - and the first block, whose sum starts at 0 -
+    // is added the slow way: a chain of 63 additions, each step adding the lane's value to the
+    // running sum of the lane below (a shift by one lane across the whole wave; lane 0 has no
+    // lane below and keeps what it has), after which every lane holds its final prefix.  The
+    // candidates' weights are at most 1 and the first is 1, so the sum crosses at most ten
+    // binades and a peaked row none.  (Restarting inside a block at the lane that leaves the
+    // binade, instead of giving the block to the chain, was slower: a round of the exact form
+    // costs a third of a chain, and a flat row then takes 25 rounds.)
     if (tid < 64u) {
         float carry = 0.0f;
         for (uint32_t r0 = 0; r0 < k; r0 += 64u) {
             const uint32_t i = r0 + tid;
             const float p = i < k ? sh.prob[i] : 0.0f;
-            float run = carry + p;  // final in lane 0
+            float run;
+            bool done = false;
+            const uint32_t sbits = lilym_f32_bits(carry), sexp = (sbits >> 23) & 0xffu;
+            // (a normal, positive sum whose last place and its inverse are normal numbers too)
+            if ((int32_t)sbits > 0 && sexp >= 24u && sexp <= 253u) {
+                const float inv_u = lilym_bits_f32((277u - sexp) << 23);   // 2^(23 - e)
+                const float u = lilym_bits_f32((sexp - 23u) << 23);        // 2^(e - 23)
+                const uint32_t m0 = (sbits & 0x7fffffu) | 0x800000u;
+                const float q = p * inv_u;
+                const uint32_t n = (uint32_t)q;
+                const float frac = q - (float)n;
+                const bool fits = p >= 0.0f && p <= carry;
+                const uint32_t m = m0 + wave_scan_u32(n + (frac > 0.5f ? 1u : 0u));
+                const uint32_t last = (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+                if (__ballot(frac == 0.5f || !fits) == 0ull && last < 0x1000000u) {
+                    run = (float)m * u;
+                    done = true;
+                }
+            }
+            if (!done) {
+                run = carry + p;  // final in lane 0
 #pragma unroll
-            for (int j = 1; j < 64; ++j) {
-                // Two idle cycles between a lane's write and the neighbour's read of it.
-                asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %1 wave_shr:1 row_mask:0xf bank_mask:0xf"
-                             : "+v"(run)
-                             : "v"(p));
+                for (int j = 1; j < 64; ++j) {
+                    // Two idle cycles between a lane's write and the neighbour's read of it.
+                    asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %1 wave_shr:1 row_mask:0xf bank_mask:0xf"
+                                 : "+v"(run)
+                                 : "v"(p));
+                }
             }
             if (i < k) {
                 sh.cum[i] = run;

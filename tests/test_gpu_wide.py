@@ -73,6 +73,34 @@ def test_plain_rows_of_many_candidates(sampler, bf16, use_plan):
             _check_logprob(r.logprobs[i], d.logprob, (k, i))
 
 
+def test_prefix_sums_that_leave_their_binade_and_round_on_ties(sampler):
+    """The left-to-right f32 sums of up to 1 024 weights are formed 64 at a time by integer
+    additions while the running sum stays in one binade and no weight lies exactly half a last
+    place above a multiple of it, and by the chain of real additions otherwise.  Rows that force
+    either way: hundreds of ids at the row's largest value (weights of exactly 1: the sum walks
+    through nine binades on integers), a flat row (the sum crosses a binade every few blocks and
+    weights within a few binades of the sum tie often), a peaked row (one binade, no ties after
+    the first block), and steps of one bf16 ulp (weights in a handful of exact ratios).  The
+    kept counts and the probabilities are bit-exact against the oracle, so is every draw."""
+    rng = np.random.default_rng(4242)
+    vocab = 151_936
+    x = np.empty((4, vocab), dtype=np.float32)
+    x[0] = rng.normal(0, 1, vocab)
+    x[0, rng.choice(vocab, 700, replace=False)] = 9.0
+    x[1] = rng.normal(0, 0.05, vocab)
+    x[2] = rng.normal(0, 1, vocab)
+    x[2, 77] = 30.0
+    x[3] = np.round(rng.normal(0, 3, vocab) * 8) / 8
+    for trial, (t, top_p) in enumerate(((1.0, 0.999), (0.7, 0.9), (1.3, 0.97))):
+        kw = [dict(temperature=t, top_k=0, top_p=top_p, seed=900 + r) for r in range(4)]
+        r, stats = _with_stats(sampler, lambda: run_rows(sampler, x, kw, [trial] * 4, logprobs=True))
+        assert stats[0] == 0 and stats[1] + stats[2] == 4, stats
+        for i in range(4):
+            d = O.sample(x[i], None, o_params(**kw[i]), trial, want_logprob=True)
+            check_row_against_oracle(r, i, d)
+            _check_logprob(r.logprobs[i], d.logprob, (trial, i))
+
+
 def test_penalised_rows_over_decode_steps(sampler):
     """Lowering penalties (repetition >= 1, presence and frequency >= 0) on the ids that matter
     most: the lanes' maxima, the row's sum and the candidates are taken on penalised worth.
