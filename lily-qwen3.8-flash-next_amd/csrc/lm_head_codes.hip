@@ -49,7 +49,7 @@ inline size_t codes_lds_bytes(uint32_t groups) { return (size_t)RING_BYTES + (si
 // loads of 1 KB (two a wave, eight whole lines each), AHEAD stages on their way in registers,
 // written to LDS one pass before they are multiplied.  (A lane's own operand would be 8 bytes of
 // each of 16 rows: the 64 lines such a load touches, not its bytes, bounded an earlier form at a
-// fifth of the memory's speed.  Loads that write LDS themselves keep only what LDS holds in
+// seventh of the memory's speed.  Loads that write LDS themselves keep only what LDS holds in
 // flight, which is too little here.)  The stage's 256 (4-bit) or 128 (8-bit) values of d are
 // split among four waves, the 128 columns between two; the four partial tiles are added through
 // LDS at the end.  The scales and biases of the whole tile are brought into LDS once, ahead of
