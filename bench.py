@@ -424,6 +424,9 @@ def main():
                 lg, tmax, tsum, pp, [99] * b_rows, ho, scratch=hs, out_logprobs=hl))
             us_rows_pen = behind_a_head(lambda i: sampler.sample_rows(lg, pp, [i] * b_rows, ho, scratch=hs,
                                                                      out_logprobs=hl))
+            # ... and config 5 in full as one call: the head and the penalised draws
+            ms_fused_pen = median_ms(stream, lambda i: sampler.lm_head_sample_rows(
+                hb, wb, lg, tmax, tsum, pp, [i] * b_rows, ho, scratch=hs, out_logprobs=hl), n_h, 3)
             sampler.synchronize()
             for sc_ in hs:
                 sc_.close()
@@ -467,6 +470,7 @@ def main():
                 "head_f32_logits_us": ms_f32 * 1e3,
                 "quantised_heads_f32_logits": quant,
                 "head_plus_draws_us": ms_fused * 1e3,
+                "head_plus_penalised_draws_us": ms_fused_pen * 1e3,
                 "draws_from_summaries_us": us_tiled,
                 "draws_from_rows_us": us_rows,
                 "penalised_draws_from_summaries_us": us_tiled_pen,

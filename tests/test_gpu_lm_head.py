@@ -334,6 +334,58 @@ def test_rows_under_lowering_penalties_are_drawn_from_summaries(sampler):
         scratch[r].close()
 
 
+def test_a_batch_of_penalised_rows_through_the_fused_call(sampler):
+    """1 024 rows under config 5's draw settings (k 64, top-p 0.9, T 0.8, penalties that only
+    lower, a 2 048-id history that holds the row's best ids, a log-probability) through the one
+    call that runs the head and draws every row: ids, kept counts and log-probabilities against
+    the oracle on the stored logits, the counts as the oracle leaves them.  Most rows are drawn
+    from the summaries, the rest from their logits by the same call."""
+    rows, d, vocab = 1024, 128, 40_000 + 72   # (rows of whole 16 bytes, a last tile of 8 columns)
+    rng = np.random.default_rng(1024)
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=50, gain=8.0)
+    params_kw = [dict(temperature=0.8, top_k=64, top_p=0.9, seed=7000 + r, repetition_penalty=1.1,
+                      presence_penalty=0.2, frequency_penalty=0.1) for r in range(rows)]
+    params = [ls_params(**kw) for kw in params_kw]
+    h, w = _bf16(hidden), _bf16(weight)
+    tiles = (vocab + TILE - 1) // TILE
+    logits = torch.zeros(rows, vocab, dtype=torch.bfloat16, device=dev())
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    # the histories need the rows' best ids: a first pass of the producer alone
+    sampler.lm_head(h, w, [0.8] * rows, logits, tmax, tsum)
+    sampler.synchronize()
+    stored = _bits(logits.contiguous())
+    best = torch.topk(logits.float(), 12, dim=1).indices.cpu().numpy().astype(np.int32)
+    scratch, hist_counts = [], []
+    for r in range(rows):
+        hh = np.concatenate([rng.integers(0, vocab, 2036).astype(np.int32), best[r]])
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(hh).to(dev()))
+        scratch.append(sc)
+        hist_counts.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+    steps = [2] * rows
+    out = torch.full((rows,), -1, dtype=torch.int32, device=dev())
+    lp = torch.zeros(rows, dtype=torch.float32, device=dev())
+    dbg_counts = torch.zeros(rows, 2, dtype=torch.int32, device=dev())
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    sampler.set_path_stats(stats)
+    sampler.lm_head_sample_rows(h, w, logits, tmax, tsum, params, steps, out, scratch=scratch,
+                                out_logprobs=lp, dbg_counts=dbg_counts)
+    sampler.synchronize()
+    sampler.set_path_stats(None)
+    assert np.array_equal(_bits(logits.contiguous()), stored), "the same head, the same logits"
+    assert stats.cpu().numpy()[2] == 0, "no row fell back to the exhaustive select"
+    ids, lps, kept = out.cpu().numpy().astype(np.int64), lp.cpu().numpy(), dbg_counts.cpu().numpy()
+    for r in range(rows):
+        dd = O.sample(stored[r], hist_counts[r], o_params(**params_kw[r]), steps[r], want_logprob=True)
+        assert ids[r] == dd.chosen and kept[r, 1] == dd.n_kept, (r, ids[r], dd.chosen, kept[r], dd.n_kept)
+        assert abs(lps[r] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (r, lps[r], dd.logprob)
+    for r in (0, 1, 511, 1023):
+        assert np.array_equal(scratch[r].read_counts().numpy().view(np.uint32), hist_counts[r]), r
+    for sc in scratch:
+        sc.close()
+
+
 def test_the_benchmarked_shape(sampler):
     """1 024 rows x 151 936 ids over d = 4 096, the shape bench.py times: a seeded subset of tiles
     against the f64 product of the same bf16 operands (logits within one bf16 step, tile_max
