@@ -33,6 +33,7 @@ namespace lily {
 // What the two launches share beyond LaunchCfg.
 struct WideArgs {
     Handed<float> lane_max;   // [rows][slices][lanes]
+    Handed<float> slice_bound;   // [rows][slices] a value that k / slices of the slice's lanes reach
     uint32_t lanes;       // values a slice leaves: NT, or NT / 2 (the larger of each pair of lanes)
     uint32_t* count;      // [rows] candidates the row's slices have left so far (0 between launches)
 };
@@ -181,6 +182,7 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
     });
     WIDE_MARK(1);
     const size_t slot = (size_t)row * S + s;
+    const float pair_max = lane_max;
     if (w.lanes == NT) {
         handed_store(w.lane_max, slot * NT + tid, lane_max);
     } else {
@@ -190,6 +192,30 @@ __global__ __launch_bounds__(NT, 4) void k_wide_bound(InlineRows rows_arg, Launc
         lane_max = fmaxf(lane_max, lilym_bits_f32((uint32_t)other));
         if ((tid & 1u) == 0u) {
             handed_store(w.lane_max, slot * (NT / 2) + tid / 2u, lane_max);
+        }
+    }
+    // ... and one value per slice that at least ceil(k / slices) of its lanes reach: in each wave
+    // the ceil(k / (4 * slices))-th largest of the 64 lane maxima (a 16-step ballot search on the
+    // leading 16 bits of the order key, as the streaming select takes its bound), the least of the
+    // four.  The least of a row's slices' values is then reached by k lanes of the row, so by k
+    // values: the second launch takes that as the row's bound without looking at the lanes'
+    // maxima.  F32_LOWEST from a wave with fewer finite lane maxima than that: the second launch
+    // then takes the bound from all the lanes' maxima.
+    {
+        const float whole = pair_max;   // (every lane's own maximum, whatever was stored above)
+        const uint32_t per_wave = (a.k + 4u * S - 1u) / (4u * S);
+        const uint32_t key16 = whole > NEG_INF ? (lilym_order_key(whole) >> 16) : 0u;
+        const uint32_t P = per_wave <= 64u ? wave_kth_key16(key16, per_wave) : 0u;
+        if ((tid & 63u) == 0u) {
+            sh.bound[0][tid >> 6] = P != 0u ? lilym_key_value(P << 16) : F32_LOWEST;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float least = sh.bound[0][0];
+            for (int i = 1; i < NWAVE; ++i) {
+                least = fminf(least, sh.bound[0][i]);
+            }
+            handed_store(w.slice_bound, slot, least);
         }
     }
     if (want_lse) {
@@ -289,7 +315,17 @@ __global__ __launch_bounds__(NT, 4) void k_wide_draw(InlineRows rows_arg, Launch
     const uint32_t step = a.step + cfg.step_delta;
     const bool want_lse = LSE && a.out_logprob != nullptr;
     const bool pen = (a.flags & F_PEN) != 0;   // (of the kind that only lowers: the host sees to it)
-    const float bound = wide_bound_of(w, row, S, a.k, sh);   // of the values' worth under the penalties
+    // The bound (of the values' worth under the penalties): the least of the slices' values, which
+    // k lanes of the row reach; where a wave of some slice had too few finite lane maxima to name
+    // one, the k-th largest of all the lanes' maxima.  Every wave reads the slices' values itself.
+    float bound;
+    {
+        const float mine = lane < S ? handed_load(w.slice_bound, (size_t)row * S + lane) : __builtin_huge_valf();
+        bound = -wave_max_dpp(-mine);
+    }
+    if (!(bound > F32_LOWEST)) {   // (the same in every wave)
+        bound = wide_bound_of(w, row, S, a.k, sh);
+    }
     Geo<DT> g;
     g.init(a.logits, vocab, s, S);
     uint64_t* cand = dyn_lds;
@@ -432,6 +468,7 @@ hipError_t launch_rows_wide(hipStream_t stream, int dtype, bool lse, uint32_t ro
     cfg.cand_cap = MERGE_CAP;
     WideArgs w;
     w.lane_max = Handed<float>{lane_max};
+    w.slice_bound = Handed<float>{lane_max + (size_t)rows * cfg.slices * NT};   // (behind the lanes' maxima)
     w.lanes = (uint64_t)cfg.slices * (NT / 2) >= 4ull * cfg.ws_k ? NT / 2 : NT;
     w.count = count;
     const bool inl = inline_rows != nullptr;

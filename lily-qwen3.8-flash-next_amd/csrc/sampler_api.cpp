@@ -383,7 +383,7 @@ uint32_t wide_slices(const lily_sampler* s, const RowArgs* rows, uint32_t n, int
     if ((uint64_t)n * MERGE_CAP > s->ws_slots) {   // a row's list of candidates: MERGE_CAP slots
         return 0;
     }
-    const uint64_t by_max = (uint64_t)WIDE_FLOATS / ((uint64_t)n * 256u);
+    const uint64_t by_max = (uint64_t)WIDE_FLOATS / ((uint64_t)n * 257u);   // 256 lane maxima and one value a slice
     sl = sl > by_max ? (uint32_t)by_max : sl;
     // the bound is the k-th largest of slices x 256 lane maxima: with twice k of them it is the
     // median of the lanes' maxima, which about 1.4 k values reach on rows of Gaussian logits
