@@ -34,6 +34,8 @@ struct HeadWeights {
     const void* scales = nullptr;
     const void* biases = nullptr;
     uint32_t group_shift = 6;   // log2 of the group size
+    unsigned long long* trace = nullptr;   // diagnostic stamps, [workgroups][8] (builds with -DLILY_HEAD_TRACE)
+    unsigned long long trace_words = 0;
 };
 hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
                                const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,

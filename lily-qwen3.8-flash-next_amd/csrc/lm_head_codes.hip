@@ -66,7 +66,16 @@ k_lm_head_codes(const uint16_t* __restrict__ hidden, uint64_t hidden_stride, con
                 uint64_t weight_stride, uint32_t rows, uint32_t d, uint32_t vocab,
                 const float* __restrict__ c2_of_row, float* __restrict__ logits, uint64_t logits_stride,
                 float* __restrict__ tile_max, float* __restrict__ tile_sum, uint32_t tiles_per_row,
-                const uint16_t* __restrict__ scales, const uint16_t* __restrict__ biases, uint32_t group_shift) {
+                const uint16_t* __restrict__ scales, const uint16_t* __restrict__ biases, uint32_t group_shift,
+                unsigned long long* trace) {
+    // Diagnostic stamps, compiled in with -DLILY_HEAD_TRACE: [workgroup][8] device-clock values
+    // (0 start, 1 scales and first stage written, 2 past the barrier, 3 loop done, 4 end).
+#ifdef LILY_HEAD_TRACE
+#define HEAD_MARK(i) do { if (trace != nullptr && threadIdx.x == 0) { trace[(size_t)blockIdx.x * 8 + (i)] = wall_clock64(); } } while (0)
+#else
+#define HEAD_MARK(i)
+#endif
+    HEAD_MARK(0);
     constexpr int STEPS = WBITS == 4 ? 2 : 1;          // products over 32 values a wave makes per stage and block
     constexpr uint32_t STAGE_K = 128u * 8u / WBITS;    // values of d in a stage
     constexpr uint32_t WAVE_K = STAGE_K / 4u;          // ... of which a wave multiplies these
@@ -249,7 +258,9 @@ k_lm_head_codes(const uint16_t* __restrict__ hidden, uint64_t hidden_stride, con
             }
         }
     }
+    HEAD_MARK(1);
     __syncthreads();   // (the scales and stage 0 are written)
+    HEAD_MARK(2);
     const uint32_t padded = (nstages + AHEAD - 1u) / AHEAD * AHEAD;
     static_assert(AHEAD % 2 == 0, "the halves of LDS alternate within a trip");
     for (uint32_t s0 = 0; s0 < padded; s0 += AHEAD) {
@@ -268,6 +279,7 @@ k_lm_head_codes(const uint16_t* __restrict__ hidden, uint64_t hidden_stride, con
     }
     __syncthreads();
 
+    HEAD_MARK(3);
     // ---- the four partial tiles, added; thread t then holds column t % 128 of the rows
     // 4 * (t / 128) .. + 3.
 #pragma unroll
@@ -342,6 +354,7 @@ k_lm_head_codes(const uint16_t* __restrict__ hidden, uint64_t hidden_stride, con
         tile_max[at] = keep_max;
         tile_sum[at] = keep_max > NEG ? sum : 0.0f;
     }
+    HEAD_MARK(4);
 }
 
 template <int WBITS>
@@ -372,7 +385,8 @@ static hipError_t launch_codes(hipStream_t stream, const void* hidden, uint64_t 
                        static_cast<const uint16_t*>(hidden), hidden_stride, static_cast<const uint32_t*>(weight),
                        weight_stride, rows, d, vocab, c2_of_row, static_cast<float*>(logits), logits_stride,
                        tile_max, tile_sum, tiles_per_row, static_cast<const uint16_t*>(wq.scales),
-                       static_cast<const uint16_t*>(wq.biases), wq.group_shift);
+                       static_cast<const uint16_t*>(wq.biases), wq.group_shift,
+                       wq.trace_words >= (unsigned long long)tiles_per_row * 8u ? wq.trace : nullptr);
     return hipGetLastError();
 }
 

@@ -1950,10 +1950,12 @@ int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* h, uint32_t rows, u
     if (int rc = stage_commit(s, slot, (size_t)rows * 4)) {
         return rc;
     }
+    HeadWeightsOf hw(h);
+    hw.trace = reinterpret_cast<unsigned long long*>(s->phase_trace);
+    hw.trace_words = s->phase_words;
     HIP_TRY(launch_lm_head_bf16(s->stream, h->hidden_dev, h->hidden_stride, h->weight_dev, h->weight_stride,
                                 rows, h->d, vocab, reinterpret_cast<const float*>(s->table_dev), logits_dev,
-                                row_stride, h->tile_max_dev, h->tile_sum_dev, h->logits_f32 != 0u,
-                                HeadWeightsOf(h)));
+                                row_stride, h->tile_max_dev, h->tile_sum_dev, h->logits_f32 != 0u, hw));
     return LILY_OK;
 }
 
