@@ -397,9 +397,11 @@ def main():
                 float((have - want).abs().max())
 
             def behind_a_head(draw, n=4):
-                """GPU time of a draw call: n of them queued while a head launch still runs, so
-                that the host's packing is off the clock."""
-                sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum)
+                """GPU time of a draw call: n of them queued while head launches still run (three
+                for a batch: the mirror packs 1 024 penalised rows for longer than one lasts),
+                so that the host's packing is off the clock."""
+                for _ in range(3 if b_rows > 64 else 1):
+                    sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum)
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
                 for i in range(n):
@@ -451,6 +453,24 @@ def main():
                 del words, qw
             ms_f32 = queued_ms(stream, lambda i: sampler.lm_head(hb, wb, [0.8] * b_rows, lg32, tmax, tsum), n_h, 3)
             del lg32
+            # which way the producer took (a batch goes through hipBLASLt and a pass that forms
+            # the summaries where that library can be opened), and this library's own kernel for
+            # the same batch beside it
+            before = sampler.lm_head_library_calls()
+            sampler.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum)
+            through_library = sampler.lm_head_library_calls() > before
+            ms_own = None
+            if through_library:
+                asked = os.environ.get("LILY_SAMPLER_HEAD")
+                os.environ["LILY_SAMPLER_HEAD"] = "own"
+                own = LS.Sampler(0, stream=stream)
+                if asked is None:
+                    del os.environ["LILY_SAMPLER_HEAD"]
+                else:
+                    os.environ["LILY_SAMPLER_HEAD"] = asked
+                ms_own = queued_ms(stream, lambda i: own.lm_head(hb, wb, [0.8] * b_rows, lg, tmax, tsum), n_h, 3)
+                own.synchronize()
+                own.close()
             # for reference only: the library's GEMM (torch.matmul, hipBLASLt) on the same
             # operands, bf16 in and out, without the summaries the head's epilogue leaves
             ref_out = torch.empty(b_rows, vocab, dtype=torch.bfloat16, device=device)
@@ -464,6 +484,8 @@ def main():
                 "head_TFLOPs": flops / (ms_head * 1e-3) / 1e12,
                 "head_frac_of_mfma_peak": flops / (ms_head * 1e-3) / 1e12 / 2500.0,
                 "head_weight_GBs": vocab * d_model * 2 / (ms_head * 1e-3) / 1e9,
+                "head_form": "hipBLASLt GEMM + k_head_summaries" if through_library else "own kernel",
+                "head_own_kernel_us": ms_own * 1e3 if ms_own is not None else ms_head * 1e3,
                 "library_gemm_us": ms_lib * 1e3,
                 "timing": f"the producers alone: per launch over {n_h} queued back to back, best of 3; "
                           f"head_plus_draws_us: median of {n_h} single calls",

@@ -466,6 +466,20 @@ uint32_t lily_lm_head_tiles(uint32_t vocab);
 int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* head, uint32_t rows, uint32_t vocab,
                       const float* temperatures, void* logits_dev, uint64_t row_stride);
 
+/* A batch of many rows (from 129 on; from 256 on over codes) is a plain matrix product of the
+ * kind the platform's GEMM library (hipBLASLt) is tuned for: where a program can open that library
+ * by its name (libhipblaslt.so.1: it is opened at run time, never linked) and the library has an
+ * algorithm for the shape, the producer forms the logits through it - codes are first turned
+ * into bf16 weights, all of them, in memory the call keeps (vocab x d x 2 bytes a device and
+ * stream; the reference does the same for a batch) - and the summaries by a pass over the stored
+ * logits; otherwise, and for fewer rows, by this library's own kernels.  Same values to the
+ * producer's bar either way (the order of the f32 additions differs).  The first call of a shape
+ * allocates (workspace, descriptors): make it outside a stream capture.  Environment,
+ * read at lily_sampler_create: LILY_SAMPLER_HEAD=own (never the library), =library (every
+ * batch it takes) or a number of rows to begin at.  lily_lm_head_library_calls: how many of this
+ * sampler's producer calls went through the library so far. */
+uint64_t lily_lm_head_library_calls(const lily_sampler_t* s);
+
 /* The draws alone: batch->logits_dev (bf16 or f32, rows at multiples of 16 bytes) and the summaries must
  * come from one producer call made with the temperatures of batch->params.  Where the summaries
  * are those of this sampler's last producer call, a row that asks for a log-probability at

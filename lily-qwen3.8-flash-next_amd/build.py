@@ -40,6 +40,7 @@ def units():
     out.append(("static_entry.hip", "static_entry.o", []))
     out.append(("lm_head.hip", "lm_head.o", []))
     out.append(("lm_head_codes.hip", "lm_head_codes.o", []))
+    out.append(("head_library.hip", "head_library.o", []))
     out.append(("rows_tiles.hip", "rows_tiles.o", []))
     out.append(("rows_wide.hip", "rows_wide.o", []))
     out.append(("sampler_api.cpp", "sampler_api.o", []))

@@ -36,6 +36,10 @@ struct HeadWeights {
     uint32_t group_shift = 6;   // log2 of the group size
     unsigned long long* trace = nullptr;   // diagnostic stamps, [workgroups][8] (builds with -DLILY_HEAD_TRACE)
     unsigned long long trace_words = 0;
+    // batches of at least this many rows go through the vendor's GEMM library where it is present
+    // and takes the shape, followed by the pass that forms the summaries (0: never)
+    uint32_t library_rows = 0;
+    unsigned long long* library_calls = nullptr;   // counts the calls that went that way
 };
 hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t hidden_stride,
                                const void* weight, uint64_t weight_stride, uint32_t rows, uint32_t d,
@@ -51,6 +55,18 @@ hipError_t launch_lm_head_codes(hipStream_t stream, const void* hidden, uint64_t
                                 uint64_t weight_stride, uint32_t rows, uint32_t d, uint32_t vocab,
                                 const float* c2_of_row, void* logits, uint64_t logits_stride, float* tile_max,
                                 float* tile_sum, const HeadWeights& wq);
+// The batch form through the vendor's GEMM library, opened by name at run time: the product alone
+// (codes are turned into bf16 weights first, in memory this call keeps per device and stream);
+// hipErrorNotSupported where the library is absent or has no algorithm for the shape - the
+// caller then runs its own kernel.  launch_head_summaries: tile_max / tile_sum of stored logits.
+constexpr uint32_t HEAD_LIBRARY_MAX_TILES = 2048;   // summaries a row that launch_head_summaries takes
+bool head_library_present();
+hipError_t launch_head_library(hipStream_t stream, const void* hidden, uint64_t hidden_stride, const void* weight,
+                               uint64_t weight_stride, uint32_t rows, uint32_t d, uint32_t vocab, void* logits,
+                               uint64_t logits_stride, bool out_f32, const HeadWeights& wq);
+hipError_t launch_head_summaries(hipStream_t stream, const void* logits, uint64_t logits_stride, uint32_t rows,
+                                 uint32_t vocab, const float* c2_of_row, float* tile_max, float* tile_sum,
+                                 bool f32);
 // The draw of `rows` rows of cfg.table from the summaries ([.., tiles] each) and the few tiles of
 // the logits (bf16 or f32) that matter; tile_row[r] = the summaries' row of table row r; served[r] is set
 // for rows under penalties (1 = drawn, 0 = declined: the row is better read whole).

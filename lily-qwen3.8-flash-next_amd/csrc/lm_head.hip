@@ -575,6 +575,24 @@ hipError_t launch_lm_head_bf16(hipStream_t stream, const void* hidden, uint64_t 
     typedef HeadTile<1, 2, 1, 64, 3, 3> Tile64;
     typedef HeadTile<2, 2, 2, 64, 3, 2> Tile128;
     typedef HeadTile<2, 4, 2, 32, 2, 2, true> Tile256;
+    // (the pass over the stored logits reads 16-byte pieces: rows that start at multiples of 16 bytes)
+    const bool rows_aligned = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0u &&
+                              (logits_stride * (out_f32 ? 4u : 2u)) % 16u == 0u;
+    if (wq.library_rows != 0u && rows >= wq.library_rows && (wq.bits == 0u || out_f32) && rows_aligned &&
+        (vocab + LILY_TILE_COLS - 1u) / LILY_TILE_COLS <= HEAD_LIBRARY_MAX_TILES) {
+        const hipError_t e = launch_head_library(stream, hidden, hidden_stride, weight, weight_stride, rows, d, vocab,
+                                                 logits, logits_stride, out_f32, wq);
+        if (e == hipSuccess) {
+            if (wq.library_calls != nullptr) {
+                ++*wq.library_calls;
+            }
+            return launch_head_summaries(stream, logits, logits_stride, rows, vocab, c2_of_row, tile_max, tile_sum,
+                                         out_f32);
+        }
+        if (e != hipErrorNotSupported) {
+            return e;
+        }
+    }
     if (wq.bits != 0u) {
         // codes: f32 logits only (what the reference's quantised head produces), and the tiles
         // whose loads pass through registers, whatever the number of rows

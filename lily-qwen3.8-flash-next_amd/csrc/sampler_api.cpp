@@ -72,6 +72,10 @@ struct DeviceScope {
     HIP_TRY(device_scope_.err)
 
 constexpr uint32_t WS_ROWS = 4096;      // rows that may span several workgroups
+// Batches of the logits' producer from this many rows on go through the vendor's GEMM library
+// where it is present (below, this library's own tiles are as fast or faster; over codes the
+// library's way begins with a pass that turns all of them into bf16 weights).
+constexpr uint32_t HEAD_LIBRARY_ROWS = 129, HEAD_LIBRARY_ROWS_CODES = 256;
 constexpr uint32_t WS_SLOTS = 1u << 22; // candidate slots of the workspace (rows x slices x k)
 constexpr uint32_t STAGE_SLOTS = 4;
 constexpr size_t STAGE_ROW_BYTES = sizeof(RowArgs) + 16;   // a staged row: descriptor + three words + slack
@@ -105,6 +109,10 @@ struct lily_sampler {
     uint32_t force_path = 0;
     uint32_t force_slices = 0;
     bool no_wide = false;   // LILY_SAMPLER_WIDE=0: rows of many candidates go the other kernels' way
+    // LILY_SAMPLER_HEAD: batches of this many rows or more are produced through the vendor's GEMM
+    // library ("own": never, "library": every batch it takes, a number: from that many rows on)
+    uint32_t head_library_rows = HEAD_LIBRARY_ROWS, head_library_rows_codes = HEAD_LIBRARY_ROWS_CODES;
+    unsigned long long head_library_calls = 0;   // producer calls that went through the vendor's library
     uint32_t handover = 0;  // LILY_SAMPLER_HANDOVER: 0 = by the launch's size, 1 = strict, 2 = relaxed
     // What the last lily_lm_head_bf16 call of this sampler left: where, and with which exponent
     // scale per row (tile_sum is only good for a log-probability at that scale).
@@ -890,6 +898,10 @@ int lily_sampler_create(int device, void* hip_stream, lily_sampler_t** out) {
     }
     if (const char* p = std::getenv("LILY_SAMPLER_WIDE")) {
         s->no_wide = std::atoi(p) == 0;
+    }
+    if (const char* p = std::getenv("LILY_SAMPLER_HEAD")) {
+        s->head_library_rows = std::strcmp(p, "own") == 0 ? 0u : std::strcmp(p, "library") == 0 ? 1u : (uint32_t)std::atoi(p);
+        s->head_library_rows_codes = s->head_library_rows;
     }
     if (const char* p = std::getenv("LILY_SAMPLER_HANDOVER")) {
         s->handover = std::strcmp(p, "strict") == 0 ? 1u : std::strcmp(p, "relaxed") == 0 ? 2u : 0u;
@@ -1764,10 +1776,12 @@ int check_head(const lily_lm_head* h, uint32_t rows, uint32_t vocab, const void*
 }
 
 struct HeadWeightsOf : HeadWeights {
-    explicit HeadWeightsOf(const lily_lm_head* h);
+    HeadWeightsOf(const lily_sampler* s, const lily_lm_head* h);
 };
-HeadWeightsOf::HeadWeightsOf(const lily_lm_head* h) {
+HeadWeightsOf::HeadWeightsOf(const lily_sampler* s, const lily_lm_head* h) {
     HeadWeights& w = *this;
+    w.library_rows = h->weight_bits != 0u ? s->head_library_rows_codes : s->head_library_rows;
+    w.library_calls = const_cast<unsigned long long*>(&s->head_library_calls);
     w.bits = h->weight_bits;
     w.scales = h->scales_dev;
     w.biases = h->biases_dev;
@@ -1900,7 +1914,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
                                     h->weight_stride, rows, h->d, b->vocab,
                                     reinterpret_cast<const float*>(dev + c2_off),
                                     const_cast<void*>(b->logits_dev), b->row_stride, h->tile_max_dev,
-                                    h->tile_sum_dev, h->logits_f32 != 0u, HeadWeightsOf(h)));
+                                    h->tile_sum_dev, h->logits_f32 != 0u, HeadWeightsOf(s, h)));
     }
     uint32_t* served_dev = reinterpret_cast<uint32_t*>(const_cast<char*>(dev) + served_off);
     if (served != 0) {
@@ -1927,6 +1941,10 @@ uint32_t lily_lm_head_tiles(uint32_t vocab) {
     return (vocab + LILY_LOGIT_TILE_COLS - 1u) / LILY_LOGIT_TILE_COLS;
 }
 
+uint64_t lily_lm_head_library_calls(const lily_sampler_t* s) {
+    return s != nullptr ? s->head_library_calls : 0u;
+}
+
 int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* h, uint32_t rows, uint32_t vocab,
                       const float* temperatures, void* logits_dev, uint64_t row_stride) {
     if (s == nullptr) {
@@ -1950,7 +1968,7 @@ int lily_lm_head_bf16(lily_sampler_t* s, const lily_lm_head* h, uint32_t rows, u
     if (int rc = stage_commit(s, slot, (size_t)rows * 4)) {
         return rc;
     }
-    HeadWeightsOf hw(h);
+    HeadWeightsOf hw(s, h);
     hw.trace = reinterpret_cast<unsigned long long*>(s->phase_trace);
     hw.trace_words = s->phase_words;
     HIP_TRY(launch_lm_head_bf16(s->stream, h->hidden_dev, h->hidden_stride, h->weight_dev, h->weight_stride,

@@ -198,6 +198,8 @@ def _load():
     L.lily_insertions_destroy.argtypes = [vp]
     L.lily_lm_head_tiles.restype = C.c_uint32
     L.lily_lm_head_tiles.argtypes = [C.c_uint32]
+    L.lily_lm_head_library_calls.restype = C.c_uint64
+    L.lily_lm_head_library_calls.argtypes = [vp]
     for name, args in sigs.items():
         getattr(L, name).restype = C.c_int
         getattr(L, name).argtypes = args
@@ -508,6 +510,11 @@ class Sampler:
         h.tile_max_dev = _ptr(tile_max, torch.float32)
         h.tile_sum_dev = _ptr(tile_sum, torch.float32)
         return h
+
+    def lm_head_library_calls(self):
+        """lily_lm_head_library_calls: producer calls of this sampler that went through the
+        platform's GEMM library."""
+        return int(_lib.lily_lm_head_library_calls(self._h))
 
     def lm_head(self, hidden, weight, temperatures, logits, tile_max, tile_sum):
         """lily_lm_head_bf16: logits[rows, V] (bf16 or f32) = hidden @ weight.T with the summaries;

@@ -590,6 +590,52 @@ def test_heads_of_affine_codes(sampler, bits, group, rows):
     _check_draws(logits.cpu().numpy(), ids, lps, cand, counts, params_kw, steps)
 
 
+@pytest.mark.parametrize("form", ["own", "library"])
+@pytest.mark.parametrize("rows,d,vocab,slack", [(130, 512, 4096 + 77, 8), (300, 128, 2000 + 3, 3),
+                                                (1024, 256, 3000, 8), (5, 64, 700, 8)])
+def test_batches_in_either_form(monkeypatch, form, rows, d, vocab, slack):
+    """A batch through this library's own tiles and through the platform's GEMM library followed
+    by the pass that forms the summaries (LILY_SAMPLER_HEAD, read when a sampler is created):
+    bf16 logits, f32 logits and both widths of codes meet the producer's bar either way, nothing
+    behind a row's last column is written, and the sampler counts the calls that took the
+    library (none under `own`; every one under `library` where the rows of the logits start at
+    multiples of 16 bytes, none where they do not: those stay with this library's own kernels)."""
+    monkeypatch.setenv("LILY_SAMPLER_HEAD", form)
+    s = LS.Sampler(0)
+    try:
+        rng = np.random.default_rng(rows + d)
+        hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(20, vocab // 8))
+        temps = [0.0 if r % 5 == 4 else 0.5 + 0.1 * (r % 7) for r in range(rows)]
+        stride = ((vocab + 7) // 8) * 8 + slack
+        h, w, buf, logits, tmax, tsum = _produce(s, hidden, weight, temps, rows, vocab, stride)
+        _check_product(h, w, logits, tmax, tsum, temps)
+        assert torch.all(buf[:, vocab:] == 7.0)
+        calls = s.lm_head_library_calls()
+        assert calls == (1 if form == "library" and slack == 8 else 0)
+        tiles = (vocab + TILE - 1) // TILE
+        buf32 = torch.full((rows, stride), 7.0, dtype=torch.float32, device=dev())
+        s.lm_head(h, w, temps, buf32[:, :vocab], tmax, tsum)
+        s.synchronize()
+        _check_f32_product(h, w, buf32[:, :vocab], tmax, tsum, temps)
+        assert torch.all(buf32[:, vocab:] == 7.0)
+        if form == "library" and slack == 8:
+            assert s.lm_head_library_calls() == 2
+        for bits, group in ((4, 64), (8, 32)):
+            qw, dense, _, _ = _quantised(rng, vocab, d, bits, group)
+            buf32.fill_(7.0)
+            before = s.lm_head_library_calls()
+            s.lm_head(h, qw, temps, buf32[:, :vocab], tmax, tsum)
+            s.synchronize()
+            if form == "library" and slack == 8:
+                assert s.lm_head_library_calls() == before + 1
+            if form == "own" and rows <= 16 and group >= 64 and (d // group) % 2 == 0 and d % (1024 // bits) == 0:
+                continue   # (the form for few rows has a test of its own)
+            _check_f32_product(h, dense, buf32[:, :vocab], tmax, tsum, temps)
+            assert torch.all(buf32[:, vocab:] == 7.0)
+    finally:
+        s.close()
+
+
 def test_codes_ask_for_f32_logits(sampler):
     rng = np.random.default_rng(5)
     qw, _, _, _ = _quantised(rng, 256, 64, 8, 64)
