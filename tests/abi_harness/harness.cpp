@@ -6,6 +6,13 @@
 //                            descriptors every call (params, steps, scratches, penalties, logprobs):
 //                            prints the host time a call takes to return and the time per call
 //                            on the device (HIP events around the N calls)
+//   harness head ROWS D V    the logits' producer on ROWS x D hidden states and V x D weights
+//                            (bf16, from the hash below), once by this library's own kernel
+//                            (LILY_SAMPLER_HEAD=own) and once the default way, which for a batch
+//                            is the platform's GEMM library opened by name - in a program that
+//                            has loaded no copy of it: prints "head library_calls N maxdiff X
+//                            maxdiff_max Y maxdiff_sum Z" (the two ways' logits and summaries
+//                            against each other, differences relative to 1 + |value|).
 //   harness gpu V SEED       two draws through lily_sample_f32, two rows through
 //                            lily_sample_rows and the same rows through a plan; prints
 //                            "ids a b c d e f" - the Python side reproduces the inputs and
@@ -306,7 +313,102 @@ static int time_mode(uint32_t rows, uint32_t vocab, uint32_t n) {
     return 0;
 }
 
+static uint16_t bf16_of(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+static float f32_of(uint16_t b) {
+    const uint32_t u = (uint32_t)b << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+static int head_mode(uint32_t rows, uint32_t d, uint32_t vocab) {
+    HIP(hipSetDevice(0));
+    hipStream_t stream;
+    HIP(hipStreamCreate(&stream));
+    const uint32_t tiles = lily_lm_head_tiles(vocab);
+    std::vector<uint16_t> hidden((size_t)rows * d), weight((size_t)vocab * d);
+    for (size_t i = 0; i < hidden.size(); ++i) {
+        hidden[i] = bf16_of(0.125f * logit_of((uint32_t)i, 5));
+    }
+    const float scale = 0.25f / std::sqrt((float)d);
+    for (size_t i = 0; i < weight.size(); ++i) {
+        weight[i] = bf16_of(scale * logit_of((uint32_t)i, 9));
+    }
+    void *h_dev, *w_dev;
+    HIP(hipMalloc(&h_dev, hidden.size() * 2));
+    HIP(hipMalloc(&w_dev, weight.size() * 2));
+    HIP(hipMemcpy(h_dev, hidden.data(), hidden.size() * 2, hipMemcpyHostToDevice));
+    HIP(hipMemcpy(w_dev, weight.data(), weight.size() * 2, hipMemcpyHostToDevice));
+    std::vector<float> temps(rows, 0.8f);
+    std::vector<uint16_t> logits[2];
+    std::vector<float> tmax[2], tsum[2];
+    unsigned long long calls = 0;
+    for (int way = 0; way < 2; ++way) {
+        if (way == 0) {
+            setenv("LILY_SAMPLER_HEAD", "own", 1);
+        } else {
+            unsetenv("LILY_SAMPLER_HEAD");
+        }
+        lily_sampler_t* s = nullptr;
+        CHECK(lily_sampler_create(0, stream, &s));
+        void *l_dev, *m_dev, *s_dev;
+        HIP(hipMalloc(&l_dev, (size_t)rows * vocab * 2));
+        HIP(hipMalloc(&m_dev, (size_t)rows * tiles * 4));
+        HIP(hipMalloc(&s_dev, (size_t)rows * tiles * 4));
+        lily_lm_head head;
+        std::memset(&head, 0, sizeof(head));
+        head.hidden_dev = h_dev;
+        head.hidden_stride = d;
+        head.weight_dev = w_dev;
+        head.weight_stride = d;
+        head.d = d;
+        head.tile_max_dev = static_cast<float*>(m_dev);
+        head.tile_sum_dev = static_cast<float*>(s_dev);
+        CHECK(lily_lm_head_bf16(s, &head, rows, vocab, temps.data(), l_dev, vocab));
+        HIP(hipStreamSynchronize(stream));
+        logits[way].resize((size_t)rows * vocab);
+        tmax[way].resize((size_t)rows * tiles);
+        tsum[way].resize((size_t)rows * tiles);
+        HIP(hipMemcpy(logits[way].data(), l_dev, logits[way].size() * 2, hipMemcpyDeviceToHost));
+        HIP(hipMemcpy(tmax[way].data(), m_dev, tmax[way].size() * 4, hipMemcpyDeviceToHost));
+        HIP(hipMemcpy(tsum[way].data(), s_dev, tsum[way].size() * 4, hipMemcpyDeviceToHost));
+        if (way == 1) {
+            calls = lily_lm_head_library_calls(s);
+        } else if (lily_lm_head_library_calls(s) != 0) {
+            std::fprintf(stderr, "the own kernel was asked for\n");
+            return 1;
+        }
+        lily_sampler_destroy(s);
+        HIP(hipFree(l_dev));
+        HIP(hipFree(m_dev));
+        HIP(hipFree(s_dev));
+    }
+    double diff = 0.0, diff_max = 0.0, diff_sum = 0.0;
+    for (size_t i = 0; i < logits[0].size(); ++i) {
+        const double a = f32_of(logits[0][i]), b = f32_of(logits[1][i]);
+        diff = std::fmax(diff, std::fabs(a - b) / (1.0 + std::fabs(a)));
+    }
+    for (size_t i = 0; i < tmax[0].size(); ++i) {
+        diff_max = std::fmax(diff_max, std::fabs((double)tmax[0][i] - tmax[1][i]) / (1.0 + std::fabs((double)tmax[0][i])));
+        diff_sum = std::fmax(diff_sum, std::fabs((double)tsum[0][i] - tsum[1][i]) / (1.0 + std::fabs((double)tsum[0][i])));
+    }
+    std::printf("head library_calls %llu maxdiff %.6f maxdiff_max %.6f maxdiff_sum %.6f\n", calls, diff, diff_max,
+                diff_sum);
+    HIP(hipFree(h_dev));
+    HIP(hipFree(w_dev));
+    HIP(hipStreamDestroy(stream));
+    return 0;
+}
+
 int main(int argc, char** argv) {
+    if (argc >= 5 && std::strcmp(argv[1], "head") == 0) {
+        return head_mode((uint32_t)std::atoi(argv[2]), (uint32_t)std::atoi(argv[3]), (uint32_t)std::atoi(argv[4]));
+    }
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) {
         return cpu_mode();
     }
@@ -316,6 +418,6 @@ int main(int argc, char** argv) {
     if (argc >= 5 && std::strcmp(argv[1], "time") == 0) {
         return time_mode((uint32_t)std::atoi(argv[2]), (uint32_t)std::atoi(argv[3]), (uint32_t)std::atoi(argv[4]));
     }
-    std::fprintf(stderr, "usage: harness cpu | harness gpu VOCAB SEED | harness time ROWS VOCAB CALLS\n");
+    std::fprintf(stderr, "usage: harness cpu | harness gpu VOCAB SEED | harness time ROWS VOCAB CALLS | harness head ROWS D VOCAB\n");
     return 2;
 }

@@ -81,3 +81,21 @@ def test_draws_from_cpp_match_the_oracle(vocab, seed):
             counts[r][d.chosen] += 1
             want.append(int(d.chosen))
     assert got == want
+
+
+@pytest.mark.gpu
+def test_a_batch_of_the_producer_from_cpp_by_either_way():
+    """A program that has loaded no copy of the platform's GEMM library: the producer opens the
+    system's by its name for a batch of 300 rows, and what it stores equals what this library's
+    own kernel stores to one bf16 step (the order of the f32 additions differs), the summaries
+    likewise (a tile's largest value is one of those values; its sum moves with them: at T 0.8 a
+    bf16 step of a value near 4 moves its term by 4 %)."""
+    _need_harness()
+    res = subprocess.run([HARNESS, "head", "300", "512", "5000"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr + res.stdout
+    words = [l for l in res.stdout.splitlines() if l.startswith("head ")][0].split()
+    got = dict(zip(words[1::2], words[2::2]))
+    assert int(got["library_calls"]) == 1, res.stdout
+    assert float(got["maxdiff"]) <= 2.0 ** -7
+    assert float(got["maxdiff_max"]) <= 2.0 ** -7
+    assert float(got["maxdiff_sum"]) <= 0.1
