@@ -44,11 +44,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // two (f32) tiles a thread with two blocks asked ahead of the one being reduced.  The arithmetic
 // is what bounds it (a 64-wide vector instruction takes four clocks, an exponential sixteen), so
 // it is kept short: the maximum skips a NaN by itself (IEEE maximum of a number and a NaN is the
-// number), 2^(x * c2 - max * c2) of a column at -inf is 0 by itself and that of a NaN becomes 0
-// by a maximum with 0.  What counts is what counts in the producer's epilogue: a NaN and a column
-// outside the vocabulary are -inf.  (A row whose c2 is not a positive finite number - its sums
-// are not to be used - gets the count of its finite values, as there.)  The row's last tile,
-// where the vocabulary ends inside it, is read value by value at the end.
+// number), 2^(x * c2 - max * c2) of a column at -inf is 0 by itself, and a tile whose sum comes
+// out as a NaN is summed again with every value tested.  What counts is what counts in the
+// producer's epilogue: a NaN and a column outside the vocabulary are -inf.  (A row whose c2 is 0
+// - its sums are not to be used - gets the count of its finite values, as there.)  The row's
+// last tile, where the vocabulary ends inside it, is read value by value at the end.
 template <bool F32>
 __global__ void __launch_bounds__(256)
 k_head_summaries(const void* __restrict__ logits, uint64_t stride, uint32_t vocab,
@@ -63,7 +63,6 @@ k_head_summaries(const void* __restrict__ logits, uint64_t stride, uint32_t voca
     const uint32_t row = blockIdx.x, sub = threadIdx.x & 15u, mine = threadIdx.x >> 4;
     const float NEG = -__builtin_huge_valf();
     const float c = c2_of_row[row];
-    const bool plain = c > 0.0f && c < __builtin_huge_valf();
     const uint32_t full = vocab / 128u;   // whole tiles
     const uint32_t all_blocks = (full + PER_BLOCK - 1u) / PER_BLOCK;
     const uint32_t b0 = blockIdx.y * blocks_per_slice;
@@ -89,21 +88,27 @@ k_head_summaries(const void* __restrict__ logits, uint64_t stride, uint32_t voca
             : "+v"(m));
         const float top = m * c;
         float sum = 0.0f;
-        if (plain) {
 #pragma unroll
-            for (uint32_t e = 0; e < 8u; ++e) {
-                sum += fmaxf(__builtin_amdgcn_exp2f(__builtin_fmaf(x[e], c, -top)), 0.0f);
-            }
-        } else {
-#pragma unroll
-            for (uint32_t e = 0; e < 8u; ++e) {
-                sum += x[e] == x[e] && x[e] > NEG ? __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], c, -top)) : 0.0f;
-            }
+        for (uint32_t e = 0; e < 8u; ++e) {
+            sum += __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], c, -top));
         }
         sum += rotated16<0x128>(sum);
         sum += rotated16<0x124>(sum);
         sum += rotated16<0x122>(sum);
         sum += rotated16<0x121>(sum);
+        // A NaN among the tile's values, a tile of nothing but -inf, a column at -inf where c2 is
+        // 0: the sum comes out as a NaN, and the rare tile is summed again value by value.
+        if (sum != sum) {
+            sum = 0.0f;
+#pragma unroll
+            for (uint32_t e = 0; e < 8u; ++e) {
+                sum += x[e] == x[e] && x[e] > NEG ? __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], c, -top)) : 0.0f;
+            }
+            sum += rotated16<0x128>(sum);
+            sum += rotated16<0x124>(sum);
+            sum += rotated16<0x122>(sum);
+            sum += rotated16<0x121>(sum);
+        }
         if (store && sub == 0u) {
             // (a tile that holds +inf: inf - inf, as in the producer's epilogue)
             const float value = m > NEG ? (m < __builtin_huge_valf() ? sum : __builtin_nanf("")) : 0.0f;

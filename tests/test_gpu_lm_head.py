@@ -632,6 +632,16 @@ def test_batches_in_either_form(monkeypatch, form, rows, d, vocab, slack):
                 continue   # (the form for few rows has a test of its own)
             _check_f32_product(h, dense, buf32[:, :vocab], tmax, tsum, temps)
             assert torch.all(buf32[:, vocab:] == 7.0)
+        # a hidden row with a NaN: every logit of the row is a NaN, which counts as -inf in the
+        # summaries (largest value -inf, sum 0); the other rows are what they were
+        h2 = h.clone()
+        h2[1, 3] = float("nan")
+        s.lm_head(h2, w, temps, logits, tmax, tsum)
+        s.synchronize()
+        assert bool(torch.all(torch.isnan(logits[1].float())))
+        assert bool(torch.all(tmax[1] == float("-inf"))) and bool(torch.all(tsum[1] == 0.0))
+        keep = [r for r in range(rows) if r != 1]
+        _check_product(h[keep], w, logits[keep], tmax[keep], tsum[keep], [temps[r] for r in keep])
     finally:
         s.close()
 
