@@ -14,8 +14,9 @@ constexpr uint32_t TILES_DECLINE = 256;                  // a penalised row that
 constexpr uint32_t SUMMED_DECLINE = 96;                  // or more tiles summed element by element
 constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated element by element
 
-// One workgroup per row (rows without mask or bias list, penalties only of the kind that can
-// but lower a value, k <= STREAM_K_MAX; bf16 or f32 logits, rows at multiples of 16 bytes).
+// One workgroup per row (rows without mask, at most STREAM_BIAS_CAP bias pairs, penalties only
+// of the kind that can but lower a value, k <= STREAM_K_MAX; bf16 or f32 logits, rows at
+// multiples of 16 bytes).
 //   * The row's largest value is the largest summary; with at least k summaries at or above
 //     x, at least k values are: the k-th largest summary bounds the k-th largest value from
 //     below, and only tiles whose summary reaches it are read (16 bytes a lane: 16 lanes a tile
@@ -24,6 +25,11 @@ constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated ele
 //   * Under penalties the bound is the k-th largest summary as the worst penalty would leave it
 //     (more tiles are read), values of listed ids are evaluated with their counts, and the tiles
 //     that matter to the row's sum are summed element by element instead of by their summaries.
+//   * A bias list (logit += delta before everything else, pairs of one id adding up in list
+//     order): a summary says nothing about a biased id.  The tiles that hold one are always
+//     read, every value of theirs evaluated (and, for the row's sum, summed one by one instead
+//     of by the summary); a tile's largest value may belong to an id with a negative bias, so
+//     the bound is the (k + pairs)-th largest summary - k of those tiles keep their largest.
 //   * More candidates than the buffer holds (ties by the thousand): the exhaustive select
 //     over the whole row takes over.
 // `tile_row[r]` is the row of the summaries that belongs to row r of the table; `served[r]` is
@@ -36,6 +42,9 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     __shared__ uint16_t listed[TILES_MAX];   // tiles to read; bit 15: summed element by element
     __shared__ uint32_t refs[REF_CAP];       // pieces to evaluate: first id; bit 31: summed
     __shared__ uint32_t n_listed, n_refs, n_summed;
+    __shared__ uint32_t bias_id[STREAM_BIAS_CAP];
+    __shared__ float bias_delta[STREAM_BIAS_CAP];
+    __shared__ uint32_t bias_tiles[TILES_MAX / 32u];   // bit t: tile t holds a biased id
     constexpr uint32_t E = (uint32_t)Geo<DT>::E;          // values in a piece of 16 bytes
     constexpr uint32_t ELEM = DT == LILY_BF16 ? 2u : 4u;  // bytes a value
     const LILY_CONST RowArgs* table = (const LILY_CONST RowArgs*)cfg.table;
@@ -58,6 +67,16 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             emit(a, a.forced, vocab);
         }
         return;
+    }
+    const uint32_t n_bias = min(a.n_bias, STREAM_BIAS_CAP);   // (the host serves no longer lists here)
+    if (n_bias != 0u) {
+        if (tid < TILES_MAX / 32u) {
+            bias_tiles[tid] = 0u;
+        }
+        if (tid < n_bias) {
+            bias_id[tid] = gload(&a.bias[tid].id);
+            bias_delta[tid] = gload(&a.bias[tid].delta);
+        }
     }
     const size_t srow = (size_t)gload(tile_row + blockIdx.y) * tiles;
     // the summaries: both arrays asked for at once (clamped, so that no load hangs on a test)
@@ -85,8 +104,24 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     for (int i = 1; i < NWAVE; ++i) {
         top = fmaxf(top, sh.red_f[i]);
     }
+    if (tid < n_bias && bias_id[tid] < vocab) {
+        const uint32_t t = bias_id[tid] / LILY_TILE_COLS;
+        atomicOr(&bias_tiles[t >> 5], 1u << (t & 31u));
+    }
     __syncthreads();
     phase(cfg, 1);
+    auto holds_bias = [&](uint32_t tile) -> bool {
+        return n_bias != 0u && ((bias_tiles[tile >> 5] >> (tile & 31u)) & 1u) != 0u;
+    };
+    // (pairs of one id add up in list order, as the row kernels add them)
+    auto with_bias = [&](uint32_t id, float x) -> float {
+        for (uint32_t j = 0; j < n_bias; ++j) {
+            if (bias_id[j] == id) {
+                x += bias_delta[j];
+            }
+        }
+        return x == x ? x : NEG_INF;
+    };
 
     if (a.mode == MODE_ARGMAX && !forced) {
         // The first of the largest values: the lowest tile that holds it, its lowest column.
@@ -146,35 +181,23 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         }
         return t;
     };
-    // The sum's cut: tiles whose summary lies below it are summed as their summaries give them
-    // (their listed ids' raw terms stand for the true ones: each is below 2^-(log2 V + 21) of
-    // the row's largest term), tiles at or above it element by element.  It hangs from a lower
-    // bound of the row's largest TRUE value: the lowered largest summary or, better where a
-    // sequence keeps coming back to one token, the true value of the scratch's most-counted id.
-    float cut = -__builtin_huge_valf();
-    if (want_lse && pen) {
-        float floor_v = lowered(top);
-        const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
-        if (heavy < vocab && max_count != 0u) {
-            floor_v = fmaxf(floor_v, true_value(heavy, load_logit<DT>(a.logits, heavy)));
-        }
-        cut = floor_v - (log2f((float)vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
-    }
+    // The summaries' part of the row's sum: every tile below the cut that holds no biased id.
     LseAcc lse;
     lse.init();
-    if (want_lse) {
+    auto add_summaries = [&](float below) {
 #pragma unroll
         for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
             const uint32_t t = tid + j * NT;
-            if (t < tiles && ms[j] > NEG_INF && (!pen || ms[j] < cut)) {
+            if (t < tiles && ms[j] > NEG_INF && (!pen || ms[j] < below) && !holds_bias(t)) {
                 // the tile's sum has the reference tile_max * c2
                 const float safe = lse.rebase(ms[j], a.c2);
                 lse.s += ss[j] * __builtin_amdgcn_exp2f(ms[j] * a.c2 - safe);
             }
         }
-    }
-    if (forced) {   // (not under penalties: the host keeps such rows off this kernel)
+    };
+    if (forced) {   // (not under penalties, no bias list: the host keeps such rows off this kernel)
         if (want_lse) {
+            add_summaries(0.0f);
             lse_reduce(sh, lse);
         }
         if (tid == 0) {
@@ -183,7 +206,8 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         return;
     }
 
-    const uint32_t k = a.k;
+    // (with a bias list: n_bias tiles more, whose largest values may be the biased ones)
+    const uint32_t k = a.k, k_tiles = a.k + n_bias;
     // with at least k summaries at or above x, at least k raw values are, and their true values
     // are at or above lowered(x)
     // (a lower bound of the k-th largest summary, as the streaming select takes it: each wave's
@@ -196,7 +220,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     }
     float kth;
     if (tiles >= NT) {
-        const uint32_t kw = (k + NWAVE - 1u) / NWAVE;
+        const uint32_t kw = (k_tiles + NWAVE - 1u) / NWAVE;
         const uint32_t key16 = lane_best > NEG_INF ? (lilym_order_key(lane_best) >> 16) : 0u;
         const uint32_t P = wave_kth_key16(key16, kw);
         if (lane == 0) {
@@ -210,7 +234,29 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         __syncthreads();
     } else {
         // a short row leaves whole waves without a summary: the exact k-th largest instead
-        kth = wg_kth_largest(ms, k, sh);
+        kth = wg_kth_largest(ms, k_tiles, sh);
+    }
+    // The sum's cut: tiles whose summary lies below it are summed as their summaries give them
+    // (their listed ids' raw terms stand for the true ones: each is below 2^-(log2 V + 21) of
+    // the row's largest term), tiles at or above it element by element.  It hangs from a lower
+    // bound of the row's largest TRUE value: the lowered largest summary (with a bias list the
+    // lowered k-th, which k tiles reach with values that carry no bias) or, better where a
+    // sequence keeps coming back to one token, the true value of the scratch's most-counted id.
+    float cut = -__builtin_huge_valf();
+    if (want_lse && pen) {
+        float floor_v = lowered(n_bias != 0u ? kth : top);
+        const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
+        if (heavy < vocab && max_count != 0u) {
+            const float raw = load_logit<DT>(a.logits, heavy);
+            const float biased = with_bias(heavy, raw == raw ? raw : NEG_INF);
+            if (biased > NEG_INF) {
+                floor_v = fmaxf(floor_v, true_value(heavy, biased));
+            }
+        }
+        cut = floor_v - (log2f((float)vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
+    }
+    if (want_lse) {
+        add_summaries(cut);
     }
     const float bound = lowered(kth);
     const float reach = (want_lse && pen) ? fminf(bound, cut) : bound;   // tiles read
@@ -220,9 +266,13 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     }
 #pragma unroll
     for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
-        if (ms[j] >= reach && ms[j] > NEG_INF) {
-            const bool sum_it = want_lse && pen && ms[j] >= cut;
-            listed[atomicAdd(&n_listed, 1u)] = (uint16_t)((tid + j * NT) | (sum_it ? 0x8000u : 0u));
+        const uint32_t t = tid + j * NT;
+        const bool biased = t < tiles && holds_bias(t);
+        if ((ms[j] >= reach && ms[j] > NEG_INF) || biased) {
+            // (bit 15: every value of the tile is evaluated, and taken into the row's sum one by
+            // one where there is a sum - the summaries' part leaves these tiles out)
+            const bool sum_it = want_lse && pen && ms[j] >= cut && ms[j] > NEG_INF;
+            listed[atomicAdd(&n_listed, 1u)] = (uint16_t)(t | (sum_it || biased ? 0x8000u : 0u));
             if (sum_it) {
                 atomicAdd(&n_summed, 1u);
             }
@@ -311,6 +361,9 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             }
             const bool summed = (ref[u] >> 31) != 0u;
             float x = raw[u] == raw[u] ? raw[u] : NEG_INF;
+            if (summed && holds_bias(id / LILY_TILE_COLS)) {
+                x = with_bias(id, x);
+            }
             if (pen && ((word[u] >> (id & 31u)) & 1u) != 0u && x > NEG_INF && (x >= bound || summed)) {
                 x = true_value(id, x);
             }

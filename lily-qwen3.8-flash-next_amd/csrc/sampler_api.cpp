@@ -1792,10 +1792,15 @@ HeadWeightsOf::HeadWeightsOf(const lily_sampler* s, const lily_lm_head* h) {
     w.group_shift = shift;
 }
 
-// Rows the summaries serve: no mask, no bias list, penalties only of the lowering kind, the row
-// given as it is, and a greedy row or a plain draw among at most STREAM_K_MAX candidates.
+// Rows the summaries serve: no mask, penalties only of the lowering kind, the row given as it
+// is, and a greedy row or a plain draw among at most STREAM_K_MAX candidates; a bias list of up
+// to STREAM_BIAS_CAP pairs on a row that draws and is not forced (a summary says nothing about
+// the largest biased value, which a greedy or a forced row's answer hangs on).
 bool tiles_serve(const RowArgs& r) {
-    if (r.allow != nullptr || r.n_bias != 0 || r.sel_row != nullptr) {
+    if (r.allow != nullptr || r.sel_row != nullptr || r.n_bias > STREAM_BIAS_CAP) {
+        return false;
+    }
+    if (r.n_bias != 0 && (r.mode == MODE_ARGMAX || (r.flags & F_FORCED))) {
         return false;
     }
     if (r.mode == MODE_ARGMAX) {

@@ -334,6 +334,123 @@ def test_rows_under_lowering_penalties_are_drawn_from_summaries(sampler):
         scratch[r].close()
 
 
+def _bias_lists(rng, stored_f, vocab):
+    """Bias lists of the kinds that matter to a draw from summaries: the row's best ids barred
+    (their tiles' summaries then overstate what the tiles hold), an id far down the row raised
+    to the top (its tile's summary says nothing of it), many small shifts, pairs of one id that
+    add up in list order, an id next to the row's best in the same tile, a full list of 64."""
+    rows = stored_f.shape[0]
+    out = []
+    for r in range(rows):
+        order = np.argsort(-stored_f[r])
+        kind = r % 5
+        if kind == 0:
+            low = int(order[vocab // 2 + r])
+            b = [(int(i), -100.0) for i in order[:3]] + [(low, 60.0)]
+        elif kind == 1:
+            ids = rng.integers(0, vocab, 40)
+            b = [(int(i), float(d)) for i, d in zip(ids, rng.normal(0, 3.0, 40))]
+            b += [b[0], b[0], (int(order[1]), 0.75), (int(order[1]), -0.25)]
+        elif kind == 2:
+            top = int(order[0])
+            near = top + 1 if (top + 1) // TILE == top // TILE and top + 1 < vocab else top - 1
+            b = [(int(i), -1.0e4) for i in order[:10]] + [(near, 25.0)]
+        elif kind == 3:
+            ids = np.concatenate([order[:20], rng.integers(0, vocab, 44)])
+            b = [(int(i), float(d)) for i, d in zip(ids, rng.normal(0, 6.0, 64))]
+        else:
+            b = [(int(order[5]), float("-inf")), (int(order[40 + r]), 3.5)]
+        out.append(b)
+    return out
+
+
+@pytest.mark.parametrize("f32", [False, True])
+def test_rows_with_bias_lists_are_drawn_from_summaries(sampler, f32):
+    """A bias list of up to 64 pairs (logit += delta before the mask and the penalties, pairs of
+    one id adding up in list order) on rows drawn from the summaries: the tiles that hold a
+    biased id are read whatever their summaries say, and the bound counts on as many tiles more
+    as there are pairs.  Rows without penalties are all served by the kernel that reads
+    summaries (one workgroup a row, where the ordinary launch cuts so few rows into slices);
+    rows under lowering penalties with a history of their best ids likewise unless that kernel
+    declines them; a greedy row and a forced row with a bias list go the ordinary way.  Ids,
+    candidates, kept counts and log-probabilities are the oracle's on the stored logits."""
+    rows, d, vocab = 15, 256, (151_936 if not f32 else 20_000)
+    rng = np.random.default_rng(77 + int(f32))
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=60, gain=9.0)
+    params_kw = [dict(temperature=0.7 + 0.05 * (r % 3), top_k=(64, 20, 5, 1 + r)[r % 4], top_p=(0.9, 1.0)[r % 2],
+                      min_p=0.01 * (r % 2), seed=900 + r) for r in range(rows)]
+    params = [ls_params(**kw) for kw in params_kw]
+    temps = [p.effective()[0] for p in params]
+    h, w = _bf16(hidden), _bf16(weight)
+    tiles = (vocab + TILE - 1) // TILE
+    logits = torch.zeros(rows, vocab, dtype=torch.float32 if f32 else torch.bfloat16, device=dev())
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    sampler.lm_head(h, w, temps, logits, tmax, tsum)
+    sampler.synchronize()
+    stored = logits.cpu().numpy() if f32 else _bits(logits.contiguous())
+    stored_f = stored if f32 else W.bf16_bits_to_f32(stored)
+    bias = _bias_lists(rng, stored_f, vocab)
+    steps = [3 + r for r in range(rows)]
+
+    def check(ids, lps, cand, counts, kws, hist=None, forced=None):
+        for r, kw in enumerate(kws):
+            if forced is not None and forced[r] is not None:
+                assert ids[r] == forced[r], r
+                continue
+            c = None if hist is None else hist[r]
+            dd = O.sample(stored[r], c, o_params(**kw), steps[r], bias=bias[r], want_logprob=True)
+            if o_params(**kw).temperature == 0.0:
+                assert ids[r] == dd.chosen, r
+                continue
+            n_fin = int(np.sum(dd.cand_adj > -np.inf))
+            assert counts[r, 0] == n_fin, (r, counts[r, 0], n_fin)
+            assert np.array_equal(cand[r, :n_fin], dd.cand_ids[:n_fin].astype(np.int64)), r
+            assert counts[r, 1] == dd.n_kept and ids[r] == dd.chosen, (r, ids[r], dd.chosen)
+            assert abs(lps[r] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (r, lps[r], dd.logprob)
+
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    sampler.set_path_stats(stats)
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, params, steps, out, bias=bias, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, steps)
+    sampler.set_path_stats(None)
+    check(ids, lps, cand, counts, params_kw)
+    st = stats.cpu().numpy()
+    assert st[0] == rows and st[1] == 0 and st[2] == 0, st.tolist()
+    # the same lists under lowering penalties, with histories that hold the rows' best ids
+    pen_kw = [dict(kw, repetition_penalty=1.1, presence_penalty=0.2, frequency_penalty=0.1) for kw in params_kw]
+    pen = [ls_params(**kw) for kw in pen_kw]
+    scratch, hist = [], []
+    for r in range(rows):
+        best = np.argsort(-stored_f[r])[:30].astype(np.int32)
+        hh = np.concatenate([rng.integers(0, vocab, 1500).astype(np.int32), np.repeat(best[:8], 3), best])
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(hh).to(dev()))
+        scratch.append(sc)
+        hist.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, pen, steps, out, scratch=scratch, bias=bias, out_logprobs=lp, dbg_ids=di,
+            dbg_counts=dc),
+        logits, pen_kw, steps)
+    check(ids, lps, cand, counts, pen_kw, hist=hist)
+    for r in range(rows):
+        assert np.array_equal(scratch[r].read_counts().numpy().view(np.uint32), hist[r]), r
+        scratch[r].close()
+    # a greedy row and a forced row with a bias list (served by the kernels that read the row)
+    odd_kw = [dict() if r % 2 else kw for r, kw in enumerate(params_kw)]
+    odd = [ls_params(**kw) for kw in odd_kw]
+    forced = [int(np.argsort(-stored_f[r])[2]) if r % 4 == 0 else None for r in range(rows)]
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, odd, steps, out, bias=bias, forced=forced, out_logprobs=lp, dbg_ids=di,
+            dbg_counts=dc),
+        logits, odd_kw, steps)
+    check(ids, lps, cand, counts, odd_kw, forced=forced)
+
+
 def test_a_batch_of_penalised_rows_through_the_fused_call(sampler):
     """1 024 rows under config 5's draw settings (k 64, top-p 0.9, T 0.8, penalties that only
     lower, a 2 048-id history that holds the row's best ids, a log-probability) through the one
