@@ -429,13 +429,17 @@ void lily_insertions_clear(lily_insertions_t* q, uint32_t row);
  * accumulated in f32 on the matrix cores and stored as f32 (what the reference's sampler reads,
  * src/kernels/sample.rs:263) or rounded to bf16 (nearest even).  Beside the logits the producer leaves,
  * for every LILY_LOGIT_TILE_COLS columns of every row, the largest value and the sum of
- * 2^((x - largest) * log2(e) / T[r]) over the tile - "summaries".  A row without allow-mask or
- * bias list that is greedy or draws among at most 64 candidates, under no penalties or under
- * penalties that can only lower a value (repetition >= 1, presence and frequency >= 0), is then
- * drawn from the summaries and the few tiles that can hold a candidate (about k tiles of 256
- * bytes instead of the row; a penalised row whose values lie too close together for that is
- * recognised on the device and read whole); every other row of the batch is drawn from the
- * logits as lily_sample_rows draws it.  Ids and log-probabilities are those of lily_sample_rows
+ * 2^((x - largest) * log2(e) / T[r]) over the tile - "summaries".  A row that is greedy or
+ * draws among at most 64 candidates, under no penalties or under penalties that can only lower
+ * a value (repetition >= 1, presence and frequency >= 0), is then drawn from the summaries and
+ * the few tiles that can hold a candidate (about k tiles of 256 bytes instead of the row; a
+ * penalised row whose values lie too close together for that is recognised on the device and
+ * read whole).  A row that draws may carry a bias list of up to 64 pairs (the tiles that hold a
+ * biased id are read besides) or an allow-mask (tiles the mask bars drop out, tiles allowed in
+ * part are tested id by id; a row whose mask bars too many of its best values, or leaves too
+ * many tiles allowed in part for its log-probability, is recognised on the device and read
+ * whole); a greedy or forced row with either, and every other row of the batch, is drawn from
+ * the logits as lily_sample_rows draws it.  Ids and log-probabilities are those of lily_sample_rows
  * on the same logits. */
 #define LILY_LOGIT_TILE_COLS 128u
 

@@ -30,10 +30,16 @@ constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated ele
 //     read, every value of theirs evaluated (and, for the row's sum, summed one by one instead
 //     of by the summary); a tile's largest value may belong to an id with a negative bias, so
 //     the bound is the (k + pairs)-th largest summary - k of those tiles keep their largest.
+//   * An allow-mask (a barred id counts as -inf): a tile none of whose ids is allowed drops out
+//     with its summary; a tile that is allowed in part has a summary that says too much - its
+//     values are tested one by one against the mask, it enters the row's sum value by value,
+//     and the bound counts on k / 2 + 8 tiles more.  That is a guess, so the row checks it: with
+//     fewer than k candidates at or above the bound it is left to the launch that follows, as is
+//     a row with more than SUMMED_DECLINE partly allowed tiles to sum.
 //   * More candidates than the buffer holds (ties by the thousand): the exhaustive select
 //     over the whole row takes over.
 // `tile_row[r]` is the row of the summaries that belongs to row r of the table; `served[r]` is
-// written for rows under penalties: 1 = drawn here, 0 = left to the launch that follows.
+// written for rows under penalties or a mask: 1 = drawn here, 0 = left to the launch that follows.
 template <int DT, bool LSE>
 __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float* tile_max,
                                                       const float* tile_sum, uint32_t tiles,
@@ -87,6 +93,37 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         const uint32_t t = min(tid + j * NT, tiles - 1u);
         ms[j] = gload(tile_max + srow + t);
         ss[j] = gload(tile_sum + srow + t);
+    }
+    // The mask's four words of every tile: a tile with no allowed id drops out, one allowed in
+    // part is marked (bit j of `partly`).
+    const bool masked = a.allow != nullptr;
+    const uint32_t words = (vocab + 31u) / 32u;
+    uint32_t partly = 0;
+    if (masked) {
+        uint32_t mw[TILES_PER_THREAD][4];
+#pragma unroll
+        for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) {
+                mw[j][q] = gload(a.allow + min((tid + j * NT) * 4u + q, words - 1u));
+            }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
+            bool any = false, all = true;
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) {
+                const uint32_t first = ((tid + j * NT) * 4u + q) * 32u;   // the word's first id
+                const uint32_t in_row = first >= vocab ? 0u : (vocab - first >= 32u ? 0xffffffffu : (1u << (vocab - first)) - 1u);
+                any = any || (mw[j][q] & in_row) != 0u;
+                all = all && (mw[j][q] & in_row) == in_row;
+            }
+            if (!any) {
+                ms[j] = NEG_INF;
+            } else if (!all) {
+                partly |= 1u << j;
+            }
+        }
     }
 #pragma unroll
     for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
@@ -161,7 +198,6 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     // summary describes raw values and bounds true ones from above.  `lowered(x)`: what a raw
     // value x is worth at least (the penalty of an id with the scratch's largest count).
     const bool pen = (a.flags & F_PEN) != 0;
-    const uint32_t words = (vocab + 31u) / 32u;
     const uint32_t max_count = pen ? *(const LILY_CONST uint32_t*)(a.touched + words) : 0u;
     auto lowered = [&](float m) -> float {
         if (pen && m > NEG_INF) {
@@ -181,14 +217,16 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         }
         return t;
     };
-    // The summaries' part of the row's sum: every tile below the cut that holds no biased id.
+    // The summaries' part of the row's sum: every tile below the cut that holds no biased id and
+    // no barred one.
     LseAcc lse;
     lse.init();
     auto add_summaries = [&](float below) {
 #pragma unroll
         for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
             const uint32_t t = tid + j * NT;
-            if (t < tiles && ms[j] > NEG_INF && (!pen || ms[j] < below) && !holds_bias(t)) {
+            if (t < tiles && ms[j] > NEG_INF && (!pen || ms[j] < below) && !holds_bias(t) &&
+                ((partly >> j) & 1u) == 0u) {
                 // the tile's sum has the reference tile_max * c2
                 const float safe = lse.rebase(ms[j], a.c2);
                 lse.s += ss[j] * __builtin_amdgcn_exp2f(ms[j] * a.c2 - safe);
@@ -207,7 +245,8 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     }
 
     // (with a bias list: n_bias tiles more, whose largest values may be the biased ones)
-    const uint32_t k = a.k, k_tiles = a.k + n_bias;
+    // (under a mask: a guess at how many of the best tiles owe their summaries to barred ids)
+    const uint32_t k = a.k, k_tiles = a.k + n_bias + (masked ? a.k / 2u + 8u : 0u);
     // with at least k summaries at or above x, at least k raw values are, and their true values
     // are at or above lowered(x)
     // (a lower bound of the k-th largest summary, as the streaming select takes it: each wave's
@@ -244,9 +283,13 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     // sequence keeps coming back to one token, the true value of the scratch's most-counted id.
     float cut = -__builtin_huge_valf();
     if (want_lse && pen) {
-        float floor_v = lowered(n_bias != 0u ? kth : top);
+        // (under a mask the lowered k-th summary is a guess; the row's check below - k candidates
+        // at or above it - confirms it as a floor of the largest true value as well)
+        float floor_v = lowered(n_bias != 0u || masked ? kth : top);
         const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
-        if (heavy < vocab && max_count != 0u) {
+        const bool heavy_allowed =
+            !masked || heavy >= vocab || ((gload(a.allow + (heavy >> 5)) >> (heavy & 31u)) & 1u) != 0u;
+        if (heavy < vocab && max_count != 0u && heavy_allowed) {
             const float raw = load_logit<DT>(a.logits, heavy);
             const float biased = with_bias(heavy, raw == raw ? raw : NEG_INF);
             if (biased > NEG_INF) {
@@ -268,10 +311,13 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     for (uint32_t j = 0; j < TILES_PER_THREAD; ++j) {
         const uint32_t t = tid + j * NT;
         const bool biased = t < tiles && holds_bias(t);
-        if ((ms[j] >= reach && ms[j] > NEG_INF) || biased) {
+        // (a tile allowed in part matters to the sum whatever its summary says; to the candidates
+        // only where the summary reaches the bound)
+        const bool part = ((partly >> j) & 1u) != 0u && ms[j] > NEG_INF;
+        if ((ms[j] >= reach && ms[j] > NEG_INF) || biased || (part && want_lse)) {
             // (bit 15: every value of the tile is evaluated, and taken into the row's sum one by
             // one where there is a sum - the summaries' part leaves these tiles out)
-            const bool sum_it = want_lse && pen && ms[j] >= cut && ms[j] > NEG_INF;
+            const bool sum_it = want_lse && ((pen && ms[j] >= cut && ms[j] > NEG_INF) || part);
             listed[atomicAdd(&n_listed, 1u)] = (uint16_t)(t | (sum_it || biased ? 0x8000u : 0u));
             if (sum_it) {
                 atomicAdd(&n_summed, 1u);
@@ -281,9 +327,10 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     __syncthreads();
     const uint32_t n_t = n_listed;
     phase(cfg, 8);
-    // A row under penalties whose bound or cut reaches a large part of its tiles (a flat row) is
-    // read faster as a whole: it is left to the launch that follows (`served` stays 0).
-    if (pen) {
+    // A row under penalties or a mask whose bound, cut or partly allowed tiles reach a large part
+    // of its tiles is read faster as a whole: it is left to the launch that follows (`served`
+    // stays 0).
+    if (pen || masked) {
         const bool decline = n_t > TILES_DECLINE || n_summed > SUMMED_DECLINE;
         if (tid == 0) {
             served[blockIdx.y] = decline ? 0u : 1u;
@@ -341,7 +388,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     const uint32_t n_r = n_refs;   // (beyond the list's capacity: the exhaustive select below)
     const uint32_t e_of = tid % E;
     for (uint32_t p0 = 0; p0 < min(n_r, REF_CAP); p0 += 4u * (NT / E)) {
-        uint32_t ref[4], word[4];
+        uint32_t ref[4], word[4], mword[4];
         float raw[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -352,6 +399,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             // (the word of the scratch's bitmap that covers the id; the summaries' first word
             // when there is no scratch to ask: the load stays unconditional)
             word[u] = gload((pen ? a.touched : reinterpret_cast<const uint32_t*>(tile_max)) + (pen ? (id >> 5) : 0u));
+            mword[u] = gload((masked ? a.allow : reinterpret_cast<const uint32_t*>(tile_max)) + (masked ? (id >> 5) : 0u));
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -363,6 +411,9 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             float x = raw[u] == raw[u] ? raw[u] : NEG_INF;
             if (summed && holds_bias(id / LILY_TILE_COLS)) {
                 x = with_bias(id, x);
+            }
+            if (masked && ((mword[u] >> (id & 31u)) & 1u) == 0u) {
+                x = NEG_INF;
             }
             if (pen && ((word[u] >> (id & 31u)) & 1u) != 0u && x > NEG_INF && (x >= bound || summed)) {
                 x = true_value(id, x);
@@ -388,6 +439,14 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     phase(cfg, 3);
     uint32_t n = sh.n_cand;
     __syncthreads();
+    // Under a mask the bound was a guess: it stands if k allowed values reach it.  (A row that
+    // has fewer allowed values altogether is drawn by the launch that follows.)
+    if (masked && n < k) {
+        if (tid == 0) {
+            served[blockIdx.y] = 0u;
+        }
+        return;
+    }
     bool sorted = false;
     uint32_t took = 0;
     if (n > TILE_CAND_CAP) {

@@ -1792,15 +1792,16 @@ HeadWeightsOf::HeadWeightsOf(const lily_sampler* s, const lily_lm_head* h) {
     w.group_shift = shift;
 }
 
-// Rows the summaries serve: no mask, penalties only of the lowering kind, the row given as it
-// is, and a greedy row or a plain draw among at most STREAM_K_MAX candidates; a bias list of up
-// to STREAM_BIAS_CAP pairs on a row that draws and is not forced (a summary says nothing about
-// the largest biased value, which a greedy or a forced row's answer hangs on).
+// Rows the summaries serve: penalties only of the lowering kind, the row given as it is, and a
+// greedy row or a plain draw among at most STREAM_K_MAX candidates; a bias list of up to
+// STREAM_BIAS_CAP pairs or an allow-mask on a row that draws and is not forced (a summary says
+// nothing about the largest biased or the largest allowed value, which a greedy or a forced
+// row's answer hangs on).  Rows under penalties or a mask may be declined on the device.
 bool tiles_serve(const RowArgs& r) {
-    if (r.allow != nullptr || r.sel_row != nullptr || r.n_bias > STREAM_BIAS_CAP) {
+    if (r.sel_row != nullptr || r.n_bias > STREAM_BIAS_CAP) {
         return false;
     }
-    if (r.n_bias != 0 && (r.mode == MODE_ARGMAX || (r.flags & F_FORCED))) {
+    if ((r.n_bias != 0 || r.allow != nullptr) && (r.mode == MODE_ARGMAX || (r.flags & F_FORCED))) {
         return false;
     }
     if (r.mode == MODE_ARGMAX) {
@@ -1884,7 +1885,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
         for (uint32_t r = 0; r < rows; ++r) {
             const RowArgs& row = packed[r];
             const bool serve = tiles_serve(row) && !sum_at_other_scale(r);
-            const bool pen = serve && row.mode != MODE_ARGMAX && (row.flags & F_PEN) != 0;
+            const bool pen = serve && row.mode != MODE_ARGMAX && ((row.flags & F_PEN) != 0 || row.allow != nullptr);
             const int g = !serve ? 2 : (pen ? 1 : 0);
             if (g != group) {
                 continue;

@@ -451,6 +451,123 @@ def test_rows_with_bias_lists_are_drawn_from_summaries(sampler, f32):
     check(ids, lps, cand, counts, odd_kw, forced=forced)
 
 
+def _masks(rng, stored_f, vocab):
+    """Allow-masks (packed u32, bit id & 31 of word id >> 5) of the kinds that matter to a draw
+    from summaries: a handful of barred ids among the row's best (their tiles are allowed in
+    part), a barred run of ids that holds the row's best tile and its neighbours (tiles that
+    drop out altogether), everything allowed, one id in thirty barred at random (every tile
+    allowed in part), and a sparse mask (a fiftieth of the ids, in runs)."""
+    rows = stored_f.shape[0]
+    words = (vocab + 31) // 32
+    out = np.zeros((rows, words), dtype=np.uint32)
+    kinds = []
+    for r in range(rows):
+        order = np.argsort(-stored_f[r])
+        allowed = np.ones(vocab, dtype=bool)
+        kind = r % 5
+        if kind == 0:
+            allowed[order[[0, 2, 3, 7, 11]]] = False
+        elif kind == 1:
+            t = int(order[0]) // TILE
+            allowed[max(0, (t - 1) * TILE + 5):min(vocab, (t + 2) * TILE - 9)] = False
+            allowed[order[1]] = False
+        elif kind == 2:
+            pass
+        elif kind == 3:
+            allowed[rng.random(vocab) < 1.0 / 30.0] = False
+        else:
+            out[r] = W.allow_mask(rng, vocab, frac=0.02)
+            kinds.append(kind)
+            continue
+        bits = np.zeros(words * 32, dtype=bool)
+        bits[:vocab] = allowed
+        out[r] = np.packbits(bits.reshape(words, 32), axis=1, bitorder="little").view(np.uint32).reshape(words)
+        kinds.append(kind)
+    return out, kinds
+
+
+@pytest.mark.parametrize("f32", [False, True])
+def test_rows_with_allow_masks_are_drawn_from_summaries(sampler, f32):
+    """An allow-mask on rows drawn from the summaries.  Tiles that the mask bars altogether drop
+    out, tiles allowed in part are evaluated id by id; the bound is a guess that the row checks
+    (k allowed values at or above it), and a row that fails the check, or has too many partly
+    allowed tiles to sum, is drawn by the launch that follows.  Whichever way a row goes, ids,
+    candidates, kept counts and log-probabilities are the oracle's on the stored logits; the
+    rows with a handful of barred ids, a barred run and no barred id are all served by the kernel
+    that reads summaries.  Then the same with bias lists and lowering penalties on top."""
+    rows, d, vocab = 15, 256, (151_936 if not f32 else 20_000 + 24)
+    rng = np.random.default_rng(131 + int(f32))
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=60, gain=9.0)
+    params_kw = [dict(temperature=0.7 + 0.05 * (r % 3), top_k=(64, 20, 5, 1 + r)[r % 4], top_p=(0.9, 1.0)[r % 2],
+                      min_p=0.01 * (r % 2), seed=300 + r) for r in range(rows)]
+    params = [ls_params(**kw) for kw in params_kw]
+    temps = [p.effective()[0] for p in params]
+    h, w = _bf16(hidden), _bf16(weight)
+    tiles = (vocab + TILE - 1) // TILE
+    logits = torch.zeros(rows, vocab, dtype=torch.float32 if f32 else torch.bfloat16, device=dev())
+    tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+    sampler.lm_head(h, w, temps, logits, tmax, tsum)
+    sampler.synchronize()
+    stored = logits.cpu().numpy() if f32 else _bits(logits.contiguous())
+    stored_f = stored if f32 else W.bf16_bits_to_f32(stored)
+    masks, kinds = _masks(rng, stored_f, vocab)
+    allow_t = torch.from_numpy(masks.view(np.int32)).to(dev())
+    steps = [9 + r for r in range(rows)]
+
+    def check(ids, lps, cand, counts, kws, which, hist=None, bias=None):
+        for i, r in enumerate(which):
+            kw = kws[r]
+            c = None if hist is None else hist[r]
+            dd = O.sample(stored[r], c, o_params(**kw), steps[r], allow=masks[r],
+                          bias=None if bias is None else bias[r], want_logprob=True)
+            n_fin = int(np.sum(dd.cand_adj > -np.inf))
+            assert counts[i, 0] == n_fin, (r, counts[i, 0], n_fin)
+            assert np.array_equal(cand[i, :n_fin], dd.cand_ids[:n_fin].astype(np.int64)), r
+            assert counts[i, 1] == dd.n_kept and ids[i] == dd.chosen, (r, ids[i], dd.chosen)
+            assert abs(lps[i] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (r, lps[i], dd.logprob)
+
+    def run(which, pp, kws, **extra):
+        sel = torch.tensor(which, device=dev())
+        lg, tm, ts = logits[sel].contiguous(), tmax[sel].contiguous(), tsum[sel].contiguous()
+        st = [steps[r] for r in which]
+        for key in ("scratch", "bias"):
+            if extra.get(key) is not None:
+                extra[key] = [extra[key][r] for r in which]
+        return _draw_all(
+            sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+                lg, tm, ts, [pp[r] for r in which], st, out, allow=allow_t[sel].contiguous(), out_logprobs=lp,
+                dbg_ids=di, dbg_counts=dc, **extra),
+            lg, [kws[r] for r in which], st)
+
+    everyone = list(range(rows))
+    check(*run(everyone, params, params_kw), params_kw, everyone)
+    light = [r for r in everyone if kinds[r] in (0, 1, 2)]
+    stats = torch.zeros(4, dtype=torch.int32, device=dev())
+    sampler.set_path_stats(stats)
+    res = run(light, params, params_kw)
+    sampler.set_path_stats(None)
+    check(*res, params_kw, light)
+    st = stats.cpu().numpy()
+    assert st[0] == len(light) and st[1] == 0 and st[2] == 0, st.tolist()
+    # bias lists and lowering penalties on top
+    bias = _bias_lists(rng, stored_f, vocab)
+    pen_kw = [dict(kw, repetition_penalty=1.1, presence_penalty=0.2, frequency_penalty=0.1) for kw in params_kw]
+    pen = [ls_params(**kw) for kw in pen_kw]
+    scratch, hist = [], []
+    for r in range(rows):
+        best = np.argsort(-stored_f[r])[:30].astype(np.int32)
+        hh = np.concatenate([rng.integers(0, vocab, 1500).astype(np.int32), np.repeat(best[:8], 3), best])
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(hh).to(dev()))
+        scratch.append(sc)
+        hist.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+    check(*run(everyone, pen, pen_kw, scratch=scratch, bias=bias), pen_kw, everyone, hist=hist, bias=bias)
+    for r in range(rows):
+        assert np.array_equal(scratch[r].read_counts().numpy().view(np.uint32), hist[r]), r
+        scratch[r].close()
+
+
 def test_a_batch_of_penalised_rows_through_the_fused_call(sampler):
     """1 024 rows under config 5's draw settings (k 64, top-p 0.9, T 0.8, penalties that only
     lower, a 2 048-id history that holds the row's best ids, a log-probability) through the one
