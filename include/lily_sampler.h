@@ -355,7 +355,8 @@ typedef struct lily_rows {
     const uint32_t* forced;              /* host [rows] or NULL; LILY_NO_TOKEN = draw */
     const float* uniforms;               /* host [rows] or NULL; NaN = uniform_for(seed, step) */
     uint32_t* out_ids_dev;               /* [rows] */
-    float* out_logprobs_dev;             /* [rows] or NULL */
+    float* out_logprobs_dev;             /* [rows] or NULL; a greedy row (exact argmax, no distribution
+                                            is formed) leaves its entry as it was */
     /* diagnostics, any may be NULL: the sorted top-k candidates before truncation */
     uint32_t* dbg_ids_dev;               /* [rows][LILY_SAMPLE_K_CAP] */
     float* dbg_probs_dev;                /* [rows][LILY_SAMPLE_K_CAP] exp(adjusted - top) */

@@ -1834,7 +1834,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
         return fail(LILY_ERR_INVALID_ARG, "tile_max and tile_sum are required");
     }
     if (reinterpret_cast<uintptr_t>(b->logits_dev) % 16u != 0 ||
-        b->row_stride % (b->dtype == LILY_BF16 ? 8u : 4u) != 0) {
+        (b->rows > 1 && b->row_stride % (b->dtype == LILY_BF16 ? 8u : 4u) != 0)) {
         return fail(LILY_ERR_INVALID_ARG, "rows of logits must start at multiples of 16 bytes");
     }
     const uint32_t rows = b->rows, tiles = lily_lm_head_tiles(b->vocab);

@@ -880,6 +880,22 @@ def test_batches_in_either_form(monkeypatch, form, rows, d, vocab, slack):
         s.close()
 
 
+def test_one_row_of_an_odd_vocabulary(sampler):
+    """A batch of one row has no second row whose start the stride would decide: 777 columns,
+    said as the stride too, are drawn from the summaries like any other row."""
+    rows, d, vocab = 1, 64, 777
+    rng = np.random.default_rng(3)
+    hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=20)
+    params_kw = [dict(temperature=0.8, top_k=20, top_p=0.9, seed=4)]
+    params = [ls_params(**kw) for kw in params_kw]
+    h, w, buf, logits, tmax, tsum = _produce(sampler, hidden, weight, [0.8], rows, vocab, stride=vocab)
+    ids, lps, cand, counts = _draw_all(
+        sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+            logits, tmax, tsum, params, [2], out, out_logprobs=lp, dbg_ids=di, dbg_counts=dc),
+        logits, params_kw, [2])
+    _check_draws(_bits(logits.contiguous()), ids, lps, cand, counts, params_kw, [2])
+
+
 def test_codes_ask_for_f32_logits(sampler):
     rng = np.random.default_rng(5)
     qw, _, _, _ = _quantised(rng, 256, 64, 8, 64)
