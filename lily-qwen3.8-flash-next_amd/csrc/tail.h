@@ -9,23 +9,48 @@ namespace lily {
 
 // ------------------------------------------------------------------ sort
 
-// The value lane ^ M holds, every lane of the wave at work.  Neighbours at distance 1 and 2
-// are inside a group of four lanes: a data-parallel move of each half; farther ones go through
-// the LDS crossbar, whose latency a sort of dependent exchanges waits out stage by stage.
+// The value lane ^ M holds, every lane of the wave at work - by moves inside the vector unit for
+// every M, never through the LDS crossbar, whose latency a sort of dependent exchanges would wait
+// out stage by stage.  1 and 2: a permutation inside each group of four lanes.  4: the lanes of
+// the even groups of four read four lanes up, those of the odd groups four lanes down (two moves,
+// each written to its groups only).  8: a rotation by eight within each row of 16.  16 and 32:
+// the swaps of whole rows and of the wave's halves (v_permlane16_swap / v_permlane32_swap with
+// the value as both operands leave one copy with rows 0 0 2 2 / the lower half twice and the
+// other with rows 1 1 3 3 / the upper half twice).
+template <uint32_t M>
+__device__ __forceinline__ uint32_t from_lane_xor32(uint32_t x) {
+    static_assert(M == 1u || M == 2u || M == 4u || M == 8u || M == 16u || M == 32u, "a power of two inside the wave");
+    const int v = (int)x;
+    if (M == 1u) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, v, 0xb1, 0xf, 0xf, true);   // quad_perm [1, 0, 3, 2]
+    }
+    if (M == 2u) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, v, 0x4e, 0xf, 0xf, true);   // quad_perm [2, 3, 0, 1]
+    }
+    if (M == 4u) {
+        const int up = __builtin_amdgcn_update_dpp(0, v, 0x104, 0xf, 0x5, false);    // row_shl:4 into groups 0 and 2
+        return (uint32_t)__builtin_amdgcn_update_dpp(up, v, 0x114, 0xf, 0xa, false); // row_shr:4 into groups 1 and 3
+    }
+    if (M == 8u) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);  // row_ror:8
+    }
+    const uint32_t lane = threadIdx.x & 63u;
+    if (M == 16u) {
+        const auto two = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+        return (lane & 16u) != 0u ? two[0] : two[1];
+    }
+    const auto two = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return (lane & 32u) != 0u ? two[0] : two[1];
+}
+
 template <uint32_t M>
 __device__ __forceinline__ uint64_t from_lane_xor(uint64_t v) {
-    if (M == 1u || M == 2u) {
-        constexpr int PERM = M == 1u ? 0xb1 : 0x4e;   // quad_perm [1, 0, 3, 2] / [2, 3, 0, 1]
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, PERM, 0xf, 0xf, true);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), PERM, 0xf, 0xf, true);
-        return ((uint64_t)hi << 32) | lo;
-    }
-    return shfl_xor_u64(v, (int)M);
+    return ((uint64_t)from_lane_xor32<M>((uint32_t)(v >> 32)) << 32) | from_lane_xor32<M>((uint32_t)v);
 }
 
 // Descending bitonic sort of cand[0..n), n <= 4 * NT, four entries per thread (entry
 // 4 * tid + r in register r; absent entries are 0, the smallest).  Exchanges at distance
-// 1 and 2 stay inside a thread, 4 .. 128 are lane shuffles inside a wave, and only the
+// 1 and 2 stay inside a thread, 4 .. 128 are moves between the lanes of a wave, and only the
 // three at distance 256 and 512 go through LDS with a barrier.
 __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
     static_assert(NT == 256, "four entries per thread cover 1024");
@@ -69,8 +94,9 @@ __device__ __forceinline__ void sort_desc_regs(uint64_t* cand, uint32_t n) {
                 const bool take_max = ((lane & m) == 0) == desc;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const uint64_t o = m == 1u ? from_lane_xor<1>(v[r])
-                                     : m == 2u ? from_lane_xor<2>(v[r]) : shfl_xor_u64(v[r], (int)m);
+                    const uint64_t o = m == 1u ? from_lane_xor<1>(v[r]) : m == 2u ? from_lane_xor<2>(v[r])
+                                     : m == 4u ? from_lane_xor<4>(v[r]) : m == 8u ? from_lane_xor<8>(v[r])
+                                     : m == 16u ? from_lane_xor<16>(v[r]) : from_lane_xor<32>(v[r]);
                     v[r] = ((o > v[r]) == take_max) ? o : v[r];
                 }
             } else if (stride == 2u) {
@@ -106,9 +132,13 @@ __device__ __forceinline__ void sort_desc(uint64_t* cand, uint32_t n) {
         if (threadIdx.x < 64) {
             const uint32_t lane = threadIdx.x;
             uint64_t c = lane < n ? cand[lane] : 0ull;
+#pragma unroll
             for (uint32_t size = 2; size <= 64; size <<= 1) {
+#pragma unroll
                 for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-                    const uint64_t o = shfl_xor_u64(c, (int)stride);
+                    const uint64_t o = stride == 1u ? from_lane_xor<1>(c) : stride == 2u ? from_lane_xor<2>(c)
+                                     : stride == 4u ? from_lane_xor<4>(c) : stride == 8u ? from_lane_xor<8>(c)
+                                     : stride == 16u ? from_lane_xor<16>(c) : from_lane_xor<32>(c);
                     const bool desc = (lane & size) == 0;
                     const bool lower = (lane & stride) == 0;
                     const bool take_max = lower == desc;
