@@ -69,10 +69,11 @@ hipError_t launch_head_summaries(hipStream_t stream, const void* logits, uint64_
                                  bool f32);
 // The draw of `rows` rows of cfg.table from the summaries ([.., tiles] each) and the few tiles of
 // the logits (bf16 or f32) that matter; tile_row[r] = the summaries' row of table row r; served[r] is set
-// for rows under penalties (1 = drawn, 0 = declined: the row is better read whole).
-hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg,
-                             const float* tile_max, const float* tile_sum, uint32_t tiles,
-                             const uint32_t* tile_row, uint32_t* served);
+// for rows under penalties or a mask (1 = drawn, 0 = declined: the row is better read whole).
+// `extra`: some row carries a bias list or a mask.
+hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, bool extra, uint32_t rows,
+                             const LaunchCfg& cfg, const float* tile_max, const float* tile_sum,
+                             uint32_t tiles, const uint32_t* tile_row, uint32_t* served);
 // Rows that draw among many candidates (k > 64), spread over cfg.slices workgroups a row: two
 // launches (the row's bound, then the values that reach it, merge, select, tail).
 // lane_max [rows][slices][256], bound [rows], count [rows][slices].

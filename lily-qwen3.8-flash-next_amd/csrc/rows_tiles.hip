@@ -40,7 +40,9 @@ constexpr uint32_t REF_CAP = 2048;                       // pieces evaluated ele
 //     over the whole row takes over.
 // `tile_row[r]` is the row of the summaries that belongs to row r of the table; `served[r]` is
 // written for rows under penalties or a mask: 1 = drawn here, 0 = left to the launch that follows.
-template <int DT, bool LSE>
+// EXTRA: rows with a bias list or a mask are among the launch's (the kernel without them keeps the
+// row's descriptor in fewer scalar registers, which the other spills).
+template <int DT, bool LSE, bool EXTRA>
 __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float* tile_max,
                                                       const float* tile_sum, uint32_t tiles,
                                                       const uint32_t* tile_row, uint32_t* served) {
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         }
         return;
     }
-    const uint32_t n_bias = min(a.n_bias, STREAM_BIAS_CAP);   // (the host serves no longer lists here)
+    const uint32_t n_bias = EXTRA ? min(a.n_bias, STREAM_BIAS_CAP) : 0u;   // (the host serves no longer lists here)
     if (n_bias != 0u) {
         if (tid < TILES_MAX / 32u) {
             bias_tiles[tid] = 0u;
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     }
     // The mask's four words of every tile: a tile with no allowed id drops out, one allowed in
     // part is marked (bit j of `partly`).
-    const bool masked = a.allow != nullptr;
+    const bool masked = EXTRA && a.allow != nullptr;
     const uint32_t words = (vocab + 31u) / 32u;
     uint32_t partly = 0;
     if (masked) {
@@ -244,8 +246,42 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         return;
     }
 
-    // (with a bias list: n_bias tiles more, whose largest values may be the biased ones)
-    // (under a mask: a guess at how many of the best tiles owe their summaries to barred ids)
+    // The sum's cut: tiles whose summary lies below it are summed as their summaries give them
+    // (their listed ids' raw terms stand for the true ones: each is below 2^-(log2 V + 21) of
+    // the row's largest term), tiles at or above it element by element.  It hangs from a lower
+    // bound of the row's largest TRUE value: the lowered largest summary (with a bias list or a
+    // mask the lowered k-th, which k tiles reach with values that carry no bias; under a mask
+    // that is a guess, which the row's check below - k candidates at or above it - confirms as
+    // a floor of the largest true value as well) or, better where a sequence keeps coming back
+    // to one token, the true value of the scratch's most-counted id.
+    float cut = -__builtin_huge_valf();
+    auto cut_below = [&](float floor_v) -> float {
+        const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
+        const bool heavy_allowed =
+            !masked || heavy >= vocab || ((gload(a.allow + (heavy >> 5)) >> (heavy & 31u)) & 1u) != 0u;
+        if (heavy < vocab && max_count != 0u && heavy_allowed) {
+            const float raw = load_logit<DT>(a.logits, heavy);
+            const float biased = with_bias(heavy, raw == raw ? raw : NEG_INF);
+            if (biased > NEG_INF) {
+                floor_v = fmaxf(floor_v, true_value(heavy, biased));
+            }
+        }
+        return floor_v - (log2f((float)vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
+    };
+    // A row without bias list and mask knows its cut from the largest summary alone: it forms
+    // it, and the summaries' part of its sum, before the search for the bound, whose barriers
+    // the loads behind the cut then wait out; the other rows need the bound first.
+    const bool cut_first = n_bias == 0u && !masked;
+    if (cut_first) {
+        if (want_lse && pen) {
+            cut = cut_below(lowered(top));
+        }
+        if (want_lse) {
+            add_summaries(cut);
+        }
+    }
+    // (with a bias list: n_bias tiles more, whose largest values may be the biased ones; under a
+    // mask: a guess at how many of the best tiles owe their summaries to barred ids)
     const uint32_t k = a.k, k_tiles = a.k + n_bias + (masked ? a.k / 2u + 8u : 0u);
     // with at least k summaries at or above x, at least k raw values are, and their true values
     // are at or above lowered(x)
@@ -275,31 +311,13 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
         // a short row leaves whole waves without a summary: the exact k-th largest instead
         kth = wg_kth_largest(ms, k_tiles, sh);
     }
-    // The sum's cut: tiles whose summary lies below it are summed as their summaries give them
-    // (their listed ids' raw terms stand for the true ones: each is below 2^-(log2 V + 21) of
-    // the row's largest term), tiles at or above it element by element.  It hangs from a lower
-    // bound of the row's largest TRUE value: the lowered largest summary (with a bias list the
-    // lowered k-th, which k tiles reach with values that carry no bias) or, better where a
-    // sequence keeps coming back to one token, the true value of the scratch's most-counted id.
-    float cut = -__builtin_huge_valf();
-    if (want_lse && pen) {
-        // (under a mask the lowered k-th summary is a guess; the row's check below - k candidates
-        // at or above it - confirms it as a floor of the largest true value as well)
-        float floor_v = lowered(n_bias != 0u || masked ? kth : top);
-        const uint32_t heavy = *(const LILY_CONST uint32_t*)(a.touched + words + 1u);
-        const bool heavy_allowed =
-            !masked || heavy >= vocab || ((gload(a.allow + (heavy >> 5)) >> (heavy & 31u)) & 1u) != 0u;
-        if (heavy < vocab && max_count != 0u && heavy_allowed) {
-            const float raw = load_logit<DT>(a.logits, heavy);
-            const float biased = with_bias(heavy, raw == raw ? raw : NEG_INF);
-            if (biased > NEG_INF) {
-                floor_v = fmaxf(floor_v, true_value(heavy, biased));
-            }
+    if (!cut_first) {
+        if (want_lse && pen) {
+            cut = cut_below(lowered(kth));
         }
-        cut = floor_v - (log2f((float)vocab) + 21.0f) * (a.temperature * 0.6931471805599453f);
-    }
-    if (want_lse) {
-        add_summaries(cut);
+        if (want_lse) {
+            add_summaries(cut);
+        }
     }
     const float bound = lowered(kth);
     const float reach = (want_lse && pen) ? fminf(bound, cut) : bound;   // tiles read
@@ -399,7 +417,7 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
             // (the word of the scratch's bitmap that covers the id; the summaries' first word
             // when there is no scratch to ask: the load stays unconditional)
             word[u] = gload((pen ? a.touched : reinterpret_cast<const uint32_t*>(tile_max)) + (pen ? (id >> 5) : 0u));
-            mword[u] = gload((masked ? a.allow : reinterpret_cast<const uint32_t*>(tile_max)) + (masked ? (id >> 5) : 0u));
+            mword[u] = masked ? gload(a.allow + (id >> 5)) : 0xffffffffu;   // (the same choice in every thread)
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -464,9 +482,9 @@ __global__ __launch_bounds__(NT, 4) void k_rows_tiles(LaunchCfg cfg, const float
     phase(cfg, 7);
 }
 
-hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, uint32_t rows, const LaunchCfg& cfg_in,
-                             const float* tile_max, const float* tile_sum, uint32_t tiles,
-                             const uint32_t* tile_row, uint32_t* served) {
+hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, bool extra, uint32_t rows,
+                             const LaunchCfg& cfg_in, const float* tile_max, const float* tile_sum,
+                             uint32_t tiles, const uint32_t* tile_row, uint32_t* served) {
     if (tiles == 0 || tiles > TILES_MAX) {
         return hipErrorInvalidValue;
     }
@@ -478,8 +496,15 @@ hipError_t launch_rows_tiles(hipStream_t stream, int dtype, bool lse, uint32_t r
     cfg.dyn_slots = (uint32_t)(dyn_bytes / 8);
     const dim3 grid(1, rows), block(NT);
 #define LILY_TILES(DT, LSE)                                                                       \
-    hipLaunchKernelGGL((k_rows_tiles<DT, LSE>), grid, block, dyn_bytes, stream, cfg, tile_max, tile_sum, \
-                       tiles, tile_row, served)
+    do {                                                                                          \
+        if (extra) {                                                                              \
+            hipLaunchKernelGGL((k_rows_tiles<DT, LSE, true>), grid, block, dyn_bytes, stream, cfg, tile_max,  \
+                               tile_sum, tiles, tile_row, served);                                \
+        } else {                                                                                  \
+            hipLaunchKernelGGL((k_rows_tiles<DT, LSE, false>), grid, block, dyn_bytes, stream, cfg, tile_max, \
+                               tile_sum, tiles, tile_row, served);                                \
+        }                                                                                         \
+    } while (0)
     if (dtype == LILY_BF16) {
         if (lse) {
             LILY_TILES(LILY_BF16, true);

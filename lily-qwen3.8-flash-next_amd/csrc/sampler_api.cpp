@@ -1869,7 +1869,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
     float* c2 = reinterpret_cast<float*>(stage + c2_off);
     uint32_t* served_flags = reinterpret_cast<uint32_t*>(stage + served_off);
     uint32_t certain = 0, maybe = 0;
-    bool lse = false;
+    bool lse = false, extra = false;
     uint32_t at = 0;
     // Summaries this sampler's lily_lm_head_bf16 produced at another temperature than the row's
     // (or at none) would give the row a wrong log-probability with the right token: such a row
@@ -1892,6 +1892,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
             }
             if (serve) {
                 lse = lse || row.out_logprob != nullptr;
+                extra = extra || row.n_bias != 0 || row.allow != nullptr;
                 tile_row[at] = r;
                 certain += group == 0 ? 1u : 0u;
                 maybe += group == 1 ? 1u : 0u;
@@ -1927,7 +1928,7 @@ int rows_with_tiles(lily_sampler* s, const lily_lm_head* h, const lily_rows* b, 
         LaunchCfg cfg;
         fill_cfg(s, &cfg, served, b->vocab, 1, 1, 0, s->table_dev);
         attach_trace(s, &cfg, served);
-        HIP_TRY(launch_rows_tiles(s->stream, (int)b->dtype, lse, served, cfg, tile_max, tile_sum, tiles,
+        HIP_TRY(launch_rows_tiles(s->stream, (int)b->dtype, lse, extra, served, cfg, tile_max, tile_sum, tiles,
                                   reinterpret_cast<const uint32_t*>(dev + idx_off), served_dev));
     }
     for (uint32_t q = 0; q < n_parts; ++q) {
