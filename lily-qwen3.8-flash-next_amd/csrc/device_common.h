@@ -475,25 +475,6 @@ struct HistRun {
     }
 };
 
-// A place in a list whose fill is *counter (an LDS word) for every lane with `has`, the lanes of
-// a wave in one addition: adds by 64 lanes to one LDS word are served one after the other.
-// Every lane of the wave calls it.
-__device__ __forceinline__ uint32_t wave_append(bool has, uint32_t* counter) {
-    const uint64_t mask = __ballot(has);
-    if (mask == 0ull) {
-        return 0u;
-    }
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t rank =
-        __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
-    const int leader = __builtin_ctzll(mask);
-    uint32_t base = 0;
-    if ((int)lane == leader) {
-        base = atomicAdd(counter, (uint32_t)__popcll(mask));
-    }
-    return (uint32_t)__shfl((int)base, leader) + rank;
-}
-
 // The top-k of cand[0..n) (zeros are invalid) compacted, unsorted, to the front;
 // returns how many there are.
 __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, uint32_t k, Shared& sh) {
@@ -573,22 +554,10 @@ __device__ __forceinline__ uint32_t wg_select_topk(uint64_t* cand, uint32_t n, u
         sh.n_cand = 0;
     }
     __syncthreads();
-    uint32_t kept = 0;
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-        kept += mine[j] != 0 && mine[j] >= floor_c ? 1u : 0u;
-    }
-    // one addition to the list's fill per wave: the lanes' counts are summed along the wave
-    const uint32_t upto = wave_scan_u32(kept);
-    uint32_t at = 0;
-    if ((tid & 63u) == 63u) {
-        at = atomicAdd(&sh.n_cand, upto);
-    }
-    at = (uint32_t)__builtin_amdgcn_readlane((int)at, 63) + upto - kept;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         if (mine[j] != 0 && mine[j] >= floor_c) {
-            cand[at++] = mine[j];
+            cand[atomicAdd(&sh.n_cand, 1u)] = mine[j];
         }
     }
     __syncthreads();

@@ -293,10 +293,8 @@ __device__ __forceinline__ void row_body(const LILY_CONST RowArgs* src, const La
             }
 #pragma unroll
             for (int q = 0; q < PER; ++q) {
-                const bool keep = mine[q] != 0ull && (uint32_t)(mine[q] >> 48) >= bound;
-                const uint32_t at = wave_append(keep, &sh.n_cand);
-                if (keep) {
-                    cand[at] = mine[q];
+                if (mine[q] != 0ull && (uint32_t)(mine[q] >> 48) >= bound) {
+                    cand[atomicAdd(&sh.n_cand, 1u)] = mine[q];
                 }
             }
             __syncthreads();
