@@ -354,13 +354,21 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         return pow2_d(d);
     };
 
-    // What a raw value is worth at least after penalties that can only lower (the penalty of an id
-    // with the scratch's largest count); the value itself for all other rows.
+    // What a raw value is worth at least after the row's penalties.  Those that can only lower:
+    // the penalty of an id with the scratch's largest count.  Any others: a listed id's value is
+    // linear in its count, so the least of the raw value (the id may not be listed) and its
+    // penalised images at a count of 1 and at the largest count - a frequency term that lowers
+    // can outweigh a presence term that raises.  Monotone in the raw value either way, so the
+    // image of the largest raw value bounds the largest true value from below.
     auto lowered = [&](float m) -> float {
-        if (pen && lowering && m > NEG_INF) {
-            float t = m > 0.0f ? m / a.repetition : m * a.repetition;
-            t -= a.presence + a.frequency * (float)max_count;
-            return t;
+        if (pen && m > NEG_INF) {
+            const float scaled = m > 0.0f ? m / a.repetition : m * a.repetition;
+            const float most = scaled - (a.presence + a.frequency * (float)max_count);
+            if (lowering) {
+                return most;
+            }
+            const float once = scaled - (a.presence + a.frequency);
+            return fminf(m, fminf(once, most));
         }
         return m;
     };
@@ -401,7 +409,7 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // largest raw value bounds the largest true value from below.  (Barred ids are -inf
             // before any maximum is taken; bias ids are few and only the sum's cut depends on
             // this bound, so a positive bias on the row's best id merely cuts less.)  Listed
-            // ids that may rise leave the raw maximum as it is.
+            // ids whose penalties may go either way: the least of what they can make of it.
             row_max = fmaxf(lowered(m), row_floor);
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
@@ -1178,7 +1186,12 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
                 cm = chunk_max<DT>(q);   // a NaN in the chunk: as its owner did
             }
             const float cut = L.blk_cut[b];
-            const bool queued = cm >= L.blk_bound[b];
+            bool queued = cm >= L.blk_bound[b];
+            if (LSE && want_lse && pen && !lowering) {
+                // (a row with a sum whose listed ids may rise queued every chunk that holds a
+                // listed id, whatever its values: none of that chunk's raw terms was summed)
+                queued = queued || (bits32_at(a.touched, row_words, (int64_t)g.id_of(c, 0)) & EMASK) != 0u;
+            }
             const bool summed = !queued && cm > cut;
             const float raw = elem_of(q, (id + g.pad) % E);
             const float t = true_value(id, raw);

@@ -126,6 +126,66 @@ def test_masks_bias_penalties_together(sampler):
         sc.close()
 
 
+def _logprobs_against_oracle(sampler, x, kw, hist, bias=None, step=3):
+    rows, vocab = x.shape
+    scratch, counts = [], []
+    for r in range(rows):
+        sc = LS.SamplerScratch(sampler, vocab)
+        sc.add_history(torch.from_numpy(hist[r]).to(dev()))
+        scratch.append(sc)
+        counts.append(np.bincount(hist[r], minlength=vocab).astype(np.uint32))
+    r = run_rows(sampler, x, kw, [step] * rows, scratch=scratch, bias=bias, logprobs=True)
+    for i in range(rows):
+        d = O.sample(x[i], counts[i], o_params(**kw[i]), step, bias=None if bias is None else bias[i],
+                     want_logprob=True)
+        check_row_against_oracle(r, i, d)
+        assert abs(r.logprobs[i] - d.logprob) <= 1e-5 * max(1.0, abs(d.logprob)), (i, r.logprobs[i], d.logprob)
+    for sc in scratch:
+        sc.close()
+
+
+def test_logprob_under_penalties_of_both_signs(sampler):
+    """Penalties that raise by one term and lower by another (presence < 0 with frequency > 0,
+    repetition on either side of 1) over a history that names every id of a short row some fifty
+    times: the frequency term takes 5 off every value, so the largest raw value says little about
+    the largest true one, which the cut of the row's sum hangs from - it must hang from what the
+    penalties can make of that value at the least."""
+    rng = np.random.default_rng(216)
+    rows, vocab = 9, 97
+    x = np.sort(rng.normal(0, 3, (rows, vocab)), axis=1).astype(np.float32)
+    x[1::2] = rng.normal(0, 3, (rows // 2, vocab)).astype(np.float32)
+    hist = rng.integers(0, vocab, (rows, 5000)).astype(np.int32)
+    kw = [dict(temperature=(0.5, 1.0, 1.7)[r % 3], top_k=(64, 7, 20)[r % 3], top_p=(1.0, 0.9)[r % 2], min_p=0.02,
+               seed=1000 + r, repetition_penalty=(1.2, 0.8)[r % 2], presence_penalty=-0.5, frequency_penalty=0.1)
+          for r in range(rows)]
+    _logprobs_against_oracle(sampler, x, kw, hist)
+    xb = W.to_bf16_bits(x)
+    _logprobs_against_oracle(sampler, xb, kw, hist)
+
+
+def test_logprob_with_a_bias_list_under_penalties_that_may_raise(sampler):
+    """A flat row half of whose ids are named by the history, penalties that raise them above
+    all others, and a bias list: the chunks that hold a named id are evaluated value by value,
+    and the id of the bias list, which is dealt with apart, must not have a raw term taken off
+    the row's sum that was never put there - one term in a thousand, 1.7e-3 of the
+    log-probability."""
+    rng = np.random.default_rng(78)
+    rows, vocab = 24, 1000
+    x = rng.normal(0, 0.02, (rows, vocab)).astype(np.float32)
+    hist = rng.integers(0, vocab, (rows, 500)).astype(np.int32)
+    bias = [[(int(rng.integers(0, vocab)), float(rng.choice([-5.0, 3.0, 0.25])))] for _ in range(rows)]
+    bias[3] = bias[3] + [(int(hist[3][0]), 0.5), (int(hist[3][1]), -0.5)]   # named by both lists
+    kw = [dict(temperature=(1.0, 0.5, 1.7)[r % 3], top_k=(64, 20, 7, 1 + r)[r % 4], top_p=(1.0, 0.9)[r % 2],
+               min_p=0.0, seed=2000 + r, repetition_penalty=0.8, presence_penalty=-0.5, frequency_penalty=0.1)
+          for r in range(rows)]
+    _logprobs_against_oracle(sampler, x, kw, hist, bias=bias)
+    big = rng.normal(0, 0.02, (5, 70_001)).astype(np.float32)
+    hist5 = rng.integers(0, 70_001, (5, 5000)).astype(np.int32)
+    bias5 = [[(int(i), float(d)) for i, d in zip(rng.integers(0, 70_001, 8), rng.choice([-5.0, 3.0, 20.0], 8))]
+             for _ in range(5)]
+    _logprobs_against_oracle(sampler, big, [dict(kw[r], top_k=(20, 64)[r % 2]) for r in range(5)], hist5, bias=bias5)
+
+
 def test_unaligned_rows_of_a_matrix(sampler):
     """Rows of a [rows, V] matrix with odd V start at every 16-byte phase."""
     rng = np.random.default_rng(12)
