@@ -354,21 +354,14 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
         return pow2_d(d);
     };
 
-    // What a raw value is worth at least after the row's penalties.  Those that can only lower:
-    // the penalty of an id with the scratch's largest count.  Any others: a listed id's value is
-    // linear in its count, so the least of the raw value (the id may not be listed) and its
-    // penalised images at a count of 1 and at the largest count - a frequency term that lowers
-    // can outweigh a presence term that raises.  Monotone in the raw value either way, so the
-    // image of the largest raw value bounds the largest true value from below.
+    // What a raw value is worth at least after penalties that can only lower (the penalty of an id
+    // with the scratch's largest count); the value itself for all other rows, whose floor
+    // refresh_bound forms apart.
     auto lowered = [&](float m) -> float {
-        if (pen && m > NEG_INF) {
-            const float scaled = m > 0.0f ? m / a.repetition : m * a.repetition;
-            const float most = scaled - (a.presence + a.frequency * (float)max_count);
-            if (lowering) {
-                return most;
-            }
-            const float once = scaled - (a.presence + a.frequency);
-            return fminf(m, fminf(once, most));
+        if (pen && lowering && m > NEG_INF) {
+            float t = m > 0.0f ? m / a.repetition : m * a.repetition;
+            t -= a.presence + a.frequency * (float)max_count;
+            return t;
         }
         return m;
     };
@@ -408,9 +401,20 @@ __device__ __forceinline__ bool select_stream(const RowArgs& a, const Geo<DT>& g
             // id with the scratch's largest count, and that map is monotone, so the image of the
             // largest raw value bounds the largest true value from below.  (Barred ids are -inf
             // before any maximum is taken; bias ids are few and only the sum's cut depends on
-            // this bound, so a positive bias on the row's best id merely cuts less.)  Listed
-            // ids whose penalties may go either way: the least of what they can make of it.
+            // this bound, so a positive bias on the row's best id merely cuts less.)
             row_max = fmaxf(lowered(m), row_floor);
+            if (pen && !lowering && m > NEG_INF) {
+                // Penalties of either sign: a listed id's value is linear in its count, so what
+                // they leave of the largest raw value at the least is the least of the value
+                // itself (its id may not be listed) and its images at a count of 1 and at the
+                // scratch's largest count - a frequency term that lowers can outweigh a presence
+                // term that raises.  Monotone in the raw value, so this bounds the largest true
+                // value from below.
+                const float scaled = m > 0.0f ? m / a.repetition : m * a.repetition;
+                const float off = a.presence + a.frequency * fmaxf(1.0f, (float)max_count);
+                const float off1 = a.presence + a.frequency;
+                row_max = fminf(m, scaled - fmaxf(off, off1));
+            }
             if (first) {
                 // Finite and far from overflow: every term is formed as 2^(v*c2 - ref_s).
                 ref_s = m > NEG_INF ? fminf(fmaxf(m * c2, -1.0e30f), 1.0e30f) : 0.0f;
