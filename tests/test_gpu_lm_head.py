@@ -880,6 +880,105 @@ def test_batches_in_either_form(monkeypatch, form, rows, d, vocab, slack):
         s.close()
 
 
+@pytest.mark.parametrize("block", range(4))
+def test_random_rows_from_summaries(sampler, block):
+    """Seeded random batches through lily_sample_rows_tiled: bf16 or f32 logits of heads with few
+    or many peaks, 1 to 23 rows, vocabularies of 777 to 151 936, any k and temperature, lowering
+    penalties over histories that may hold the rows' best ids, bias lists of 0 to 64 pairs with
+    deltas from -inf to +60, and six kinds of allow-mask (a few of the best ids barred, a run
+    around one of the best tiles, ids barred at random with any density, a sparse set, the best
+    ids barred by the dozen, none).  Whatever way each row goes - the summaries, a decline on the
+    device, the kernels that read the row - ids, candidates, kept counts, counts of the scratch
+    and log-probabilities are the oracle's on the stored logits."""
+    for trial in range(block * 10, block * 10 + 10):
+        rng = np.random.default_rng(990_000 + trial)
+        f32 = bool(rng.integers(0, 2))
+        rows, d = int(rng.integers(1, 24)), int(rng.choice([64, 128, 256]))
+        vocab = int(rng.choice([777, 5000, 20000 + int(rng.integers(0, 130)), 151936]))
+        hidden, weight = _peaked_head(rng, rows, d, vocab, peaks=min(int(rng.choice([5, 40, 200])), vocab // 8),
+                                      gain=float(rng.choice([3.0, 6.0, 9.0, 14.0])))
+        kws = []
+        for r in range(rows):
+            kw = dict(temperature=float(rng.choice([0.3, 0.7, 1.0, 1.5])),
+                      top_k=int(rng.choice([1, 2, 5, 20, 64, 64, 100])), top_p=float(rng.choice([1.0, 0.9, 0.5])),
+                      min_p=float(rng.choice([0.0, 0.0, 0.05])), seed=int(rng.integers(0, 1 << 30)))
+            if rng.random() < 0.5:
+                kw.update(repetition_penalty=float(rng.choice([1.0, 1.1, 1.3])),
+                          presence_penalty=float(rng.choice([0.0, 0.2])),
+                          frequency_penalty=float(rng.choice([0.0, 0.1])))
+            kws.append(dict() if rng.random() < 0.1 else kw)
+        params = [ls_params(**kw) for kw in kws]
+        temps = [p.effective()[0] for p in params]
+        h, w = _bf16(hidden), _bf16(weight)
+        tiles = (vocab + TILE - 1) // TILE
+        stride = ((vocab + 7) // 8) * 8
+        buf = torch.zeros(rows, stride, dtype=torch.float32 if f32 else torch.bfloat16, device=dev())
+        logits = buf[:, :vocab]
+        tmax = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+        tsum = torch.zeros(rows, tiles, dtype=torch.float32, device=dev())
+        sampler.lm_head(h, w, temps, logits, tmax, tsum)
+        sampler.synchronize()
+        stored = logits.contiguous().cpu().numpy() if f32 else _bits(logits.contiguous())
+        stored_f = stored if f32 else W.bf16_bits_to_f32(stored)
+        words = (vocab + 31) // 32
+        masks = np.zeros((rows, words), dtype=np.uint32)
+        use_mask = rng.random() < 0.6
+        bias, scratch, hist = [], [], []
+        for r in range(rows):
+            order = np.argsort(-stored_f[r])
+            allowed = np.ones(vocab, dtype=bool)
+            kind = int(rng.integers(0, 6))
+            if kind == 0:
+                allowed[order[rng.choice(min(30, vocab), 6, replace=False)]] = False
+            elif kind == 1:
+                t = int(order[int(rng.integers(0, 3))]) // TILE
+                allowed[max(0, t * TILE - int(rng.integers(0, 200))):min(vocab, (t + 1) * TILE + int(rng.integers(0, 200)))] = False
+            elif kind == 2:
+                allowed[rng.random(vocab) < rng.choice([0.001, 0.03, 0.5])] = False
+            elif kind == 3:
+                allowed[:] = False
+                allowed[order[rng.choice(min(200, vocab), int(rng.integers(1, 100)), replace=False)]] = True
+            elif kind == 4:
+                allowed[order[:int(rng.integers(1, 80))]] = False
+            bits = np.zeros(words * 32, dtype=bool)
+            bits[:vocab] = allowed
+            masks[r] = np.packbits(bits.reshape(words, 32), axis=1, bitorder="little").view(np.uint32).reshape(words)
+            nb = int(rng.choice([0, 0, 1, 5, 40, 64]))
+            ids = np.concatenate([order[rng.integers(0, min(100, vocab), nb // 2)], rng.integers(0, vocab, nb - nb // 2)])
+            deltas = rng.choice([-100.0, -5.0, -0.5, 0.25, 3.0, 20.0, 60.0, float("-inf")], nb)
+            bias.append([(int(i), float(dl)) for i, dl in zip(ids, deltas)])
+            best = order[:20].astype(np.int32)
+            hh = np.concatenate([rng.integers(0, vocab, int(rng.integers(0, 2000))).astype(np.int32),
+                                 np.repeat(best[:5], int(rng.integers(0, 4))), best[:int(rng.integers(0, 20))]])
+            sc = LS.SamplerScratch(sampler, vocab)
+            if len(hh):
+                sc.add_history(torch.from_numpy(hh).to(dev()))
+            scratch.append(sc)
+            hist.append(np.bincount(hh, minlength=vocab).astype(np.uint32))
+        steps = [int(rng.integers(0, 1000)) for _ in range(rows)]
+        allow_t = torch.from_numpy(masks.view(np.int32)).to(dev()) if use_mask else None
+        ids, lps, cand, counts = _draw_all(
+            sampler, lambda out, lp, di, dc: sampler.sample_rows_tiled(
+                logits, tmax, tsum, params, steps, out, scratch=scratch, bias=bias, allow=allow_t, out_logprobs=lp,
+                dbg_ids=di, dbg_counts=dc),
+            logits, kws, steps)
+        for r, kw in enumerate(kws):
+            p = o_params(**kw)
+            dd = O.sample(stored[r], hist[r], p, steps[r], allow=masks[r] if use_mask else None, bias=bias[r],
+                          want_logprob=True)
+            assert ids[r] == dd.chosen, (trial, r)
+            if p.temperature == 0.0 or kw.get("top_k") == 1:
+                continue   # (a greedy row reports its token only)
+            n_fin = int(np.sum(dd.cand_adj > -np.inf))
+            assert counts[r, 0] == n_fin and counts[r, 1] == dd.n_kept, (trial, r)
+            assert np.array_equal(cand[r, :n_fin], dd.cand_ids[:n_fin].astype(np.int64)), (trial, r)
+            if np.isfinite(dd.logprob):
+                assert abs(lps[r] - dd.logprob) <= LOGPROB_RTOL * max(1.0, abs(dd.logprob)), (trial, r, lps[r], dd.logprob)
+        for r in range(rows):
+            assert np.array_equal(scratch[r].read_counts().numpy().view(np.uint32), hist[r]), (trial, r)
+            scratch[r].close()
+
+
 def test_one_row_of_an_odd_vocabulary(sampler):
     """A batch of one row has no second row whose start the stride would decide: 777 columns,
     said as the stride too, are drawn from the summaries like any other row."""
